@@ -1,0 +1,142 @@
+"""ctypes binding of libprimus_turbo_amd.so (the C-ABI library with the gfx950 kernels).
+
+The library is the only compute backend: there is no CPU or eager fallback. If it
+has not been built, every op raises ``RuntimeError`` naming the build command.
+``import torch`` happens first so that the library binds to the HIP runtime that
+PyTorch already loaded (one HIP runtime per process).
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from pathlib import Path
+from typing import Optional
+
+import torch
+
+_PKG_ROOT = Path(__file__).resolve().parent.parent  # .../primus-turbo_amd
+LIB_PATH = Path(os.environ.get("PRIMUS_TURBO_AMD_LIB", _PKG_ROOT / "lib" / "libprimus_turbo_amd.so"))
+
+# element type codes of include/primus_turbo_amd.h
+DT_BF16, DT_F16, DT_F32, DT_E4M3, DT_E5M2, DT_E2M1X2, DT_E8M0 = range(7)
+
+_DTYPE_CODE = {
+    torch.bfloat16: DT_BF16,
+    torch.float16: DT_F16,
+    torch.float32: DT_F32,
+    torch.float8_e4m3fn: DT_E4M3,
+    torch.float8_e5m2: DT_E5M2,
+}
+if hasattr(torch, "float4_e2m1fn_x2"):
+    _DTYPE_CODE[torch.float4_e2m1fn_x2] = DT_E2M1X2
+if hasattr(torch, "float8_e8m0fnu"):
+    _DTYPE_CODE[torch.float8_e8m0fnu] = DT_E8M0
+
+_lib: Optional[ctypes.CDLL] = None
+_lock = threading.Lock()
+
+c_void_p, c_int, c_i64, c_size_t, c_float = (
+    ctypes.c_void_p,
+    ctypes.c_int,
+    ctypes.c_int64,
+    ctypes.c_size_t,
+    ctypes.c_float,
+)
+
+# name -> (restype, argtypes); must match include/primus_turbo_amd.h
+_SIGNATURES = {
+    "pt_last_error": (ctypes.c_char_p, []),
+    "pt_abi_version": (c_int, []),
+    "pt_device_cu_count": (c_int, []),
+    "pt_quantize_fp8_tensorwise_workspace_bytes": (c_size_t, []),
+    "pt_quantize_fp8_tensorwise": (
+        c_int,
+        [c_void_p, c_int, c_i64, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
+    ),
+    "pt_dequantize_fp8_tensorwise": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p, c_int, c_void_p]),
+    "pt_quantize_fp8_rowwise": (
+        c_int,
+        [c_void_p, c_int, c_i64, c_i64, c_i64, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
+    ),
+    "pt_dequantize_fp8_rowwise": (
+        c_int,
+        [c_void_p, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_int, c_void_p],
+    ),
+}
+
+
+def exported_symbols():
+    """Names every build of the library must export (used by the load test)."""
+    return sorted(_SIGNATURES)
+
+
+def lib() -> ctypes.CDLL:
+    """Load (once) and return the native library; raise loudly if it is missing."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not LIB_PATH.exists():
+            raise RuntimeError(
+                f"primus_turbo: native library {LIB_PATH} is missing. Build it with "
+                f"`python {_PKG_ROOT / 'build_native.py'}` (hipcc, --offload-arch=gfx950). "
+                "There is no CPU fallback."
+            )
+        handle = ctypes.CDLL(str(LIB_PATH))
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(handle, name)  # AttributeError if the build is stale
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise RuntimeError(f"primus_turbo: dtype {dtype} is not supported by the gfx950 kernels") from None
+
+
+def check(status: int) -> None:
+    if status != 0:
+        msg = lib().pt_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"primus_turbo native error {status}: {msg}")
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def stream_of(t: torch.Tensor) -> int:
+    """Raw hipStream_t of torch's current stream on ``t``'s device."""
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def require_cuda(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "primus_turbo: tensors must live on a ROCm GPU (the kernels are gfx950 HIP; there is no CPU path)"
+            )
+
+
+# ---------------------------------------------------------------------------
+# Small persistent device workspaces (zero-filled once, left zeroed by the kernels).
+# One per (device, stream) so launches on different streams never share one.
+# ---------------------------------------------------------------------------
+_workspaces: dict = {}
+
+
+def zeroed_workspace(device: torch.device, nbytes: int, tag: str) -> torch.Tensor:
+    stream = torch.cuda.current_stream(device)
+    key = (tag, device.index if device.index is not None else torch.cuda.current_device(), stream.cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws

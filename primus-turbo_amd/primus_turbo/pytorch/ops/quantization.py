@@ -1,0 +1,230 @@
+"""Public quantize / dequantize entry points (reference: primus_turbo/pytorch/ops/quantization.py).
+
+Same names, argument meaning and error behaviour as the reference ops; each call lands in
+one gfx950 HIP kernel family through the impl layer.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from primus_turbo.pytorch.core.low_precision import (
+    MXFP4_BLOCK_SIZE,
+    MXFP8_BLOCK_SIZE,
+    ScalingGranularity,
+    ScalingRecipe,
+)
+from primus_turbo.pytorch.kernels.quantization import quantization_impl as _impl
+
+__all__ = [
+    "quantize_fp8",
+    "quantize_fp8_with_trans",
+    "dequantize_fp8",
+    "quantize_fp4",
+    "quantize_fp4_with_trans",
+    "dequantize_fp4",
+    "grouped_quantize_fp8",
+    "grouped_quantize_fp8_with_trans",
+    "grouped_dequantize_fp8",
+    "grouped_quantize_fp4",
+    "grouped_dequantize_fp4",
+]
+
+_G = ScalingGranularity
+
+
+def _unknown(granularity):
+    return NotImplementedError(f"Unknown granularity {granularity}")
+
+
+def _need_mx_block(block_size, expect, what):
+    assert block_size == expect, f"The block size must be {expect} for {what} quantization"
+
+
+def quantize_fp8(
+    x: torch.Tensor,
+    out_dtype: torch.dtype,
+    granularity: ScalingGranularity,
+    *,
+    block_size: Optional[int] = None,
+    axis: Optional[int] = None,
+    scaling_recipe: Optional[ScalingRecipe] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Quantize ``x`` to FP8; returns ``(x_fp8, scale_inv)``.
+
+    ROWWISE needs ``axis``; BLOCKWISE needs ``block_size`` and either ``axis`` (1-D blocks)
+    or ``scaling_recipe.use_2d_block`` (one scale per square tile, for weights);
+    MX_BLOCKWISE needs a 2-D/3-D ``x``, ``block_size == 32`` and ``axis`` as the direction.
+    """
+    if granularity == _G.TENSORWISE:
+        return _impl.quantize_fp8_tensorwise_impl(x, out_dtype)
+    if granularity == _G.ROWWISE:
+        return _impl.quantize_fp8_rowwise_impl(x, out_dtype, axis)
+    if granularity == _G.BLOCKWISE:
+        assert block_size is not None, "block_size must be specified for BLOCKWISE quantization"
+        if scaling_recipe is not None and scaling_recipe.use_2d_block:
+            return _impl.quant_fp8_blockwise_for_weight_impl(x, out_dtype, block_size=block_size)
+        assert axis is not None, "axis must be specified for 1D BLOCKWISE quantization"
+        return _impl.quant_fp8_blockwise_impl(x, out_dtype, axis=axis, block_size=block_size)
+    if granularity == _G.MX_BLOCKWISE:
+        _need_mx_block(block_size, MXFP8_BLOCK_SIZE, "MXFP8")
+        return _impl.quantize_mxfp8_impl(x, out_dtype, axis, block_size, False, scaling_recipe)
+    raise _unknown(granularity)
+
+
+def quantize_fp8_with_trans(
+    x: torch.Tensor,
+    out_dtype: torch.dtype,
+    granularity: ScalingGranularity,
+    *,
+    block_size: Optional[int] = None,
+    scaling_recipe: Optional[ScalingRecipe] = None,
+    scaling_recipe_for_trans: Optional[ScalingRecipe] = None,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Quantize along both directions from one read of ``x``.
+
+    Returns ``(x_rowwise, scale_inv_rowwise, x_colwise, scale_inv_colwise)``.
+    """
+    if granularity == _G.MX_BLOCKWISE:
+        _need_mx_block(block_size, MXFP8_BLOCK_SIZE, "MXFP8")
+        return _impl.quantize_mxfp8_impl(
+            x, out_dtype, None, block_size, True, scaling_recipe, scaling_recipe_for_trans
+        )
+    if granularity == _G.BLOCKWISE:
+        return _impl.quant_fp8_blockwise_dual_impl(x, out_dtype, block_size=block_size)
+    raise _unknown(granularity)
+
+
+def dequantize_fp8(
+    x: torch.Tensor,
+    out_dtype: torch.dtype,
+    granularity: ScalingGranularity,
+    *,
+    block_size: Optional[int] = None,
+    axis: Optional[int] = None,
+    scale_inv: torch.Tensor,
+    scaling_recipe: Optional[ScalingRecipe] = None,
+):
+    """Inverse of :func:`quantize_fp8` for the same granularity / axis / recipe."""
+    if granularity == _G.TENSORWISE:
+        return _impl.dequantize_fp8_tensorwise_impl(x, out_dtype, scale_inv)
+    if granularity == _G.ROWWISE:
+        if axis is None:
+            raise ValueError("axis must be specified for rowwise FP8 de-quantization")
+        return _impl.dequantize_fp8_rowwise_impl(x, out_dtype, axis, scale_inv)
+    if granularity == _G.BLOCKWISE:
+        assert block_size is not None, "block_size must be specified for BLOCKWISE de-quantization"
+        if scaling_recipe is not None and scaling_recipe.use_2d_block:
+            return _impl.dequant_fp8_blockwise_for_weight_impl(x, scale_inv, out_dtype, block_size)
+        assert axis is not None, "axis must be specified for 1D BLOCKWISE de-quantization"
+        return _impl.dequant_fp8_blockwise_impl(x, scale_inv, out_dtype, axis, block_size)
+    if granularity == _G.MX_BLOCKWISE:
+        _need_mx_block(block_size, MXFP8_BLOCK_SIZE, "MXFP8")
+        return _impl.dequantize_mxfp8_impl(x, out_dtype, axis, block_size, scale_inv)
+    raise _unknown(granularity)
+
+
+def quantize_fp4(
+    x: torch.Tensor,
+    out_dtype: torch.dtype,
+    granularity: ScalingGranularity,
+    *,
+    block_size: Optional[int] = None,
+    axis: Optional[int] = None,
+    scaling_recipe: Optional[ScalingRecipe] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """MXFP4 quantize in one direction (2-D: axis 1 = along rows, axis 0 = transposed output)."""
+    if granularity == _G.MX_BLOCKWISE:
+        _need_mx_block(block_size, MXFP4_BLOCK_SIZE, "MXFP4")
+        assert axis is not None, "axis must be specified for MXFP4 quantization"
+        return _impl.quantize_mxfp4_impl(
+            x, out_dtype, axis, block_size, with_trans=False, scaling_recipe=scaling_recipe
+        )
+    raise _unknown(granularity)
+
+
+def quantize_fp4_with_trans(
+    x: torch.Tensor,
+    out_dtype: torch.dtype,
+    granularity: ScalingGranularity,
+    *,
+    block_size: Optional[int] = None,
+    axis: Optional[int] = None,
+    scaling_recipe: Optional[ScalingRecipe] = None,
+    scaling_recipe_for_trans: Optional[ScalingRecipe] = None,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """MXFP4 quantize in both directions from one read of ``x``."""
+    if granularity == _G.MX_BLOCKWISE:
+        _need_mx_block(block_size, MXFP4_BLOCK_SIZE, "MXFP4")
+        return _impl.quantize_mxfp4_impl(
+            x,
+            out_dtype,
+            axis,
+            block_size,
+            with_trans=True,
+            scaling_recipe=scaling_recipe,
+            scaling_recipe_for_trans=scaling_recipe_for_trans,
+        )
+    raise _unknown(granularity)
+
+
+def dequantize_fp4(
+    x: torch.Tensor,
+    out_dtype: torch.dtype,
+    granularity: ScalingGranularity,
+    *,
+    block_size: Optional[int] = None,
+    axis: Optional[int] = None,
+    scale_inv: torch.Tensor,
+    scaling_recipe: Optional[ScalingRecipe] = None,
+) -> torch.Tensor:
+    if granularity == _G.MX_BLOCKWISE:
+        _need_mx_block(block_size, MXFP4_BLOCK_SIZE, "MXFP4")
+        return _impl.dequantize_mxfp4_impl(x, out_dtype, axis, block_size, scale_inv)
+    raise _unknown(granularity)
+
+
+# --- grouped MX quantizers: not part of this build's hot path ---------------------------
+def _grouped_mx_not_built(name):
+    raise NotImplementedError(
+        f"{name}: the grouped MX quantizers (per-group padded MXFP8/MXFP4 layouts) are not built; "
+        "the grouped path of this library is the FP8 128-blockwise one (grouped_gemm_fp8 with BLOCKWISE)."
+    )
+
+
+def grouped_quantize_fp8(x, out_dtype, granularity, group_lens, group_offs, *, block_size=None, axis=None,
+                         scaling_recipe=None):
+    if granularity == _G.MX_BLOCKWISE:
+        _grouped_mx_not_built("grouped_quantize_fp8")
+    raise _unknown(granularity)
+
+
+def grouped_quantize_fp8_with_trans(x, out_dtype, granularity, group_lens, group_offs, *, block_size=None,
+                                    scaling_recipe=None, scaling_recipe_for_trans=None):
+    if granularity == _G.MX_BLOCKWISE:
+        _grouped_mx_not_built("grouped_quantize_fp8_with_trans")
+    raise _unknown(granularity)
+
+
+def grouped_dequantize_fp8(x, out_dtype, granularity, group_offs, group_offs_padded, *, block_size=None, axis=None,
+                           scale_inv=None, scaling_recipe=None, total_M=None):
+    if granularity == _G.MX_BLOCKWISE:
+        _grouped_mx_not_built("grouped_dequantize_fp8")
+    raise _unknown(granularity)
+
+
+def grouped_quantize_fp4(x, out_dtype, granularity, group_lens, group_offs, *, block_size=None, axis=None,
+                         scaling_recipe=None):
+    if granularity == _G.MX_BLOCKWISE:
+        _grouped_mx_not_built("grouped_quantize_fp4")
+    raise _unknown(granularity)
+
+
+def grouped_dequantize_fp4(x, out_dtype, granularity, *, block_size=None, axis=None, scale_inv=None,
+                           scaling_recipe=None):
+    if granularity == _G.MX_BLOCKWISE:
+        _need_mx_block(block_size, MXFP4_BLOCK_SIZE, "MXFP4")
+        return _impl.dequantize_mxfp4_impl(x, out_dtype, axis, block_size, scale_inv)
+    raise _unknown(granularity)

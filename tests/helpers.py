@@ -1,0 +1,42 @@
+"""Shared helpers for the parity tests (seeded inputs, torch <-> numpy views)."""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+
+def bf16_randn(shape, seed, scale=1.0, outlier_frac=0.0, outlier_mul=100.0, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(shape, generator=g, dtype=torch.float32) * scale
+    if outlier_frac > 0:
+        g2 = torch.Generator().manual_seed(seed + 1)
+        n = max(1, int(x.numel() * outlier_frac))
+        idx = torch.randperm(x.numel(), generator=g2)[:n]
+        x.view(-1)[idx] *= outlier_mul
+    return x.to(dtype)
+
+
+def to_f32_np(t: torch.Tensor) -> np.ndarray:
+    return t.detach().cpu().to(torch.float32).numpy()
+
+
+def codes_np(t: torch.Tensor) -> np.ndarray:
+    """uint8 view of an fp8 / fp4x2 / e8m0 tensor."""
+    return t.detach().cpu().contiguous().view(torch.uint8).numpy()
+
+
+def bits_np(t: torch.Tensor) -> np.ndarray:
+    """Bit pattern of a float32 / bf16 / fp16 tensor as unsigned ints."""
+    t = t.detach().cpu().contiguous()
+    if t.dtype == torch.float32:
+        return t.view(torch.int32).numpy().view(np.uint32)
+    return t.view(torch.int16).numpy().view(np.uint16)
+
+
+def round_to(t_f32: np.ndarray, dtype: torch.dtype) -> torch.Tensor:
+    """fp32 -> dtype with round-to-nearest-even (torch CPU cast)."""
+    return torch.from_numpy(np.ascontiguousarray(t_f32)).to(dtype)
+
+
+FMT = {torch.float8_e4m3fn: "e4m3", torch.float8_e5m2: "e5m2"}
