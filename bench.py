@@ -1,0 +1,224 @@
+#!/usr/bin/env python3
+"""Throughput of the low-precision hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+
+Prints ONE JSON line. A "step" is one pass of the hot path over one batch of
+synthetic input that is already resident in HBM. ``roofline`` prices the dominant
+kernel of the workload (algorithmic bytes or flops per launch / its average launch
+duration, timed with HIP events on the launch stream) against MI355X's published
+peak; ``cpu_baseline`` times the reference's own pure-PyTorch formulas
+(oracle/cpu_reference.py) on the host cores over a bounded sample.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for _p in (ROOT, ROOT / "primus-turbo_amd"):
+    if str(_p) not in sys.path:
+        sys.path.insert(0, str(_p))
+
+import torch  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0
+FP8_PEAK_TFLOPS = 5000.0
+FP4_PEAK_TFLOPS = 10100.0
+
+
+def _events_ms(fn, iters):
+    """Average duration (ms) of ``fn`` over ``iters`` back-to-back launches, HIP events on
+    torch's current stream (the stream every kernel of this library is launched on)."""
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def _outlier_randn(shape, seed, frac=0.001, mul=100.0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(shape, generator=g, dtype=torch.float32)
+    g2 = torch.Generator().manual_seed(seed + 1)
+    n = max(1, int(x.numel() * frac))
+    idx = torch.randperm(x.numel(), generator=g2)[:n]
+    x.view(-1)[idx] *= mul
+    return x.to(torch.bfloat16)
+
+
+# ---------------------------------------------------------------------------------------
+# workloads
+# ---------------------------------------------------------------------------------------
+class QuantTensorwise:
+    """BASELINE config 0: E4M3 tensorwise quantize + dequantize of a 4096x4096 bf16 tensor."""
+
+    name = "fp8_e4m3_tensorwise_quant_dequant_4096x4096_bf16"
+    metric = "quantize+dequantize GB/s (algorithmic bytes)"
+    unit = "GB/s"
+    dtype = "f32"
+    bound = "hbm"
+
+    def __init__(self, dev):
+        import primus_turbo.pytorch as turbo
+        from primus_turbo.pytorch.core.low_precision import ScalingGranularity as G
+
+        self.turbo, self.G = turbo, G
+        self.x_cpu = _outlier_randn((4096, 4096), 0)
+        self.x = self.x_cpu.to(dev)
+        self.n = self.x.numel()
+        self.q, self.sinv = turbo.ops.quantize_fp8(self.x, turbo.float8_e4m3, G.TENSORWISE)
+
+    # bytes: quant reads 2 B + writes 1 B per element, dequant reads 1 B + writes 2 B
+    def step_work(self):
+        return 6.0 * self.n
+
+    def step(self):
+        q, sinv = self.turbo.ops.quantize_fp8(self.x, self.turbo.float8_e4m3, self.G.TENSORWISE)
+        return self.turbo.ops.dequantize_fp8(q, torch.bfloat16, self.G.TENSORWISE, scale_inv=sinv)
+
+    dominant_name = "quant_tensorwise_kernel (fused amax + scale + cast)"
+
+    def dominant(self):
+        return self.turbo.ops.quantize_fp8(self.x, self.turbo.float8_e4m3, self.G.TENSORWISE)
+
+    def dominant_work(self):
+        return 3.0 * self.n  # bytes per launch
+
+    def check(self):
+        import numpy as np
+
+        from oracle import quantize as Q
+
+        oq, osinv = Q.fp8_tensorwise(self.x_cpu.float().numpy(), "e4m3")
+        same = np.array_equal(self.q.cpu().view(torch.uint8).numpy(), oq)
+        same = same and self.sinv.cpu().view(torch.int32).item() == osinv.view(np.int32).item()
+        return bool(same), "bytes and scale_inv bit-exact vs oracle"
+
+    def cpu_baseline(self):
+        from oracle import cpu_reference as R
+
+        x = self.x_cpu
+        R.quantize_fp8_tensorwise_ref(x, torch.float8_e4m3fn)  # warm-up
+        times = []
+        t_end = time.perf_counter() + 10.0
+        while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 40):
+            t0 = time.perf_counter()
+            q, _, sinv = R.quantize_fp8_tensorwise_ref(x, torch.float8_e4m3fn)
+            R.dequantize_fp8_ref(q, torch.bfloat16, sinv)
+            times.append(time.perf_counter() - t0)
+        med = sorted(times)[len(times) // 2]
+        return dict(
+            value=6.0 * self.n / med / 1e9,
+            unit="GB/s",
+            cores=torch.get_num_threads(),
+            kind="port",
+            sample=f"full 4096x4096 quantize+dequantize, median of {len(times)} runs, "
+            f"{os.cpu_count()} logical CPUs visible",
+        )
+
+
+WORKLOADS = {"quant_tensorwise": QuantTensorwise}
+try:  # the GEMM workloads register themselves once their ops exist
+    from bench_workloads import register as _register  # noqa: E402
+
+    _register(WORKLOADS)
+except ImportError:
+    pass
+
+DEFAULT_ORDER = ["gemm_fp8_rowwise", "quant_tensorwise"]
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="auto", help="one of: auto, " + ", ".join(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print(
+            "bench.py: this build measures the one-GPU hot path only; run it with --gpus 1 "
+            "(no collectives or sharding are part of it).",
+            file=sys.stderr,
+        )
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the hot path has no CPU fallback.", file=sys.stderr)
+        sys.exit(3)
+
+    name = args.workload
+    if name == "auto":
+        name = next(w for w in DEFAULT_ORDER if w in WORKLOADS)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    wl = WORKLOADS[name](dev)
+
+    ok, what = wl.check()
+    for _ in range(args.warmup):
+        wl.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        wl.step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    scale = 1e12 if wl.unit == "TFLOP/s" else 1e9
+    value = wl.step_work() / (ms_per_step * 1e-3) / scale
+
+    # dominant kernel, HIP events on the launch stream
+    for _ in range(max(3, args.warmup)):
+        wl.dominant()
+    dom_ms = _events_ms(wl.dominant, max(args.steps, 20))
+    achieved = wl.dominant_work() / (dom_ms * 1e-3) / scale
+    peak = {"hbm": HBM_PEAK_GBS, "mfma": getattr(wl, "peak", FP8_PEAK_TFLOPS)}[wl.bound]
+    roofline = dict(
+        bound=wl.bound,
+        achieved=round(achieved, 2),
+        peak=peak,
+        unit="GB/s" if wl.bound == "hbm" else "TFLOP/s",
+        frac=round(achieved / peak, 4),
+        traffic=getattr(wl, "traffic", None),
+        kernel=wl.dominant_name,
+        kernel_ms=round(dom_ms, 5),
+    )
+
+    out = dict(
+        metric=wl.metric,
+        value=round(value, 2),
+        unit=wl.unit,
+        n_gpus=1,
+        steps=args.steps,
+        warmup=args.warmup,
+        ms_per_step=round(ms_per_step, 5),
+        higher_is_better=True,
+        scaling="weak",
+        vs_baseline=None,
+        dtype=wl.dtype,
+        data="synthetic",
+        config=dict(workload=wl.name),
+        parity=dict(ok=ok, what=what),
+        roofline=roofline,
+    )
+    if not args.no_cpu:
+        out["cpu_baseline"] = wl.cpu_baseline()
+    extra = getattr(wl, "extra", None)
+    if extra:
+        out["extra"] = extra() if callable(extra) else extra
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -75,9 +75,10 @@ PT_API int pt_device_cu_count(void);
  * scale_inv : device fp32[1] output.
  * workspace : device memory of at least pt_quantize_fp8_tensorwise_workspace_bytes()
  *             bytes, 16-byte aligned, ZERO-FILLED before its first use. The
- *             kernel leaves it zero-filled on exit, so one buffer can be reused
- *             by successive calls on the same stream without clearing it again;
- *             calls that may overlap (different streams) need separate buffers.
+ *             kernels keep an epoch counter and per-workgroup slots in it and
+ *             maintain them from then on, so one buffer serves any number of
+ *             successive calls on one stream without being cleared again; calls
+ *             that may overlap (different streams) need separate buffers.
  */
 PT_API size_t pt_quantize_fp8_tensorwise_workspace_bytes(void);
 PT_API int    pt_quantize_fp8_tensorwise(const void *x, int x_dtype, int64_t numel, void *q,
@@ -97,11 +98,10 @@ PT_API int pt_dequantize_fp8_tensorwise(const void *q, int q_dtype, int64_t nume
  * dequantize_fp8_rowwise (bindings_pytorch.cpp:36,40; quantization.cpp:110-208,232-282;
  * kernels quantization_rowwise.cu:59-183,188-286,288-503, reduce/reduce_col.cuh).
  *
- * The tensor is viewed as [B, M, N] with the reduced axis = M when N > 1
- * ("column" scales, one per (b, n)) or as [outer, inner] rows when the reduced
- * axis is the last one (B*M rows of length N... expressed as B = outer, M = inner,
- * N = 1). scale / scale_inv hold B*N floats; numerics per scale as tensorwise
- * (eps 1e-12).
+ * The tensor is viewed as [B, M, N] with M the reduced axis: B = product of the
+ * dimensions before it, N = product of those after it (N == 1 when the reduced
+ * axis is the last, contiguous one). One scale per (b, n): scale_inv holds B*N
+ * floats; numerics per scale as tensorwise (eps 1e-12).
  *
  * scale_in : optional precomputed scales (B*N floats); NULL = dynamic amax.
  */
@@ -110,6 +110,66 @@ PT_API int pt_quantize_fp8_rowwise(const void *x, int x_dtype, int64_t B, int64_
                                    void *stream);
 PT_API int pt_dequantize_fp8_rowwise(const void *q, int q_dtype, int64_t B, int64_t M, int64_t N,
                                      const float *scale_inv, void *y, int y_dtype, void *stream);
+
+/* FP8 128-blockwise (fp32 scales, eps 1e-4) -----------------------------------
+ *
+ * Numerics per block: scale = qmax / max(amax, 1e-4); the stored scale is
+ * 1.0f / scale; q = fp8_rne(clamp(float(x) * scale, -qmax, qmax)). Elements
+ * beyond the tensor edge count as zeros.
+ *
+ * pt_quantize_fp8_blockwise replaces primus_turbo::quant_fp8_blockwise_impl and
+ * primus_turbo::quant_fp8_blockwise_dual_impl
+ * (primus_turbo/pytorch/kernels/quantization/quantization_impl.py:81-125,236-281;
+ * kernels primus_turbo/triton/quantization/quant_blockwise.py:11-112) for block 128.
+ * x is [M, N]. Give q_row + scale_inv_row ([M, ceil(N/128)]) for 1 x 128 row
+ * blocks, q_col + scale_inv_col ([ceil(M/128), N]) for 128 x 1 column blocks, or
+ * both ("dual": x is read once).
+ */
+PT_API int pt_quantize_fp8_blockwise(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype,
+                                     void *q_row, float *scale_inv_row, void *q_col,
+                                     float *scale_inv_col, void *stream);
+
+/* Replaces torch.ops.primus_turbo_cpp_extension.quantize_fp8_blockwise_for_weight
+ * (bindings_pytorch.cpp:52-93, csrc/pytorch/quantization/quantization.cpp:1443-1480,
+ * csrc/kernels/quantization/quantization_blockwise.cu:248-346): w is [B, M, N], one
+ * scale per 128 x 128 tile, scale_inv is [B, ceil(M/128), ceil(N/128)]. */
+PT_API int pt_quantize_fp8_blockwise_weight(const void *w, int w_dtype, int64_t B, int64_t M,
+                                            int64_t N, void *q, int q_dtype, float *scale_inv,
+                                            void *stream);
+
+/* Prefix sums of group lengths, each rounded up to `align` first:
+ *   padded_lens[i] = round_up(group_lens[i], align)   (optional output, may be NULL)
+ *   group_offs[0] = 0, group_offs[i+1] = group_offs[i] + padded_lens[i]
+ * align = 1 replaces torch.ops.primus_turbo_cpp_extension.grouped_gemm_compute_offs
+ * (bindings_pytorch.cpp:134, csrc/kernels/grouped_gemm/compute_group_offs.cu:15-42);
+ * align = 128 replaces compute_padded_group_offs
+ * (csrc/kernels/quantization/quantization_blockwise.cu:18-48). All int64, on device. */
+PT_API int pt_compute_group_offs(const int64_t *group_lens, int64_t num_groups, int64_t align,
+                                 int64_t *padded_lens, int64_t *group_offs, void *stream);
+
+/* Replaces torch.ops.primus_turbo_cpp_extension.quantize_fp8_blockwise_segment_m_row_col
+ * (csrc/pytorch/quantization/quantization.cpp:1384-1441,
+ * csrc/kernels/quantization/quantization_blockwise.cu:60-232): one read of the
+ * packed-M activation x [M, N] gives
+ *   q_row [M, N] + scale_inv_row stored transposed [ceil(N/128), M]   (1 x 128 blocks)
+ *   q_col_padded [M + G*128, N] + scale_inv_col_padded [(M + G*128)/128, N]
+ *     (128 x 1 blocks of the segment-padded tensor: group g starts at row
+ *      padded_group_offs[g], its pad rows are zero codes; rows at and beyond
+ *      padded_group_offs[G] are left untouched).
+ * group_offs / padded_group_offs are device int64 [G+1] (see pt_compute_group_offs). */
+PT_API int pt_quantize_fp8_blockwise_segment_m_row_col(
+    const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype, const int64_t *group_offs,
+    const int64_t *padded_group_offs, int64_t num_groups, void *q_row, float *scale_inv_row,
+    void *q_col_padded, float *scale_inv_col_padded, void *stream);
+
+/* De-quantize with one fp32 scale per (block_m x block_n) block of a [B, M, N] tensor:
+ *   y[b, m, n] = T(float(q[b, m, n]) * scale_inv[b, m / block_m, n / block_n]).
+ * (1, 128) / (128, 1) replace primus_turbo::dequant_fp8_blockwise_impl, (128, 128)
+ * replaces primus_turbo::dequant_fp8_blockwise_for_weight_impl
+ * (quantization_impl.py:146-234; quant_blockwise.py:162-234). */
+PT_API int pt_dequantize_fp8_block(const void *q, int q_dtype, int64_t B, int64_t M, int64_t N,
+                                   const float *scale_inv, int64_t block_m, int64_t block_n,
+                                   void *y, int y_dtype, void *stream);
 
 #ifdef __cplusplus
 }

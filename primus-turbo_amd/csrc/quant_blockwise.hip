@@ -1,0 +1,491 @@
+// FP8 128-blockwise quantizers (fp32 scales) for gfx950:
+//   1 x 128 row blocks, 128 x 1 column blocks, both at once ("dual"),
+//   128 x 128 weight tiles, and the fused grouped row + segment-padded column
+//   quantizer that feeds the MoE grouped GEMM, plus their de-quantizers and the
+//   group-offset prefix sums.
+//
+// Numerics (identical for every variant): per block
+//   scale = qmax / max(amax, 1e-4), stored value = 1.0f / scale,
+//   q = fp8_rne(clamp(float(x) * scale, -qmax, qmax)),
+// following primus_turbo/triton/quantization/quant_blockwise.py:11-327 and
+// csrc/kernels/quantization/quantization_blockwise.cu:18-346 of Primus-Turbo.
+//
+// One workgroup (256 threads, 4 wavefronts) owns one 128 x 128 tile and reads it
+// from HBM once; all requested outputs come from the register copy. A tile row is
+// spread over the 16 lanes of one DPP row, so the 1 x 128 amax is four DPP steps;
+// column maxima meet through 8 KB of LDS.
+#include "pt_common.h"
+
+namespace pt {
+
+constexpr int BQ        = 128; // block edge
+constexpr int BQ_PACK   = 8;   // elements per thread per row visit
+constexpr int BQ_ROUNDS = 8;   // 16 rows per round x 8 rounds = 128 rows
+constexpr float BQ_EPS  = 1e-4f;
+
+enum : int { MODE_ROW = 1, MODE_COL = 2, MODE_TILE = 4 };
+
+struct BlockQuantArgs {
+    const void *x;
+    uint8_t    *q_row;     // MODE_ROW / MODE_TILE output codes
+    float      *s_row;     // MODE_ROW: 1/scale per (row, n-block); MODE_TILE: per tile
+    uint8_t    *q_col;     // MODE_COL output codes
+    float      *s_col;     // MODE_COL: 1/scale per (m-block, col)
+    int64_t     M, N;      // rows / cols of one batch slice of x
+    int64_t     rs_m, rs_n; // s_row index = m * rs_m + nblock * rs_n
+    // grouped (segment-padded) mode
+    const int64_t *group_offs;  // [G+1] row offsets of the groups in x
+    const int64_t *padded_offs; // [G+1] offsets with every group rounded up to 128 rows
+    int            num_groups;
+    float          qmax;
+};
+
+template <typename T> __device__ __forceinline__ void load8(const T *p, float (&f)[8]) {
+    if constexpr (sizeof(T) == 4) {
+        const u32x4 a = ld128(p), b = ld128(p + 4);
+        f[0] = __uint_as_float(a.x); f[1] = __uint_as_float(a.y);
+        f[2] = __uint_as_float(a.z); f[3] = __uint_as_float(a.w);
+        f[4] = __uint_as_float(b.x); f[5] = __uint_as_float(b.y);
+        f[6] = __uint_as_float(b.z); f[7] = __uint_as_float(b.w);
+    } else {
+        const u32x4 a = ld128(p);
+        unpack2<T>(a.x, f[0], f[1]);
+        unpack2<T>(a.y, f[2], f[3]);
+        unpack2<T>(a.z, f[4], f[5]);
+        unpack2<T>(a.w, f[6], f[7]);
+    }
+}
+
+template <bool E5M2>
+__device__ __forceinline__ u32x2 quant8(const float (&f)[8], const float (&s)[8], float qmax) {
+    u32x2 o;
+    o.x = cvt4_fp8<E5M2>(scale_clamp(f[0], s[0], qmax), scale_clamp(f[1], s[1], qmax),
+                         scale_clamp(f[2], s[2], qmax), scale_clamp(f[3], s[3], qmax));
+    o.y = cvt4_fp8<E5M2>(scale_clamp(f[4], s[4], qmax), scale_clamp(f[5], s[5], qmax),
+                         scale_clamp(f[6], s[6], qmax), scale_clamp(f[7], s[7], qmax));
+    return o;
+}
+
+__device__ __forceinline__ void store8(uint8_t *p, u32x2 v, bool vec, int64_t gn, int64_t N) {
+    if (vec) {
+        *reinterpret_cast<u32x2 *>(p) = v;
+    } else {
+        const uint32_t w[2] = {v.x, v.y};
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (gn + i < N)
+                p[i] = static_cast<uint8_t>((w[i >> 2] >> (8 * (i & 3))) & 0xffu);
+    }
+}
+
+// MODE: bitmask of MODE_ROW / MODE_COL / MODE_TILE.  GROUPED: tiles live in the
+// segment-padded row space and map back to input rows through the group offsets.
+// VEC8: N % 8 == 0 and all pointers 16-byte aligned (128-bit loads, 64-bit stores).
+template <typename T, bool E5M2, int MODE, bool GROUPED, bool VEC8>
+__global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArgs a) {
+    const int     tid   = threadIdx.x;
+    const int     cseg  = tid & 15; // which 8-column segment of the tile row
+    const int     rslot = tid >> 4; // row within a round
+    const int64_t tn = blockIdx.x, tm = blockIdx.y, batch = blockIdx.z;
+    const int64_t M = a.M, N = a.N;
+    const float   qmax = a.qmax;
+
+    const T *x     = static_cast<const T *>(a.x) + batch * M * N;
+    int64_t  in_m0 = tm * BQ; // input row of tile row 0
+    int64_t  in_end = M;      // first invalid input row
+    int64_t  M_out  = M;      // rows of the (padded) column output that exist
+    if constexpr (GROUPED) {
+        M_out = a.padded_offs[a.num_groups];
+        const int64_t pad_start_tile = tm * BQ;
+        if (pad_start_tile >= M_out)
+            return;
+        int g = 0;
+        for (int i = 0; i < a.num_groups; ++i)
+            if (pad_start_tile >= a.padded_offs[i] && pad_start_tile < a.padded_offs[i + 1])
+                g = i;
+        const int64_t o0 = a.group_offs[g], o1 = a.group_offs[g + 1];
+        in_m0  = o0 + (pad_start_tile - a.padded_offs[g]);
+        in_end = o1 < M ? o1 : M;
+    }
+
+    const int64_t gn   = tn * BQ + cseg * BQ_PACK;
+    const bool    full = VEC8 && (gn + BQ_PACK <= N);
+
+    float vals[BQ_ROUNDS][BQ_PACK];
+    float col_amax[BQ_PACK];
+    float tile_amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < BQ_PACK; ++i)
+        col_amax[i] = 0.f;
+
+#pragma unroll
+    for (int r = 0; r < BQ_ROUNDS; ++r) {
+        const int     lm    = rslot + 16 * r;
+        const int64_t in_m  = in_m0 + lm;
+        const bool    valid = in_m < in_end;
+        if (valid && full) {
+            load8<T>(x + in_m * N + gn, vals[r]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < BQ_PACK; ++i)
+                vals[r][i] = (valid && gn + i < N) ? HP<T>::to_f32(x[in_m * N + gn + i]) : 0.f;
+        }
+        float amax = 0.f;
+#pragma unroll
+        for (int i = 0; i < BQ_PACK; ++i) {
+            const float av = fabsf(vals[r][i]);
+            amax           = fmaxf(amax, av);
+            if constexpr (MODE & MODE_COL)
+                col_amax[i] = fmaxf(col_amax[i], av);
+        }
+        if constexpr (MODE & MODE_TILE)
+            tile_amax = fmaxf(tile_amax, amax);
+        if constexpr (MODE & MODE_ROW) {
+            amax              = row16_max(amax); // the 16 lanes of this tile row
+            const float scale = qmax / fmaxf(amax, BQ_EPS);
+            if (valid) {
+                const float s[8] = {scale, scale, scale, scale, scale, scale, scale, scale};
+                store8(a.q_row + batch * M * N + in_m * N + gn, quant8<E5M2>(vals[r], s, qmax),
+                       full, gn, N);
+                if (cseg == 0)
+                    a.s_row[in_m * a.rs_m + tn * a.rs_n] = 1.0f / scale;
+            }
+        }
+    }
+
+    if constexpr (MODE & MODE_TILE) {
+        __shared__ float s_red[4];
+        tile_amax         = block_max(tile_amax, s_red);
+        const float scale = qmax / fmaxf(tile_amax, BQ_EPS);
+        if (tid == 0)
+            a.s_row[(batch * gridDim.y + tm) * gridDim.x + tn] = 1.0f / scale;
+        const float s[8] = {scale, scale, scale, scale, scale, scale, scale, scale};
+#pragma unroll
+        for (int r = 0; r < BQ_ROUNDS; ++r) {
+            const int64_t in_m = in_m0 + rslot + 16 * r;
+            if (in_m < in_end)
+                store8(a.q_row + batch * M * N + in_m * N + gn, quant8<E5M2>(vals[r], s, qmax),
+                       full, gn, N);
+        }
+    }
+
+    if constexpr (MODE & MODE_COL) {
+        __shared__ float s_part[16][BQ];
+        __shared__ float s_cscale[BQ];
+#pragma unroll
+        for (int i = 0; i < BQ_PACK; ++i)
+            s_part[rslot][cseg * BQ_PACK + i] = col_amax[i];
+        __syncthreads();
+        if (tid < BQ) {
+            float m = 0.f;
+#pragma unroll
+            for (int k = 0; k < 16; ++k)
+                m = fmaxf(m, s_part[k][tid]);
+            const float scale = qmax / fmaxf(m, BQ_EPS);
+            s_cscale[tid]     = scale;
+            const int64_t c   = tn * BQ + tid;
+            if (c < N)
+                a.s_col[tm * N + c] = 1.0f / scale;
+        }
+        __syncthreads();
+        float s[8];
+#pragma unroll
+        for (int i = 0; i < BQ_PACK; ++i)
+            s[i] = s_cscale[cseg * BQ_PACK + i];
+#pragma unroll
+        for (int r = 0; r < BQ_ROUNDS; ++r) {
+            const int64_t out_m = tm * BQ + rslot + 16 * r;
+            if (out_m < M_out) // grouped: pad rows carry zeros -> code 0
+                store8(a.q_col + out_m * N + gn, quant8<E5M2>(vals[r], s, qmax), full, gn, N);
+        }
+    }
+}
+
+template <typename T, bool E5M2, int MODE, bool GROUPED>
+static int launch_block128(const BlockQuantArgs &a, int64_t tiles_m, int64_t tiles_n, int64_t batch,
+                           bool vec, hipStream_t stream) {
+    if (tiles_m * tiles_n * batch == 0)
+        return PT_OK;
+    dim3 g(static_cast<unsigned>(tiles_n), static_cast<unsigned>(tiles_m),
+           static_cast<unsigned>(batch));
+    if (vec)
+        quant_block128_kernel<T, E5M2, MODE, GROUPED, true><<<g, 256, 0, stream>>>(a);
+    else
+        quant_block128_kernel<T, E5M2, MODE, GROUPED, false><<<g, 256, 0, stream>>>(a);
+    return check_launch("quant_block128_kernel");
+}
+
+// ---------------------------------------------------------------------------
+// De-quantize with one fp32 scale per (bm x bn) block:
+//   y[b, m, n] = T(float(q[b, m, n]) * s[b, m / bm, n / bn])
+// (bm, bn) = (1, 128) row blocks, (128, 1) column blocks, (128, 128) tiles.
+// ---------------------------------------------------------------------------
+template <typename T, bool E5M2>
+__global__ __launch_bounds__(256) void dequant_block_kernel(
+    const uint8_t *__restrict__ q, const float *__restrict__ s, T *__restrict__ y, const int64_t B,
+    const int64_t M, const int64_t N, const int bm, const int bn) {
+    const int64_t sm = (M + bm - 1) / bm, sn = (N + bn - 1) / bn;
+    const int64_t total  = B * M * N;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total;
+         i += stride) {
+        const int64_t n = i % N, m = (i / N) % M, b = i / (M * N);
+        const float   sc = s[(b * sm + m / bm) * sn + n / bn];
+        y[i]             = HP<T>::from_f32(fp8_to_f32<E5M2>(q[i], 0) * sc);
+    }
+}
+
+// 16 consecutive columns per thread; requires N % 16 == 0 and 16-byte aligned q / y.
+template <typename T, bool E5M2, bool PER_COL>
+__global__ __launch_bounds__(256) void dequant_block_vec_kernel(
+    const uint8_t *__restrict__ q, const float *__restrict__ s, T *__restrict__ y, const int64_t B,
+    const int64_t M, const int64_t N, const int bm, const int bn) {
+    const int64_t sm = (M + bm - 1) / bm, sn = (N + bn - 1) / bn;
+    const int64_t units  = B * M * N / 16;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t u = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; u < units;
+         u += stride) {
+        const int64_t  i = u * 16;
+        const int64_t  n = i % N, m = (i / N) % M, b = i / (M * N);
+        const u32x4    w = ld128(q + i);
+        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+        float          f[16];
+        if constexpr (PER_COL) { // bn == 1: sixteen different scales
+            const float *sp = s + (b * sm + m / bm) * sn + n;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                f[4 * k + 0] = fp8_to_f32<E5M2>(ww[k], 0) * sp[4 * k + 0];
+                f[4 * k + 1] = fp8_to_f32<E5M2>(ww[k], 1) * sp[4 * k + 1];
+                f[4 * k + 2] = fp8_to_f32<E5M2>(ww[k], 2) * sp[4 * k + 2];
+                f[4 * k + 3] = fp8_to_f32<E5M2>(ww[k], 3) * sp[4 * k + 3];
+            }
+        } else { // bn == 128: one scale for the 16 columns
+            const float sc = s[(b * sm + m / bm) * sn + n / bn];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                f[4 * k + 0] = fp8_to_f32<E5M2>(ww[k], 0) * sc;
+                f[4 * k + 1] = fp8_to_f32<E5M2>(ww[k], 1) * sc;
+                f[4 * k + 2] = fp8_to_f32<E5M2>(ww[k], 2) * sc;
+                f[4 * k + 3] = fp8_to_f32<E5M2>(ww[k], 3) * sc;
+            }
+        }
+        char *dst = reinterpret_cast<char *>(y + i);
+        if constexpr (sizeof(T) == 4) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                st128(dst + 16 * k,
+                      u32x4{__float_as_uint(f[4 * k]), __float_as_uint(f[4 * k + 1]),
+                            __float_as_uint(f[4 * k + 2]), __float_as_uint(f[4 * k + 3])});
+        } else {
+#pragma unroll
+            for (int k = 0; k < 2; ++k)
+                st128(dst + 16 * k,
+                      u32x4{pack2<T>(f[8 * k], f[8 * k + 1]), pack2<T>(f[8 * k + 2], f[8 * k + 3]),
+                            pack2<T>(f[8 * k + 4], f[8 * k + 5]),
+                            pack2<T>(f[8 * k + 6], f[8 * k + 7])});
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Group offsets: offs[0] = 0, offs[i+1] = offs[i] + round_up(lens[i], align).
+// One wavefront; each lane owns a strided slice, partial sums meet in LDS.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void group_offs_kernel(const int64_t *__restrict__ lens,
+                                                        int64_t *__restrict__ padded_lens,
+                                                        int64_t *__restrict__ offs, const int G,
+                                                        const int64_t align) {
+    __shared__ int64_t s_sum[64];
+    const int          lane  = threadIdx.x;
+    const int          chunk = (G + 63) / 64;
+    const int          i0 = lane * chunk, i1 = (i0 + chunk < G) ? i0 + chunk : G;
+    int64_t            sum = 0;
+    for (int i = i0; i < i1; ++i)
+        sum += (lens[i] + align - 1) / align * align;
+    s_sum[lane] = sum;
+    __syncthreads();
+    int64_t base = 0;
+    for (int k = 0; k < lane; ++k)
+        base += s_sum[k];
+    if (lane == 0)
+        offs[0] = 0;
+    for (int i = i0; i < i1; ++i) {
+        const int64_t p = (lens[i] + align - 1) / align * align;
+        if (padded_lens)
+            padded_lens[i] = p;
+        base += p;
+        offs[i + 1] = base;
+    }
+}
+
+#define PT_DISPATCH_T_E5(hp, fp8, CALL)                                                            \
+    do {                                                                                           \
+        if (hp == PT_DTYPE_BF16 && fp8 == PT_DTYPE_E4M3) { CALL(bf16_t, false); }                  \
+        else if (hp == PT_DTYPE_BF16 && fp8 == PT_DTYPE_E5M2) { CALL(bf16_t, true); }              \
+        else if (hp == PT_DTYPE_F16 && fp8 == PT_DTYPE_E4M3) { CALL(f16_t, false); }               \
+        else if (hp == PT_DTYPE_F16 && fp8 == PT_DTYPE_E5M2) { CALL(f16_t, true); }                \
+        else if (hp == PT_DTYPE_F32 && fp8 == PT_DTYPE_E4M3) { CALL(float, false); }               \
+        else { CALL(float, true); }                                                                \
+    } while (0)
+
+static bool vec_ok(const BlockQuantArgs &a, int elem_bytes) {
+    return a.N % 8 == 0 && aligned_to(a.x, 16) && (a.q_row == nullptr || aligned_to(a.q_row, 8)) &&
+           (a.q_col == nullptr || aligned_to(a.q_col, 8)) && elem_bytes > 0;
+}
+
+} // namespace pt
+
+using namespace pt;
+
+extern "C" {
+
+int pt_quantize_fp8_blockwise(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype,
+                              void *q_row, float *scale_inv_row, void *q_col, float *scale_inv_col,
+                              void *stream) {
+    PT_REQUIRE(is_hp_dtype(x_dtype), "input must be bf16, fp16 or fp32");
+    PT_REQUIRE(is_fp8_dtype(q_dtype), "output must be e4m3 or e5m2");
+    PT_REQUIRE(M >= 0 && N >= 0, "dimensions must be non-negative");
+    const bool row = q_row != nullptr, col = q_col != nullptr;
+    PT_REQUIRE(row || col, "at least one of q_row / q_col must be given");
+    PT_REQUIRE(!row || scale_inv_row, "scale_inv_row must accompany q_row");
+    PT_REQUIRE(!col || scale_inv_col, "scale_inv_col must accompany q_col");
+    if (M * N == 0)
+        return PT_OK;
+    PT_REQUIRE(x != nullptr, "x must not be NULL");
+    const int64_t tm = cdiv(M, BQ), tn = cdiv(N, BQ);
+    PT_REQUIRE(tm < 65536, "too many row tiles");
+    BlockQuantArgs a{};
+    a.x = x;
+    a.q_row = static_cast<uint8_t *>(q_row);
+    a.s_row = scale_inv_row;
+    a.q_col = static_cast<uint8_t *>(q_col);
+    a.s_col = scale_inv_col;
+    a.M = M;
+    a.N = N;
+    a.rs_m = tn;
+    a.rs_n = 1;
+    a.qmax = fp8_max_of(q_dtype);
+    auto       st  = static_cast<hipStream_t>(stream);
+    const bool vec = vec_ok(a, 1);
+#define CALL(T, E5)                                                                                \
+    do {                                                                                           \
+        if (row && col)                                                                            \
+            return launch_block128<T, E5, MODE_ROW | MODE_COL, false>(a, tm, tn, 1, vec, st);      \
+        if (row)                                                                                   \
+            return launch_block128<T, E5, MODE_ROW, false>(a, tm, tn, 1, vec, st);                 \
+        return launch_block128<T, E5, MODE_COL, false>(a, tm, tn, 1, vec, st);                     \
+    } while (0)
+    PT_DISPATCH_T_E5(x_dtype, q_dtype, CALL);
+#undef CALL
+}
+
+int pt_quantize_fp8_blockwise_weight(const void *w, int w_dtype, int64_t B, int64_t M, int64_t N,
+                                     void *q, int q_dtype, float *scale_inv, void *stream) {
+    PT_REQUIRE(is_hp_dtype(w_dtype), "input must be bf16, fp16 or fp32");
+    PT_REQUIRE(is_fp8_dtype(q_dtype), "output must be e4m3 or e5m2");
+    PT_REQUIRE(B >= 0 && M >= 0 && N >= 0, "dimensions must be non-negative");
+    if (B * M * N == 0)
+        return PT_OK;
+    PT_REQUIRE(w && q && scale_inv, "NULL tensor pointer");
+    const int64_t tm = cdiv(M, BQ), tn = cdiv(N, BQ);
+    PT_REQUIRE(tm < 65536 && B < 65536, "too many tiles / batches");
+    BlockQuantArgs a{};
+    a.x = w;
+    a.q_row = static_cast<uint8_t *>(q);
+    a.s_row = scale_inv;
+    a.M = M;
+    a.N = N;
+    a.qmax = fp8_max_of(q_dtype);
+    auto       st  = static_cast<hipStream_t>(stream);
+    const bool vec = vec_ok(a, 1) && (M * N) % 8 == 0;
+#define CALL(T, E5) return launch_block128<T, E5, MODE_TILE, false>(a, tm, tn, B, vec, st)
+    PT_DISPATCH_T_E5(w_dtype, q_dtype, CALL);
+#undef CALL
+}
+
+int pt_compute_group_offs(const int64_t *group_lens, int64_t num_groups, int64_t align,
+                          int64_t *padded_lens, int64_t *group_offs, void *stream) {
+    PT_REQUIRE(num_groups >= 0 && num_groups < (1 << 24), "bad group count");
+    PT_REQUIRE(align >= 1, "align must be >= 1");
+    PT_REQUIRE(group_offs != nullptr && (num_groups == 0 || group_lens != nullptr),
+               "NULL tensor pointer");
+    group_offs_kernel<<<1, 64, 0, static_cast<hipStream_t>(stream)>>>(
+        group_lens, padded_lens, group_offs, static_cast<int>(num_groups), align);
+    return check_launch("group_offs_kernel");
+}
+
+int pt_quantize_fp8_blockwise_segment_m_row_col(const void *x, int x_dtype, int64_t M, int64_t N,
+                                                int q_dtype, const int64_t *group_offs,
+                                                const int64_t *padded_group_offs,
+                                                int64_t num_groups, void *q_row,
+                                                float *scale_inv_row, void *q_col_padded,
+                                                float *scale_inv_col_padded, void *stream) {
+    PT_REQUIRE(is_hp_dtype(x_dtype), "input must be bf16, fp16 or fp32");
+    PT_REQUIRE(is_fp8_dtype(q_dtype), "output must be e4m3 or e5m2");
+    PT_REQUIRE(M >= 0 && N >= 0 && num_groups >= 1, "bad dimensions");
+    PT_REQUIRE(group_offs && padded_group_offs, "group offsets must not be NULL");
+    PT_REQUIRE(q_row && scale_inv_row && q_col_padded && scale_inv_col_padded,
+               "NULL output pointer");
+    if (N == 0)
+        return PT_OK;
+    PT_REQUIRE(x != nullptr || M == 0, "x must not be NULL");
+    const int64_t tm = cdiv(M + num_groups * BQ, BQ), tn = cdiv(N, BQ);
+    PT_REQUIRE(tm < 65536, "too many row tiles");
+    BlockQuantArgs a{};
+    a.x = x;
+    a.q_row = static_cast<uint8_t *>(q_row);
+    a.s_row = scale_inv_row;
+    a.q_col = static_cast<uint8_t *>(q_col_padded);
+    a.s_col = scale_inv_col_padded;
+    a.M = M;
+    a.N = N;
+    a.rs_m = 1; // row scales are stored transposed: [N / 128, M]
+    a.rs_n = M;
+    a.group_offs = group_offs;
+    a.padded_offs = padded_group_offs;
+    a.num_groups = static_cast<int>(num_groups);
+    a.qmax = fp8_max_of(q_dtype);
+    auto       st  = static_cast<hipStream_t>(stream);
+    const bool vec = vec_ok(a, 1);
+#define CALL(T, E5) return launch_block128<T, E5, MODE_ROW | MODE_COL, true>(a, tm, tn, 1, vec, st)
+    PT_DISPATCH_T_E5(x_dtype, q_dtype, CALL);
+#undef CALL
+}
+
+int pt_dequantize_fp8_block(const void *q, int q_dtype, int64_t B, int64_t M, int64_t N,
+                            const float *scale_inv, int64_t block_m, int64_t block_n, void *y,
+                            int y_dtype, void *stream) {
+    PT_REQUIRE(is_fp8_dtype(q_dtype), "input must be e4m3 or e5m2");
+    PT_REQUIRE(is_hp_dtype(y_dtype), "output must be bf16, fp16 or fp32");
+    PT_REQUIRE(B >= 0 && M >= 0 && N >= 0, "dimensions must be non-negative");
+    PT_REQUIRE(block_m >= 1 && block_n >= 1, "block sizes must be positive");
+    if (B * M * N == 0)
+        return PT_OK;
+    PT_REQUIRE(q && y && scale_inv, "NULL tensor pointer");
+    auto          st    = static_cast<hipStream_t>(stream);
+    const int64_t total = B * M * N;
+    const bool    vec   = N % 16 == 0 && aligned_to(q, 16) && aligned_to(y, 16) &&
+                     (block_n == 1 || block_n % 16 == 0);
+    const int bm = static_cast<int>(block_m), bn = static_cast<int>(block_n);
+    int64_t   grid = cdiv(vec ? total / 16 : total, 256);
+    if (grid > 16384)
+        grid = 16384;
+    const unsigned g = static_cast<unsigned>(grid);
+#define CALL(T, E5)                                                                                \
+    do {                                                                                           \
+        if (vec && bn == 1)                                                                        \
+            dequant_block_vec_kernel<T, E5, true><<<g, 256, 0, st>>>(                              \
+                static_cast<const uint8_t *>(q), scale_inv, static_cast<T *>(y), B, M, N, bm, bn); \
+        else if (vec)                                                                              \
+            dequant_block_vec_kernel<T, E5, false><<<g, 256, 0, st>>>(                             \
+                static_cast<const uint8_t *>(q), scale_inv, static_cast<T *>(y), B, M, N, bm, bn); \
+        else                                                                                       \
+            dequant_block_kernel<T, E5><<<g, 256, 0, st>>>(                                        \
+                static_cast<const uint8_t *>(q), scale_inv, static_cast<T *>(y), B, M, N, bm, bn); \
+        return check_launch("dequant_block_kernel");                                               \
+    } while (0)
+    PT_DISPATCH_T_E5(y_dtype, q_dtype, CALL);
+#undef CALL
+}
+
+} // extern "C"

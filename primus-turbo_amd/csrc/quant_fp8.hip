@@ -19,26 +19,43 @@ namespace pt {
 constexpr int TW_THREADS = 1024;
 constexpr int TW_VEC     = 16; // elements per thread per unit (16 fp8 bytes = one 128-bit store)
 
-// workspace words
-enum { WS_AMAX = 0, WS_ARRIVE = 1, WS_DEPART = 2, WS_TIMEOUT = 3, WS_WORDS = 4 };
-
-// Spin bound of the grid-wide wait (each probe sleeps ~64 cycles + one L2 atomic).
+// Grid-wide abs-max exchange without read-modify-write atomics (same-address
+// device-scope atomics serialise at ~12 ns each on this part, far too slow for a
+// 256-workgroup launch). Workspace layout, in 32-bit words:
+//   [0]            epoch k, advanced by one per launch
+//   [1]            sticky time-out flag
+//   [64 + s*1024 + b]  slot of workgroup b in slot set s (s = 0, 1)
+// Launch k publishes into set k & 1: workgroup b stores its abs-max bit pattern
+// with bit 31 raised (abs-max >= 0, so bit 31 is free to mean "published"), then
+// thread t polls slot t until it is published and the block reduces what it read.
+// Workgroup 0 clears the other set for launch k + 1 (nobody reads it during launch
+// k, and launch k - 1, its last user, has finished) and advances the epoch once it
+// is past the exchange, i.e. after every workgroup has read the old epoch.
+constexpr int      WS_EPOCH = 0, WS_TIMEOUT = 1, WS_SLOTS = 64, WS_MAX_BLOCKS = 1024;
+constexpr int      WS_WORDS = WS_SLOTS + 2 * WS_MAX_BLOCKS;
+// Probe bound of the poll (each probe sleeps ~64 cycles plus one memory round trip).
 // Every workgroup of the launch is resident (grid <= CU count, one workgroup per
-// CU), so the wait normally ends within microseconds; the bound only guarantees
-// that every wave exits even if residency is broken by something outside this
-// library. A timed-out launch raises WS_TIMEOUT (sticky) and its output is invalid.
-constexpr uint32_t GRID_WAIT_MAX_PROBES = 1u << 22;
+// CU), so the wait normally ends within microseconds; the bound only guarantees that
+// every wave exits even if residency is broken by something outside this library.
+// A timed-out launch raises WS_TIMEOUT (sticky) and its output is invalid.
+constexpr uint32_t GRID_WAIT_MAX_PROBES = 1u << 21;
 
 __device__ __forceinline__ float grid_max_exchange(float block_amax, uint32_t *ws,
-                                                   uint32_t nblocks) {
-    __shared__ float s_amax;
-    if (threadIdx.x == 0) {
-        __hip_atomic_fetch_max(&ws[WS_AMAX], __float_as_uint(block_amax), __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_fetch_add(&ws[WS_ARRIVE], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-        uint32_t probes = 0;
-        while (__hip_atomic_load(&ws[WS_ARRIVE], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) <
-               nblocks) {
+                                                   uint32_t nblocks, float *s_red) {
+    const uint32_t k   = ws[WS_EPOCH];
+    uint32_t      *cur = ws + WS_SLOTS + (k & 1u) * WS_MAX_BLOCKS;
+    uint32_t      *nxt = ws + WS_SLOTS + ((k + 1u) & 1u) * WS_MAX_BLOCKS;
+    if (blockIdx.x == 0)
+        for (int t = threadIdx.x; t < WS_MAX_BLOCKS; t += blockDim.x)
+            nxt[t] = 0u;
+    if (threadIdx.x == 0)
+        __hip_atomic_store(&cur[blockIdx.x], __float_as_uint(block_amax) | 0x80000000u,
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    float v = 0.f;
+    for (uint32_t t = threadIdx.x; t < nblocks; t += blockDim.x) {
+        uint32_t probes = 0, w;
+        while (((w = __hip_atomic_load(&cur[t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) &
+                0x80000000u) == 0u) {
             __builtin_amdgcn_s_sleep(1);
             if (++probes >= GRID_WAIT_MAX_PROBES) {
                 __hip_atomic_store(&ws[WS_TIMEOUT], 1u, __ATOMIC_RELAXED,
@@ -46,20 +63,12 @@ __device__ __forceinline__ float grid_max_exchange(float block_amax, uint32_t *w
                 break;
             }
         }
-        const uint32_t bits =
-            __hip_atomic_load(&ws[WS_AMAX], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_amax = __uint_as_float(bits);
-        // last workgroup to leave puts the workspace back to zero for the next launch
-        const uint32_t left = __hip_atomic_fetch_add(&ws[WS_DEPART], 1u, __ATOMIC_ACQ_REL,
-                                                     __HIP_MEMORY_SCOPE_AGENT);
-        if (left == nblocks - 1) {
-            __hip_atomic_store(&ws[WS_AMAX], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(&ws[WS_ARRIVE], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(&ws[WS_DEPART], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+        v = fmaxf(v, __uint_as_float(w & 0x7fffffffu));
     }
-    __syncthreads();
-    return s_amax;
+    v = block_max(v, s_red);
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+        ws[WS_EPOCH] = k + 1u;
+    return v;
 }
 
 // Register image of one 16-element unit.
@@ -163,7 +172,7 @@ __global__ __launch_bounds__(TW_THREADS) void quant_tensorwise_kernel(
             if (blockIdx.x == 0 && tail0 + threadIdx.x < n)
                 amax = fmaxf(amax, fabsf(HP<T>::to_f32(x[tail0 + threadIdx.x])));
             amax = block_max(amax, s_red);
-            amax = grid_max_exchange(amax, ws, gridDim.x);
+            amax = grid_max_exchange(amax, ws, gridDim.x, s_red);
         }
         float scale;
         if constexpr (DYNAMIC)
@@ -195,7 +204,7 @@ __global__ __launch_bounds__(TW_THREADS) void quant_tensorwise_kernel(
             for (int64_t i = tid0; i < n; i += stride)
                 amax = fmaxf(amax, fabsf(HP<T>::to_f32(x[i])));
             amax = block_max(amax, s_red);
-            amax = grid_max_exchange(amax, ws, gridDim.x);
+            amax = grid_max_exchange(amax, ws, gridDim.x, s_red);
         }
         float scale;
         if constexpr (DYNAMIC)
@@ -222,6 +231,8 @@ static int launch_quant_tensorwise(const void *x, int64_t n, void *q, const floa
         grid = 1;
     if (grid > cus)
         grid = cus; // one workgroup per CU: all of them are resident at the grid exchange
+    if (grid > WS_MAX_BLOCKS)
+        grid = WS_MAX_BLOCKS;
     const T *xp = static_cast<const T *>(x);
     auto    *qp = static_cast<uint8_t *>(q);
     dim3     g(static_cast<unsigned>(grid)), b(TW_THREADS);

@@ -64,6 +64,24 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_int, c_void_p],
     ),
+    "pt_quantize_fp8_blockwise": (
+        c_int,
+        [c_void_p, c_int, c_i64, c_i64, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    ),
+    "pt_quantize_fp8_blockwise_weight": (
+        c_int,
+        [c_void_p, c_int, c_i64, c_i64, c_i64, c_void_p, c_int, c_void_p, c_void_p],
+    ),
+    "pt_compute_group_offs": (c_int, [c_void_p, c_i64, c_i64, c_void_p, c_void_p, c_void_p]),
+    "pt_quantize_fp8_blockwise_segment_m_row_col": (
+        c_int,
+        [c_void_p, c_int, c_i64, c_i64, c_int, c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_void_p,
+         c_void_p, c_void_p],
+    ),
+    "pt_dequantize_fp8_block": (
+        c_int,
+        [c_void_p, c_int, c_i64, c_i64, c_i64, c_void_p, c_i64, c_i64, c_void_p, c_int, c_void_p],
+    ),
 }
 
 

@@ -238,3 +238,323 @@ def dequantize_fp8_rowwise_impl(x: torch.Tensor, out_dtype: torch.dtype, axis: i
     assert x.is_contiguous(), "The x tensor must be contiguous."
     assert scale_inv.is_contiguous(), "The scale_inv tensor must be contiguous."
     return torch.ops.primus_turbo_cpp_extension.dequantize_fp8_rowwise(x, scale_inv, axis, out_dtype)
+
+
+# ===========================================================================
+# FP8 128-blockwise
+# ===========================================================================
+def ceil_div(a: int, b: int) -> int:
+    return (a + b - 1) // b
+
+
+def _need_block_128(block_size: int) -> None:
+    _check(block_size == 128, f"only block_size=128 is built for the FP8 blockwise kernels, got {block_size}")
+
+
+def _blockwise_launch(x, dtype, want_row: bool, want_col: bool):
+    N.require_cuda(x)
+    _check(x.dtype in _HP_DTYPES, "input must be bfloat16, float16 or float32")
+    _check_fp8_out(dtype)
+    M, Nn = x.shape
+    dev = x.device
+    q_row = s_row = q_col = s_col = None
+    if want_row:
+        q_row = torch.empty((M, Nn), dtype=dtype, device=dev)
+        s_row = torch.empty((M, ceil_div(Nn, 128)), dtype=torch.float32, device=dev)
+    if want_col:
+        q_col = torch.empty((M, Nn), dtype=dtype, device=dev)
+        s_col = torch.empty((ceil_div(M, 128), Nn), dtype=torch.float32, device=dev)
+    N.check(
+        N.lib().pt_quantize_fp8_blockwise(
+            N.ptr(x), N.dtype_code(x.dtype), M, Nn, N.dtype_code(dtype),
+            N.ptr(q_row), N.ptr(s_row), N.ptr(q_col), N.ptr(s_col), N.stream_of(x),
+        )
+    )
+    return q_row, s_row, q_col, s_col
+
+
+@torch.library.custom_op("primus_turbo::quant_fp8_blockwise_impl", mutates_args=())
+def quant_fp8_blockwise_impl(
+    x: torch.Tensor, dtype: torch.dtype, axis: int, block_size: int = 128
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """1-D blockwise quantization of a contiguous 2-D tensor along ``axis``.
+
+    axis 1 / -1: scales ``[M, cdiv(N, block)]``; axis 0 / -2: scales ``[cdiv(M, block), N]``.
+    Returns ``(x_fp8, scale_inv)`` (the stored scale is 1/scale)."""
+    assert x.is_contiguous() and x.dim() == 2, "Input must be 2D and contiguous"
+    assert axis in (-2, -1, 0, 1), f"axis must be 0 or 1 (or -1, -2), got {axis}"
+    _need_block_128(block_size)
+    if axis % 2 == 1:
+        q, s, _, _ = _blockwise_launch(x, dtype, True, False)
+    else:
+        _, _, q, s = _blockwise_launch(x, dtype, False, True)
+    return q, s
+
+
+@quant_fp8_blockwise_impl.register_fake
+def _quant_fp8_blockwise_impl_fake(x, dtype, axis, block_size=128):
+    assert x.dim() == 2, "Input must be 2D"
+    assert axis in (-2, -1, 0, 1), f"axis must be 0 or 1 (or -1, -2), got {axis}"
+    M, Nn = x.shape
+    shape = (M, ceil_div(Nn, block_size)) if axis % 2 == 1 else (ceil_div(M, block_size), Nn)
+    return (
+        torch.empty((M, Nn), dtype=dtype, device=x.device),
+        torch.empty(shape, dtype=torch.float32, device=x.device),
+    )
+
+
+@torch.library.custom_op("primus_turbo::quant_fp8_blockwise_dual_impl", mutates_args=())
+def quant_fp8_blockwise_dual_impl(
+    x: torch.Tensor, dtype: torch.dtype, block_size: int = 128
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Row (1 x block) and column (block x 1) quantization from one read of ``x``.
+
+    Returns ``(x_fp8_row, scales_row [M, N/b], x_fp8_col, scales_col [M/b, N])``."""
+    assert x.is_contiguous() and x.dim() == 2, "Input must be 2D and contiguous"
+    _need_block_128(block_size)
+    return _blockwise_launch(x, dtype, True, True)
+
+
+@quant_fp8_blockwise_dual_impl.register_fake
+def _quant_fp8_blockwise_dual_impl_fake(x, dtype, block_size=128):
+    assert x.dim() == 2, "Input must be 2D"
+    M, Nn = x.shape
+    dev = x.device
+    return (
+        torch.empty((M, Nn), dtype=dtype, device=dev),
+        torch.empty((M, ceil_div(Nn, block_size)), dtype=torch.float32, device=dev),
+        torch.empty((M, Nn), dtype=dtype, device=dev),
+        torch.empty((ceil_div(M, block_size), Nn), dtype=torch.float32, device=dev),
+    )
+
+
+# quantize_fp8_blockwise_for_weight(Tensor input, ScalarType dest_dtype, int block_size) -> Tensor[]
+_ext.define("quantize_fp8_blockwise_for_weight(Tensor input, ScalarType dest_dtype, int block_size) -> Tensor[]")
+
+
+def _weight_shapes(w, block_size):
+    if w.dim() == 2:
+        B, (M, Nn) = 1, w.shape
+        sshape = [ceil_div(M, block_size), ceil_div(Nn, block_size)]
+    else:
+        B, M, Nn = w.shape
+        sshape = [B, ceil_div(M, block_size), ceil_div(Nn, block_size)]
+    return B, M, Nn, sshape
+
+
+def _quantize_fp8_blockwise_for_weight(input: torch.Tensor, dest_dtype: torch.dtype, block_size: int):
+    N.require_cuda(input)
+    _check(input.dtype in _HP_DTYPES, "input must be bfloat16, float16 or float32")
+    _check_fp8_out(dest_dtype)
+    _check(input.dim() in (2, 3), "weight quant requires 2D or 3D input")
+    _need_block_128(block_size)
+    w = input.contiguous()
+    B, M, Nn, sshape = _weight_shapes(w, block_size)
+    q = torch.empty_like(w, dtype=dest_dtype)
+    s = torch.empty(sshape, dtype=torch.float32, device=w.device)
+    N.check(
+        N.lib().pt_quantize_fp8_blockwise_weight(
+            N.ptr(w), N.dtype_code(w.dtype), B, M, Nn, N.ptr(q), N.dtype_code(dest_dtype), N.ptr(s), N.stream_of(w)
+        )
+    )
+    return [q, s]
+
+
+def _quantize_fp8_blockwise_for_weight_meta(input, dest_dtype, block_size):
+    _, _, _, sshape = _weight_shapes(input, block_size)
+    return [
+        torch.empty(input.shape, dtype=dest_dtype, device=input.device),
+        torch.empty(sshape, dtype=torch.float32, device=input.device),
+    ]
+
+
+_ext.impl("quantize_fp8_blockwise_for_weight", _quantize_fp8_blockwise_for_weight, "CUDA")
+_ext.impl("quantize_fp8_blockwise_for_weight", _quantize_fp8_blockwise_for_weight, "CPU")
+_ext.impl("quantize_fp8_blockwise_for_weight", _quantize_fp8_blockwise_for_weight_meta, "Meta")
+
+
+@torch.library.custom_op("primus_turbo::quant_fp8_blockwise_for_weight_impl", mutates_args=())
+def quant_fp8_blockwise_for_weight_impl(
+    w: torch.Tensor, dtype: torch.dtype, block_size: int = 128
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One scale per block x block tile of a 2-D or 3-D weight -> ``(w_fp8, scale_inv)``."""
+    assert w.dim() in (2, 3)
+    q, s = torch.ops.primus_turbo_cpp_extension.quantize_fp8_blockwise_for_weight(w.contiguous(), dtype, block_size)
+    return q, s
+
+
+@quant_fp8_blockwise_for_weight_impl.register_fake
+def _quant_fp8_blockwise_for_weight_impl_fake(w, dtype, block_size=128):
+    assert w.dim() in (2, 3)
+    q, s = _quantize_fp8_blockwise_for_weight_meta(w, dtype, block_size)
+    return q, s
+
+
+def _dequant_block(q: torch.Tensor, scale_inv: torch.Tensor, out_dtype, B, M, Nn, bm, bn):
+    N.require_cuda(q, scale_inv)
+    _check(q.dtype in _FP8_DTYPES, "input must be float8_e4m3fn or float8_e5m2")
+    _check(out_dtype in _HP_DTYPES, "out_dtype must be bfloat16, float16 or float32")
+    _check(scale_inv.dtype == torch.float32, "scale_inv must be float32")
+    s = scale_inv.contiguous()
+    _check(s.numel() == B * ceil_div(M, bm) * ceil_div(Nn, bn), "scale_inv has the wrong number of elements")
+    out = torch.empty(q.shape, dtype=out_dtype, device=q.device)
+    N.check(
+        N.lib().pt_dequantize_fp8_block(
+            N.ptr(q), N.dtype_code(q.dtype), B, M, Nn, N.ptr(s), bm, bn, N.ptr(out), N.dtype_code(out_dtype),
+            N.stream_of(q),
+        )
+    )
+    return out
+
+
+@torch.library.custom_op("primus_turbo::dequant_fp8_blockwise_impl", mutates_args=())
+def dequant_fp8_blockwise_impl(
+    x_fp8: torch.Tensor, scale_inv: torch.Tensor, out_dtype: torch.dtype, axis: int, block_size: int = 128
+) -> torch.Tensor:
+    """Inverse of :func:`quant_fp8_blockwise_impl` for the same ``axis``."""
+    assert x_fp8.is_contiguous() and x_fp8.dim() == 2, "Input must be 2D and contiguous"
+    assert axis in (-2, -1, 0, 1), f"axis must be 0 or 1 (or -1, -2), got {axis}"
+    M, Nn = x_fp8.shape
+    bm, bn = (1, block_size) if axis % 2 == 1 else (block_size, 1)
+    return _dequant_block(x_fp8, scale_inv, out_dtype, 1, M, Nn, bm, bn)
+
+
+@dequant_fp8_blockwise_impl.register_fake
+def _dequant_fp8_blockwise_impl_fake(x_fp8, scale_inv, out_dtype, axis, block_size=128):
+    assert x_fp8.dim() == 2, "Input must be 2D"
+    return torch.empty(x_fp8.shape, dtype=out_dtype, device=x_fp8.device)
+
+
+@torch.library.custom_op("primus_turbo::dequant_fp8_blockwise_for_weight_impl", mutates_args=())
+def dequant_fp8_blockwise_for_weight_impl(
+    w_fp8: torch.Tensor, scale_inv: torch.Tensor, out_dtype: torch.dtype, block_size: int = 128
+) -> torch.Tensor:
+    """Inverse of :func:`quant_fp8_blockwise_for_weight_impl` (2-D or 3-D)."""
+    assert w_fp8.dim() in (2, 3)
+    w = w_fp8.contiguous()
+    B, M, Nn, _ = _weight_shapes(w, block_size)
+    return _dequant_block(w, scale_inv, out_dtype, B, M, Nn, block_size, block_size)
+
+
+@dequant_fp8_blockwise_for_weight_impl.register_fake
+def _dequant_fp8_blockwise_for_weight_impl_fake(w_fp8, scale_inv, out_dtype, block_size=128):
+    assert w_fp8.dim() in (2, 3)
+    return torch.empty(w_fp8.shape, dtype=out_dtype, device=w_fp8.device)
+
+
+# ---------------------------------------------------------------------------
+# group offsets and the fused grouped row + segment-padded column quantizer
+# ---------------------------------------------------------------------------
+_ext.define("grouped_gemm_compute_offs(Tensor group_lens) -> Tensor")
+
+
+def _group_offs(group_lens: torch.Tensor, align: int, want_padded_lens: bool):
+    N.require_cuda(group_lens)
+    _check(group_lens.dtype == torch.int64 and group_lens.dim() == 1, "group_lens must be a 1-D int64 tensor")
+    gl = group_lens.contiguous()
+    G = gl.numel()
+    offs = torch.empty(G + 1, dtype=torch.int64, device=gl.device)
+    padded = torch.empty(G, dtype=torch.int64, device=gl.device) if want_padded_lens else None
+    N.check(N.lib().pt_compute_group_offs(N.ptr(gl), G, align, N.ptr(padded), N.ptr(offs), N.stream_of(gl)))
+    return padded, offs
+
+
+def _grouped_gemm_compute_offs(group_lens: torch.Tensor) -> torch.Tensor:
+    return _group_offs(group_lens, 1, False)[1]
+
+
+def _grouped_gemm_compute_offs_meta(group_lens):
+    return torch.empty(group_lens.numel() + 1, dtype=torch.int64, device=group_lens.device)
+
+
+_ext.impl("grouped_gemm_compute_offs", _grouped_gemm_compute_offs, "CUDA")
+_ext.impl("grouped_gemm_compute_offs", _grouped_gemm_compute_offs, "CPU")
+_ext.impl("grouped_gemm_compute_offs", _grouped_gemm_compute_offs_meta, "Meta")
+
+_ext.define(
+    "quantize_fp8_blockwise_segment_m_row_col(Tensor input, ScalarType dest_dtype, int block_size, "
+    "Tensor group_lens, Tensor group_offs) -> Tensor[]"
+)
+
+
+def _segment_shapes(M, Nn, G, block_size):
+    Mp = M + G * block_size
+    return Mp, (ceil_div(Nn, block_size), M), (ceil_div(Mp, block_size), Nn)
+
+
+def _quantize_fp8_blockwise_segment_m_row_col(input, dest_dtype, block_size, group_lens, group_offs):
+    N.require_cuda(input, group_lens, group_offs)
+    _check(input.dtype in _HP_DTYPES, "input must be bfloat16, float16 or float32")
+    _check_fp8_out(dest_dtype)
+    _check(input.dim() == 2, "input must be 2D")
+    _need_block_128(block_size)
+    for t in (group_lens, group_offs):
+        _check(t.dtype == torch.int64, "group_lens / group_offs must be int64")
+        _check(t.is_contiguous(), "group_lens / group_offs must be contiguous")
+    G = group_lens.numel()
+    _check(group_offs.numel() == G + 1, "group_offs must have one more element than group_lens")
+    x = input.contiguous()
+    M, Nn = x.shape
+    Mp, rs_shape, cs_shape = _segment_shapes(M, Nn, G, block_size)
+    dev = x.device
+    padded_lens, padded_offs = _group_offs(group_lens, block_size, True)
+    q_row = torch.empty((M, Nn), dtype=dest_dtype, device=dev)
+    q_col = torch.empty((Mp, Nn), dtype=dest_dtype, device=dev)
+    s_row = torch.empty(rs_shape, dtype=torch.float32, device=dev)
+    s_col = torch.empty(cs_shape, dtype=torch.float32, device=dev)
+    N.check(
+        N.lib().pt_quantize_fp8_blockwise_segment_m_row_col(
+            N.ptr(x), N.dtype_code(x.dtype), M, Nn, N.dtype_code(dest_dtype), N.ptr(group_offs), N.ptr(padded_offs),
+            G, N.ptr(q_row), N.ptr(s_row), N.ptr(q_col), N.ptr(s_col), N.stream_of(x),
+        )
+    )
+    return [q_row, q_col, s_row, s_col, padded_lens, padded_offs]
+
+
+def _quantize_fp8_blockwise_segment_m_row_col_meta(input, dest_dtype, block_size, group_lens, group_offs):
+    M, Nn = input.shape
+    G = group_lens.numel()
+    Mp, rs_shape, cs_shape = _segment_shapes(M, Nn, G, block_size)
+    dev = input.device
+    return [
+        torch.empty((M, Nn), dtype=dest_dtype, device=dev),
+        torch.empty((Mp, Nn), dtype=dest_dtype, device=dev),
+        torch.empty(rs_shape, dtype=torch.float32, device=dev),
+        torch.empty(cs_shape, dtype=torch.float32, device=dev),
+        torch.empty(G, dtype=torch.int64, device=dev),
+        torch.empty(G + 1, dtype=torch.int64, device=dev),
+    ]
+
+
+_ext.impl("quantize_fp8_blockwise_segment_m_row_col", _quantize_fp8_blockwise_segment_m_row_col, "CUDA")
+_ext.impl("quantize_fp8_blockwise_segment_m_row_col", _quantize_fp8_blockwise_segment_m_row_col, "CPU")
+_ext.impl("quantize_fp8_blockwise_segment_m_row_col", _quantize_fp8_blockwise_segment_m_row_col_meta, "Meta")
+
+
+@torch.library.custom_op("primus_turbo::quant_fp8_blockwise_segment_m_row_col_impl", mutates_args=())
+def quant_fp8_blockwise_segment_m_row_col_impl(
+    x: torch.Tensor,
+    dtype: torch.dtype,
+    block_size: int,
+    group_lens: torch.Tensor,
+    group_offs: torch.Tensor,
+    gemm_other_dim: Optional[int] = None,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Fused grouped quantizer: one read of the packed-M activation ``x [M, N]`` yields the
+    row-quantized tensor (fwd / dgrad operand, scales stored ``[N/b, M]``) and the
+    segment-padded column-quantized tensor (variable-K wgrad operand).
+
+    Returns ``(x_fp8_row [M,N], x_fp8_col_padded [M+G*b,N], scales_row [N/b,M],
+    scales_col_padded [(M+G*b)/b,N], padded_group_lens [G], padded_group_offs [G+1])``.
+    ``gemm_other_dim`` is accepted for signature parity; there is a single kernel here."""
+    assert x.is_contiguous() and x.dim() == 2
+    r = torch.ops.primus_turbo_cpp_extension.quantize_fp8_blockwise_segment_m_row_col(
+        x, dtype, block_size, group_lens, group_offs
+    )
+    return r[0], r[1], r[2], r[3], r[4], r[5]
+
+
+@quant_fp8_blockwise_segment_m_row_col_impl.register_fake
+def _quant_fp8_blockwise_segment_m_row_col_impl_fake(x, dtype, block_size, group_lens, group_offs, gemm_other_dim=None):
+    r = _quantize_fp8_blockwise_segment_m_row_col_meta(x, dtype, block_size, group_lens, group_offs)
+    return r[0], r[1], r[2], r[3], r[4], r[5]

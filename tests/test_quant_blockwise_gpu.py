@@ -1,0 +1,154 @@
+"""GPU parity: FP8 128-blockwise quantizers vs the CPU oracle (bit-exact bytes and scales)."""
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import FMT, bf16_randn, bits_np, codes_np, round_to, to_f32_np
+from oracle import quantize as Q
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _turbo(native_lib):
+    global turbo, G, ScalingRecipe
+    import primus_turbo.pytorch as turbo
+    from primus_turbo.pytorch.core.low_precision import ScalingGranularity as G
+    from primus_turbo.pytorch.core.low_precision import ScalingRecipe
+
+
+def _eq_scales(got: torch.Tensor, want: np.ndarray):
+    assert tuple(got.shape) == want.shape, (got.shape, want.shape)
+    assert np.array_equal(bits_np(got), want.view(np.uint32))
+
+
+SHAPES = [(16384, 2048), (256, 256), (128, 128), (1, 1), (1, 300), (300, 1), (129, 257), (200, 128), (555, 1000), (64, 4104)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_blockwise_row_col_dual(shape, dtype):
+    if shape[0] == 16384 and dtype != torch.float8_e4m3fn:
+        pytest.skip("headline size only for e4m3")
+    x = bf16_randn(shape, seed=21, outlier_frac=0.001)
+    xf = to_f32_np(x)
+    xg = x.cuda()
+    f = FMT[dtype]
+    oqr, osr = Q.fp8_blockwise(xf, 1, f)
+    oqc, osc = Q.fp8_blockwise(xf, 0, f)
+    q, s = turbo.ops.quantize_fp8(xg, dtype, G.BLOCKWISE, block_size=128, axis=1)
+    assert np.array_equal(codes_np(q), oqr)
+    _eq_scales(s, osr)
+    q0, s0 = turbo.ops.quantize_fp8(xg, dtype, G.BLOCKWISE, block_size=128, axis=0)
+    assert np.array_equal(codes_np(q0), oqc)
+    _eq_scales(s0, osc)
+    qr, sr, qc, sc = turbo.ops.quantize_fp8_with_trans(xg, dtype, G.BLOCKWISE, block_size=128)
+    assert np.array_equal(codes_np(qr), oqr) and np.array_equal(codes_np(qc), oqc)
+    _eq_scales(sr, osr)
+    _eq_scales(sc, osc)
+    # negative axis aliases
+    qn, sn = turbo.ops.quantize_fp8(xg, dtype, G.BLOCKWISE, block_size=128, axis=-2)
+    assert torch.equal(qn.view(torch.uint8), q0.view(torch.uint8)) and torch.equal(sn, s0)
+    # de-quantize both directions
+    y1 = turbo.ops.dequantize_fp8(q, torch.bfloat16, G.BLOCKWISE, block_size=128, axis=1, scale_inv=s)
+    assert np.array_equal(bits_np(y1), bits_np(round_to(Q.fp8_blockwise_dequant(oqr, osr, 1, f), torch.bfloat16)))
+    y0 = turbo.ops.dequantize_fp8(q0, torch.float32, G.BLOCKWISE, block_size=128, axis=0, scale_inv=s0)
+    assert np.array_equal(bits_np(y0), Q.fp8_blockwise_dequant(oqc, osc, 0, f).view(np.uint32))
+    # every full-magnitude block holds a code of magnitude qmax (0x7E e4m3 / 0x7B e5m2)
+    top = 0x7E if dtype == torch.float8_e4m3fn else 0x7B
+    if shape[1] % 128 == 0:
+        blocks = (codes_np(q) & 0x7F).reshape(shape[0], -1, 128).max(axis=2)
+        amax = np.abs(xf).reshape(shape[0], -1, 128).max(axis=2)
+        assert np.all(blocks[amax >= 1e-4] == top)
+
+
+@pytest.mark.parametrize("src", [torch.float16, torch.float32])
+def test_blockwise_other_sources(src):
+    x = bf16_randn((300, 520), 22, dtype=src)
+    qr, sr, qc, sc = turbo.ops.quantize_fp8_with_trans(x.cuda(), torch.float8_e4m3fn, G.BLOCKWISE, block_size=128)
+    oqr, osr, oqc, osc = Q.fp8_blockwise_dual(to_f32_np(x), "e4m3")
+    assert np.array_equal(codes_np(qr), oqr) and np.array_equal(codes_np(qc), oqc)
+    _eq_scales(sr, osr)
+    _eq_scales(sc, osc)
+
+
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+@pytest.mark.parametrize("shape", [(7168, 2048), (4, 512, 384), (2, 130, 260), (100, 100), (3, 1, 1), (32, 4096, 7168)])
+def test_blockwise_weight(shape, dtype):
+    if shape[0] in (32, 7168) and dtype != torch.float8_e4m3fn:
+        pytest.skip("large size only for e4m3")
+    x = bf16_randn(shape, seed=23)
+    f = FMT[dtype]
+    rec = ScalingRecipe(use_2d_block=True)
+    q, s = turbo.ops.quantize_fp8(x.cuda(), dtype, G.BLOCKWISE, block_size=128, scaling_recipe=rec)
+    torch.cuda.synchronize()
+    oq, os_ = Q.fp8_blockwise_weight(to_f32_np(x), f)
+    assert np.array_equal(codes_np(q), oq)
+    _eq_scales(s, os_)
+    if shape[0] != 32:
+        y = turbo.ops.dequantize_fp8(q, torch.bfloat16, G.BLOCKWISE, block_size=128, scale_inv=s, scaling_recipe=rec)
+        want = round_to(Q.fp8_blockwise_weight_dequant(oq, os_, f), torch.bfloat16)
+        assert np.array_equal(bits_np(y), bits_np(want))
+
+
+def _lens(kind, G_, total, seed):
+    rng = np.random.default_rng(seed)
+    if kind == "balanced":
+        return np.full(G_, total // G_, dtype=np.int64)
+    if kind == "ragged":
+        w = 0.2 + 0.8 * rng.random(G_)
+        lens = np.floor(w / w.sum() * total).astype(np.int64)
+        lens[-1] += total - lens.sum()
+        return lens
+    if kind == "zeros":
+        lens = np.zeros(G_, dtype=np.int64)
+        lens[0] = total // 2
+        lens[1] = total - total // 2
+        return lens
+    if kind == "zipf":
+        w = (1.0 + np.arange(G_)) ** -1.2
+        w = rng.permutation(w)
+        w[rng.choice(G_, 2, replace=False)] = 0
+        lens = np.floor(w / w.sum() * total).astype(np.int64)
+        lens[np.argmax(lens)] += total - lens.sum()
+        return lens
+    raise ValueError(kind)
+
+
+@pytest.mark.parametrize(
+    "kind,G_,M,N",
+    [
+        ("balanced", 4, 1024, 512),
+        ("ragged", 8, 3000, 384),
+        ("zeros", 8, 16384, 256),
+        ("zipf", 32, 32768, 2048),
+        ("ragged", 3, 77, 100),
+        ("zipf", 32, 8192, 7168),
+    ],
+)
+def test_grouped_segment_row_col(kind, G_, M, N):
+    lens = _lens(kind, G_, M, 24)
+    assert lens.sum() == M
+    x = bf16_randn((M, N), seed=25, outlier_frac=0.001)
+    gl = torch.from_numpy(lens).cuda()
+    offs = torch.ops.primus_turbo_cpp_extension.grouped_gemm_compute_offs(gl)
+    assert np.array_equal(offs.cpu().numpy(), Q.group_offs(lens))
+    from primus_turbo.pytorch.kernels.quantization.quantization_impl import (
+        quant_fp8_blockwise_segment_m_row_col_impl as seg,
+    )
+
+    qr, qc, sr, sc, plens, poffs = seg(x.cuda(), torch.float8_e4m3fn, 128, gl, offs, N)
+    torch.cuda.synchronize()
+    o = Q.fp8_blockwise_segment_m_row_col(to_f32_np(x), lens, "e4m3")
+    assert np.array_equal(plens.cpu().numpy(), o["padded_lens"])
+    assert np.array_equal(poffs.cpu().numpy(), o["padded_offs"])
+    assert np.array_equal(codes_np(qr), o["row"])
+    _eq_scales(sr, o["row_scale"])
+    w = o["written_rows"]
+    assert tuple(qc.shape) == o["col"].shape and tuple(sc.shape) == o["col_scale"].shape
+    assert np.array_equal(codes_np(qc)[:w], o["col"][:w])
+    assert np.array_equal(bits_np(sc)[: w // 128], o["col_scale"].view(np.uint32)[: w // 128])
+    # row scales are the plain 1x128 scales transposed
+    _, s_plain = turbo.ops.quantize_fp8(x.cuda(), torch.float8_e4m3fn, G.BLOCKWISE, block_size=128, axis=1)
+    assert torch.equal(sr, s_plain.t().contiguous())
