@@ -1,0 +1,242 @@
+"""Pins for oracle/quantize.py: closed forms, the reference's own pure-PyTorch formula on
+fp32 input, brute-force per-block loops written independently, and invariants."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cpu_reference as R
+from oracle import formats as F
+from oracle import quantize as Q
+
+
+def _f32(a):
+    return np.asarray(a, dtype=np.float32)
+
+
+def _rng_x(shape, seed, scale=1.0):
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal(shape) * scale).astype(np.float32)
+    return F.bf16_bits_to_f32(F.f32_to_bf16_bits(x))  # bf16-representable values
+
+
+# ---------------------------------------------------------------- tensorwise / rowwise
+def test_tensorwise_closed_forms():
+    # all zero: scale = 448 / 1e-12, scale_inv = 1 / scale, all codes 0
+    q, si = Q.fp8_tensorwise(np.zeros(100, np.float32), "e4m3")
+    assert q.max() == 0
+    s = np.float32(448.0) / np.float32(1e-12)
+    assert si == np.float32(1.0) / s
+    # power-of-two amax: scale is exact, element = amax -> +-448 -> 0x7E / 0xFE
+    x = _f32([0.5, -4.0, 4.0, 1.0, 0.0])
+    q, si = Q.fp8_tensorwise(x, "e4m3")
+    assert si == np.float32(4.0 / 448.0) or si == np.float32(1.0) / np.float32(112.0)
+    assert q.tolist() == [F.encode_rne(_f32([56.0]), F.E4M3)[0], 0xFE, 0x7E, F.encode_rne(_f32([112.0]), F.E4M3)[0], 0]
+    # single spike: everything else collapses towards zero codes
+    x = np.full(1000, 1e-3, np.float32)
+    x[17] = -300.0
+    q, si = Q.fp8_tensorwise(x, "e4m3")
+    assert q[17] == 0xFE
+    small = np.float32(1e-3) * (np.float32(448.0) / np.float32(300.0))
+    assert q[0] == F.encode_rne(_f32([small]), F.E4M3)[0]
+    # NaN -> +max and is ignored by the amax; inf -> scale 0
+    x = _f32([1.0, np.nan, -2.0])
+    q, si = Q.fp8_tensorwise(x, "e4m3")
+    assert q.tolist() == [F.encode_rne(_f32([224.0]), F.E4M3)[0], 0x7E, 0xFE]
+    q, si = Q.fp8_tensorwise(_f32([1.0, np.inf, -np.inf]), "e4m3")
+    assert np.isinf(si) and q.tolist() == [0, 0x7E, 0x7E]
+    # given scale
+    q, si = Q.fp8_tensorwise(_f32([1.0, 2.0]), "e4m3", scale=_f32(2.0))
+    assert si == np.float32(0.5) and q.tolist() == F.encode_rne(_f32([2.0, 4.0]), F.E4M3).tolist()
+
+
+@pytest.mark.parametrize("tdtype,fmt", [(torch.float8_e4m3fn, "e4m3"), (torch.float8_e5m2, "e5m2")])
+def test_tensorwise_equals_reference_formula_on_fp32(tdtype, fmt):
+    """On fp32 input the reference's pure-PyTorch test formula has no extra rounding and
+    must agree bit for bit (tests/pytorch/ref/quantization_ref.py:31-40 of the reference)."""
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(513, 257, generator=g) * 3
+    x.view(-1)[::1001] *= 100
+    rq, _, rsi = R.quantize_fp8_tensorwise_ref(x, tdtype)
+    q, si = Q.fp8_tensorwise(x.numpy(), fmt)
+    assert np.array_equal(q, rq.view(torch.uint8).numpy())
+    assert si.view(np.uint32) == rsi.numpy().view(np.uint32)
+    for axis in (0, 1, -1):
+        # torch evaluates `scalar / tensor` as tensor.reciprocal() * scalar, i.e. with one more
+        # rounding than the IEEE division of the device kernel: scales may differ by an ulp or
+        # two, and only slices whose scale agrees must agree in every code.
+        rq, rs, rsi = R.quantize_fp8_rowwise_ref(x, tdtype, axis)
+        q, si = Q.fp8_rowwise(x.numpy(), axis, fmt)
+        ulp = np.abs(si.view(np.int32).astype(np.int64) - rsi.numpy().view(np.int32).astype(np.int64))
+        assert ulp.max() <= 2
+        amax = np.abs(x.numpy()).max(axis=axis, keepdims=True)
+        ieee_scale = (np.float32(torch.finfo(tdtype).max) / np.maximum(amax, np.float32(1e-12))).astype(np.float32)
+        same_scale = ieee_scale.view(np.uint32) == rs.numpy().view(np.uint32)
+        same_scale = np.broadcast_to(same_scale, q.shape)
+        eq = q == rq.view(torch.uint8).numpy()
+        assert np.all(eq[same_scale]) and same_scale.mean() > 0.5 and eq.mean() > 0.999
+    # dequantize
+    y = Q.fp8_dequant(rq.view(torch.uint8).numpy(), rsi.numpy(), fmt)
+    ry = R.dequantize_fp8_ref(rq, torch.float32, rsi)
+    assert np.array_equal(y.view(np.uint32), ry.numpy().view(np.uint32))
+
+
+def test_rowwise_is_tensorwise_per_slice():
+    x = _rng_x((5, 7, 33), 4)
+    for axis in (0, 1, 2, -1, -3):
+        q, si = Q.fp8_rowwise(x, axis, "e4m3")
+        ax = axis % 3
+        assert si.shape == tuple(1 if i == ax else s for i, s in enumerate(x.shape))
+        xm, qm, sm = np.moveaxis(x, ax, -1), np.moveaxis(q, ax, -1), np.moveaxis(si, ax, -1)
+        for idx in np.ndindex(xm.shape[:-1]):
+            tq, tsi = Q.fp8_tensorwise(xm[idx], "e4m3")
+            assert np.array_equal(tq, qm[idx]) and tsi == sm[idx][0]
+
+
+# ---------------------------------------------------------------- blockwise
+def _block_loop(x, r0, r1, c0, c1, qmax, fmt):
+    """Independent scalar evaluation of one block (python floats + np.float32 rounding)."""
+    blk = x[r0:r1, c0:c1]
+    amax = np.float32(max(float(np.max(np.abs(blk))) if blk.size else 0.0, 0.0))
+    scale = np.float32(qmax) / np.float32(max(amax, np.float32(1e-4)))
+    v = np.clip((blk * scale).astype(np.float32), -qmax, qmax)
+    return F.encode_rne(v, fmt), np.float32(1.0) / scale
+
+
+@pytest.mark.parametrize("shape", [(256, 384), (130, 257), (1, 5), (300, 128)])
+def test_blockwise_bruteforce(shape):
+    x = _rng_x(shape, 5)
+    x[0, 0] = 1000.0
+    M, N = shape
+    qr, sr, qc, sc = Q.fp8_blockwise_dual(x, "e4m3")
+    assert sr.shape == (M, math.ceil(N / 128)) and sc.shape == (math.ceil(M / 128), N)
+    for m in range(0, M, max(1, M // 7)):
+        for nb in range(sr.shape[1]):
+            c, s = _block_loop(x, m, m + 1, nb * 128, min(N, nb * 128 + 128), 448.0, F.E4M3)
+            assert np.array_equal(c[0], qr[m, nb * 128 : nb * 128 + 128]) and s == sr[m, nb]
+    for n in range(0, N, max(1, N // 7)):
+        for mb in range(sc.shape[0]):
+            c, s = _block_loop(x, mb * 128, min(M, mb * 128 + 128), n, n + 1, 448.0, F.E4M3)
+            assert np.array_equal(c[:, 0], qc[mb * 128 : mb * 128 + 128, n]) and s == sc[mb, n]
+    # weight tiles
+    qw, sw = Q.fp8_blockwise_weight(x, "e4m3")
+    for mb in range(sw.shape[0]):
+        for nb in range(sw.shape[1]):
+            c, s = _block_loop(x, mb * 128, min(M, mb * 128 + 128), nb * 128, min(N, nb * 128 + 128), 448.0, F.E4M3)
+            assert np.array_equal(c, qw[mb * 128 : mb * 128 + 128, nb * 128 : nb * 128 + 128]) and s == sw[mb, nb]
+    # round trip error bound: |x - deq| <= amax_block * 2^-4 (e4m3 has 3 mantissa bits)
+    d = Q.fp8_blockwise_dequant(qr, sr, 1, "e4m3")
+    amax = np.repeat(np.abs(np.pad(x, ((0, 0), (0, -N % 128)))).reshape(M, -1, 128).max(2), 128, axis=1)[:, :N]
+    assert np.all(np.abs(d - x) <= amax * 2.0**-4 + 1e-6)
+
+
+def test_blockwise_invariants():
+    x = _rng_x((384, 512), 6)
+    qr, sr, qc, sc = Q.fp8_blockwise_dual(x, "e5m2")
+    assert (qr & 0x7F).reshape(384, 4, 128).max(2).min() == 0x7B  # every row block saturates one code
+    assert (qc & 0x7F).reshape(3, 128, 512).max(1).min() == 0x7B
+    a, sa = Q.fp8_blockwise(x, 1, "e5m2")
+    b, sb = Q.fp8_blockwise(x, 0, "e5m2")
+    assert np.array_equal(a, qr) and np.array_equal(b, qc) and np.array_equal(sa, sr) and np.array_equal(sb, sc)
+    # tiny block: eps 1e-4 clamps the amax, 3-D weights are per-batch
+    z = np.full((128, 128), 1e-6, np.float32)
+    q, s = Q.fp8_blockwise_weight(z, "e4m3")
+    assert s[0, 0] == np.float32(1.0) / (np.float32(448.0) / np.float32(1e-4))
+    w = _rng_x((3, 200, 130), 7)
+    q3, s3 = Q.fp8_blockwise_weight(w, "e4m3")
+    for b_ in range(3):
+        q2, s2 = Q.fp8_blockwise_weight(w[b_], "e4m3")
+        assert np.array_equal(q3[b_], q2) and np.array_equal(s3[b_], s2)
+    d = Q.fp8_blockwise_weight_dequant(q3, s3, "e4m3")
+    assert d.shape == w.shape and np.max(np.abs(d - w)) < 0.3
+
+
+@pytest.mark.parametrize("lens", [[128, 128], [100, 0, 30, 300], [0, 0, 5], [1] * 7, [513, 0, 127, 129]])
+def test_grouped_segment_layout(lens):
+    lens = np.asarray(lens, np.int64)
+    M, N = int(lens.sum()), 200
+    x = _rng_x((M, N), 8)
+    o = Q.fp8_blockwise_segment_m_row_col(x, lens, "e4m3")
+    pl, po = o["padded_lens"], o["padded_offs"]
+    assert pl.tolist() == [((int(v) + 127) // 128) * 128 for v in lens]
+    assert po.tolist() == [0] + np.cumsum(pl).tolist()
+    Mp = M + len(lens) * 128
+    assert o["col"].shape == (Mp, N) and o["col_scale"].shape == (math.ceil(Mp / 128), N)
+    rq, rs = Q.fp8_blockwise(x, 1, "e4m3")
+    assert np.array_equal(o["row"], rq) and np.array_equal(o["row_scale"], rs.T)
+    offs = Q.group_offs(lens)
+    for g, n in enumerate(lens):
+        seg = o["col"][po[g] : po[g + 1]]
+        assert np.all(seg[n:] == 0)  # pad rows are zero codes
+        if n:
+            xp = np.zeros((int(pl[g]), N), np.float32)
+            xp[:n] = x[offs[g] : offs[g] + n]
+            cq, cs = Q.fp8_blockwise(xp, 0, "e4m3")
+            assert np.array_equal(seg, cq)
+            assert np.array_equal(o["col_scale"][po[g] // 128 : po[g + 1] // 128], cs)
+
+
+# ---------------------------------------------------------------- MX
+@pytest.mark.parametrize("fmt,qmax", [("e4m3", 448.0), ("e5m2", 57344.0), ("e2m1", 6.0)])
+def test_mx_rowwise_bruteforce(fmt, qmax):
+    f = Q._fmt(fmt)
+    x = _rng_x((37, 96), 9, scale=3.0)
+    x[3, :32] = 0.0  # an all-zero block
+    x[5, 40] = 2.0**20
+    codes, sc = Q.mx_quant_rowwise(x, fmt)
+    Kp = 128
+    assert sc.shape == (37, Kp // 32)
+    assert codes.shape == ((37, Kp // 2) if fmt == "e2m1" else (37, Kp))
+    un = Q.unpack_fp4(codes) if fmt == "e2m1" else codes
+    add, tgt = F.E8M0_RULE[fmt]
+    for m in range(37):
+        for kb in range(Kp // 32):
+            blk = np.zeros(32, np.float32)
+            lo, hi = kb * 32, min(96, kb * 32 + 32)
+            if lo < 96:
+                blk[: hi - lo] = x[m, lo:hi]
+            amax = float(np.max(np.abs(blk)))
+            if amax == 0:
+                e = -127
+            else:
+                mm, ex = math.frexp(amax)
+                bits = int(np.float32(amax).view(np.uint32))
+                e = (((bits + add) >> 23) & 0x1FF) - 127 - tgt
+                e = max(-127, min(128, e))
+                assert e in (ex - 1 - tgt, ex - tgt)
+            assert sc[m, kb] == e + 127
+            want = F.encode_rne(np.clip(blk.astype(np.float64) * 2.0 ** (-e), -qmax, qmax), f)
+            assert np.array_equal(un[m, kb * 32 : kb * 32 + 32], want)
+    assert sc[3, 0] == 0 and np.all(un[3, :32] == 0)
+    assert np.all(sc[:, 3] == 0) and np.all(un[:, 96:] == 0)  # K padding
+    # round trip: |x - deq| <= 2^e * (half a step at the top binade)
+    d = Q.mx_dequant(codes, sc, fmt)[:, :96]
+    # e4m3: the block maximum may sit in the saturating sliver [448, 496) -> up to 9.7 % off
+    step = {"e4m3": 0.1, "e5m2": 2.0**-3, "e2m1": 2.0**-2}[fmt]
+    blk_amax = np.repeat(np.abs(np.pad(x, ((0, 0), (0, 32)))).reshape(37, 4, 32).max(2), 32, axis=1)[:, :96]
+    assert np.all(np.abs(d - x) <= blk_amax * step * 1.0001 + 1e-30)
+
+
+def test_mx_colwise_and_2d():
+    x = _rng_x((96, 64), 10)
+    c, s = Q.mx_quant_colwise(x, "e4m3")
+    c2, s2 = Q.mx_quant_rowwise(np.ascontiguousarray(x.T), "e4m3")
+    assert c.shape == (64, 128) and s.shape == (64, 4)
+    assert np.array_equal(c, c2) and np.array_equal(s, s2)
+    # 2-D blocks: one exponent per 32x32 tile, equal to the 1-D rule on the tile amax
+    c, s = Q.mx_quant_rowwise(x, "e2m1", use_2d_block=True)
+    for tm in range(3):
+        for tk in range(2):
+            tile = x[tm * 32 : tm * 32 + 32, tk * 32 : tk * 32 + 32]
+            e = F.e8m0_exponent(np.float32(np.abs(tile).max()), F.E2M1)
+            assert np.all(s[tm * 32 : tm * 32 + 32, tk] == e + 127)
+    assert np.all(s[:, 2:] == 0)
+
+
+def test_fp4_packing_order():
+    codes = np.arange(16, dtype=np.uint8)[None, :]
+    p = Q._pack_fp4(codes)
+    assert p.tolist() == [[0x10, 0x32, 0x54, 0x76, 0x98, 0xBA, 0xDC, 0xFE]]  # even element in the low nibble
+    assert np.array_equal(Q.unpack_fp4(p), codes)
