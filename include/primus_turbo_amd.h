@@ -171,6 +171,46 @@ PT_API int pt_dequantize_fp8_block(const void *q, int q_dtype, int64_t B, int64_
                                    const float *scale_inv, int64_t block_m, int64_t block_n,
                                    void *y, int y_dtype, void *stream);
 
+/* Scaled FP8 GEMM -------------------------------------------------------------
+ *
+ * Replaces primus_turbo::gemm_fp8_impl / gemm_fp8_accum_impl
+ * (primus_turbo/pytorch/kernels/gemm/gemm_fp8_impl.py:518-585) for the TENSORWISE,
+ * ROWWISE and BLOCKWISE granularities, i.e. the Triton kernels of
+ * primus_turbo/triton/gemm/gemm_fp8_kernel.py:123-243,446-565,871-1183 and the
+ * CK / hipBLASLt instantiations behind the same op.
+ *
+ *   C[M, N] (+)= scale( op(A) . op(B) ),  fp32 accumulation, C in c_dtype.
+ *   trans_a == 0: A is stored [M, K];  trans_a != 0: A is stored [K, M].
+ *   trans_b != 0: B is stored [N, K];  trans_b == 0: B is stored [K, N].
+ * The MFMA kernel contracts along contiguous K in steps of 128; an operand stored with
+ * K as its row axis is transposed into `workspace` first, and when K is not a multiple
+ * of 128 both operands are copied there with a zero-filled K tail
+ * (pt_gemm_fp8_workspace_bytes(M, N, K, trans_a, trans_b) bytes, 16-byte aligned;
+ * zero bytes, and `workspace` may be NULL, for trans_a == 0, trans_b != 0, K % 128 == 0).
+ *
+ * scale_mode 0 (vector):  C = (A.B) * a_scale[m * sa_m] * b_scale[n * sb_n]
+ *     tensorwise: sa_m = sb_n = 0;  rowwise: sa_m = sb_n = 1.
+ * scale_mode 1 (128-block along K; kb runs over ceil(K / 128) blocks):
+ *     C = sum_kb (A_kb.B_kb) * a_scale[(m / sa_block) * sa_m + kb * sa_k]
+ *                            * b_scale[(n / sb_block) * sb_n + kb * sb_k]
+ *     sa_block / sb_block are 1 (1 x 128 activation blocks) or 128 (128 x 128 tiles).
+ * accumulate != 0 adds into C (beta = 1) instead of overwriting it.
+ * tile_cfg: 0 = automatic, 1 = 256x256, 2 = 256x128, 3 = 128x128 workgroup tile.
+ * Requirements: a, b, c 16-byte aligned.
+ */
+PT_API size_t pt_gemm_fp8_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans_a,
+                                          int trans_b);
+PT_API int pt_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const void *b, int b_dtype,
+                       const float *b_scale, void *c, int c_dtype, int64_t M, int64_t N, int64_t K,
+                       int trans_a, int trans_b, int scale_mode, int64_t sa_m, int64_t sa_k,
+                       int64_t sb_n, int64_t sb_k, int sa_block, int sb_block, int accumulate,
+                       void *workspace, size_t workspace_bytes, int tile_cfg, void *stream);
+
+/* Byte-matrix transpose out[b, c, r] = in[b, r, c] (fp8 payloads; replaces the 2-D
+ * transpose used for tensorwise `.t()` copies, csrc/kernels/transpose/). */
+PT_API int pt_transpose_u8(const void *in, void *out, int64_t batch, int64_t R, int64_t C,
+                           void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -61,12 +61,20 @@ def _deps_mtime() -> float:
     return max(p.stat().st_mtime for p in deps)
 
 
+def _extra_flags(src: Path) -> list[str]:
+    """Per-file compiler flags: a leading ``// hipcc-flags: ...`` comment line in the source."""
+    with open(src) as f:
+        first = f.readline()
+    tag = "// hipcc-flags:"
+    return first[len(tag):].split() if first.startswith(tag) else []
+
+
 def _compile_one(hipcc: str, src: Path, force: bool, verbose: bool) -> Path:
     obj = BUILD / (src.stem + ".o")
     if not force and obj.exists():
         if obj.stat().st_mtime >= max(src.stat().st_mtime, _deps_mtime()):
             return obj
-    cmd = [hipcc, *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)]
+    cmd = [hipcc, *HIPCC_FLAGS, *_extra_flags(src), "-c", str(src), "-o", str(obj)]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)

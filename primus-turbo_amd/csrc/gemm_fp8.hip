@@ -1,0 +1,195 @@
+// Scaled FP8 GEMM entry points: operand preparation (transposes / K padding), the
+// VECTOR-scale (tensorwise, rowwise) kernel instantiations and the C ABI. The BLOCK-scale
+// instantiations live in gemm_fp8_block.hip, which is compiled with MFMA results in VGPRs.
+#include "gemm_fp8_kernel.h"
+
+namespace pt {
+
+int launch_gemm_block(const GemmArgs &a, int fa, int fb, bool sb_vec, int tile_cfg, hipStream_t stream);
+
+// ---------------------------------------------------------------------------
+// fp8 byte matrix transpose in[R, C] -> out[C, ldo] through a padded 64 x 64 LDS tile;
+// columns [R, ldo) of every output row are zero-filled. Brings operands whose reduction
+// axis is not contiguous into NT form (and pads K to a multiple of 128 on the way).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void transpose_u8_kernel(const uint8_t *__restrict__ in,
+                                                           uint8_t *__restrict__ out,
+                                                           const int64_t R, const int64_t C,
+                                                           const int64_t ldo) {
+    __shared__ uint8_t t[64][64 + 4];
+    const int64_t      r0 = static_cast<int64_t>(blockIdx.y) * 64, c0 = static_cast<int64_t>(blockIdx.x) * 64;
+    const int64_t      bi = static_cast<int64_t>(blockIdx.z) * R * C, bo = static_cast<int64_t>(blockIdx.z) * C * ldo;
+    const int          tx = threadIdx.x & 15, ty = threadIdx.x >> 4; // 16 x 16 threads, 4 bytes each
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int     r  = ty + 16 * p;
+        const int64_t gr = r0 + r, gc = c0 + tx * 4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            t[r][tx * 4 + e] = (gr < R && gc + e < C) ? in[bi + gr * C + gc + e] : 0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int     c  = ty + 16 * p; // output row = input column
+        const int64_t gc = c0 + c, gr = r0 + tx * 4;
+        if (gc < C) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (gr + e < ldo)
+                    out[bo + gc * ldo + gr + e] = t[tx * 4 + e][c]; // rows >= R were loaded as 0
+        }
+    }
+}
+
+// in[R, C] -> out[R, ldo], columns [C, ldo) zero-filled (K padding of a K-contiguous operand)
+__global__ __launch_bounds__(256) void pad_rows_u8_kernel(const uint8_t *__restrict__ in,
+                                                          uint8_t *__restrict__ out, const int64_t R,
+                                                          const int64_t C, const int64_t ldo) {
+    const int64_t total  = R * ldo;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t r = i / ldo, c = i % ldo;
+        out[i]          = c < C ? in[r * C + c] : 0;
+    }
+}
+
+static void launch_transpose(const uint8_t *in, uint8_t *out, int64_t batch, int64_t R, int64_t C,
+                             int64_t ldo, hipStream_t st) {
+    // the grid covers ldo (>= R) input-row positions so that the zero tail gets written too
+    dim3 g(static_cast<unsigned>(cdiv(C, 64)), static_cast<unsigned>(cdiv(ldo, 64)),
+           static_cast<unsigned>(batch));
+    transpose_u8_kernel<<<g, 256, 0, st>>>(in, out, R, C, ldo);
+}
+
+template <int FA, int FB>
+static int launch_vector_tiles(const GemmArgs &a, int tile_cfg, hipStream_t stream) {
+    // tile_cfg: 0 = auto, 1 = 256x256, 2 = 256x128, 3 = 128x128
+    if (tile_cfg == 0)
+        tile_cfg = (a.M >= 2048 && a.N >= 2048) ? 1 : 3;
+    if (tile_cfg == 1)
+        return launch_gemm_cfg<8, 8, SCALE_VECTOR, false, FA, FB>(a, stream);
+    if (tile_cfg == 2)
+        return launch_gemm_cfg<8, 4, SCALE_VECTOR, false, FA, FB>(a, stream);
+    return launch_gemm_cfg<4, 4, SCALE_VECTOR, false, FA, FB>(a, stream);
+}
+
+static int launch_gemm_vector(const GemmArgs &a, int fa, int fb, int tile_cfg, hipStream_t stream) {
+    if (fa == 0 && fb == 0)
+        return launch_vector_tiles<0, 0>(a, tile_cfg, stream);
+    if (fa == 0 && fb == 1)
+        return launch_vector_tiles<0, 1>(a, tile_cfg, stream);
+    if (fa == 1 && fb == 0)
+        return launch_vector_tiles<1, 0>(a, tile_cfg, stream);
+    return launch_vector_tiles<1, 1>(a, tile_cfg, stream);
+}
+
+static inline int64_t round_up(int64_t x, int64_t m) {
+    return (x + m - 1) / m * m;
+}
+
+} // namespace pt
+
+using namespace pt;
+
+extern "C" {
+
+size_t pt_gemm_fp8_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans_a, int trans_b) {
+    // An operand is copied into the workspace when its reduction axis is not contiguous
+    // (transpose) or when K is not a multiple of 128 (zero padding of the K tail).
+    const int64_t Kp    = round_up(K, KSTEP);
+    const bool    pad   = Kp != K;
+    size_t        bytes = 0;
+    if (trans_a || pad)
+        bytes += static_cast<size_t>(round_up(M * Kp, 256));
+    if (!trans_b || pad)
+        bytes += static_cast<size_t>(round_up(N * Kp, 256));
+    return bytes;
+}
+
+int pt_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const void *b, int b_dtype,
+                const float *b_scale, void *c, int c_dtype, int64_t M, int64_t N, int64_t K,
+                int trans_a, int trans_b, int scale_mode, int64_t sa_m, int64_t sa_k, int64_t sb_n,
+                int64_t sb_k, int sa_block, int sb_block, int accumulate, void *workspace,
+                size_t workspace_bytes, int tile_cfg, void *stream) {
+    PT_REQUIRE(is_fp8_dtype(a_dtype) && is_fp8_dtype(b_dtype), "operands must be e4m3 or e5m2");
+    PT_REQUIRE(is_hp_dtype(c_dtype), "output must be bf16, fp16 or fp32");
+    PT_REQUIRE(M >= 0 && N >= 0 && K >= 0, "dimensions must be non-negative");
+    PT_REQUIRE(scale_mode == SCALE_VECTOR || scale_mode == SCALE_BLOCK, "unknown scale mode");
+    PT_REQUIRE(scale_mode != SCALE_BLOCK || ((sa_block == 1 || sa_block == 128) && (sb_block == 1 || sb_block == 128)),
+               "sa_block / sb_block must be 1 or 128");
+    PT_REQUIRE(tile_cfg >= 0 && tile_cfg <= 3, "tile_cfg must be 0..3");
+    if (M == 0 || N == 0)
+        return PT_OK;
+    PT_REQUIRE(a && b && c && a_scale && b_scale, "NULL tensor pointer");
+    PT_REQUIRE(aligned_to(a, 16) && aligned_to(b, 16) && aligned_to(c, 16), "operands must be 16-byte aligned");
+    PT_REQUIRE(cdiv(M, 128) * cdiv(N, 128) < (1LL << 31), "too many tiles");
+    auto st = static_cast<hipStream_t>(stream);
+
+    const int64_t  Kp  = round_up(K, KSTEP);
+    const bool     pad = Kp != K;
+    const uint8_t *A   = static_cast<const uint8_t *>(a);
+    const uint8_t *B   = static_cast<const uint8_t *>(b);
+    if (trans_a || !trans_b || pad) {
+        const size_t need = pt_gemm_fp8_workspace_bytes(M, N, K, trans_a, trans_b);
+        if (workspace == nullptr || workspace_bytes < need || !aligned_to(workspace, 16))
+            return fail(PT_ERR_WORKSPACE, "pt_gemm_fp8: workspace missing, too small or misaligned");
+        uint8_t *ws = static_cast<uint8_t *>(workspace);
+        if (trans_a || pad) {
+            if (M * Kp > 0) {
+                if (trans_a) // stored [K, M] -> [M, Kp]
+                    launch_transpose(A, ws, 1, K, M, Kp, st);
+                else
+                    pad_rows_u8_kernel<<<static_cast<unsigned>(cdiv(M * Kp, 256 * 16)), 256, 0, st>>>(A, ws, M, K, Kp);
+            }
+            A = ws;
+            ws += round_up(M * Kp, 256);
+        }
+        if (!trans_b || pad) {
+            if (N * Kp > 0) {
+                if (!trans_b) // stored [K, N] -> [N, Kp]
+                    launch_transpose(B, ws, 1, K, N, Kp, st);
+                else
+                    pad_rows_u8_kernel<<<static_cast<unsigned>(cdiv(N * Kp, 256 * 16)), 256, 0, st>>>(B, ws, N, K, Kp);
+            }
+            B = ws;
+        }
+    }
+
+    GemmArgs g{};
+    g.A = A;
+    g.B = B;
+    g.C = c;
+    g.sA = a_scale;
+    g.sB = b_scale;
+    g.M = M;
+    g.N = N;
+    g.K = Kp;
+    g.lda = Kp;
+    g.ldb = Kp;
+    g.sa_m = sa_m;
+    g.sa_k = sa_k;
+    g.sb_n = sb_n;
+    g.sb_k = sb_k;
+    g.sa_shift = sa_block == 128 ? 7 : 0;
+    g.sb_shift = sb_block == 128 ? 7 : 0;
+    g.out_dtype = c_dtype;
+    g.accumulate = accumulate;
+    const int fa = a_dtype == PT_DTYPE_E5M2 ? 1 : 0, fb = b_dtype == PT_DTYPE_E5M2 ? 1 : 0;
+    if (scale_mode == SCALE_VECTOR)
+        return launch_gemm_vector(g, fa, fb, tile_cfg, st);
+    return launch_gemm_block(g, fa, fb, sb_block == 1, tile_cfg, st);
+}
+
+int pt_transpose_u8(const void *in, void *out, int64_t batch, int64_t R, int64_t C, void *stream) {
+    PT_REQUIRE(batch >= 0 && R >= 0 && C >= 0, "dimensions must be non-negative");
+    if (batch * R * C == 0)
+        return PT_OK;
+    PT_REQUIRE(in && out, "NULL tensor pointer");
+    PT_REQUIRE(batch < 65536 && cdiv(R, 64) < 65536, "grid dimension out of range");
+    launch_transpose(static_cast<const uint8_t *>(in), static_cast<uint8_t *>(out), batch, R, C, R,
+                     static_cast<hipStream_t>(stream));
+    return check_launch("transpose_u8_kernel");
+}
+
+} // extern "C"

@@ -1,0 +1,267 @@
+"""``gemm_fp8``: FP8 GEMM with autograd (reference: primus_turbo/pytorch/ops/gemm_fp8.py).
+
+Which quantizer feeds which GEMM layout, per granularity (same recipes as the reference):
+
+  TENSORWISE  fwd  C = Aq . Bq            one scale per tensor; backward runs NT GEMMs on
+                   physically transposed fp8 copies when the forward is NT (ref :96-276)
+  ROWWISE     fwd  A, B quantized along K; backward re-quantizes the de-quantized
+                   operands along the other axis and quantizes grad_out twice (ref :278-426)
+  BLOCKWISE   fwd  A 1x128 (+128x1 for wgrad from the same read), B 128x128 tiles;
+                   dgrad = NN with the same weight tiles, wgrad = TN on the 128x1 casts
+                   (ref :429-553)
+  MX_BLOCKWISE     A 1x32, B 32x32 two-direction MXFP8 casts, every GEMM is NT (ref :556-717)
+
+HYBRID format: forward operands E4M3, gradients E5M2.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Union
+
+import torch
+
+from primus_turbo.pytorch.core.backend import BackendType
+from primus_turbo.pytorch.core.low_precision import (
+    Float8QuantConfig,
+    ScalingGranularity,
+    ScalingRecipe,
+    check_mxfp8_support,
+)
+from primus_turbo.pytorch.core.quantized_tensor import (
+    QuantizedTensor,
+    QuantizedTensorPair,
+    check_quantized_tensor,
+)
+from primus_turbo.pytorch.kernels.gemm.gemm_fp8_impl import gemm_fp8_accum_impl, gemm_fp8_impl
+from primus_turbo.pytorch.ops.quantization import quantize_fp8, quantize_fp8_with_trans
+from primus_turbo.pytorch.ops.utils import _get_dummy_wgrad, _get_fp8_dtype, _setup_fused_grad_accum
+
+__all__ = ["gemm_fp8"]
+
+_NATIVE = BackendType.TURBO.value  # single backend; the value is informational
+
+
+def _gemm(a, a_s, trans_a, b, b_s, trans_b, out_dtype, trans_c, granularity):
+    return gemm_fp8_impl(a, a_s, trans_a, b, b_s, trans_b, out_dtype, trans_c, granularity.value, _NATIVE)
+
+
+def _wgrad_gemm(a, a_s, trans_a, b, b_s, trans_b, out_dtype, trans_c, granularity, accumulate_into=None):
+    """Weight-gradient GEMM; with ``accumulate_into`` the result is added to that buffer in
+    the GEMM epilogue and a cached dummy tensor of the weight's shape is returned (the
+    framework's own accumulation was switched off in forward)."""
+    if accumulate_into is None:
+        return _gemm(a, a_s, trans_a, b, b_s, trans_b, out_dtype, trans_c, granularity)
+    gemm_fp8_accum_impl(a, a_s, trans_a, b, b_s, trans_b, accumulate_into.dtype, trans_c, granularity.value,
+                        accumulate_into, _NATIVE)
+    return _get_dummy_wgrad(accumulate_into.shape, out_dtype)
+
+
+def _as_quantized(x, config, fwd: bool, axis, recipe=None) -> QuantizedTensor:
+    if isinstance(x, QuantizedTensor):
+        check_quantized_tensor(x, config, axis=axis, scaling_recipe=recipe)
+        return x
+    return QuantizedTensor.quantize(
+        x, _get_fp8_dtype(config.format, fwd), config.granularity, axis=axis, block_size=config.block_size,
+        scaling_recipe=recipe,
+    )
+
+
+class FP8GemmTensorFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, a, b, a_t, b_t, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum_pattern=None):
+        fuse, main_grad = _setup_fused_grad_accum(b, fuse_bgrad_accum_pattern)
+        qa = _as_quantized(a, config, True, -1)
+        qb = _as_quantized(b, config, True, -1)
+        out = _gemm(qa.qdata, qa.scale_inv, trans_a, qb.qdata, qb.scale_inv, trans_b, out_dtype, False, config.granularity)
+        # NT forward: keep physically transposed fp8 copies so that both backward GEMMs
+        # are NT as well (contiguous-K operands need no transposition pass inside the GEMM)
+        nt_bwd = (not trans_a) and trans_b
+        if nt_bwd:
+            qa_t = a_t if isinstance(a_t, QuantizedTensor) else qa.t()
+            qb_t = b_t if isinstance(b_t, QuantizedTensor) else qb.t()
+            ctx.save_for_backward(qa_t.qdata, qa_t.scale_inv, qb_t.qdata, qb_t.scale_inv)
+        else:
+            ctx.save_for_backward(qa.qdata, qa.scale_inv, qb.qdata, qb.scale_inv)
+        ctx.meta = (trans_a, trans_b, out_dtype, config, nt_bwd, fuse, main_grad)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        trans_a, trans_b, out_dtype, config, nt_bwd, fuse, main_grad = ctx.meta
+        sa, sa_s, sb, sb_s = ctx.saved_tensors
+        g = QuantizedTensor.quantize(grad_out.contiguous(), _get_fp8_dtype(config.format, False), config.granularity, axis=-1)
+        gran = config.granularity
+        acc = main_grad if fuse else None
+        if nt_bwd:
+            # saved: A^T [K, M], B^T [K, N]
+            grad_a = _gemm(g.qdata, g.scale_inv, False, sb, sb_s, True, out_dtype, False, gran)
+            g_t = g.t()
+            grad_b = _wgrad_gemm(sa, sa_s, False, g_t.qdata, g_t.scale_inv, True, out_dtype, trans_b, gran, acc)
+        else:
+            grad_a = _gemm(g.qdata, g.scale_inv, False, sb, sb_s, not trans_b, out_dtype, trans_a, gran)
+            grad_b = _wgrad_gemm(sa, sa_s, not trans_a, g.qdata, g.scale_inv, False, out_dtype, trans_b, gran, acc)
+        return grad_a, grad_b, None, None, None, None, None, None, None
+
+
+class FP8GemmRowFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, a, b, a_t, b_t, trans_a, trans_b, out_dtype, config):
+        assert trans_a == False, "trans_a has to be False"  # noqa: E712
+        b_axis = -1 if trans_b else -2
+        qa = _as_quantized(a, config, True, -1)
+        qb = _as_quantized(b, config, True, b_axis)
+
+        def other_axis(q: QuantizedTensor, given, axis):
+            if given is not None:
+                assert isinstance(given, QuantizedTensor)
+                return given
+            return QuantizedTensor.quantize(q.dequantize(), q.real_dtype, config.granularity, axis=axis,
+                                            block_size=config.block_size)
+
+        qa_t = other_axis(qa, a_t, -2)
+        qb_t = other_axis(qb, b_t, -2 if trans_b else -1)
+        out = _gemm(qa.qdata, qa.scale_inv, trans_a, qb.qdata, qb.scale_inv, trans_b, out_dtype, False, config.granularity)
+        ctx.save_for_backward(qa_t.qdata, qa_t.scale_inv, qb_t.qdata, qb_t.scale_inv)
+        ctx.meta = (trans_a, trans_b, out_dtype, config)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        trans_a, trans_b, out_dtype, config = ctx.meta
+        a_c, a_cs, b_c, b_cs = ctx.saved_tensors
+        grad_out = grad_out.contiguous()
+        gdt = _get_fp8_dtype(config.format, False)
+        gran = config.granularity
+        g_row = QuantizedTensor.quantize(grad_out, gdt, gran, axis=-1, block_size=config.block_size)
+        grad_a = _gemm(g_row.qdata, g_row.scale_inv, False, b_c, b_cs, not trans_b, out_dtype, trans_a, gran)
+        g_col = QuantizedTensor.quantize(grad_out, gdt, gran, axis=-2, block_size=config.block_size)
+        grad_b = _gemm(a_c, a_cs, not trans_a, g_col.qdata, g_col.scale_inv, False, out_dtype, trans_b, gran)
+        return grad_a, grad_b, None, None, None, None, None, None
+
+
+class FP8GemmBlockFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, a, b, a_t, b_t, trans_a, trans_b, out_dtype, config):
+        assert trans_a == False, "trans_a has to be False"  # noqa: E712
+        fdt = _get_fp8_dtype(config.format, True)
+        gran, bs = config.granularity, config.block_size
+        if isinstance(a, QuantizedTensor):
+            check_quantized_tensor(a, config, axis=-1)
+            a_row, a_row_s = a.qdata, a.scale_inv
+            if a_t is None:
+                a_t = QuantizedTensor.quantize(a.dequantize(), fdt, gran, axis=-2, block_size=bs)
+            a_col, a_col_s = a_t.qdata, a_t.scale_inv
+        else:
+            a_row, a_row_s, a_col, a_col_s = quantize_fp8_with_trans(a, fdt, gran, block_size=bs)
+        w_recipe = ScalingRecipe(use_2d_block=True)  # weight tiles serve forward and backward unchanged
+        if isinstance(b, QuantizedTensor):
+            check_quantized_tensor(b, config, scaling_recipe=w_recipe)
+            b_q, b_s = b.qdata, b.scale_inv
+        else:
+            b_q, b_s = quantize_fp8(b, fdt, gran, block_size=bs, scaling_recipe=w_recipe)
+        out = _gemm(a_row, a_row_s, trans_a, b_q, b_s, trans_b, out_dtype, False, gran)
+        ctx.save_for_backward(a_col, a_col_s, b_q, b_s)
+        ctx.meta = (trans_a, trans_b, out_dtype, config)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        trans_a, trans_b, out_dtype, config = ctx.meta
+        a_col, a_col_s, b_q, b_s = ctx.saved_tensors
+        gran = config.granularity
+        g_row, g_row_s, g_col, g_col_s = quantize_fp8_with_trans(
+            grad_out.contiguous(), _get_fp8_dtype(config.format, False), gran, block_size=config.block_size
+        )
+        grad_a = _gemm(g_row, g_row_s, False, b_q, b_s, not trans_b, out_dtype, False, gran)
+        grad_b = _gemm(a_col, a_col_s, not trans_a, g_col, g_col_s, False, out_dtype, trans_b, gran)
+        return grad_a, grad_b, None, None, None, None, None, None
+
+
+class FP8GemmMXFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, a, b, a_t, b_t, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum_pattern=None):
+        from primus_turbo.pytorch.kernels.quantization.quantization_impl import quantize_mxfp8_impl
+
+        ok, why = check_mxfp8_support()
+        assert ok, why
+        assert trans_a == False and trans_b == True, "trans_a has to be False and trans_b has to be True"  # noqa: E712
+        fuse, main_grad = _setup_fused_grad_accum(b, fuse_bgrad_accum_pattern)
+        fdt = _get_fp8_dtype(config.format, True)
+        gran, bs = config.granularity, config.block_size
+
+        def both_ways(x, x_t, recipe):
+            if isinstance(x, QuantizedTensor):
+                check_quantized_tensor(x, config, axis=-1, scaling_recipe=recipe)
+                if x_t is None:
+                    x_t = QuantizedTensor.quantize(x.dequantize(), x.real_dtype, gran, axis=-2, block_size=bs,
+                                                   scaling_recipe=recipe)
+                return x.qdata, x.scale_inv, x_t.qdata, x_t.scale_inv
+            return quantize_mxfp8_impl(x, fdt, None, bs, with_trans=True, scaling_recipe=recipe,
+                                       scaling_recipe_for_trans=recipe)
+
+        a_row, a_row_s, a_col, a_col_s = both_ways(a, a_t, ScalingRecipe())
+        b_row, b_row_s, b_col, b_col_s = both_ways(b, b_t, ScalingRecipe(use_2d_block=True))
+        out = _gemm(a_row, a_row_s, False, b_row, b_row_s, True, out_dtype, False, gran)
+        ctx.save_for_backward(a_col, a_col_s, b_col, b_col_s)
+        ctx.meta = (out_dtype, config, fuse, main_grad)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        from primus_turbo.pytorch.kernels.quantization.quantization_impl import quantize_mxfp8_impl
+
+        out_dtype, config, fuse, main_grad = ctx.meta
+        a_col, a_col_s, b_col, b_col_s = ctx.saved_tensors
+        gran = config.granularity
+        g = grad_out.reshape(grad_out.shape[0], -1).contiguous()
+        g_row, g_row_s, g_col, g_col_s = quantize_mxfp8_impl(
+            g, _get_fp8_dtype(config.format, False), None, config.block_size, with_trans=True,
+            scaling_recipe=ScalingRecipe(), scaling_recipe_for_trans=ScalingRecipe(),
+        )
+        # the two-direction casts are stored transposed, so dgrad and wgrad are NT GEMMs too
+        grad_a = _gemm(g_row, g_row_s, False, b_col, b_col_s, True, out_dtype, False, gran)
+        grad_b = _wgrad_gemm(g_col, g_col_s, False, a_col, a_col_s, True, out_dtype, False, gran,
+                             main_grad if fuse else None)
+        return grad_a, grad_b, None, None, None, None, None, None, None
+
+
+def gemm_fp8(
+    a: Union[torch.Tensor, QuantizedTensor, QuantizedTensorPair],
+    b: Union[torch.Tensor, QuantizedTensor, QuantizedTensorPair],
+    trans_a: bool = False,
+    trans_b: bool = False,
+    out_dtype: Optional[torch.dtype] = None,
+    config: Optional[Float8QuantConfig] = None,
+    fuse_bgrad_accum_pattern: Optional[str] = None,
+) -> torch.Tensor:
+    """FP8 GEMM with autograd: ``a`` is ``(M, K)``, ``b`` is ``(K, N)`` or, with
+    ``trans_b``, ``(N, K)``; returns ``(M, N)`` in ``out_dtype``.
+
+    ``config`` selects format (E4M3 / E5M2 / HYBRID) and granularity (TENSORWISE default,
+    ROWWISE, BLOCKWISE with ``block_size=128``, MX_BLOCKWISE with ``block_size=32`` and E8M0
+    scales). Operands may be pre-quantized ``QuantizedTensor`` / ``QuantizedTensorPair``.
+    ``fuse_bgrad_accum_pattern="megatron"`` (TENSORWISE and MX_BLOCKWISE) adds the weight
+    gradient into ``b.main_grad`` inside the wgrad GEMM epilogue.
+    """
+    if config is None:
+        config = Float8QuantConfig()
+    a_data, a_t = (a.data, a.data_t) if isinstance(a, QuantizedTensorPair) else (a, None)
+    b_data, b_t = (b.data, b.data_t) if isinstance(b, QuantizedTensorPair) else (b, None)
+    assert a_data.ndim == 2, "Only 2D tensors are supported"
+    assert b_data.ndim == 2, "Only 2D tensors are supported"
+    if out_dtype is None:
+        out_dtype = torch.promote_types(a_data.dtype, b_data.dtype)
+
+    g = config.granularity
+    if g == ScalingGranularity.TENSORWISE:
+        return FP8GemmTensorFunction.apply(a_data, b_data, a_t, b_t, trans_a, trans_b, out_dtype, config,
+                                           fuse_bgrad_accum_pattern)
+    if g == ScalingGranularity.MX_BLOCKWISE:
+        return FP8GemmMXFunction.apply(a_data, b_data, a_t, b_t, trans_a, trans_b, out_dtype, config,
+                                       fuse_bgrad_accum_pattern)
+    assert fuse_bgrad_accum_pattern is None, f"fuse_bgrad_accum_pattern is not supported for {g}"
+    if g == ScalingGranularity.ROWWISE:
+        return FP8GemmRowFunction.apply(a_data, b_data, a_t, b_t, trans_a, trans_b, out_dtype, config)
+    if g == ScalingGranularity.BLOCKWISE:
+        return FP8GemmBlockFunction.apply(a_data, b_data, a_t, b_t, trans_a, trans_b, out_dtype, config)
+    raise ValueError(f"Unsupported FP8 ScalingGranularity: {g}")
