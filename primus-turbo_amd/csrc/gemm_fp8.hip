@@ -88,6 +88,27 @@ static inline int64_t round_up(int64_t x, int64_t m) {
     return (x + m - 1) / m * m;
 }
 
+// The kernel wants K as a multiple of 128 and at least three 128-byte slabs.
+static inline int64_t padded_k(int64_t K) {
+    const int64_t kp = round_up(K, KSTEP);
+    return kp < 3 * KSTEP ? 3 * KSTEP : kp;
+}
+
+// zero `bytes` bytes at a 16-byte aligned address (a fill kernel rather than a memset node,
+// so that callers may capture the launch in a graph)
+__global__ __launch_bounds__(256) void zero16_kernel(u32x4 *p, int64_t n16, int64_t bytes) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i < n16) {
+        if ((i + 1) * 16 <= bytes) {
+            p[i] = u32x4{0u, 0u, 0u, 0u};
+        } else {
+            uint8_t *b = reinterpret_cast<uint8_t *>(p);
+            for (int64_t k = i * 16; k < bytes; ++k)
+                b[k] = 0;
+        }
+    }
+}
+
 } // namespace pt
 
 using namespace pt;
@@ -97,7 +118,7 @@ extern "C" {
 size_t pt_gemm_fp8_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans_a, int trans_b) {
     // An operand is copied into the workspace when its reduction axis is not contiguous
     // (transpose) or when K is not a multiple of 128 (zero padding of the K tail).
-    const int64_t Kp    = round_up(K, KSTEP);
+    const int64_t Kp    = padded_k(K);
     const bool    pad   = Kp != K;
     size_t        bytes = 0;
     if (trans_a || pad)
@@ -124,9 +145,19 @@ int pt_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const void *b,
     PT_REQUIRE(a && b && c && a_scale && b_scale, "NULL tensor pointer");
     PT_REQUIRE(aligned_to(a, 16) && aligned_to(b, 16) && aligned_to(c, 16), "operands must be 16-byte aligned");
     PT_REQUIRE(cdiv(M, 128) * cdiv(N, 128) < (1LL << 31), "too many tiles");
+    // the kernel addresses a tile's rows with 32-bit byte offsets: 255 rows x K must fit
+    PT_REQUIRE(K < (1LL << 24), "K must be below 2^24");
     auto st = static_cast<hipStream_t>(stream);
+    if (K == 0) { // empty sum
+        if (!accumulate) {
+            const int64_t n16 = cdiv(M * N * (c_dtype == PT_DTYPE_F32 ? 4 : 2), 16);
+            zero16_kernel<<<static_cast<unsigned>(cdiv(n16, 256)), 256, 0, st>>>(static_cast<u32x4 *>(c), n16, M * N * (c_dtype == PT_DTYPE_F32 ? 4 : 2));
+            return check_launch("zero16_kernel");
+        }
+        return PT_OK;
+    }
 
-    const int64_t  Kp  = round_up(K, KSTEP);
+    const int64_t  Kp  = padded_k(K);
     const bool     pad = Kp != K;
     const uint8_t *A   = static_cast<const uint8_t *>(a);
     const uint8_t *B   = static_cast<const uint8_t *>(b);

@@ -10,13 +10,13 @@
 //   * one workgroup = 4 wavefronts in a 2 x 2 grid; each wavefront owns a
 //     (16 TM) x (16 TN) sub-tile built from v_mfma_f32_16x16x128_f8f6f4;
 //   * K advances 128 bytes per step; A and B tiles go HBM/L2 -> LDS directly
-//     (global_load_lds_dwordx4, no VGPR staging) into a double buffer, so the loads of
-//     step k+1 fly during the MFMAs of step k and one barrier per step suffices;
+//     (global_load_lds_dwordx4, no VGPR staging) into a double buffer, requested two steps
+//     ahead; the MFMA operand fragments of step k+1 are read from LDS into a second
+//     register set while the last MFMAs of step k run; one barrier per step;
 //   * LDS rows are 128 B; the 16-byte chunk c of row r sits at chunk c ^ ((r >> 1) & 7),
 //     which makes the 16 lanes of an MFMA operand read hit 16 different bank groups;
 //   * the MFMA is issued with B as the "row" operand, so a lane ends up holding four
-//     consecutive n for one m; the epilogue regroups them through LDS into whole output
-//     rows and stores 16 bytes per lane;
+//     consecutive n for one m and stores them without any exchange between lanes;
 //   * workgroup ids are remapped so that the 8 XCDs (one L2 each) work on compact
 //     neighbourhoods of the tile grid.
 #pragma once
@@ -30,12 +30,6 @@
 #define PT_GEMM_TRACE_DECL
 #define PT_GEMM_TRACE_POINT(id)
 #endif
-// Development switch (timing experiments only, results are wrong when non-zero):
-// bit 0 = no tile prefetch inside the K loop, bit 1 = no MFMA, bit 2 = no fragment reads.
-#ifndef PT_GEMM_EXP
-#define PT_GEMM_EXP 0
-#endif
-
 namespace pt {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -70,25 +64,10 @@ __device__ __forceinline__ int swz(int row) {
 typedef __attribute__((address_space(3))) void       *lds_ptr_t;
 typedef const __attribute__((address_space(1))) void *glb_ptr_t;
 
-// Copy `ROWS` rows x 128 bytes from global (row stride ld bytes) into LDS, swizzled.
-// Each wave instruction moves 8 rows (1 KB); rows at or beyond `rows_valid` re-read the
-// last valid row (their products are never stored).
-template <int ROWS>
-__device__ __forceinline__ void tile_to_lds(const uint8_t *__restrict__ g, int64_t ld,
-                                            int rows_valid, uint8_t *lds, int wave, int lane) {
-    constexpr int INSTR = ROWS / 8 / GEMM_WAVES;
-    const int     lrow  = lane >> 3; // row within the 8-row group
-    const int     pchk  = lane & 7;  // physical chunk this lane fills
-#pragma unroll
-    for (int j = 0; j < INSTR; ++j) {
-        const int r8  = j * GEMM_WAVES + wave;
-        int       row = r8 * 8 + lrow;
-        const int lch = pchk ^ swz(row);
-        int       src = row < rows_valid ? row : rows_valid - 1;
-        const uint8_t *p = g + static_cast<int64_t>(src) * ld + lch * 16;
-        __builtin_amdgcn_global_load_lds((glb_ptr_t)p, (lds_ptr_t)(lds + r8 * 1024), 16, 0, 0);
-    }
-}
+// Direct-to-LDS copies: each wave instruction moves 8 tile rows x 128 B = 1 KB to
+// contiguous LDS; lane l fills physical chunk l % 8 of row l / 8, reading the logical chunk
+// that the swizzle maps there. Rows at or beyond the matrix edge re-read the last valid
+// row (their products are never stored).
 
 // MFMA operand fragment of 16 tile rows: lane (r = lane % 16, g = lane / 16) takes K bytes
 // [16g, 16g+16) and [64+16g, 64+16g+16) of row r, i.e. two 16-byte LDS reads. The swizzle
@@ -140,30 +119,6 @@ __device__ __forceinline__ f32x4 mfma_fp8(const i32x8 &rowop, const i32x8 &colop
                                                             0, 0x7f7f7f7f);
 }
 
-template <typename T> __device__ __forceinline__ void store4(T *p, f32x4 v, bool vec4, int nvalid, bool accumulate) {
-    if (accumulate) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-            if (e < nvalid)
-                v[e] += HP<T>::to_f32(p[e]);
-    }
-    if (vec4) {
-        if constexpr (sizeof(T) == 4) {
-            *reinterpret_cast<f32x4 *>(p) = v;
-        } else {
-            u32x2 o;
-            o.x = pack2<T>(v[0], v[1]);
-            o.y = pack2<T>(v[2], v[3]);
-            *reinterpret_cast<u32x2 *>(p) = o;
-        }
-    } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-            if (e < nvalid)
-                p[e] = HP<T>::from_f32(v[e]);
-    }
-}
-
 // Tile coordinates of a workgroup: XCD-contiguous ids, then groups of GROUP_M tile rows
 // walked column-major so that concurrently running tiles share A and B panels in L2.
 __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, int &tm, int &tn) {
@@ -187,126 +142,145 @@ __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, i
     tn                 = r / gsz;
 }
 
-// Epilogue. A lane holds, for tile (i, j), C[wm_base + 16 i + lm][wn_base + 16 j + 4 lg + e],
-// e = 0..3: written directly that is 32-byte pieces scattered over 16 rows per instruction.
-// Instead every wavefront passes its sub-tile, 16 rows x 64 (or 32) columns (fp32) at a time,
-// through a private LDS strip and writes it back out row-wise: a lane scales, converts
-// and stores 16 bytes of one row, so HBM sees full 128-byte lines.
-// Strip width: 64 columns where one workgroup per CU leaves room for it, 32 columns for the
-// 128 x 128 tile so that two workgroups still fit into the 160 KB of LDS.
-template <int TM, int TN> struct EpiGeom {
-    static constexpr int COLS  = (TM * TN >= 32) ? 64 : 32;
-    static constexpr int ROWB  = COLS * 4 + 16; // padded LDS row pitch in bytes
-    static constexpr int BYTES = 16 * ROWB;     // per wavefront
-};
-
-template <typename T, int TM, int TN, int MODE>
-__device__ __forceinline__ void epilogue(const GemmArgs &a, const f32x4 (&acc)[TM][TN],
-                                         int64_t wm_base, int64_t wn_base, int lane,
-                                         uint8_t *strip) {
-    constexpr int EPI_COLS = EpiGeom<TM, TN>::COLS, EPI_ROWB = EpiGeom<TM, TN>::ROWB;
-    constexpr int ES  = sizeof(T);
-    constexpr int EPC = 16 / ES;        // output elements per 16-byte chunk
-    constexpr int CPR = EPI_COLS / EPC; // chunks per strip row
-    constexpr int RPI = 64 / CPR;       // rows written per store instruction
-    constexpr int JH  = EPI_COLS / 16;  // MFMA tiles per strip width
-    static_assert(TN % JH == 0, "sub-tile width must be a multiple of the strip width");
-    const int  lm = lane & 15, lg = lane >> 4;
-    T         *C    = static_cast<T *>(a.C);
-    const bool accu = a.accumulate != 0;
-    // 16-byte global accesses need every row start on a 16-byte boundary
-    const bool vec  = (a.N * ES) % 16 == 0;
-    const int  crow = lane / CPR, cchk = lane % CPR; // this lane's (row, chunk) in the write-out
-    // VECTOR mode: fetch every scale this lane will need before the first store is issued
-    // (a load issued behind stores cannot complete before they are acknowledged)
-    constexpr int NR = 16 / RPI, NH = TN / JH;
-    [[maybe_unused]] float sa_e[TM][NR], sb_e[NH][EPC];
-    if constexpr (MODE == SCALE_VECTOR) {
+// Epilogue. A lane holds, for MFMA tile (i, j), C[wm_base + 16 i + lm][wn_base + 16 j + 4 lg + e],
+// e = 0..3. It scales, converts and stores those four values itself (8 bytes of bf16/fp16,
+// 16 bytes of fp32): per instruction the wavefront writes 16 rows x 32 (64) contiguous bytes,
+// the neighbouring j tiles complete the 128-byte lines in the write-back L2, and the
+// accumulators need no exchange between lanes, which keeps the instruction count per
+// output near its minimum (two multiplies and half a convert).
+//
+// One straight-line loop nest per output type serves sub-tiles that lie wholly inside the
+// matrix with aligned rows; a generic nest (per-element bounds checks, run-time type)
+// serves the rest. The accumulators are read with hand-written v_accvgpr_read where they
+// are needed: left to itself the compiler copies all of them out of the AGPRs ahead of the
+// case distinction and spills everything else.
+template <bool ACC_IN_AGPR> __device__ __forceinline__ f32x4 read_acc(const f32x4 &c) {
+    f32x4 v;
+    if constexpr (ACC_IN_AGPR) {
+#if defined(__HIP_DEVICE_COMPILE__) // the host pass cannot parse the AGPR constraint
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int q = 0; q < NR; ++q) {
-                const int64_t m = wm_base + i * 16 + q * RPI + crow;
-                sa_e[i][q]      = a.sA[(m < a.M ? m : a.M - 1) * a.sa_m];
-            }
-#pragma unroll
-        for (int h = 0; h < NH; ++h)
-#pragma unroll
-            for (int e = 0; e < EPC; ++e) {
-                const int64_t ne = wn_base + h * EPI_COLS + cchk * EPC + e;
-                sb_e[h][e]       = a.sB[(ne < a.N ? ne : a.N - 1) * a.sb_n];
-            }
+        for (int e = 0; e < 4; ++e)
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[e]) : "a"(c[e]));
+#endif
+    } else {
+        v = c;
     }
+    return v;
+}
+
+template <typename T, int TM, int TN, int MODE, bool ACC_IN_AGPR>
+__device__ __forceinline__ void epilogue_inner(T *row, int64_t step, bool accu, const f32x4 (&acc)[TM][TN],
+                                               const float (&sa)[TM], const f32x4 (&sb)[TN]) {
+    static_for<0, TM>([&](auto ic) {
+        constexpr int i = ic;
+        static_for<0, TN>([&](auto jc) {
+            constexpr int j = jc;
+            f32x4         v = read_acc<ACC_IN_AGPR>(acc[i][j]);
+            if constexpr (MODE == SCALE_VECTOR) {
 #pragma unroll
-    for (int h = 0; h < NH; ++h) {
-        const int64_t n = wn_base + h * EPI_COLS + cchk * EPC;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            // 1. accumulators -> LDS strip [16][64] fp32
-#pragma unroll
-            for (int jj = 0; jj < JH; ++jj)
-                *reinterpret_cast<f32x4 *>(strip + lm * EPI_ROWB + (jj * 16 + lg * 4) * 4) = acc[i][h * JH + jj];
-            // 2. LDS strip -> global, row-wise (the same wavefront wrote and reads; LDS keeps
-            //    its accesses in program order)
-#pragma unroll
-            for (int r0 = 0; r0 < 16; r0 += RPI) {
-                const int     r = r0 + crow;
-                const int64_t m = wm_base + i * 16 + r;
-                float         f[EPC];
-#pragma unroll
-                for (int q = 0; q < EPC / 4; ++q) {
-                    const f32x4 t = *reinterpret_cast<const f32x4 *>(strip + r * EPI_ROWB + (cchk * EPC + q * 4) * 4);
-                    f[4 * q] = t[0]; f[4 * q + 1] = t[1]; f[4 * q + 2] = t[2]; f[4 * q + 3] = t[3];
-                }
-                if (m < a.M && n < a.N) {
-                    if constexpr (MODE == SCALE_VECTOR) {
-                        const float sa = sa_e[i][r0 / RPI];
-#pragma unroll
-                        for (int e = 0; e < EPC; ++e)
-                            f[e] = f[e] * sa * sb_e[h][e];
-                    }
-                    T *gp = C + m * a.N + n;
-                    if (vec && n + EPC <= a.N) {
-                        if (accu) {
-                            const u32x4 old = ld128(gp);
-                            if constexpr (ES == 4) {
-                                f[0] += __uint_as_float(old.x); f[1] += __uint_as_float(old.y);
-                                f[2] += __uint_as_float(old.z); f[3] += __uint_as_float(old.w);
-                            } else {
-                                const uint32_t ow[4] = {old.x, old.y, old.z, old.w};
-#pragma unroll
-                                for (int q = 0; q < 4; ++q) {
-                                    float o0, o1;
-                                    unpack2<T>(ow[q], o0, o1);
-                                    f[2 * q] += o0;
-                                    f[2 * q + 1] += o1;
-                                }
-                            }
-                        }
-                        u32x4 w;
-                        if constexpr (ES == 4) {
-                            w = u32x4{__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3])};
-                        } else {
-                            w = u32x4{pack2<T>(f[0], f[1]), pack2<T>(f[2], f[3]), pack2<T>(f[4], f[5]), pack2<T>(f[6], f[7])};
-                        }
-                        st128(gp, w);
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < EPC; ++e)
-                            if (n + e < a.N) {
-                                float v = f[e];
-                                if (accu)
-                                    v += HP<T>::to_f32(gp[e]);
-                                gp[e] = HP<T>::from_f32(v);
-                            }
-                    }
-                }
+                for (int e = 0; e < 4; ++e)
+                    v[e] = v[e] * sa[i] * sb[j][e];
             }
-        }
+            T *q = row + j * 16;
+            if constexpr (sizeof(T) == 4) {
+                if (accu)
+                    v += *reinterpret_cast<const f32x4 *>(q);
+                *reinterpret_cast<f32x4 *>(q) = v;
+            } else {
+                if (accu) {
+                    const u32x2 old = *reinterpret_cast<const u32x2 *>(q);
+                    float       o0, o1, o2, o3;
+                    unpack2<T>(old.x, o0, o1);
+                    unpack2<T>(old.y, o2, o3);
+                    v[0] += o0; v[1] += o1; v[2] += o2; v[3] += o3;
+                }
+                u32x2 w;
+                w.x = pack2<T>(v[0], v[1]);
+                w.y = pack2<T>(v[2], v[3]);
+                *reinterpret_cast<u32x2 *>(q) = w;
+            }
+            // keep each accumulator's read next to its store (register pressure)
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        row += step;
+    });
+}
+
+__device__ __forceinline__ void store_elem(float f, uint8_t *q, int out_dtype, bool accu) {
+    if (out_dtype == PT_DTYPE_F32) {
+        float *p = reinterpret_cast<float *>(q);
+        *p       = accu ? f + *p : f;
+    } else if (out_dtype == PT_DTYPE_BF16) {
+        bf16_t *p = reinterpret_cast<bf16_t *>(q);
+        *p        = HP<bf16_t>::from_f32(accu ? f + HP<bf16_t>::to_f32(*p) : f);
+    } else {
+        f16_t *p = reinterpret_cast<f16_t *>(q);
+        *p       = HP<f16_t>::from_f32(accu ? f + HP<f16_t>::to_f32(*p) : f);
     }
 }
 
-// Where a workgroup's current tile lives.
+template <int TM, int TN, int MODE, bool ACC_IN_AGPR>
+__device__ __forceinline__ void epilogue(const GemmArgs &a, const f32x4 (&acc)[TM][TN],
+                                         int64_t wm_base, int64_t wn_base, int lane) {
+    const int     ES = a.out_dtype == PT_DTYPE_F32 ? 4 : 2;
+    const int     lm = lane & 15, lg = lane >> 4;
+    uint8_t      *C    = static_cast<uint8_t *>(a.C);
+    const bool    accu = a.accumulate != 0;
+    const int64_t m0 = wm_base + lm, n0 = wn_base + lg * 4;
+
+    [[maybe_unused]] float sa[TM];
+    [[maybe_unused]] f32x4 sb[TN];
+    if constexpr (MODE == SCALE_VECTOR) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int64_t m = m0 + i * 16;
+            sa[i]           = a.sA[(m < a.M ? m : a.M - 1) * a.sa_m];
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int64_t n = n0 + j * 16 + e;
+                sb[j][e]        = a.sB[(n < a.N ? n : a.N - 1) * a.sb_n];
+            }
+    }
+    // whole sub-tile inside the matrix and every 4-element group aligned: no per-element checks
+    const bool fast = wm_base + TM * 16 <= a.M && wn_base + TN * 16 <= a.N && (a.N & 3) == 0 &&
+                      (reinterpret_cast<uintptr_t>(C) & 15) == 0;
+    uint8_t      *row  = C + (m0 * a.N + n0) * ES;
+    const int64_t step = 16 * a.N;
+    if (fast) {
+        if (a.out_dtype == PT_DTYPE_BF16)
+            epilogue_inner<bf16_t, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<bf16_t *>(row), step, accu, acc, sa, sb);
+        else if (a.out_dtype == PT_DTYPE_F16)
+            epilogue_inner<f16_t, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<f16_t *>(row), step, accu, acc, sa, sb);
+        else
+            epilogue_inner<float, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<float *>(row), step, accu, acc, sa, sb);
+    } else {
+        static_for<0, TM>([&](auto ic) {
+            constexpr int i = ic;
+            static_for<0, TN>([&](auto jc) {
+                constexpr int j = jc;
+                f32x4         v = read_acc<ACC_IN_AGPR>(acc[i][j]);
+                if constexpr (MODE == SCALE_VECTOR) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        v[e] = v[e] * sa[i] * sb[j][e];
+                }
+                if (m0 + i * 16 < a.M) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (n0 + j * 16 + e < a.N)
+                            store_elem(v[e], row + (j * 16 + e) * ES, a.out_dtype, accu);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            row += step * ES;
+        });
+    }
+}
+
+// Where a workgroup's tile lives.
 struct TileCtx {
     const uint8_t *Ag, *Bg; // first row of the tile in A / B
     int            rows_a, rows_b;
@@ -328,16 +302,31 @@ __device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile) {
 }
 
 // Persistent kernel: the grid is sized to the machine and every workgroup walks tiles
-// blockIdx.x, blockIdx.x + gridDim.x, ... . The K pipeline runs across tile boundaries: the
-// first K slab of the next tile is already being loaded while the current tile's last
-// slab is multiplied and its result written out, so the matrix cores only pause for the
-// epilogue's own instructions.
+// blockIdx.x, blockIdx.x + gridDim.x, ... as one uninterrupted sequence of K steps
+// ("slabs" of 128 bytes of K, double-buffered in LDS stages s % 2). With one wavefront per
+// SIMD nothing hides a stall, so a slab is scheduled such that no MFMA ever waits for an
+// LDS round trip:
+//   * the A fragments of a wavefront's sub-tile live in one register set, the B fragments
+//     stream through a ring of four; every LDS read is issued at least one fragment
+//     (8 MFMAs) before its first use;
+//   * the MFMA tiles (i, j) are walked column by column up to column TN - 3; then the stage
+//     is released (barrier: everyone is done reading it and everyone's part of the next slab
+//     has landed), and the last two columns are walked row by row: after (i, TN-2), (i, TN-1)
+//     A fragment i is dead and is refilled at once from the next slab, together with a share
+//     of the copies that bring the slab after that into the stage just released;
+//   * tile boundaries do not drain the pipeline: while a tile's result is written out, the
+//     first fragments of the next tile are already in registers and its second slab is in
+//     flight.
 template <int TM, int TN, int MODE, bool SB_VEC, int FA, int FB>
 __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
+    static_assert(TN % 4 == 0, "the B fragment ring assumes TN = 4 or 8");
     constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
     constexpr int A_BYTES = BM * KSTEP, B_BYTES = BN * KSTEP, STAGE = A_BYTES + B_BYTES;
+    constexpr int LA = BM / 8 / GEMM_WAVES, LB = BN / 8 / GEMM_WAVES; // copies per wave and slab
+    constexpr int NL  = LA + LB;
+    constexpr int JR  = TN - 2; // columns [0, JR) before the release point, [JR, TN) after
+    constexpr int NSB = SB_VEC ? 4 : 1;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-    uint8_t *strips = smem + 2 * STAGE; // epilogue staging, outside the pipeline buffers
 
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
@@ -352,18 +341,61 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     const int total = a.tiles_m * a.tiles_n;
     const int KT    = static_cast<int>(a.K / KSTEP);
     int       tile  = blockIdx.x;
-    if (tile >= total)
+    if (tile >= total || KT < 3)
         return;
     TileCtx cur_t = make_tile<BM, BN>(a, tile);
 
-    f32x4 acc[TM][TN];
+    // ---- loader: two slabs ahead of the MFMAs ----
+    // Copies are buffer loads: a lane's offset inside a slab (row * pitch + swizzled chunk)
+    // is the same for every tile; the tile and the K position live in the (uniform) buffer
+    // descriptor, whose size makes rows beyond the matrix edge read as zero. The loader
+    // therefore changes tile by swapping scalars -- no branch in the K loop, which the
+    // compiler would use to sink MFMAs -- and it does so after requesting the tile's last
+    // slab, at step KT - 3 of the MFMAs (the host guarantees KT >= 3).
+    uint32_t off[NL];
+    {
+        const int lrow = lane >> 3, pchk = lane & 7;
+#pragma unroll
+        for (int j = 0; j < NL; ++j) {
+            const bool isA = j < LA;
+            const int  row = ((isA ? j : j - LA) * GEMM_WAVES + wave) * 8 + lrow;
+            off[j] = static_cast<uint32_t>(row * (isA ? a.lda : a.ldb)) + ((pchk ^ swz(row)) << 4);
+        }
+    }
+    const uint8_t *ld_ga = cur_t.Ag, *ld_gb = cur_t.Bg; // slab the loader points at
+    uint32_t       ld_na = cur_t.rows_a * static_cast<uint32_t>(a.lda); // bytes from there to the
+    uint32_t       ld_nb = cur_t.rows_b * static_cast<uint32_t>(a.ldb); // end of the tile's rows
+    int            ld_kt = 0;
+    TileCtx        nxt_t = cur_t; // tile after the MFMAs' tile (the same tile after the last one)
+    // copy number L of the loader's slab into stage `b`
+    auto issue_copy = [&](auto lc, int b) {
+        constexpr int L   = lc;
+        uint8_t      *dst = smem + b * STAGE;
+#if defined(__HIP_DEVICE_COMPILE__) // the buffer resource type only exists in the device pass
+        constexpr uint32_t RSRC_FLAGS = 0x00020000; // raw buffer, 32-bit data format
+        if constexpr (L < LA) {
+            __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(ld_ga), 0, ld_na, RSRC_FLAGS);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr_t)(dst + (L * GEMM_WAVES + wave) * 1024), 16, off[L], 0, 0, 0);
+        } else {
+            __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(ld_gb), 0, ld_nb, RSRC_FLAGS);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr_t)(dst + A_BYTES + ((L - LA) * GEMM_WAVES + wave) * 1024), 16, off[L], 0, 0, 0);
+        }
+#endif
+    };
+    auto advance_loader = [&]() {
+        const bool wrap = ld_kt + 1 == KT;
+        ld_kt = wrap ? 0 : ld_kt + 1;
+        ld_ga = wrap ? nxt_t.Ag : ld_ga + KSTEP;
+        ld_gb = wrap ? nxt_t.Bg : ld_gb + KSTEP;
+        ld_na = wrap ? nxt_t.rows_a * static_cast<uint32_t>(a.lda) : ld_na - KSTEP;
+        ld_nb = wrap ? nxt_t.rows_b * static_cast<uint32_t>(a.ldb) : ld_nb - KSTEP;
+    };
 
-    // BLOCK mode: the fp32 scales of the next K block are fetched one step ahead (before
-    // the tile prefetch is issued, so that the tile loads stay the youngest entries of the
-    // vector-memory counter) and are in registers when their step starts.
-    [[maybe_unused]] float sa_cur[TM], sa_nxt[TM];
-    [[maybe_unused]] float sb_cur[TN][SB_VEC ? 4 : 1], sb_nxt[TN][SB_VEC ? 4 : 1];
-    auto fetch_scales = [&](const TileCtx &t, int kt, float (&sa)[TM], float (&sb)[TN][SB_VEC ? 4 : 1]) {
+    // BLOCK mode: the fp32 scales of a K block are fetched one slab ahead, at the release
+    // point and before that slab's tile copies are issued (so the copies stay the youngest
+    // entries of the vector-memory counter).
+    [[maybe_unused]] float sa_cur[TM], sa_nxt[TM], sb_cur[TN][NSB], sb_nxt[TN][NSB];
+    auto fetch_scales = [&](const TileCtx &t, int kt, float (&sa)[TM], float (&sb)[TN][NSB]) {
         if constexpr (MODE == SCALE_BLOCK) {
             const int64_t wm_base = t.m0 + wm * (TM * 16), wn_base = t.n0 + wn * (TN * 16);
 #pragma unroll
@@ -390,18 +422,41 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             }
         }
     };
-    auto load_stage = [&](const TileCtx &t, int kt, uint8_t *buf) {
-        tile_to_lds<BM>(t.Ag + static_cast<int64_t>(kt) * KSTEP, a.lda, t.rows_a, buf, wave, lane);
-        tile_to_lds<BN>(t.Bg + static_cast<int64_t>(kt) * KSTEP, a.ldb, t.rows_b, buf + A_BYTES, wave, lane);
-    };
 
-    int buf = 0;
+    f32x4 acc[TM][TN];
+    // MFMA operand fragments (8 VGPRs each). Loop-carried: fa = the A fragments of the slab
+    // about to be multiplied, fb[0] and fb[1] = its first two B fragments.
+    i32x8 fa[TM], fb[4];
+    int   buf = 0;
+
+    // fragment f (16 rows) of the A or B part of a stage: two 16-byte LDS reads per lane
+    auto ldfrag = [&](const uint8_t *part, int f) {
+        const uint8_t *p  = part + f * 16 * KSTEP;
+        const u32x4    lo = *reinterpret_cast<const u32x4 *>(p + frag_off_lo);
+        const u32x4    hh = *reinterpret_cast<const u32x4 *>(p + frag_off_hi);
+        i32x8          r;
+        r[0] = lo.x; r[1] = lo.y; r[2] = lo.z; r[3] = lo.w;
+        r[4] = hh.x; r[5] = hh.y; r[6] = hh.z; r[7] = hh.w;
+        return r;
+    };
+    const uint32_t a_part = wm * (TM * 16) * KSTEP;
+    const uint32_t b_part = A_BYTES + wn * (TN * 16) * KSTEP;
+
+    // ---- prologue: slabs 0 and 1 requested, the first fragments of slab 0 on their way ----
     PT_GEMM_TRACE_DECL;
     PT_GEMM_TRACE_POINT(0);
-    if (KT > 0) {
-        fetch_scales(cur_t, 0, sa_nxt, sb_nxt);
-        load_stage(cur_t, 0, smem);
-    }
+    fetch_scales(cur_t, 0, sa_nxt, sb_nxt);
+    static_for<0, NL>([&](auto l) { issue_copy(l, 0); });
+    advance_loader();
+    static_for<0, NL>([&](auto l) { issue_copy(l, 1); });
+    advance_loader();
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
+    __builtin_amdgcn_s_barrier();
+    fb[0] = ldfrag(smem + b_part, 0);
+    fb[1] = ldfrag(smem + b_part, 1);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+        fa[i] = ldfrag(smem + a_part, i);
 
     while (true) {
 #pragma unroll
@@ -411,17 +466,15 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                 acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
         const int next_tile = tile + gridDim.x;
-        TileCtx   nxt_t     = cur_t;
+        nxt_t               = cur_t;
         if (next_tile < total)
             nxt_t = make_tile<BM, BN>(a, next_tile);
 
+        // one K slab per iteration; the body must stay a single basic block (no branches), or
+        // the compiler sinks the MFMAs behind them
         for (int kt = 0; kt < KT; ++kt) {
-            uint8_t *cur = smem + buf * STAGE;
-            PT_GEMM_TRACE_POINT(1);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            PT_GEMM_TRACE_POINT(2);
-            __builtin_amdgcn_s_barrier();
-            PT_GEMM_TRACE_POINT(3);
+            const uint8_t *cur = smem + buf * STAGE;
+            const uint8_t *nxt = smem + (buf ^ 1) * STAGE;
             if constexpr (MODE == SCALE_BLOCK) {
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
@@ -429,43 +482,19 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
 #pragma unroll
-                    for (int e = 0; e < (SB_VEC ? 4 : 1); ++e)
+                    for (int e = 0; e < NSB; ++e)
                         sb_cur[j][e] = sb_nxt[j][e];
             }
-            // prefetch the next step of the pipeline: same tile, or the next tile's first slab
-            if ((PT_GEMM_EXP & 1) && kt > 0) {
-            } else if (kt + 1 < KT) {
-                fetch_scales(cur_t, kt + 1, sa_nxt, sb_nxt);
-                load_stage(cur_t, kt + 1, smem + (buf ^ 1) * STAGE);
-            } else if (next_tile < total) {
-                fetch_scales(nxt_t, 0, sa_nxt, sb_nxt);
-                load_stage(nxt_t, 0, smem + (buf ^ 1) * STAGE);
-            }
-            // lane addresses of the A / B fragments of this wavefront in the current stage
-            const uint32_t la = lds_addr(cur) + wm * (TM * 16) * KSTEP + frag_off_lo;
-            const uint32_t lb = lds_addr(cur) + A_BYTES + wn * (TN * 16) * KSTEP + frag_off_lo;
-            const uint32_t hi = frag_off_hi - frag_off_lo; // same for A and B
 
-            Frag fa[TM], fb[2];
-            if ((PT_GEMM_EXP & 4) && kt > 0) {
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-                    fa[i].lo = fa[i].hi = u32x4{la, lb, hi, (uint32_t)kt};
-                fb[0].lo = fb[0].hi = fb[1].lo = fb[1].hi = u32x4{la, lb, hi, (uint32_t)kt};
-            } else {
-            static_for<0, TM>([&](auto i) { frag_issue<i * 16 * KSTEP>(fa[i], la, la + hi); });
-            frag_issue<0>(fb[0], lb, lb + hi);
-            if constexpr (TN > 1)
-                frag_issue<16 * KSTEP>(fb[1], lb, lb + hi);
-            }
-            i32x8 af[TM];
-
+            // BLOCK mode: MFMA t (in issue order) writes ring[t % RING]; DEPTH MFMAs later its
+            // product is folded into the running sum with the block scales (VALU work in
+            // the shadow of later MFMAs).
             [[maybe_unused]] constexpr int DEPTH = 2, RING = DEPTH + 1, TILES = TM * TN;
             [[maybe_unused]] f32x4 ring[RING];
+            // issue order -> tile: columns [0, JR) column-major, then rows of the last two columns
             [[maybe_unused]] auto  fold = [&](int t) {
-                // BLOCK mode: fold the finished product of one 128-wide K block into the
-                // running sum with its block scale (VALU work in the shadow of later MFMAs)
-                const int    i = t % TM, j = t / TM;
+                const int    i = t < JR * TM ? t % TM : (t - JR * TM) / 2;
+                const int    j = t < JR * TM ? t / TM : JR + (t - JR * TM) % 2;
                 const f32x4 &p = ring[t % RING];
                 if constexpr (SB_VEC) {
 #pragma unroll
@@ -478,58 +507,70 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                         acc[i][j][e] = fmaf(p[e], sc, acc[i][j][e]);
                 }
             };
+            auto mma = [&](int t, int i, int j, const i32x8 &af, const i32x8 &bf) {
+                if constexpr (MODE == SCALE_BLOCK) {
+                    ring[t % RING] = mfma_fp8<FA, FB>(bf, af, f32x4{0.f, 0.f, 0.f, 0.f});
+                    if (t >= DEPTH)
+                        fold(t - DEPTH);
+                } else {
+                    acc[i][j] = mfma_fp8<FA, FB>(bf, af, acc[i][j]);
+                }
+            };
 
-            static_for<0, TN>([&](auto jc) {
-                constexpr int j = jc;
-                // B fragment j (and, for j == 0, every A fragment) must have landed; the two
-                // reads of fragment j + 1 may still be in flight
-                if constexpr (j + 1 < TN)
-                    frag_wait<2>();
-                else
-                    frag_wait<0>();
-                if constexpr (j == 0) {
+            // ---- columns 0 .. JR-1: B fragment j + 2 is requested before column j is multiplied ----
 #pragma unroll
-                    for (int i = 0; i < TM; ++i)
-                        af[i] = frag_ready(fa[i]);
-                }
-                const i32x8 bf = frag_ready(fb[j & 1]);
+            for (int j = 0; j < JR; ++j) {
+                fb[(j + 2) % 4] = ldfrag(cur + b_part, j + 2);
+                // keep the instruction scheduler from moving MFMAs and LDS reads across each other
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int i = 0; i < TM; ++i) {
-                    if constexpr (MODE == SCALE_BLOCK) {
-                        const int t    = j * TM + i;
-                        ring[t % RING] = mfma_fp8<FA, FB>(bf, af[i], f32x4{0.f, 0.f, 0.f, 0.f});
-                        if (t >= DEPTH)
-                            fold(t - DEPTH);
-                    } else if (PT_GEMM_EXP & 2) {
-                        acc[i][j][0] += __builtin_bit_cast(float, bf[i & 7] ^ af[i][j & 7]);
-                    } else {
-                        acc[i][j] = mfma_fp8<FA, FB>(bf, af[i], acc[i][j]);
-                    }
-                }
-                if constexpr (j + 2 < TN) {
-                    if (!((PT_GEMM_EXP & 4) && kt > 0))
-                        frag_issue<(j + 2) * 16 * KSTEP>(fb[j & 1], lb, lb + hi);
-                }
+                for (int i = 0; i < TM; ++i)
+                    mma(j * TM + i, i, j, fa[i], fb[j % 4]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+
+            // ---- release point ----
+            // my reads of this stage are done and my copies of the next slab have landed
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            PT_GEMM_TRACE_POINT(3);
+            // (after the last slab of the last tile the following fetch and read leftovers: harmless)
+            if constexpr (MODE == SCALE_BLOCK) {
+                const bool same = kt + 1 < KT;
+                TileCtx    st   = nxt_t;
+                st.m0           = same ? cur_t.m0 : nxt_t.m0;
+                st.n0           = same ? cur_t.n0 : nxt_t.n0;
+                fetch_scales(st, same ? kt + 1 : 0, sa_nxt, sb_nxt);
+            }
+            fb[0] = ldfrag(nxt + b_part, 0);
+            fb[1] = ldfrag(nxt + b_part, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- last two columns, row by row: A fragment i is refilled as soon as it is dead ----
+            static_for<0, TM>([&](auto ic) {
+                constexpr int i = ic;
+                mma(JR * TM + 2 * i, i, JR, fa[i], fb[JR % 4]);
+                mma(JR * TM + 2 * i + 1, i, JR + 1, fa[i], fb[(JR + 1) % 4]);
+                __builtin_amdgcn_sched_barrier(0);
+                fa[i] = ldfrag(nxt + a_part, i);
+                static_for<i * NL / TM, (i + 1) * NL / TM>([&](auto l) { issue_copy(l, buf); });
+                __builtin_amdgcn_sched_barrier(0);
             });
             if constexpr (MODE == SCALE_BLOCK) {
 #pragma unroll
                 for (int t = TILES - DEPTH; t < TILES; ++t)
                     fold(t);
             }
+            advance_loader();
             buf ^= 1;
-            PT_GEMM_TRACE_POINT(4);
         }
 
+        // the epilogue reads the accumulators with hand-written instructions the compiler's
+        // hazard tracking does not see: let the last MFMA's write-back finish first
+        if constexpr (MODE == SCALE_VECTOR)
+            asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
         PT_GEMM_TRACE_POINT(5);
-        // epilogue through this wavefront's private strip (no workgroup barrier needed)
         const int64_t wm_base = cur_t.m0 + wm * (TM * 16), wn_base = cur_t.n0 + wn * (TN * 16);
-        uint8_t      *strip   = strips + wave * EpiGeom<TM, TN>::BYTES;
-        if (a.out_dtype == PT_DTYPE_BF16)
-            epilogue<bf16_t, TM, TN, MODE>(a, acc, wm_base, wn_base, lane, strip);
-        else if (a.out_dtype == PT_DTYPE_F16)
-            epilogue<f16_t, TM, TN, MODE>(a, acc, wm_base, wn_base, lane, strip);
-        else
-            epilogue<float, TM, TN, MODE>(a, acc, wm_base, wn_base, lane, strip);
+        epilogue<TM, TN, MODE, MODE == SCALE_VECTOR>(a, acc, wm_base, wn_base, lane);
 
         PT_GEMM_TRACE_POINT(6);
         if (next_tile >= total)
@@ -537,12 +578,14 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         tile  = next_tile;
         cur_t = nxt_t;
     }
+    // no copy into this workgroup's LDS may still be in flight when the LDS is handed on
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 template <int TM, int TN, int MODE, bool SB_VEC, int FA, int FB>
 static int launch_gemm_cfg(const GemmArgs &args_in, hipStream_t stream) {
     constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
-    constexpr int LDS = 2 * (BM + BN) * KSTEP + GEMM_WAVES * EpiGeom<TM, TN>::BYTES;
+    constexpr int LDS = 2 * (BM + BN) * KSTEP;
     GemmArgs      a   = args_in;
     a.tiles_m         = static_cast<int>(cdiv(a.M, BM));
     a.tiles_n         = static_cast<int>(cdiv(a.N, BN));

@@ -61,16 +61,10 @@ template <> struct HP<bf16_t> {
     static __device__ __forceinline__ float to_f32(bf16_t x) {
         return __uint_as_float(static_cast<uint32_t>(x.bits) << 16);
     }
-    // round-to-nearest-even, NaN stays NaN
+    // round-to-nearest-even in hardware (v_cvt_pk_bf16_f32), NaN stays NaN
     static __device__ __forceinline__ bf16_t from_f32(float f) {
-        uint32_t u = __float_as_uint(f);
-        bf16_t   r;
-        if ((u & 0x7fffffffu) > 0x7f800000u) {
-            r.bits = static_cast<uint16_t>((u >> 16) | 0x0040u);
-        } else {
-            u += 0x7fffu + ((u >> 16) & 1u);
-            r.bits = static_cast<uint16_t>(u >> 16);
-        }
+        bf16_t r;
+        r.bits = __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
         return r;
     }
 };
@@ -225,15 +219,14 @@ template <> __device__ __forceinline__ void unpack2<f16_t>(uint32_t w, float &a,
 
 template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b);
 template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float a, float b) {
-    return static_cast<uint32_t>(HP<bf16_t>::from_f32(a).bits) |
-           (static_cast<uint32_t>(HP<bf16_t>::from_f32(b).bits) << 16);
+    typedef float  f2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2{a, b}, b2));
 }
 template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
+    typedef float    f2 __attribute__((ext_vector_type(2)));
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-    h2               h;
-    h.x = static_cast<_Float16>(a);
-    h.y = static_cast<_Float16>(b);
-    return __builtin_bit_cast(uint32_t, h);
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2{a, b}, h2));
 }
 
 } // namespace pt
