@@ -206,6 +206,50 @@ PT_API int pt_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const v
                        int64_t sb_n, int64_t sb_k, int sa_block, int sb_block, int accumulate,
                        void *workspace, size_t workspace_bytes, int tile_cfg, void *stream);
 
+/* MoE grouped FP8 GEMM, 128-blockwise scales -------------------------------
+ *
+ * pt_grouped_gemm_fp8 replaces primus_turbo::grouped_gemm_fp8_impl
+ * (primus_turbo/pytorch/kernels/grouped_gemm/grouped_gemm_fp8_impl.py:888-930; Triton kernels
+ * primus_turbo/triton/grouped_gemm/grouped_gemm_fp8_kernel.py:1405-1556,1809-1944) for the
+ * BLOCKWISE granularity, the forward and dgrad product of a grouped linear layer:
+ *
+ *   out[offs[g] : offs[g+1], :] = A[offs[g] : offs[g+1], :] . W_g^T      g = 0 .. G-1
+ *   out[offs[G] : out_rows, :]  = 0
+ *
+ * A is [M, K] fp8 with one scale per row and 128-wide K block stored K-block major,
+ * a_scale[kb * M + m] (the "pre-shuffled" row scales of
+ * pt_quantize_fp8_blockwise_segment_m_row_col). trans_b != 0: W is [G, N, K] with tile scales
+ * [G, ceil(N/128), ceil(K/128)]; trans_b == 0: W is [G, K, N] with [G, ceil(K/128), ceil(N/128)].
+ * group_offs: device int64 [G + 1] prefix sums of the per-group row counts (no host sync; groups
+ * may be empty). The workspace (pt_grouped_gemm_fp8_workspace_bytes) holds the K-contiguous
+ * copy of W when trans_b == 0 and zero-padded copies when K % 128 != 0 or K < 384.
+ *
+ * pt_grouped_gemm_fp8_variable_k replaces primus_turbo::grouped_gemm_fp8_variable_k_impl and
+ * ..._variable_k_accum_impl (grouped_gemm_fp8_impl.py:933-1022; Triton
+ * grouped_gemm_fp8_kernel.py:1656-1802,1951-2103), the wgrad product:
+ *
+ *   C[g] (+)= LHS[p[g] : p[g+1], :]^T . RHS[p[g] : p[g+1], :]     ([Ml, Nr]; [Nr, Ml] if trans_c)
+ *
+ * LHS [Mp, Ml] and RHS [Mp, Nr] are the segment-padded column quantizations (each group's rows
+ * rounded up to a multiple of 128, pad rows zero) with scales [Mp / 128, cols]; p = padded
+ * group offsets (device int64 [G + 1], multiples of 128). An empty group yields C[g] = 0
+ * (or leaves it unchanged when accumulating). The workspace holds both transposed operands.
+ */
+PT_API size_t pt_grouped_gemm_fp8_workspace_bytes(int64_t G, int64_t M, int64_t N, int64_t K,
+                                                  int trans_b);
+PT_API int pt_grouped_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const void *b,
+                               int b_dtype, const float *b_scale, void *c, int c_dtype,
+                               const int64_t *group_offs, int64_t G, int64_t M, int64_t out_rows,
+                               int64_t N, int64_t K, int trans_b, void *workspace,
+                               size_t workspace_bytes, int tile_cfg, void *stream);
+PT_API size_t pt_grouped_gemm_fp8_variable_k_workspace_bytes(int64_t Mp, int64_t Ml, int64_t Nr);
+PT_API int pt_grouped_gemm_fp8_variable_k(const void *lhs, int lhs_dtype, const float *lhs_scale,
+                                          const void *rhs, int rhs_dtype, const float *rhs_scale,
+                                          void *c, int c_dtype, const int64_t *group_offs, int64_t G,
+                                          int64_t Mp, int64_t Ml, int64_t Nr, int trans_c,
+                                          int accumulate, void *workspace, size_t workspace_bytes,
+                                          int tile_cfg, void *stream);
+
 /* Byte-matrix transpose out[b, c, r] = in[b, r, c] (fp8 payloads; replaces the 2-D
  * transpose used for tensorwise `.t()` copies, csrc/kernels/transpose/). */
 PT_API int pt_transpose_u8(const void *in, void *out, int64_t batch, int64_t R, int64_t C,

@@ -49,6 +49,35 @@ def gemm_fp8_rowwise_ref(a: torch.Tensor, b: torch.Tensor, dtype=torch.float8_e4
     return (ad @ bd.t()).to(out_dtype)
 
 
+def quantize_fp8_blockwise_ref(x: torch.Tensor, dtype: torch.dtype, block_m: int, block_n: int):
+    """Blockwise quantization of a 2-D tensor with block_m x block_n tiles (1 x 128 for
+    activations, 128 x 128 for weights), the formula of the reference's Triton quantizers
+    (/root/reference/primus_turbo/triton/quantization/quant_blockwise.py:35-66): scale =
+    fp8_max / max(amax, 1e-4), the stored scale is its reciprocal. Returns (codes, scale_inv)
+    with scale_inv of shape [ceil(M / block_m), ceil(N / block_n)]."""
+    M, N = x.shape
+    fp8_max = torch.finfo(dtype).max
+    pm, pn = (-M) % block_m, (-N) % block_n
+    xp = torch.nn.functional.pad(x.float(), (0, pn, 0, pm))
+    t = xp.view((M + pm) // block_m, block_m, (N + pn) // block_n, block_n)
+    amax = t.abs().amax(dim=(1, 3), keepdim=True)
+    scale = fp8_max / torch.clamp(amax, min=1e-4)
+    q = torch.clamp(t * scale, -fp8_max, fp8_max).to(dtype)
+    q = q.view(M + pm, N + pn)[:M, :N]
+    return q, (1.0 / scale).view((M + pm) // block_m, (N + pn) // block_n)
+
+
+def gemm_fp8_blockwise_ref(a: torch.Tensor, b: torch.Tensor, dtype=torch.float8_e4m3fn, block: int = 128,
+                           out_dtype=torch.bfloat16):
+    """DeepSeek-style blockwise GEMM on the CPU: A [M, K] with 1 x block scales, B [N, K] with
+    block x block scales, fp32 matmul of the de-quantized operands."""
+    aq, asi = quantize_fp8_blockwise_ref(a, dtype, 1, block)
+    bq, bsi = quantize_fp8_blockwise_ref(b, dtype, block, block)
+    ad = aq.float() * asi.repeat_interleave(block, dim=1)[:, : a.shape[1]]
+    bd = bq.float() * bsi.repeat_interleave(block, dim=0)[: b.shape[0]].repeat_interleave(block, dim=1)[:, : b.shape[1]]
+    return (ad @ bd.t()).to(out_dtype)
+
+
 def grouped_gemm_ref(a: torch.Tensor, b: torch.Tensor, seg_lens, trans_b=True):
     out = []
     start = 0

@@ -5,7 +5,6 @@
 
 namespace pt {
 
-int launch_gemm_block(const GemmArgs &a, int fa, int fb, bool sb_vec, int tile_cfg, hipStream_t stream);
 
 // ---------------------------------------------------------------------------
 // fp8 byte matrix transpose in[R, C] -> out[C, ldo] through a padded 64 x 64 LDS tile;
@@ -54,8 +53,8 @@ __global__ __launch_bounds__(256) void pad_rows_u8_kernel(const uint8_t *__restr
     }
 }
 
-static void launch_transpose(const uint8_t *in, uint8_t *out, int64_t batch, int64_t R, int64_t C,
-                             int64_t ldo, hipStream_t st) {
+void launch_transpose(const uint8_t *in, uint8_t *out, int64_t batch, int64_t R, int64_t C,
+                      int64_t ldo, hipStream_t st) {
     // the grid covers ldo (>= R) input-row positions so that the zero tail gets written too
     dim3 g(static_cast<unsigned>(cdiv(C, 64)), static_cast<unsigned>(cdiv(ldo, 64)),
            static_cast<unsigned>(batch));
@@ -84,14 +83,8 @@ static int launch_gemm_vector(const GemmArgs &a, int fa, int fb, int tile_cfg, h
     return launch_vector_tiles<1, 1>(a, tile_cfg, stream);
 }
 
-static inline int64_t round_up(int64_t x, int64_t m) {
-    return (x + m - 1) / m * m;
-}
-
-// The kernel wants K as a multiple of 128 and at least three 128-byte slabs.
-static inline int64_t padded_k(int64_t K) {
-    const int64_t kp = round_up(K, KSTEP);
-    return kp < 3 * KSTEP ? 3 * KSTEP : kp;
+void launch_pad_rows(const uint8_t *in, uint8_t *out, int64_t R, int64_t C, int64_t ldo, hipStream_t st) {
+    pad_rows_u8_kernel<<<static_cast<unsigned>(cdiv(R * ldo, 256 * 16)), 256, 0, st>>>(in, out, R, C, ldo);
 }
 
 // zero `bytes` bytes at a 16-byte aligned address (a fill kernel rather than a memset node,
@@ -171,7 +164,7 @@ int pt_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const void *b,
                 if (trans_a) // stored [K, M] -> [M, Kp]
                     launch_transpose(A, ws, 1, K, M, Kp, st);
                 else
-                    pad_rows_u8_kernel<<<static_cast<unsigned>(cdiv(M * Kp, 256 * 16)), 256, 0, st>>>(A, ws, M, K, Kp);
+                    launch_pad_rows(A, ws, M, K, Kp, st);
             }
             A = ws;
             ws += round_up(M * Kp, 256);
@@ -181,7 +174,7 @@ int pt_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const void *b,
                 if (!trans_b) // stored [K, N] -> [N, Kp]
                     launch_transpose(B, ws, 1, K, N, Kp, st);
                 else
-                    pad_rows_u8_kernel<<<static_cast<unsigned>(cdiv(N * Kp, 256 * 16)), 256, 0, st>>>(B, ws, N, K, Kp);
+                    launch_pad_rows(B, ws, N, K, Kp, st);
             }
             B = ws;
         }
@@ -204,6 +197,7 @@ int pt_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const void *b,
     g.sb_k = sb_k;
     g.sa_shift = sa_block == 128 ? 7 : 0;
     g.sb_shift = sb_block == 128 ? 7 : 0;
+    g.kb_valid = static_cast<int>(cdiv(K, 128));
     g.out_dtype = c_dtype;
     g.accumulate = accumulate;
     const int fa = a_dtype == PT_DTYPE_E5M2 ? 1 : 0, fb = b_dtype == PT_DTYPE_E5M2 ? 1 : 0;

@@ -49,10 +49,24 @@ struct GemmArgs {
     // BLOCK : sA[(m >> sa_shift) * sa_m + kb * sa_k], sB[(n >> sb_shift) * sb_n + kb * sb_k]
     int64_t sa_m, sa_k, sb_n, sb_k;
     int     sa_shift, sb_shift; // 0 (one scale per row) or 7 (one per 128 rows)
+    int     kb_valid;           // BLOCK: K blocks the scale arrays hold (K slabs beyond are zero padding)
     int     out_dtype;
     int     accumulate; // C += result (beta = 1) instead of C = result
     int     tiles_m, tiles_n;
+    // Grouped problems (MoE experts); group_offs is a device array of G + 1 int64 prefix sums.
+    //   GROUP_ROWS: rows [offs[g], offs[g+1]) of A and C belong to group g, which multiplies
+    //               with B + g * b_gstride (scales sB + g * sb_gstride); M is the row count of A.
+    //   GROUP_K   : group g reduces over K columns [offs[g], offs[g+1]) of A and B (multiples
+    //               of 128) into C + g * c_gstride; scales start at K block offs[g] / 128.
+    int            gmode;
+    int            G;
+    const int64_t *group_offs;
+    int64_t        b_gstride;  // bytes
+    int64_t        sb_gstride; // floats
+    int64_t        c_gstride;  // elements
 };
+
+enum : int { GROUP_NONE = 0, GROUP_ROWS = 1, GROUP_K = 2 };
 
 constexpr int KSTEP      = 128; // bytes of K per pipeline step (= one MFMA K)
 constexpr int GEMM_WAVES = 4;
@@ -121,11 +135,11 @@ __device__ __forceinline__ f32x4 mfma_fp8(const i32x8 &rowop, const i32x8 &colop
 
 // Tile coordinates of a workgroup: XCD-contiguous ids, then groups of GROUP_M tile rows
 // walked column-major so that concurrently running tiles share A and B panels in L2.
+__device__ __forceinline__ void tile_coords_local(int lid, int tiles_m, int tiles_n, int &tm, int &tn);
 __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, int &tm, int &tn) {
-    constexpr int NXCD    = 8;
-    constexpr int GROUP_M = 8;
-    const int     total   = tiles_m * tiles_n;
-    int           lid     = pid;
+    constexpr int NXCD  = 8;
+    const int     total = tiles_m * tiles_n;
+    int           lid   = pid;
     if (total >= NXCD * 4) {
         // workgroup i runs on XCD i % 8: give each XCD one contiguous id range
         const int per  = total / NXCD, rem = total % NXCD;
@@ -133,7 +147,11 @@ __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, i
         // XCDs [0, rem) own per + 1 ids
         lid = xcd * per + (xcd < rem ? xcd : rem) + slot;
     }
-    const int in_group = GROUP_M * tiles_n;
+    tile_coords_local(lid, tiles_m, tiles_n, tm, tn);
+}
+__device__ __forceinline__ void tile_coords_local(int lid, int tiles_m, int tiles_n, int &tm, int &tn) {
+    constexpr int GROUP_M  = 8;
+    const int     in_group = GROUP_M * tiles_n;
     const int gid      = lid / in_group;
     const int first_m  = gid * GROUP_M;
     const int gsz      = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
@@ -219,12 +237,15 @@ __device__ __forceinline__ void store_elem(float f, uint8_t *q, int out_dtype, b
     }
 }
 
+// `Cm` / `sAm` / `sBm` / `m_end` describe the matrix the tile belongs to (the whole problem,
+// or one group's share of it).
 template <int TM, int TN, int MODE, bool ACC_IN_AGPR>
-__device__ __forceinline__ void epilogue(const GemmArgs &a, const f32x4 (&acc)[TM][TN],
+__device__ __forceinline__ void epilogue(const GemmArgs &a, const f32x4 (&acc)[TM][TN], uint8_t *Cm,
+                                         const float *sAm, const float *sBm, int64_t m_end,
                                          int64_t wm_base, int64_t wn_base, int lane) {
     const int     ES = a.out_dtype == PT_DTYPE_F32 ? 4 : 2;
     const int     lm = lane & 15, lg = lane >> 4;
-    uint8_t      *C    = static_cast<uint8_t *>(a.C);
+    uint8_t      *C    = Cm;
     const bool    accu = a.accumulate != 0;
     const int64_t m0 = wm_base + lm, n0 = wn_base + lg * 4;
 
@@ -234,18 +255,18 @@ __device__ __forceinline__ void epilogue(const GemmArgs &a, const f32x4 (&acc)[T
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             const int64_t m = m0 + i * 16;
-            sa[i]           = a.sA[(m < a.M ? m : a.M - 1) * a.sa_m];
+            sa[i]           = sAm[(m < a.M ? m : a.M - 1) * a.sa_m];
         }
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int64_t n = n0 + j * 16 + e;
-                sb[j][e]        = a.sB[(n < a.N ? n : a.N - 1) * a.sb_n];
+                sb[j][e]        = sBm[(n < a.N ? n : a.N - 1) * a.sb_n];
             }
     }
     // whole sub-tile inside the matrix and every 4-element group aligned: no per-element checks
-    const bool fast = wm_base + TM * 16 <= a.M && wn_base + TN * 16 <= a.N && (a.N & 3) == 0 &&
+    const bool fast = wm_base + TM * 16 <= m_end && wn_base + TN * 16 <= a.N && (a.N & 3) == 0 &&
                       (reinterpret_cast<uintptr_t>(C) & 15) == 0;
     uint8_t      *row  = C + (m0 * a.N + n0) * ES;
     const int64_t step = 16 * a.N;
@@ -267,7 +288,7 @@ __device__ __forceinline__ void epilogue(const GemmArgs &a, const f32x4 (&acc)[T
                     for (int e = 0; e < 4; ++e)
                         v[e] = v[e] * sa[i] * sb[j][e];
                 }
-                if (m0 + i * 16 < a.M) {
+                if (m0 + i * 16 < m_end) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         if (n0 + j * 16 + e < a.N)
@@ -280,24 +301,67 @@ __device__ __forceinline__ void epilogue(const GemmArgs &a, const f32x4 (&acc)[T
     }
 }
 
-// Where a workgroup's tile lives.
+// Where a workgroup's tile lives. The second half only varies between tiles of grouped
+// problems; in the dense case it repeats the kernel arguments.
 struct TileCtx {
-    const uint8_t *Ag, *Bg; // first row of the tile in A / B
+    const uint8_t *Ag, *Bg; // first row of the tile in A / B (at the tile's first K column)
     int            rows_a, rows_b;
-    int64_t        m0, n0;
+    int64_t        m0, n0;  // first output row / column (row index in the tile's C matrix)
+    int64_t        m_end;   // rows of C at or beyond this belong to someone else
+    const float   *sA, *sB; // scale arrays of the tile's matrix (BLOCK: at its first K block)
+    uint8_t       *C;       // the tile's output matrix
+    int            KT;      // K slabs of this tile
 };
 
-template <int BM, int BN>
-__device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile) {
-    int tm, tn;
-    tile_coords(tile, a.tiles_m, a.tiles_n, tm, tn);
+// GROUP_ROWS: prefix[g] = number of tiles of the groups before g (in LDS), `g` is a search
+// hint that only moves forward as a workgroup walks its tiles.
+template <int BM, int BN, int GMODE>
+__device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile, const int *prefix, int &g) {
     TileCtx t;
-    t.m0     = static_cast<int64_t>(tm) * BM;
+    int     tm, tn;
+    if constexpr (GMODE == GROUP_NONE) {
+        tile_coords(tile, a.tiles_m, a.tiles_n, tm, tn);
+        t.m0    = static_cast<int64_t>(tm) * BM;
+        t.m_end = a.M;
+        t.Ag    = a.A + t.m0 * a.lda;
+        t.Bg    = a.B;
+        t.sA    = a.sA;
+        t.sB    = a.sB;
+        t.C     = static_cast<uint8_t *>(a.C);
+        t.KT    = static_cast<int>(a.K / KSTEP);
+    } else if constexpr (GMODE == GROUP_ROWS) {
+        while (g + 1 < a.G && tile >= __builtin_amdgcn_readfirstlane(prefix[g + 1]))
+            ++g;
+        const int     local = tile - __builtin_amdgcn_readfirstlane(prefix[g]);
+        const int64_t lo = a.group_offs[g], hi = a.group_offs[g + 1];
+        const int     gtm = static_cast<int>((hi - lo + BM - 1) / BM);
+        tile_coords_local(local, gtm, a.tiles_n, tm, tn);
+        t.m0    = lo + static_cast<int64_t>(tm) * BM;
+        t.m_end = hi;
+        t.Ag    = a.A + t.m0 * a.lda;
+        t.Bg    = a.B + g * a.b_gstride;
+        t.sA    = a.sA;
+        t.sB    = a.sB + g * a.sb_gstride;
+        t.C     = static_cast<uint8_t *>(a.C);
+        t.KT    = static_cast<int>(a.K / KSTEP);
+    } else {
+        const int per = a.tiles_m * a.tiles_n;
+        g             = tile / per;
+        tile_coords_local(tile - g * per, a.tiles_m, a.tiles_n, tm, tn);
+        const int64_t lo = a.group_offs[g], hi = a.group_offs[g + 1];
+        t.m0    = static_cast<int64_t>(tm) * BM;
+        t.m_end = a.M;
+        t.Ag    = a.A + t.m0 * a.lda + lo;
+        t.Bg    = a.B + lo;
+        t.sA    = a.sA + (lo / KSTEP) * a.sa_k;
+        t.sB    = a.sB + (lo / KSTEP) * a.sb_k;
+        t.C     = static_cast<uint8_t *>(a.C) + g * a.c_gstride * (a.out_dtype == PT_DTYPE_F32 ? 4 : 2);
+        t.KT    = static_cast<int>((hi - lo) / KSTEP);
+    }
     t.n0     = static_cast<int64_t>(tn) * BN;
-    t.rows_a = (a.M - t.m0) < BM ? static_cast<int>(a.M - t.m0) : BM;
+    t.rows_a = (t.m_end - t.m0) < BM ? static_cast<int>(t.m_end - t.m0) : BM;
     t.rows_b = (a.N - t.n0) < BN ? static_cast<int>(a.N - t.n0) : BN;
-    t.Ag     = a.A + t.m0 * a.lda;
-    t.Bg     = a.B + t.n0 * a.ldb;
+    t.Bg += t.n0 * a.ldb;
     return t;
 }
 
@@ -317,7 +381,7 @@ __device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile) {
 //   * tile boundaries do not drain the pipeline: while a tile's result is written out, the
 //     first fragments of the next tile are already in registers and its second slab is in
 //     flight.
-template <int TM, int TN, int MODE, bool SB_VEC, int FA, int FB>
+template <int TM, int TN, int MODE, bool SB_VEC, int FA, int FB, int GMODE>
 __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     static_assert(TN % 4 == 0, "the B fragment ring assumes TN = 4 or 8");
     constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
@@ -326,6 +390,9 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     constexpr int NL  = LA + LB;
     constexpr int JR  = TN - 2; // columns [0, JR) before the release point, [JR, TN) after
     constexpr int NSB = SB_VEC ? 4 : 1;
+    // GROUP_K tiles have their own K extent (possibly none at all): they run the pipeline per
+    // tile instead of across tile boundaries
+    constexpr bool XPIPE = GMODE != GROUP_K;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
     const int tid  = threadIdx.x;
@@ -338,20 +405,46 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     const uint32_t frag_off_lo = lm * KSTEP + ((lg ^ swz(lm)) << 4);
     const uint32_t frag_off_hi = lm * KSTEP + (((4 + lg) ^ swz(lm)) << 4);
 
-    const int total = a.tiles_m * a.tiles_n;
-    const int KT    = static_cast<int>(a.K / KSTEP);
-    int       tile  = blockIdx.x;
-    if (tile >= total || KT < 3)
+    // ---- tile list ----
+    int *prefix = reinterpret_cast<int *>(smem + 2 * STAGE); // GROUP_ROWS: tiles before group g
+    int  total;
+    if constexpr (GMODE == GROUP_ROWS) {
+        for (int g = tid; g < a.G; g += 256) {
+            const int64_t rows = a.group_offs[g + 1] - a.group_offs[g];
+            prefix[g + 1]      = static_cast<int>((rows + BM - 1) / BM) * a.tiles_n;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            int run = 0;
+            prefix[0] = 0;
+            for (int g = 1; g <= a.G; ++g) {
+                run += prefix[g];
+                prefix[g] = run;
+            }
+        }
+        __syncthreads();
+        total = __builtin_amdgcn_readfirstlane(prefix[a.G]);
+    } else if constexpr (GMODE == GROUP_K) {
+        total = a.G * a.tiles_m * a.tiles_n;
+    } else {
+        total = a.tiles_m * a.tiles_n;
+    }
+    const int KT_ALL = static_cast<int>(a.K / KSTEP); // XPIPE: every tile has this many slabs (>= 3)
+    int       tile   = blockIdx.x;
+    if (tile >= total || (XPIPE && KT_ALL < 3))
         return;
-    TileCtx cur_t = make_tile<BM, BN>(a, tile);
+    int     g_cur = 0, g_nxt = 0;
+    TileCtx cur_t = make_tile<BM, BN, GMODE>(a, tile, prefix, g_cur);
+    g_nxt         = g_cur;
 
     // ---- loader: two slabs ahead of the MFMAs ----
     // Copies are buffer loads: a lane's offset inside a slab (row * pitch + swizzled chunk)
     // is the same for every tile; the tile and the K position live in the (uniform) buffer
-    // descriptor, whose size makes rows beyond the matrix edge read as zero. The loader
-    // therefore changes tile by swapping scalars -- no branch in the K loop, which the
-    // compiler would use to sink MFMAs -- and it does so after requesting the tile's last
-    // slab, at step KT - 3 of the MFMAs (the host guarantees KT >= 3).
+    // descriptor, whose size makes rows beyond the tile's share of the matrix read as zero.
+    // The loader therefore changes tile by swapping scalars -- no branch in the K loop, which
+    // the compiler would use to sink MFMAs -- and it does so after requesting the tile's last
+    // slab, at step KT - 3 of the MFMAs (the host guarantees KT >= 3). Without cross-tile
+    // pipelining it stops at the tile's last slab and keeps re-reading that one.
     uint32_t off[NL];
     {
         const int lrow = lane >> 3, pchk = lane & 7;
@@ -362,11 +455,17 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             off[j] = static_cast<uint32_t>(row * (isA ? a.lda : a.ldb)) + ((pchk ^ swz(row)) << 4);
         }
     }
-    const uint8_t *ld_ga = cur_t.Ag, *ld_gb = cur_t.Bg; // slab the loader points at
-    uint32_t       ld_na = cur_t.rows_a * static_cast<uint32_t>(a.lda); // bytes from there to the
-    uint32_t       ld_nb = cur_t.rows_b * static_cast<uint32_t>(a.ldb); // end of the tile's rows
-    int            ld_kt = 0;
+    const uint8_t *ld_ga, *ld_gb; // slab the loader points at
+    uint32_t       ld_na, ld_nb;  // bytes from there to the end of the tile's rows
+    int            ld_kt;
     TileCtx        nxt_t = cur_t; // tile after the MFMAs' tile (the same tile after the last one)
+    auto           loader_to = [&](const TileCtx &t) {
+        ld_ga = t.Ag;
+        ld_gb = t.Bg;
+        ld_na = t.rows_a * static_cast<uint32_t>(a.lda);
+        ld_nb = t.rows_b * static_cast<uint32_t>(a.ldb);
+        ld_kt = 0;
+    };
     // copy number L of the loader's slab into stage `b`
     auto issue_copy = [&](auto lc, int b) {
         constexpr int L   = lc;
@@ -383,26 +482,37 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
 #endif
     };
     auto advance_loader = [&]() {
-        const bool wrap = ld_kt + 1 == KT;
-        ld_kt = wrap ? 0 : ld_kt + 1;
-        ld_ga = wrap ? nxt_t.Ag : ld_ga + KSTEP;
-        ld_gb = wrap ? nxt_t.Bg : ld_gb + KSTEP;
-        ld_na = wrap ? nxt_t.rows_a * static_cast<uint32_t>(a.lda) : ld_na - KSTEP;
-        ld_nb = wrap ? nxt_t.rows_b * static_cast<uint32_t>(a.ldb) : ld_nb - KSTEP;
+        if constexpr (XPIPE) {
+            const bool wrap = ld_kt + 1 == KT_ALL;
+            ld_kt = wrap ? 0 : ld_kt + 1;
+            ld_ga = wrap ? nxt_t.Ag : ld_ga + KSTEP;
+            ld_gb = wrap ? nxt_t.Bg : ld_gb + KSTEP;
+            ld_na = wrap ? nxt_t.rows_a * static_cast<uint32_t>(a.lda) : ld_na - KSTEP;
+            ld_nb = wrap ? nxt_t.rows_b * static_cast<uint32_t>(a.ldb) : ld_nb - KSTEP;
+        } else {
+            const int adv = ld_kt + 1 < cur_t.KT ? KSTEP : 0;
+            ld_kt += adv / KSTEP;
+            ld_ga += adv;
+            ld_gb += adv;
+            ld_na -= adv;
+            ld_nb -= adv;
+        }
     };
 
     // BLOCK mode: the fp32 scales of a K block are fetched one slab ahead, at the release
     // point and before that slab's tile copies are issued (so the copies stay the youngest
     // entries of the vector-memory counter).
     [[maybe_unused]] float sa_cur[TM], sa_nxt[TM], sb_cur[TN][NSB], sb_nxt[TN][NSB];
-    auto fetch_scales = [&](const TileCtx &t, int kt, float (&sa)[TM], float (&sb)[TN][NSB]) {
+    auto fetch_scales = [&](int64_t m0, int64_t n0, const float *sAm, const float *sBm, int kt, float (&sa)[TM],
+                            float (&sb)[TN][NSB]) {
         if constexpr (MODE == SCALE_BLOCK) {
-            const int64_t wm_base = t.m0 + wm * (TM * 16), wn_base = t.n0 + wn * (TN * 16);
+            const int64_t wm_base = m0 + wm * (TM * 16), wn_base = n0 + wn * (TN * 16);
+            kt = kt < a.kb_valid ? kt : a.kb_valid - 1; // zero-padded slabs: any valid scale will do
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
                 int64_t m = wm_base + i * 16 + lm;
                 m         = m < a.M ? m : a.M - 1;
-                sa[i]     = a.sA[(m >> a.sa_shift) * a.sa_m + kt * a.sa_k];
+                sa[i]     = sAm[(m >> a.sa_shift) * a.sa_m + kt * a.sa_k];
             }
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
@@ -411,13 +521,13 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                     for (int e = 0; e < 4; ++e) {
                         int64_t n = wn_base + j * 16 + lg * 4 + e;
                         n         = n < a.N ? n : a.N - 1;
-                        sb[j][e]  = a.sB[n * a.sb_n + kt * a.sb_k];
+                        sb[j][e]  = sBm[n * a.sb_n + kt * a.sb_k];
                     }
                 } else {
                     int64_t       nb    = (wn_base + j * 16) >> a.sb_shift;
                     const int64_t nbmax = (a.N - 1) >> a.sb_shift;
                     nb                  = nb < nbmax ? nb : nbmax;
-                    sb[j][0]            = a.sB[nb * a.sb_n + kt * a.sb_k];
+                    sb[j][0]            = sBm[nb * a.sb_n + kt * a.sb_k];
                 }
             }
         }
@@ -442,21 +552,27 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     const uint32_t a_part = wm * (TM * 16) * KSTEP;
     const uint32_t b_part = A_BYTES + wn * (TN * 16) * KSTEP;
 
-    // ---- prologue: slabs 0 and 1 requested, the first fragments of slab 0 on their way ----
+    // pipeline start at tile t: slabs 0 and 1 requested, the first fragments of slab 0 on their way
+    auto start_pipeline = [&](const TileCtx &t) {
+        loader_to(t);
+        fetch_scales(t.m0, t.n0, t.sA, t.sB, 0, sa_nxt, sb_nxt);
+        static_for<0, NL>([&](auto l) { issue_copy(l, 0); });
+        advance_loader();
+        static_for<0, NL>([&](auto l) { issue_copy(l, 1); });
+        advance_loader();
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
+        __builtin_amdgcn_s_barrier();
+        buf   = 0;
+        fb[0] = ldfrag(smem + b_part, 0);
+        fb[1] = ldfrag(smem + b_part, 1);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+            fa[i] = ldfrag(smem + a_part, i);
+    };
     PT_GEMM_TRACE_DECL;
     PT_GEMM_TRACE_POINT(0);
-    fetch_scales(cur_t, 0, sa_nxt, sb_nxt);
-    static_for<0, NL>([&](auto l) { issue_copy(l, 0); });
-    advance_loader();
-    static_for<0, NL>([&](auto l) { issue_copy(l, 1); });
-    advance_loader();
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
-    __builtin_amdgcn_s_barrier();
-    fb[0] = ldfrag(smem + b_part, 0);
-    fb[1] = ldfrag(smem + b_part, 1);
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-        fa[i] = ldfrag(smem + a_part, i);
+    if constexpr (XPIPE)
+        start_pipeline(cur_t);
 
     while (true) {
 #pragma unroll
@@ -468,7 +584,12 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         const int next_tile = tile + gridDim.x;
         nxt_t               = cur_t;
         if (next_tile < total)
-            nxt_t = make_tile<BM, BN>(a, next_tile);
+            nxt_t = make_tile<BM, BN, GMODE>(a, next_tile, prefix, g_nxt);
+        const int KT = XPIPE ? KT_ALL : cur_t.KT;
+        if constexpr (!XPIPE) {
+            if (KT > 0)
+                start_pipeline(cur_t);
+        }
 
         // one K slab per iteration; the body must stay a single basic block (no branches), or
         // the compiler sinks the MFMAs behind them
@@ -534,13 +655,16 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_s_barrier();
             PT_GEMM_TRACE_POINT(3);
-            // (after the last slab of the last tile the following fetch and read leftovers: harmless)
+            // (after a tile's last slab without a successor the following fetch and read leftovers:
+            // harmless)
             if constexpr (MODE == SCALE_BLOCK) {
-                const bool same = kt + 1 < KT;
-                TileCtx    st   = nxt_t;
-                st.m0           = same ? cur_t.m0 : nxt_t.m0;
-                st.n0           = same ? cur_t.n0 : nxt_t.n0;
-                fetch_scales(st, same ? kt + 1 : 0, sa_nxt, sb_nxt);
+                if constexpr (XPIPE) {
+                    const bool same = kt + 1 < KT;
+                    fetch_scales(same ? cur_t.m0 : nxt_t.m0, same ? cur_t.n0 : nxt_t.n0, same ? cur_t.sA : nxt_t.sA,
+                                 same ? cur_t.sB : nxt_t.sB, same ? kt + 1 : 0, sa_nxt, sb_nxt);
+                } else {
+                    fetch_scales(cur_t.m0, cur_t.n0, cur_t.sA, cur_t.sB, kt + 1 < KT ? kt + 1 : kt, sa_nxt, sb_nxt);
+                }
             }
             fb[0] = ldfrag(nxt + b_part, 0);
             fb[1] = ldfrag(nxt + b_part, 1);
@@ -563,6 +687,12 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             advance_loader();
             buf ^= 1;
         }
+        if constexpr (!XPIPE) {
+            // the re-read copies of the last slab must have landed everywhere before the next
+            // tile's first copies go into the same stages
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+        }
 
         // the epilogue reads the accumulators with hand-written instructions the compiler's
         // hazard tracking does not see: let the last MFMA's write-back finish first
@@ -570,7 +700,8 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
         PT_GEMM_TRACE_POINT(5);
         const int64_t wm_base = cur_t.m0 + wm * (TM * 16), wn_base = cur_t.n0 + wn * (TN * 16);
-        epilogue<TM, TN, MODE, MODE == SCALE_VECTOR>(a, acc, wm_base, wn_base, lane);
+        epilogue<TM, TN, MODE, MODE == SCALE_VECTOR>(a, acc, cur_t.C, cur_t.sA, cur_t.sB, cur_t.m_end, wm_base, wn_base,
+                                                     lane);
 
         PT_GEMM_TRACE_POINT(6);
         if (next_tile >= total)
@@ -582,29 +713,62 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-template <int TM, int TN, int MODE, bool SB_VEC, int FA, int FB>
+// Upper bound on the number of tiles (exact for the ungrouped case): GROUP_ROWS cannot know
+// the per-group row counts on the host, but every group adds at most one partial tile row.
+template <int TM, int TN, int MODE, bool SB_VEC, int FA, int FB, int GMODE = GROUP_NONE>
 static int launch_gemm_cfg(const GemmArgs &args_in, hipStream_t stream) {
     constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
-    constexpr int LDS = 2 * (BM + BN) * KSTEP;
-    GemmArgs      a   = args_in;
-    a.tiles_m         = static_cast<int>(cdiv(a.M, BM));
-    a.tiles_n         = static_cast<int>(cdiv(a.N, BN));
-    auto kern         = gemm_fp8_nt_kernel<TM, TN, MODE, SB_VEC, FA, FB>;
+    constexpr int STAGES  = 2 * (BM + BN) * KSTEP;
+    constexpr int MAX_G   = 4096;
+    constexpr int LDS_MAX = STAGES + (GMODE == GROUP_ROWS ? (MAX_G + 2) * 4 : 0);
+    static_assert(LDS_MAX <= 160 * 1024, "tile configuration does not fit the LDS");
+    GemmArgs a = args_in;
+    a.gmode    = GMODE;
+    a.tiles_m  = static_cast<int>(cdiv(a.M, BM));
+    a.tiles_n  = static_cast<int>(cdiv(a.N, BN));
+    if (GMODE != GROUP_NONE && a.G > MAX_G)
+        return fail(PT_ERR_INVALID_ARGUMENT, "grouped gemm: at most 4096 groups");
+    auto kern            = gemm_fp8_nt_kernel<TM, TN, MODE, SB_VEC, FA, FB, GMODE>;
     static bool attr_set = false;
     if (!attr_set) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess)
+                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_MAX) != hipSuccess)
             return fail(PT_ERR_LAUNCH, "gemm_fp8: cannot raise the dynamic LDS limit");
         attr_set = true;
     }
+    const int lds = STAGES + (GMODE == GROUP_ROWS ? (a.G + 2) * 4 : 0);
     // persistent grid: as many workgroups as fit on the machine at once (LDS-limited)
-    const int     per_cu = (160 * 1024) / LDS;
-    const int64_t total  = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
-    int64_t       grid   = static_cast<int64_t>(device_cu_count()) * (per_cu < 1 ? 1 : per_cu);
+    const int per_cu = (160 * 1024) / lds;
+    int64_t   total;
+    if (GMODE == GROUP_ROWS)
+        total = (static_cast<int64_t>(a.tiles_m) + a.G) * a.tiles_n;
+    else if (GMODE == GROUP_K)
+        total = static_cast<int64_t>(a.G) * a.tiles_m * a.tiles_n;
+    else
+        total = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
+    int64_t grid = static_cast<int64_t>(device_cu_count()) * (per_cu < 1 ? 1 : per_cu);
     if (grid > total)
         grid = total;
-    kern<<<static_cast<unsigned>(grid), 256, LDS, stream>>>(a);
+    if (grid <= 0)
+        return PT_OK;
+    kern<<<static_cast<unsigned>(grid), 256, lds, stream>>>(a);
     return check_launch("gemm_fp8_nt_kernel");
 }
+
+// ---- host helpers shared by the translation units that instantiate the kernel ----
+static inline int64_t round_up(int64_t x, int64_t m) {
+    return (x + m - 1) / m * m;
+}
+// The kernel wants K as a multiple of 128 and at least three 128-byte slabs.
+static inline int64_t padded_k(int64_t K) {
+    const int64_t kp = round_up(K, KSTEP);
+    return kp < 3 * KSTEP ? 3 * KSTEP : kp;
+}
+// in[batch][R, C] -> out[batch][C, ldo] (columns [R, ldo) zero-filled), fp8 bytes
+void launch_transpose(const uint8_t *in, uint8_t *out, int64_t batch, int64_t R, int64_t C, int64_t ldo,
+                      hipStream_t st);
+// in[R, C] -> out[R, ldo] (columns [C, ldo) zero-filled)
+void launch_pad_rows(const uint8_t *in, uint8_t *out, int64_t R, int64_t C, int64_t ldo, hipStream_t st);
+int  launch_gemm_block(const GemmArgs &a, int fa, int fb, bool sb_vec, int tile_cfg, hipStream_t stream);
 
 } // namespace pt

@@ -1,0 +1,191 @@
+"""Grouped FP8 GEMM impl layer: the reference's ``grouped_gemm_fp8_impl`` /
+``grouped_gemm_fp8_variable_k_impl`` / ``..._variable_k_accum_impl`` contracts
+(primus_turbo/pytorch/kernels/grouped_gemm/grouped_gemm_fp8_impl.py:888-1022 of the reference)
+on top of ``pt_grouped_gemm_fp8`` and ``pt_grouped_gemm_fp8_variable_k``.
+
+One backend exists here, so ``default_backend``, ``num_cu`` and ``maybe_pre_sync`` are accepted
+and ignored (the kernel is persistent over all CUs and never needs the group sizes on the
+host). BLOCKWISE is the granularity these kernels implement.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from primus_turbo import _native as N
+from primus_turbo.pytorch.core.low_precision import ScalingGranularity
+
+_FP8 = (torch.float8_e4m3fn, torch.float8_e5m2)
+
+TILE_CFG = 0  # 0 = automatic; tests and the benchmark may pin 2 (256x128) or 3 (128x128)
+
+
+def _check(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _require_blockwise(granularity: int):
+    if ScalingGranularity(granularity) != ScalingGranularity.BLOCKWISE:
+        raise NotImplementedError(
+            f"grouped FP8 GEMM: only BLOCKWISE scaling is implemented, got {ScalingGranularity(granularity)}"
+        )
+
+
+@torch.library.custom_op("primus_turbo::grouped_gemm_fp8_impl", mutates_args=(), device_types="cuda")
+def grouped_gemm_fp8_impl(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    a_scales: torch.Tensor,
+    b_scales: torch.Tensor,
+    group_lens: torch.Tensor,
+    group_offs: torch.Tensor,
+    trans_a: bool,
+    trans_b: bool,
+    out_dtype: torch.dtype,
+    granularity: int,
+    num_cu: Optional[int],
+    default_backend: int,
+    maybe_pre_sync: bool = False,
+    group_offs_out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """``out[offs[g]:offs[g+1]] = a[offs[g]:offs[g+1]] @ op(b[g])``; rows past ``offs[G]`` are zero.
+
+    ``a`` ``[M, K]`` fp8 with row scales stored ``[K/128, M]``; ``b`` ``[G, N, K]`` (``trans_b``)
+    or ``[G, K, N]`` fp8 with 128 x 128 tile scales."""
+    _require_blockwise(granularity)
+    _check(not trans_a, "Only trans_a=False is supported.")
+    _check(group_offs_out is None, "group_offs_out belongs to the MX grouped path")
+    N.require_cuda(a, b, a_scales, b_scales, group_offs)
+    _check(a.dim() == 2 and b.dim() == 3, "a must be 2-D and b 3-D")
+    _check(a.dtype in _FP8 and b.dtype in _FP8, "operands must be float8_e4m3fn / float8_e5m2")
+    _check(out_dtype in (torch.float16, torch.bfloat16), "out_dtype must be float16 or bfloat16")
+    _check(group_offs.dtype == torch.int64 and group_offs.numel() == b.shape[0] + 1, "group_offs must be int64 [G + 1]")
+    a, b = a.contiguous(), b.contiguous()
+    a_scales, b_scales = a_scales.contiguous(), b_scales.contiguous()
+    G = b.shape[0]
+    M, K = a.shape
+    Nn, Kb = (b.shape[1], b.shape[2]) if trans_b else (b.shape[2], b.shape[1])
+    _check(K == Kb, f"reduction dims differ: {K} vs {Kb}")
+    kb, nb = (K + 127) // 128, (Nn + 127) // 128
+    _check(tuple(a_scales.shape) == (kb, M), f"a_scales must be [K/128, M] = {(kb, M)}, got {tuple(a_scales.shape)}")
+    want_b = (G, nb, kb) if trans_b else (G, kb, nb)
+    _check(tuple(b_scales.shape) == want_b, f"b_scales must be {want_b}, got {tuple(b_scales.shape)}")
+    out = torch.empty((M, Nn), dtype=out_dtype, device=a.device)
+    lib = N.lib()
+    ws = None
+    ws_bytes = lib.pt_grouped_gemm_fp8_workspace_bytes(G, M, Nn, K, int(trans_b))
+    if ws_bytes:
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
+    N.check(
+        lib.pt_grouped_gemm_fp8(
+            N.ptr(a), N.dtype_code(a.dtype), N.ptr(a_scales),
+            N.ptr(b), N.dtype_code(b.dtype), N.ptr(b_scales),
+            N.ptr(out), N.dtype_code(out.dtype), N.ptr(group_offs), G, M, M, Nn, K, int(trans_b),
+            N.ptr(ws), ws_bytes, TILE_CFG, N.stream_of(a),
+        )
+    )
+    return out
+
+
+@grouped_gemm_fp8_impl.register_fake
+def _grouped_gemm_fp8_impl_fake(a, b, a_scales, b_scales, group_lens, group_offs, trans_a, trans_b, out_dtype,
+                                granularity, num_cu, default_backend, maybe_pre_sync=False, group_offs_out=None):
+    assert a.dim() == 2 and b.dim() == 3
+    n = b.shape[-2] if trans_b else b.shape[-1]
+    return torch.empty((a.shape[0], n), device=a.device, dtype=out_dtype)
+
+
+def _variable_k(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, accumulate):
+    _check(trans_a and not trans_b, "variable-K grouped GEMM computes a^T @ b (trans_a=True, trans_b=False)")
+    N.require_cuda(a, b, a_scales, b_scales, group_offs, out)
+    _check(a.dim() == 2 and b.dim() == 2 and a.shape[0] == b.shape[0], "a and b must be 2-D with the same row count")
+    _check(a.dtype in _FP8 and b.dtype in _FP8, "operands must be float8_e4m3fn / float8_e5m2")
+    a, b = a.contiguous(), b.contiguous()
+    a_scales, b_scales = a_scales.contiguous(), b_scales.contiguous()
+    Mp, Ml = a.shape
+    Nr = b.shape[1]
+    G = group_offs.numel() - 1
+    _check(tuple(a_scales.shape) == ((Mp + 127) // 128, Ml) or a_scales.shape[1] == Ml, "a_scales must be [rows/128, a.shape[1]]")
+    _check(b_scales.shape[1] == Nr, "b_scales must be [rows/128, b.shape[1]]")
+    want = (G, Nr, Ml) if trans_c else (G, Ml, Nr)
+    _check(tuple(out.shape) == want and out.is_contiguous(), f"out must be a contiguous {want} tensor")
+    lib = N.lib()
+    ws_bytes = lib.pt_grouped_gemm_fp8_variable_k_workspace_bytes(Mp, Ml, Nr)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=a.device)
+    N.check(
+        lib.pt_grouped_gemm_fp8_variable_k(
+            N.ptr(a), N.dtype_code(a.dtype), N.ptr(a_scales),
+            N.ptr(b), N.dtype_code(b.dtype), N.ptr(b_scales),
+            N.ptr(out), N.dtype_code(out.dtype), N.ptr(group_offs), G, Mp, Ml, Nr, int(trans_c), int(accumulate),
+            N.ptr(ws), ws_bytes, TILE_CFG, N.stream_of(a),
+        )
+    )
+    return out
+
+
+@torch.library.custom_op("primus_turbo::grouped_gemm_fp8_variable_k_impl", mutates_args=(), device_types="cuda")
+def grouped_gemm_fp8_variable_k_impl(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    a_scales: torch.Tensor,
+    b_scales: torch.Tensor,
+    group_lens: torch.Tensor,
+    group_offs: torch.Tensor,
+    trans_a: bool,
+    trans_b: bool,
+    trans_c: bool,
+    out_dtype: torch.dtype,
+    granularity: int,
+    num_cu: Optional[int],
+    default_backend: int,
+    maybe_pre_sync: bool = False,
+) -> torch.Tensor:
+    """``out[g] = a[p[g]:p[g+1]]^T @ b[p[g]:p[g+1]]`` (transposed when ``trans_c``) over the
+    segment-padded column quantizations; ``group_offs`` holds the padded offsets ``p``."""
+    _require_blockwise(granularity)
+    G = group_offs.numel() - 1
+    shape = (G, b.shape[1], a.shape[1]) if trans_c else (G, a.shape[1], b.shape[1])
+    out = torch.empty(shape, dtype=out_dtype, device=a.device)
+    return _variable_k(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, False)
+
+
+@grouped_gemm_fp8_variable_k_impl.register_fake
+def _grouped_gemm_fp8_variable_k_impl_fake(a, b, a_scales, b_scales, group_lens, group_offs, trans_a, trans_b,
+                                           trans_c, out_dtype, granularity, num_cu, default_backend,
+                                           maybe_pre_sync=False):
+    G = group_offs.numel() - 1
+    shape = (G, b.shape[1], a.shape[1]) if trans_c else (G, a.shape[1], b.shape[1])
+    return torch.empty(shape, dtype=out_dtype, device=a.device)
+
+
+@torch.library.custom_op("primus_turbo::grouped_gemm_fp8_variable_k_accum_impl", mutates_args={"out"}, device_types="cuda")
+def grouped_gemm_fp8_variable_k_accum_impl(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    a_scales: torch.Tensor,
+    b_scales: torch.Tensor,
+    group_lens: torch.Tensor,
+    group_offs: torch.Tensor,
+    trans_a: bool,
+    trans_b: bool,
+    trans_c: bool,
+    out_dtype: torch.dtype,
+    granularity: int,
+    num_cu: Optional[int],
+    default_backend: int,
+    out: torch.Tensor,
+    maybe_pre_sync: bool = False,
+) -> None:
+    """Same product, added into ``out`` in the GEMM epilogue (beta = 1)."""
+    _require_blockwise(granularity)
+    _variable_k(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, True)
+
+
+@grouped_gemm_fp8_variable_k_accum_impl.register_fake
+def _grouped_gemm_fp8_variable_k_accum_impl_fake(a, b, a_scales, b_scales, group_lens, group_offs, trans_a, trans_b,
+                                                 trans_c, out_dtype, granularity, num_cu, default_backend, out,
+                                                 maybe_pre_sync=False):
+    return None

@@ -118,10 +118,13 @@ class FP8GemmRowFunction(torch.autograd.Function):
             return QuantizedTensor.quantize(q.dequantize(), q.real_dtype, config.granularity, axis=axis,
                                             block_size=config.block_size)
 
-        qa_t = other_axis(qa, a_t, -2)
-        qb_t = other_axis(qb, b_t, -2 if trans_b else -1)
         out = _gemm(qa.qdata, qa.scale_inv, trans_a, qb.qdata, qb.scale_inv, trans_b, out_dtype, False, config.granularity)
-        ctx.save_for_backward(qa_t.qdata, qa_t.scale_inv, qb_t.qdata, qb_t.scale_inv)
+        # the operands quantized along their other axis only feed backward: skip them when no
+        # input asks for a gradient (same outputs, two quantizer passes less)
+        if any(ctx.needs_input_grad[:2]):
+            qa_t = other_axis(qa, a_t, -2)
+            qb_t = other_axis(qb, b_t, -2 if trans_b else -1)
+            ctx.save_for_backward(qa_t.qdata, qa_t.scale_inv, qb_t.qdata, qb_t.scale_inv)
         ctx.meta = (trans_a, trans_b, out_dtype, config)
         return out
 

@@ -1,0 +1,150 @@
+"""``grouped_gemm_fp8``: MoE grouped linear layer in FP8 with autograd
+(reference: primus_turbo/pytorch/ops/grouped_gemm_fp8.py:99-265,853-960).
+
+BLOCKWISE (128) is the granularity implemented here: one fused pass over the bf16 activation
+yields the row quantization (forward / dgrad operand) and the segment-padded column
+quantization (wgrad operand); the weight is quantized in 128 x 128 tiles that serve forward
+and backward unchanged.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Union
+
+import torch
+
+from primus_turbo.pytorch.core.backend import BackendType
+from primus_turbo.pytorch.core.low_precision import (
+    Float8QuantConfig,
+    ScalingGranularity,
+    ScalingRecipe,
+)
+from primus_turbo.pytorch.core.quantized_tensor import (
+    QuantizedTensor,
+    QuantizedTensorPair,
+    check_quantized_tensor,
+)
+from primus_turbo.pytorch.kernels.grouped_gemm.grouped_gemm_fp8_impl import (
+    grouped_gemm_fp8_impl,
+    grouped_gemm_fp8_variable_k_accum_impl,
+    grouped_gemm_fp8_variable_k_impl,
+)
+from primus_turbo.pytorch.kernels.grouped_gemm.grouped_gemm_utils import group_offs_from_lens
+from primus_turbo.pytorch.kernels.quantization.quantization_impl import (
+    quant_fp8_blockwise_for_weight_impl,
+    quant_fp8_blockwise_segment_m_row_col_impl,
+)
+from primus_turbo.pytorch.ops.utils import (
+    _ensure_contiguous_grad_out,
+    _get_dummy_wgrad,
+    _get_fp8_dtype,
+    _setup_fused_grad_accum,
+)
+
+__all__ = ["grouped_gemm_fp8"]
+
+_NATIVE = BackendType.TRITON.value  # placeholder id: a single backend exists here
+
+
+def _grouped_gemm_fp8_variable_k_impl_wrapper(a, b, a_scales, b_scales, group_lens, group_offs, trans_a, trans_b,
+                                              trans_c, out_dtype, granularity, num_cu, default_backend,
+                                              inplace_add_to_out=False, out=None):
+    """Variable-K wgrad GEMM; with ``inplace_add_to_out`` the product is added into ``out``
+    (fp32 ``main_grad``) and a placeholder in the weight's dtype is returned for autograd."""
+    if not inplace_add_to_out:
+        return grouped_gemm_fp8_variable_k_impl(a, b, a_scales, b_scales, group_lens, group_offs, trans_a, trans_b,
+                                                trans_c, out_dtype, granularity, num_cu, default_backend)
+    assert out is not None, "out should not be None when inplace_add_to_out is True"
+    grouped_gemm_fp8_variable_k_accum_impl(a, b, a_scales, b_scales, group_lens, group_offs, trans_a, trans_b,
+                                           trans_c, out.dtype, granularity, num_cu, default_backend, out)
+    return _get_dummy_wgrad(out.shape, out_dtype)
+
+
+class FP8GroupedGemmBlockFunc(torch.autograd.Function):
+    """BLOCKWISE grouped GEMM autograd."""
+
+    @staticmethod
+    def forward(ctx, a, b, a_t, b_t, group_lens, group_offs, trans_b, out_dtype, config, num_cu,
+                fuse_bgrad_accum_pattern=None):
+        fuse_bgrad_accum, main_grad = _setup_fused_grad_accum(b, fuse_bgrad_accum_pattern)
+        assert config.granularity == ScalingGranularity.BLOCKWISE
+        assert config.block_size in [128], "Only block_size 128 is supported currently."
+        if isinstance(a, QuantizedTensor):
+            raise NotImplementedError("FP8GroupedGemmBlockFunc does not support a pre-quantized activation `a`")
+        assert a.ndim == 2, "Input tensor must be 2-dimensional."
+        assert b.ndim == 3, "Weight tensor must be 3-dimensional."
+        assert group_lens.size(0) == b.size(0), "group_lens size must match b size(0)."
+        assert out_dtype in [torch.float16, torch.bfloat16]
+        a_dtype = _get_fp8_dtype(config.format, True)
+        b_dtype = _get_fp8_dtype(config.format, True)
+
+        gemm_n = b.size(-2) if trans_b else b.size(-1)
+        a_fp8_row, a_fp8_col, a_scale_row, a_scale_col, _, _ = quant_fp8_blockwise_segment_m_row_col_impl(
+            a.contiguous(), a_dtype, config.block_size, group_lens, group_offs, gemm_other_dim=gemm_n
+        )
+        b_recipe = ScalingRecipe(use_2d_block=True)
+        if isinstance(b, QuantizedTensor):
+            check_quantized_tensor(b, config, scaling_recipe=b_recipe)
+            b_fp8, b_scale = b.qdata, b.scale_inv
+        else:
+            b_fp8, b_scale = quant_fp8_blockwise_for_weight_impl(b, b_dtype, block_size=config.block_size)
+
+        out = grouped_gemm_fp8_impl(a_fp8_row, b_fp8, a_scale_row, b_scale, group_lens, group_offs, False, trans_b,
+                                    out_dtype, config.granularity.value, num_cu, _NATIVE)
+        ctx.save_for_backward(a_fp8_col, a_scale_col, b_fp8, b_scale, group_lens, group_offs)
+        ctx.meta = (trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        grad_out = _ensure_contiguous_grad_out(grad_out)
+        a_fp8_col, a_scale_col, b_fp8, b_scale, group_lens, group_offs = ctx.saved_tensors
+        trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad = ctx.meta
+        g_dtype = _get_fp8_dtype(config.format, False)
+        gran = config.granularity.value
+
+        gemm_k = b_fp8.size(-1) if trans_b else b_fp8.size(-2)
+        g_row, g_col, g_scale_row, g_scale_col, var_k_lens, var_k_offs = quant_fp8_blockwise_segment_m_row_col_impl(
+            grad_out, g_dtype, config.block_size, group_lens, group_offs, gemm_other_dim=gemm_k
+        )
+        # grad_a = grad_out @ b^T
+        grad_a = grouped_gemm_fp8_impl(g_row, b_fp8, g_scale_row, b_scale, group_lens, group_offs, False, not trans_b,
+                                       out_dtype, gran, num_cu, _NATIVE)
+        # grad_b[g] = a_g^T @ grad_out_g
+        grad_b = _grouped_gemm_fp8_variable_k_impl_wrapper(
+            a_fp8_col, g_col, a_scale_col, g_scale_col, var_k_lens, var_k_offs, True, False, trans_b, out_dtype, gran,
+            num_cu, _NATIVE, inplace_add_to_out=fuse_bgrad_accum, out=main_grad,
+        )
+        return grad_a, grad_b, None, None, None, None, None, None, None, None, None
+
+
+def grouped_gemm_fp8(
+    a: Union[torch.Tensor, QuantizedTensor, QuantizedTensorPair],
+    b: Union[torch.Tensor, QuantizedTensor, QuantizedTensorPair],
+    group_lens: torch.Tensor,
+    group_offs: Optional[torch.Tensor] = None,
+    trans_b: bool = True,
+    out_dtype: Optional[torch.dtype] = None,
+    config: Optional[Float8QuantConfig] = None,
+    num_cu: Optional[int] = None,
+    fuse_bgrad_accum_pattern: Optional[str] = None,
+) -> torch.Tensor:
+    """Grouped GEMM with FP8 quantization: ``out[rows of group g] = a[rows of group g] @ op(b[g])``.
+
+    ``a``: ``[sum(group_lens), k]`` (fp16 / bf16); ``b``: ``[G, n, k]`` if ``trans_b`` else
+    ``[G, k, n]`` (or a pre-quantized 2-D-block ``QuantizedTensor``); ``group_lens``: int64 ``[G]``
+    on the device (groups may be empty); ``config``: BLOCKWISE with ``block_size=128``."""
+    if config is None:
+        config = Float8QuantConfig()
+    if group_offs is None:
+        group_offs = group_offs_from_lens(group_lens)
+    a_data, a_data_t = (a.data, a.data_t) if isinstance(a, QuantizedTensorPair) else (a, None)
+    b_data, b_data_t = (b.data, b.data_t) if isinstance(b, QuantizedTensorPair) else (b, None)
+    if out_dtype is None:
+        out_dtype = torch.promote_types(a_data.dtype, b_data.dtype)
+    if config.granularity == ScalingGranularity.BLOCKWISE:
+        return FP8GroupedGemmBlockFunc.apply(a_data, b_data, a_data_t, b_data_t, group_lens, group_offs, trans_b,
+                                             out_dtype, config, num_cu, fuse_bgrad_accum_pattern)
+    raise NotImplementedError(
+        f"grouped_gemm_fp8: granularity {config.granularity} is not implemented (BLOCKWISE with block_size=128 is)"
+    )

@@ -40,3 +40,29 @@ def round_to(t_f32: np.ndarray, dtype: torch.dtype) -> torch.Tensor:
 
 
 FMT = {torch.float8_e4m3fn: "e4m3", torch.float8_e5m2: "e5m2"}
+
+
+def group_lens(kind, G_, total, seed):
+    """Per-group row counts summing to ``total``: balanced, ragged, two non-empty groups, or
+    Zipf(1.2)-skewed with two groups forced empty."""
+    rng = np.random.default_rng(seed)
+    if kind == "balanced":
+        return np.full(G_, total // G_, dtype=np.int64)
+    if kind == "ragged":
+        w = 0.2 + 0.8 * rng.random(G_)
+        lens = np.floor(w / w.sum() * total).astype(np.int64)
+        lens[-1] += total - lens.sum()
+        return lens
+    if kind == "zeros":
+        lens = np.zeros(G_, dtype=np.int64)
+        lens[0] = total // 2
+        lens[1] = total - total // 2
+        return lens
+    if kind == "zipf":
+        w = (1.0 + np.arange(G_)) ** -1.2
+        w = rng.permutation(w)
+        w[rng.choice(G_, 2, replace=False)] = 0
+        lens = np.floor(w / w.sum() * total).astype(np.int64)
+        lens[np.argmax(lens)] += total - lens.sum()
+        return lens
+    raise ValueError(kind)

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import FMT, bf16_randn, bits_np, codes_np, round_to, to_f32_np
+from helpers import FMT, bf16_randn, bits_np, codes_np, round_to, to_f32_np, group_lens
 from oracle import quantize as Q
 
 pytestmark = pytest.mark.gpu
@@ -92,30 +92,6 @@ def test_blockwise_weight(shape, dtype):
         assert np.array_equal(bits_np(y), bits_np(want))
 
 
-def _lens(kind, G_, total, seed):
-    rng = np.random.default_rng(seed)
-    if kind == "balanced":
-        return np.full(G_, total // G_, dtype=np.int64)
-    if kind == "ragged":
-        w = 0.2 + 0.8 * rng.random(G_)
-        lens = np.floor(w / w.sum() * total).astype(np.int64)
-        lens[-1] += total - lens.sum()
-        return lens
-    if kind == "zeros":
-        lens = np.zeros(G_, dtype=np.int64)
-        lens[0] = total // 2
-        lens[1] = total - total // 2
-        return lens
-    if kind == "zipf":
-        w = (1.0 + np.arange(G_)) ** -1.2
-        w = rng.permutation(w)
-        w[rng.choice(G_, 2, replace=False)] = 0
-        lens = np.floor(w / w.sum() * total).astype(np.int64)
-        lens[np.argmax(lens)] += total - lens.sum()
-        return lens
-    raise ValueError(kind)
-
-
 @pytest.mark.parametrize(
     "kind,G_,M,N",
     [
@@ -128,7 +104,7 @@ def _lens(kind, G_, total, seed):
     ],
 )
 def test_grouped_segment_row_col(kind, G_, M, N):
-    lens = _lens(kind, G_, M, 24)
+    lens = group_lens(kind, G_, M, 24)
     assert lens.sum() == M
     x = bf16_randn((M, N), seed=25, outlier_frac=0.001)
     gl = torch.from_numpy(lens).cuda()
