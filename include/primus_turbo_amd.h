@@ -171,6 +171,37 @@ PT_API int pt_dequantize_fp8_block(const void *q, int q_dtype, int64_t B, int64_
                                    const float *scale_inv, int64_t block_m, int64_t block_n,
                                    void *y, int y_dtype, void *stream);
 
+/* MX (microscaling) quantizers ------------------------------------------------
+ *
+ * pt_quantize_mx replaces the dispatcher ops quantize_mxfp8 / quantize_mxfp8_dual /
+ * quantize_mxfp4 / quantize_mxfp4_dual (csrc/pytorch/quantization/quantization.cpp:511-969,
+ * schemas csrc/pytorch/bindings_pytorch.cpp:52-93) and the FlyDSL kernels the Python layer
+ * prefers for them (primus_turbo/flydsl/quantization/mxfp8_quant_flydsl.py:337-525,
+ * mxfp4_quant_kernel.py:354-481), for round-to-nearest-even without RHT, stochastic rounding
+ * or output shuffling.
+ *
+ * x is [B, M, N] bf16 / fp16 (B = 1 for a matrix). q_dtype: PT_DTYPE_E4M3, PT_DTYPE_E5M2
+ * (MXFP8) or PT_DTYPE_E2M1X2 (MXFP4, two codes per byte). One E8M0 byte per 32 elements:
+ *   e = clamp((((bits(amax) + R) >> 23) & 0x1FF) - 127 - T, -127, 128),  byte = e + 127,
+ *   q = rne_sat(clamp(x * 2^-e, +-qmax));  (R, T) = (1<<19, 8) E4M3, (1<<20, 15) E5M2,
+ *   (1<<21, 2) E2M1.
+ * Row direction (blocks of 32 along N): row_q [B, M, Npad] codes (FP4: Npad / 2 bytes per
+ * row), row_scale [B, M, Npad / 32]; Npad = N rounded up to 128, the padding is zero data
+ * with scale byte 0. Column direction (blocks of 32 along M), emitted transposed:
+ * col_q [B, N, Mpad], col_scale [B, N, Mpad / 32]. Either pair may be NULL. row_2d / col_2d
+ * != 0 share one exponent per 32 x 32 tile (weights).
+ *
+ * pt_dequantize_mx replaces dequantize_mxfp8 / dequantize_mxfp4 (quantization.cpp:285-359,
+ * 436-508; kernels dequantization_mxfp8.cu:29-113, dequantization_mxfp4.cu:28-160):
+ *   y[r, c] = T(float(q[r, c]) * bits_to_f32(scale[r, c / 32] << 23))
+ * over q [rows, cols] (cols % 32 == 0; FP4 packed), written as y [rows, cols] or, for
+ * column-direction data, transposed back as y [cols, rows]. */
+PT_API int pt_quantize_mx(const void *x, int x_dtype, int64_t B, int64_t M, int64_t N, int q_dtype,
+                          void *row_q, void *row_scale, int row_2d, void *col_q, void *col_scale,
+                          int col_2d, void *stream);
+PT_API int pt_dequantize_mx(const void *q, int q_dtype, const void *scale, int64_t rows,
+                            int64_t cols, void *y, int y_dtype, int transpose, void *stream);
+
 /* Scaled FP8 GEMM -------------------------------------------------------------
  *
  * Replaces primus_turbo::gemm_fp8_impl / gemm_fp8_accum_impl

@@ -1,0 +1,397 @@
+// MX (microscaling) quantizers and de-quantizers for gfx950: MXFP8 (E4M3 / E5M2) and MXFP4
+// (E2M1), one E8M0 shared exponent per 32 elements.
+//
+// Numerics (Primus-Turbo's MX quantizers: flydsl/quantization/mxfp8_quant_flydsl.py:44-66,
+// flydsl/quantization/mxfp4_quant_kernel.py:78-89,121-149; de-quantizers
+// csrc/kernels/quantization/dequantization_mxfp8.cu:29-113, dequantization_mxfp4.cu:28-160):
+//   amax  = max |x| over the block (NaN ignored)
+//   e     = clamp((((bits(amax) + R) >> 23) & 0x1FF) - 127 - T, -127, 128)   (integers)
+//           (R, T) = (1 << 19, 8) E4M3, (1 << 20, 15) E5M2, (1 << 21, 2) E2M1
+//   scale byte = e + 127;  q = rne_sat(clamp(x * 2^-e, +-qmax))  (NaN -> +qmax)
+//   FP4: element 2p in the low nibble, 2p + 1 in the high nibble of byte p
+//   de-quantize: y = T(float(q) * bits_to_f32(byte << 23))
+//
+// One workgroup handles a 128 x 128 tile: it is read once into LDS (raw 16-bit), then
+// quantized along rows (blocks of 32 columns) and/or along columns (blocks of 32 rows, output
+// transposed), so the dual quantizer reads HBM once. The "2-D block" variants share one
+// exponent per 32 x 32 tile.
+#include "pt_common.h"
+
+namespace pt {
+
+enum : int { MX_E4M3 = 0, MX_E5M2 = 1, MX_E2M1 = 2 };
+
+template <int FMT> struct MxFmt;
+template <> struct MxFmt<MX_E4M3> {
+    static constexpr uint32_t R = 1u << 19;
+    static constexpr int      T = 8;
+    static constexpr float    QMAX = 448.f;
+};
+template <> struct MxFmt<MX_E5M2> {
+    static constexpr uint32_t R = 1u << 20;
+    static constexpr int      T = 15;
+    static constexpr float    QMAX = 57344.f;
+};
+template <> struct MxFmt<MX_E2M1> {
+    static constexpr uint32_t R = 1u << 21;
+    static constexpr int      T = 2;
+    static constexpr float    QMAX = 6.f;
+};
+
+// shared exponent of a block (unbiased) from its abs-max
+template <int FMT> __device__ __forceinline__ int mx_exponent(float amax) {
+    const uint32_t b = __float_as_uint(amax);
+    int            e = static_cast<int>(((b + MxFmt<FMT>::R) >> 23) & 0x1FFu) - 127 - MxFmt<FMT>::T;
+    e                = e < -127 ? -127 : e;
+    return e > 128 ? 128 : e;
+}
+
+// 2^-e as a float; e stays within [-127, 126] for every finite or infinite abs-max
+__device__ __forceinline__ float mx_inv_scale(int e) {
+    return __uint_as_float(static_cast<uint32_t>(127 - e) << 23);
+}
+
+// 32 scaled values -> packed codes. FP8: 8 dwords, FP4: 4 dwords.
+template <int FMT> __device__ __forceinline__ void mx_encode32(const float (&v)[32], float inv, uint32_t (&out)[8]) {
+    constexpr float Q = MxFmt<FMT>::QMAX;
+    if constexpr (FMT == MX_E2M1) {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            uint32_t w = 0;
+            // byte k of the dword holds elements 8 d + 2 k (low nibble) and 8 d + 2 k + 1
+            w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp(v[8 * d + 0], inv, Q), scale_clamp(v[8 * d + 1], inv, Q), 1.0f, 0);
+            w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp(v[8 * d + 2], inv, Q), scale_clamp(v[8 * d + 3], inv, Q), 1.0f, 1);
+            w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp(v[8 * d + 4], inv, Q), scale_clamp(v[8 * d + 5], inv, Q), 1.0f, 2);
+            w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp(v[8 * d + 6], inv, Q), scale_clamp(v[8 * d + 7], inv, Q), 1.0f, 3);
+            out[d] = w;
+        }
+    } else {
+#pragma unroll
+        for (int d = 0; d < 8; ++d)
+            out[d] = cvt4_fp8<FMT == MX_E5M2>(scale_clamp(v[4 * d], inv, Q), scale_clamp(v[4 * d + 1], inv, Q),
+                                              scale_clamp(v[4 * d + 2], inv, Q), scale_clamp(v[4 * d + 3], inv, Q));
+    }
+}
+
+constexpr int MX_TILE  = 128;
+constexpr int MX_PITCH = MX_TILE + 8; // 16-bit elements per LDS row (272 B: 16-byte aligned rows)
+
+struct MxArgs {
+    const void *x; // [B, M, N] bf16 / fp16
+    int64_t     B, M, N, Mpad, Npad;
+    uint8_t    *row_q; // [B, M, Npad] (FP4: Npad / 2 bytes per row) or NULL
+    uint8_t    *row_s; // [B, M, Npad / 32] or NULL
+    uint8_t    *col_q; // [B, N, Mpad] (FP4: Mpad / 2) or NULL
+    uint8_t    *col_s; // [B, N, Mpad / 32] or NULL
+};
+
+// fabsf(x) with NaN mapped to 0 (fmaxf-style abs-max ignores NaN)
+__device__ __forceinline__ float abs_or_zero(float x) {
+    const float a = fabsf(x);
+    return a == a ? a : 0.f;
+}
+
+template <typename T, int FMT, bool ROW, bool COL, bool ROW2D, bool COL2D>
+__global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
+    constexpr bool ANY2D = (ROW && ROW2D) || (COL && COL2D);
+    __shared__ __attribute__((aligned(16))) uint16_t tile[MX_TILE * MX_PITCH];
+    __shared__ float                                 amax_rc[ANY2D ? MX_TILE * 4 : 1]; // [row][32-col block]
+    const int     tid = threadIdx.x;
+    const int64_t n0 = static_cast<int64_t>(blockIdx.x) * MX_TILE, m0 = static_cast<int64_t>(blockIdx.y) * MX_TILE;
+    const int64_t b  = blockIdx.z;
+    const uint16_t *x = static_cast<const uint16_t *>(a.x) + b * a.M * a.N;
+
+    // ---- tile -> LDS (zeros outside the matrix) ----
+    const bool vec = (a.N & 7) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+        const int     r = p * 16 + (tid >> 4), c = (tid & 15) * 8;
+        const int64_t m = m0 + r, n = n0 + c;
+        u32x4         v = u32x4{0u, 0u, 0u, 0u};
+        if (m < a.M && n < a.N) {
+            if (vec) {
+                v = ld128(x + m * a.N + n);
+            } else {
+                uint16_t e[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    e[k] = n + k < a.N ? x[m * a.N + n + k] : uint16_t(0);
+                v = u32x4{e[0] | (uint32_t(e[1]) << 16), e[2] | (uint32_t(e[3]) << 16), e[4] | (uint32_t(e[5]) << 16),
+                          e[6] | (uint32_t(e[7]) << 16)};
+            }
+        }
+        *reinterpret_cast<u32x4 *>(&tile[r * MX_PITCH + c]) = v;
+    }
+    __syncthreads();
+
+    auto elem = [&](uint16_t raw) -> float {
+        T t;
+        __builtin_memcpy(&t, &raw, 2);
+        return HP<T>::to_f32(t);
+    };
+
+    // ---- row direction: task = (row r, 32-column block c) ----
+    float rv[2][32];
+    float ram[2];
+    if constexpr (ROW || ANY2D) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const int t = tid + 256 * p, r = t >> 2, c = t & 3;
+            float     am = 0.f;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const u32x4    w    = *reinterpret_cast<const u32x4 *>(&tile[r * MX_PITCH + c * 32 + q * 8]);
+                const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float lo = elem(static_cast<uint16_t>(ww[k] & 0xffffu)), hi = elem(static_cast<uint16_t>(ww[k] >> 16));
+                    rv[p][q * 8 + 2 * k]     = lo;
+                    rv[p][q * 8 + 2 * k + 1] = hi;
+                    am = fmaxf(am, fmaxf(abs_or_zero(lo), abs_or_zero(hi)));
+                }
+            }
+            ram[p] = am;
+            if constexpr (ANY2D)
+                amax_rc[r * 4 + c] = am;
+        }
+    }
+    if constexpr (ANY2D)
+        __syncthreads();
+    if constexpr (ROW) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const int     t = tid + 256 * p, r = t >> 2, c = t & 3;
+            const int64_t m = m0 + r;
+            float         am = ram[p];
+            if constexpr (ROW2D) {
+                const int rb = r & ~31;
+                am           = 0.f;
+#pragma unroll 8
+                for (int i = 0; i < 32; ++i)
+                    am = fmaxf(am, amax_rc[(rb + i) * 4 + c]);
+            }
+            const int e = mx_exponent<FMT>(am);
+            uint32_t  code[8];
+            mx_encode32<FMT>(rv[p], mx_inv_scale(e), code);
+            if (m < a.M) {
+                const int64_t nb = (n0 >> 5) + c; // 32-column block index in the padded row
+                a.row_s[(b * a.M + m) * (a.Npad >> 5) + nb] = static_cast<uint8_t>(e + 127);
+                if constexpr (FMT == MX_E2M1) {
+                    uint8_t *q = a.row_q + (b * a.M + m) * (a.Npad >> 1) + nb * 16;
+                    st128(q, u32x4{code[0], code[1], code[2], code[3]});
+                } else {
+                    uint8_t *q = a.row_q + (b * a.M + m) * a.Npad + nb * 32;
+                    st128(q, u32x4{code[0], code[1], code[2], code[3]});
+                    st128(q + 16, u32x4{code[4], code[5], code[6], code[7]});
+                }
+            }
+        }
+    }
+
+    // ---- column direction: task = (column n, 32-row block rb); output transposed ----
+    if constexpr (COL) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const int     t = tid + 256 * p, c = t & 127, rb = t >> 7;
+            const int64_t n = n0 + c;
+            float         v[32];
+            float         am = 0.f;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                v[i] = elem(tile[(rb * 32 + i) * MX_PITCH + c]);
+                am   = fmaxf(am, abs_or_zero(v[i]));
+            }
+            if constexpr (COL2D) {
+                am = 0.f;
+#pragma unroll 8
+                for (int i = 0; i < 32; ++i)
+                    am = fmaxf(am, amax_rc[(rb * 32 + i) * 4 + (c >> 5)]);
+            }
+            const int e = mx_exponent<FMT>(am);
+            uint32_t  code[8];
+            mx_encode32<FMT>(v, mx_inv_scale(e), code);
+            if (n < a.N) {
+                const int64_t mb = (m0 >> 5) + rb;
+                a.col_s[(b * a.N + n) * (a.Mpad >> 5) + mb] = static_cast<uint8_t>(e + 127);
+                if constexpr (FMT == MX_E2M1) {
+                    uint8_t *q = a.col_q + (b * a.N + n) * (a.Mpad >> 1) + mb * 16;
+                    st128(q, u32x4{code[0], code[1], code[2], code[3]});
+                } else {
+                    uint8_t *q = a.col_q + (b * a.N + n) * a.Mpad + mb * 32;
+                    st128(q, u32x4{code[0], code[1], code[2], code[3]});
+                    st128(q + 16, u32x4{code[4], code[5], code[6], code[7]});
+                }
+            }
+        }
+    }
+}
+
+template <typename T, int FMT, bool ROW, bool COL>
+static void launch_mx_2d(const MxArgs &a, bool row2d, bool col2d, dim3 grid, hipStream_t st) {
+    if (row2d && col2d)
+        mx_quant_kernel<T, FMT, ROW, COL, ROW, COL><<<grid, 256, 0, st>>>(a);
+    else if (row2d)
+        mx_quant_kernel<T, FMT, ROW, COL, ROW, false><<<grid, 256, 0, st>>>(a);
+    else if (col2d)
+        mx_quant_kernel<T, FMT, ROW, COL, false, COL><<<grid, 256, 0, st>>>(a);
+    else
+        mx_quant_kernel<T, FMT, ROW, COL, false, false><<<grid, 256, 0, st>>>(a);
+}
+
+template <typename T, int FMT>
+static void launch_mx_dir(const MxArgs &a, bool row2d, bool col2d, dim3 grid, hipStream_t st) {
+    const bool row = a.row_q != nullptr, col = a.col_q != nullptr;
+    if (row && col)
+        launch_mx_2d<T, FMT, true, true>(a, row2d, col2d, grid, st);
+    else if (row)
+        launch_mx_2d<T, FMT, true, false>(a, row2d, false, grid, st);
+    else
+        launch_mx_2d<T, FMT, false, true>(a, false, col2d, grid, st);
+}
+
+template <typename T> static void launch_mx_fmt(const MxArgs &a, int fmt, bool row2d, bool col2d, dim3 grid, hipStream_t st) {
+    if (fmt == MX_E4M3)
+        launch_mx_dir<T, MX_E4M3>(a, row2d, col2d, grid, st);
+    else if (fmt == MX_E5M2)
+        launch_mx_dir<T, MX_E5M2>(a, row2d, col2d, grid, st);
+    else
+        launch_mx_dir<T, MX_E2M1>(a, row2d, col2d, grid, st);
+}
+
+// ---------------------------------------------------------------------------
+// de-quantize: q [rows, cols] codes (FP4 packed) with scales [rows, cols / 32]
+//   -> y [rows, cols], or y [cols, rows] when `transpose` (column-direction data)
+// One workgroup per 64 x 64 tile through LDS so that both layouts store whole lines.
+// ---------------------------------------------------------------------------
+template <typename T, int FMT>
+__global__ __launch_bounds__(256) void mx_dequant_kernel(const uint8_t *__restrict__ q, const uint8_t *__restrict__ s,
+                                                         T *__restrict__ y, const int64_t rows, const int64_t cols,
+                                                         const int transpose) {
+    __shared__ float t[64][65];
+    const int64_t    r0 = static_cast<int64_t>(blockIdx.y) * 64, c0 = static_cast<int64_t>(blockIdx.x) * 64;
+    const int        tx = threadIdx.x & 15, ty = threadIdx.x >> 4; // thread: row ty + 16 p, columns 4 tx .. 4 tx + 3
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int     r  = ty + 16 * p;
+        const int64_t gr = r0 + r, gc = c0 + tx * 4;
+        float         v[4] = {0.f, 0.f, 0.f, 0.f};
+        if (gr < rows && gc < cols) { // cols is a multiple of 32: a group of 4 is all in or all out
+            const float sc = __uint_as_float(static_cast<uint32_t>(s[gr * (cols >> 5) + (gc >> 5)]) << 23);
+            if constexpr (FMT == MX_E2M1) {
+                const uint16_t w = *reinterpret_cast<const uint16_t *>(q + gr * (cols >> 1) + (gc >> 1));
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t nib = (w >> (4 * k)) & 0xFu;
+                    // E2M1: 1 sign, 2 exponent, 1 mantissa bits: {0, .5, 1, 1.5, 2, 3, 4, 6}
+                    const uint32_t mag = nib & 7u;
+                    const float    f   = mag < 2 ? 0.5f * mag : __uint_as_float(((126u + (mag >> 1)) << 23) | ((mag & 1u) << 22));
+                    v[k]               = (nib & 8u ? -f : f) * sc;
+                }
+            } else {
+                const uint32_t w = *reinterpret_cast<const uint32_t *>(q + gr * cols + gc);
+                v[0] = fp8_to_f32<FMT == MX_E5M2>(w, 0) * sc;
+                v[1] = fp8_to_f32<FMT == MX_E5M2>(w, 1) * sc;
+                v[2] = fp8_to_f32<FMT == MX_E5M2>(w, 2) * sc;
+                v[3] = fp8_to_f32<FMT == MX_E5M2>(w, 3) * sc;
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            t[r][tx * 4 + k] = v[k];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int r = ty + 16 * p; // output row within the tile
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int c = tx * 4 + k;
+            if (!transpose) {
+                if (r0 + r < rows && c0 + c < cols)
+                    y[(r0 + r) * cols + c0 + c] = HP<T>::from_f32(t[r][c]);
+            } else {
+                if (c0 + r < cols && r0 + c < rows)
+                    y[(c0 + r) * rows + r0 + c] = HP<T>::from_f32(t[c][r]);
+            }
+        }
+    }
+}
+
+template <int FMT>
+static void launch_mx_dequant(const uint8_t *q, const uint8_t *s, void *y, int ydtype, int64_t rows, int64_t cols,
+                              int transpose, hipStream_t st) {
+    dim3 grid(static_cast<unsigned>(cdiv(cols, 64)), static_cast<unsigned>(cdiv(rows, 64)));
+    if (ydtype == PT_DTYPE_BF16)
+        mx_dequant_kernel<bf16_t, FMT><<<grid, 256, 0, st>>>(q, s, static_cast<bf16_t *>(y), rows, cols, transpose);
+    else if (ydtype == PT_DTYPE_F16)
+        mx_dequant_kernel<f16_t, FMT><<<grid, 256, 0, st>>>(q, s, static_cast<f16_t *>(y), rows, cols, transpose);
+    else
+        mx_dequant_kernel<float, FMT><<<grid, 256, 0, st>>>(q, s, static_cast<float *>(y), rows, cols, transpose);
+}
+
+static int mx_fmt_of(int dtype) {
+    return dtype == PT_DTYPE_E4M3 ? MX_E4M3 : dtype == PT_DTYPE_E5M2 ? MX_E5M2 : dtype == PT_DTYPE_E2M1X2 ? MX_E2M1 : -1;
+}
+
+} // namespace pt
+
+using namespace pt;
+
+extern "C" {
+
+int pt_quantize_mx(const void *x, int x_dtype, int64_t B, int64_t M, int64_t N, int q_dtype, void *row_q,
+                   void *row_scale, int row_2d, void *col_q, void *col_scale, int col_2d, void *stream) {
+    PT_REQUIRE(x_dtype == PT_DTYPE_BF16 || x_dtype == PT_DTYPE_F16, "input must be bf16 or fp16");
+    const int fmt = mx_fmt_of(q_dtype);
+    PT_REQUIRE(fmt >= 0, "q_dtype must be e4m3, e5m2 or e2m1x2");
+    PT_REQUIRE(B >= 0 && M >= 0 && N >= 0, "dimensions must be non-negative");
+    PT_REQUIRE((row_q != nullptr) == (row_scale != nullptr) && (col_q != nullptr) == (col_scale != nullptr),
+               "codes and scales come in pairs");
+    PT_REQUIRE(row_q || col_q, "nothing to produce");
+    if (B == 0 || M == 0 || N == 0)
+        return PT_OK;
+    PT_REQUIRE(x, "NULL input");
+    PT_REQUIRE(aligned_to(row_q, 16) && aligned_to(col_q, 16), "outputs must be 16-byte aligned");
+    MxArgs a;
+    a.x     = x;
+    a.B     = B;
+    a.M     = M;
+    a.N     = N;
+    a.Mpad  = cdiv(M, 128) * 128;
+    a.Npad  = cdiv(N, 128) * 128;
+    a.row_q = static_cast<uint8_t *>(row_q);
+    a.row_s = static_cast<uint8_t *>(row_scale);
+    a.col_q = static_cast<uint8_t *>(col_q);
+    a.col_s = static_cast<uint8_t *>(col_scale);
+    PT_REQUIRE(a.Mpad / 128 < 65536 && B < 65536, "grid dimension out of range");
+    dim3 grid(static_cast<unsigned>(a.Npad / 128), static_cast<unsigned>(a.Mpad / 128), static_cast<unsigned>(B));
+    auto st = static_cast<hipStream_t>(stream);
+    if (x_dtype == PT_DTYPE_BF16)
+        launch_mx_fmt<bf16_t>(a, fmt, row_2d != 0, col_2d != 0, grid, st);
+    else
+        launch_mx_fmt<f16_t>(a, fmt, row_2d != 0, col_2d != 0, grid, st);
+    return check_launch("mx_quant_kernel");
+}
+
+int pt_dequantize_mx(const void *q, int q_dtype, const void *scale, int64_t rows, int64_t cols, void *y, int y_dtype,
+                     int transpose, void *stream) {
+    const int fmt = mx_fmt_of(q_dtype);
+    PT_REQUIRE(fmt >= 0, "q_dtype must be e4m3, e5m2 or e2m1x2");
+    PT_REQUIRE(is_hp_dtype(y_dtype), "output must be bf16, fp16 or fp32");
+    PT_REQUIRE(rows >= 0 && cols >= 0 && cols % 32 == 0, "cols must be a non-negative multiple of 32");
+    if (rows == 0 || cols == 0)
+        return PT_OK;
+    PT_REQUIRE(q && scale && y, "NULL pointer");
+    PT_REQUIRE(cdiv(rows, 64) < 65536, "grid dimension out of range");
+    auto           st = static_cast<hipStream_t>(stream);
+    const uint8_t *qq = static_cast<const uint8_t *>(q), *ss = static_cast<const uint8_t *>(scale);
+    if (fmt == MX_E4M3)
+        launch_mx_dequant<MX_E4M3>(qq, ss, y, y_dtype, rows, cols, transpose, st);
+    else if (fmt == MX_E5M2)
+        launch_mx_dequant<MX_E5M2>(qq, ss, y, y_dtype, rows, cols, transpose, st);
+    else
+        launch_mx_dequant<MX_E2M1>(qq, ss, y, y_dtype, rows, cols, transpose, st);
+    return check_launch("mx_dequant_kernel");
+}
+
+} // extern "C"

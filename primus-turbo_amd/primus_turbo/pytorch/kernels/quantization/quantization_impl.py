@@ -558,3 +558,146 @@ def quant_fp8_blockwise_segment_m_row_col_impl(
 def _quant_fp8_blockwise_segment_m_row_col_impl_fake(x, dtype, block_size, group_lens, group_offs, gemm_other_dim=None):
     r = _quantize_fp8_blockwise_segment_m_row_col_meta(x, dtype, block_size, group_lens, group_offs)
     return r[0], r[1], r[2], r[3], r[4], r[5]
+
+
+# ---------------------------------------------------------------------------------------
+# MX quantizers (E8M0 scale per 32 elements): MXFP8 and MXFP4
+# reference: primus_turbo/pytorch/kernels/quantization/quantization_impl.py:496-569,814-835,
+#            868-1010; shapes from csrc/pytorch/quantization/quantization.cpp:511-969
+# ---------------------------------------------------------------------------------------
+_MX_PAD = 128
+_E8M0 = getattr(torch, "float8_e8m0fnu", torch.uint8)
+_FP4X2 = getattr(torch, "float4_e2m1fn_x2", None)
+
+
+def _mx_recipes(with_trans, scaling_recipe, scaling_recipe_for_trans, what):
+    from primus_turbo.pytorch.core.low_precision import ScalingRecipe
+
+    r = ScalingRecipe() if scaling_recipe is None else scaling_recipe
+    rt = (ScalingRecipe() if scaling_recipe_for_trans is None else scaling_recipe_for_trans) if with_trans else r
+    for rec in (r, rt):
+        if rec.use_sr or rec.use_rht or rec.shuffle_scale or rec.shuffle_out:
+            raise NotImplementedError(
+                f"{what}: stochastic rounding, RHT and shuffled layouts are not implemented "
+                "(round-to-nearest-even, plain layouts are)"
+            )
+    return r, rt
+
+
+def _mx_check_axis(x, axis, with_trans):
+    if not with_trans:
+        if x.ndim == 2:
+            assert axis in (0, 1), "The axis must be 0 or 1 when with_trans is False and x is 2D."
+        elif x.ndim == 3:
+            assert axis in (1, 2), "The axis must be 1 or 2 when with_trans is False and x is 3D."
+        else:
+            raise ValueError(f"The input tensor must be 2D or 3D but got {x.ndim}D.")
+    else:
+        assert axis is None, "The axis must be None when with_trans is True."
+        assert x.ndim in (2, 3), f"The input tensor must be 2D or 3D but got {x.ndim}D."
+
+
+def _mx_quantize(x: torch.Tensor, out_dtype: torch.dtype, want_row: bool, want_col: bool, row_2d: bool, col_2d: bool):
+    """-> (row_q, row_scale, col_q, col_scale); the pair of an unwanted direction is None."""
+    N.require_cuda(x)
+    if x.dtype not in (torch.bfloat16, torch.float16):
+        raise RuntimeError("Input must be BFloat16 or Half")
+    if not x.is_contiguous():
+        raise RuntimeError("Input must be contiguous")
+    fp4 = _FP4X2 is not None and out_dtype == _FP4X2
+    if not fp4 and out_dtype not in (torch.float8_e4m3fn, torch.float8_e5m2):
+        raise RuntimeError("Output must be Float8_e4m3fn, Float8_e5m2 or Float4_e2m1fn_x2")
+    batched = x.dim() == 3
+    B = x.shape[0] if batched else 1
+    M, Nn = x.shape[-2], x.shape[-1]
+    if Nn % 32 != 0:
+        raise RuntimeError(f"N must be divisible by 32, got N={Nn}")
+    Mp, Np = -(-M // _MX_PAD) * _MX_PAD, -(-Nn // _MX_PAD) * _MX_PAD
+    pack = 2 if fp4 else 1
+    lead = (B,) if batched else ()
+    dev = x.device
+    row_q = row_s = col_q = col_s = None
+    if want_row:
+        row_q = torch.empty(lead + (M, Np // pack), dtype=torch.uint8, device=dev)
+        row_s = torch.empty(lead + (M, Np // 32), dtype=torch.uint8, device=dev)
+    if want_col:
+        col_q = torch.empty(lead + (Nn, Mp // pack), dtype=torch.uint8, device=dev)
+        col_s = torch.empty(lead + (Nn, Mp // 32), dtype=torch.uint8, device=dev)
+    N.check(
+        N.lib().pt_quantize_mx(
+            N.ptr(x), N.dtype_code(x.dtype), B, M, Nn, N.dtype_code(out_dtype),
+            N.ptr(row_q), N.ptr(row_s), int(row_2d), N.ptr(col_q), N.ptr(col_s), int(col_2d), N.stream_of(x),
+        )
+    )
+    view = lambda t, dt: None if t is None else t.view(dt)  # noqa: E731
+    return view(row_q, out_dtype), view(row_s, _E8M0), view(col_q, out_dtype), view(col_s, _E8M0)
+
+
+def _quantize_mx_impl(x, out_dtype, axis, block_size, with_trans, scaling_recipe, scaling_recipe_for_trans, what):
+    assert block_size == 32, f"The block size must be 32 for {what} quantization"
+    r, rt = _mx_recipes(with_trans, scaling_recipe, scaling_recipe_for_trans, what)
+    _mx_check_axis(x, axis, with_trans)
+    if with_trans:
+        return _mx_quantize(x, out_dtype, True, True, r.use_2d_block, rt.use_2d_block)
+    rowwise = axis == x.ndim - 1
+    rq, rs, cq, cs = _mx_quantize(x, out_dtype, rowwise, not rowwise, r.use_2d_block, r.use_2d_block)
+    return (rq, rs) if rowwise else (cq, cs)
+
+
+def quantize_mxfp8_impl(x, out_dtype, axis, block_size, with_trans=False, scaling_recipe=None,
+                        scaling_recipe_for_trans=None):
+    """MXFP8 quantization. One direction (``axis``: last = along rows, else the transposed,
+    column-direction output) -> ``(q, scale)``; ``with_trans`` -> ``(q_row, scale_row, q_col,
+    scale_col)`` from a single read of ``x``. Shapes: row ``[.., M, N_pad]`` / ``[.., M, N_pad/32]``,
+    col ``[.., N, M_pad]`` / ``[.., N, M_pad/32]`` with the pads rounding up to 128."""
+    return _quantize_mx_impl(x, out_dtype, axis, block_size, with_trans, scaling_recipe, scaling_recipe_for_trans, "MXFP8")
+
+
+def quantize_mxfp4_impl(x, out_dtype, axis, block_size, with_trans=False, scaling_recipe=None,
+                        scaling_recipe_for_trans=None):
+    """MXFP4 (E2M1, two codes per byte, even element in the low nibble); shapes as MXFP8 with
+    the code tensors half as wide."""
+    assert x.is_contiguous(), "The x tensor must be contiguous."
+    return _quantize_mx_impl(x, out_dtype, axis, block_size, with_trans, scaling_recipe, scaling_recipe_for_trans, "MXFP4")
+
+
+def _dequantize_mx(x, out_dtype, axis, block_size, scale_inv, fp4):
+    assert x.is_contiguous(), "The x tensor must be contiguous."
+    assert x.dim() in (2, 3), "The x must be a 2D or 3D tensor."
+    assert scale_inv.dim() == x.dim(), "The scale_inv rank must match x."
+    assert scale_inv.is_contiguous(), "The scale_inv tensor must be contiguous."
+    if x.dim() == 2:
+        assert axis in (0, 1), "The axis must be 0 or 1 for 2D input."
+    else:
+        assert axis in (1, 2), "The axis must be 1 or 2 for 3D input."
+    assert out_dtype in (torch.float16, torch.bfloat16, torch.float32), f"unsupported out dtype {out_dtype}"
+    assert block_size == 32
+    N.require_cuda(x, scale_inv)
+    rowwise = axis == x.dim() - 1
+    rows = x.shape[0] if x.dim() == 2 else x.shape[0] * x.shape[1]
+    cols = x.shape[-1] * (2 if fp4 else 1)
+    assert cols % block_size == 0, "The last dimension of the x tensor must be divisible by the block size."
+    assert scale_inv.numel() == rows * (cols // 32), "scale_inv does not match x"
+    out = torch.empty((rows, cols) if rowwise else (cols, rows), dtype=out_dtype, device=x.device)
+    N.check(
+        N.lib().pt_dequantize_mx(
+            N.ptr(x), N.dtype_code(x.dtype), N.ptr(scale_inv), rows, cols, N.ptr(out), N.dtype_code(out_dtype),
+            int(not rowwise), N.stream_of(x),
+        )
+    )
+    if x.dim() == 3:
+        if rowwise:
+            return out.reshape(x.shape[0], x.shape[1], cols)
+        return out.reshape(cols, x.shape[0], x.shape[1]).permute(1, 2, 0)
+    return out
+
+
+def dequantize_mxfp8_impl(x, out_dtype, axis, block_size, scale_inv):
+    """``y = float(q) * 2^(byte - 127)`` per 32-element block of the last axis; ``axis`` other
+    than the last means ``x`` holds column-direction (transposed) data and the result is
+    transposed back."""
+    return _dequantize_mx(x, out_dtype, axis, block_size, scale_inv, fp4=False)
+
+
+def dequantize_mxfp4_impl(x, out_dtype, axis, block_size, scale_inv):
+    return _dequantize_mx(x, out_dtype, axis, block_size, scale_inv, fp4=True)

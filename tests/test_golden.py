@@ -71,3 +71,23 @@ def test_hip_reproduces_golden_fp8(gold, native_lib):
     assert np.array_equal(_bits(sr), gold["segment_row_sinv"].view(np.uint32))
     assert np.array_equal(_codes(qc)[:w], gold["segment_col_q"])
     assert np.array_equal(_bits(sc)[: w // 128], gold["segment_col_sinv"].view(np.uint32))
+
+
+@pytest.mark.gpu
+def test_hip_reproduces_golden_mx(gold, native_lib):
+    from primus_turbo.pytorch.core.low_precision import ScalingRecipe
+    from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+    x = torch.from_numpy(F.bf16_bits_to_f32(gold["x_bf16_bits"])).to(torch.bfloat16).cuda()
+    fmts = [("e4m3", torch.float8_e4m3fn, qi.quantize_mxfp8_impl), ("e5m2", torch.float8_e5m2, qi.quantize_mxfp8_impl)]
+    if hasattr(torch, "float4_e2m1fn_x2"):
+        fmts.append(("e2m1", torch.float4_e2m1fn_x2, qi.quantize_mxfp4_impl))
+    for fmt, dt, fn in fmts:
+        for two_d in (False, True):
+            tag = f"mx_{fmt}_{'2d' if two_d else '1d'}"
+            rec = ScalingRecipe(use_2d_block=two_d)
+            rq, rs, cq, cs = fn(x, dt, None, 32, with_trans=True, scaling_recipe=rec, scaling_recipe_for_trans=rec)
+            assert np.array_equal(_codes(rq), gold[f"{tag}_row_q"]), tag
+            assert np.array_equal(_codes(rs), gold[f"{tag}_row_scale"]), tag
+            assert np.array_equal(_codes(cq), gold[f"{tag}_col_q"]), tag
+            assert np.array_equal(_codes(cs), gold[f"{tag}_col_scale"]), tag

@@ -1,0 +1,142 @@
+"""GPU parity of the MX quantizers (MXFP8 E4M3 / E5M2, MXFP4 E2M1): codes and E8M0 scale
+bytes bit-exact against the oracle, single direction and dual, 1-D (1 x 32) and 2-D (32 x 32)
+blocks, padded and batched shapes, special values; de-quantizers bit-exact as well."""
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import bf16_randn, codes_np, to_f32_np
+from oracle import quantize as Q
+
+pytestmark = pytest.mark.gpu
+
+FP4 = getattr(torch, "float4_e2m1fn_x2", None)
+FMTS = [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)] + ([("e2m1", FP4)] if FP4 is not None else [])
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _turbo(native_lib):
+    global qi, ScalingRecipe, turbo, G
+    import primus_turbo.pytorch as turbo
+    from primus_turbo.pytorch.core.low_precision import ScalingGranularity as G
+    from primus_turbo.pytorch.core.low_precision import ScalingRecipe
+    from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+
+def _fn(fmt):
+    return qi.quantize_mxfp4_impl if fmt == "e2m1" else qi.quantize_mxfp8_impl
+
+
+def _dq(fmt):
+    return qi.dequantize_mxfp4_impl if fmt == "e2m1" else qi.dequantize_mxfp8_impl
+
+
+SHAPES = [(128, 128), (256, 512), (200, 96), (33, 32), (1000, 2080), (4096, 1024)]
+
+
+@pytest.mark.parametrize("fmt,dt", FMTS)
+@pytest.mark.parametrize("two_d", [False, True])
+@pytest.mark.parametrize("M,N", SHAPES)
+def test_mx_dual_matches_oracle(fmt, dt, two_d, M, N):
+    x = bf16_randn((M, N), seed=50, outlier_frac=0.002)
+    rec = ScalingRecipe(use_2d_block=two_d)
+    rq, rs, cq, cs = _fn(fmt)(x.cuda(), dt, None, 32, with_trans=True, scaling_recipe=rec, scaling_recipe_for_trans=rec)
+    torch.cuda.synchronize()
+    xf = to_f32_np(x)
+    oq, os_ = Q.mx_quant_rowwise(xf, fmt, two_d)
+    assert codes_np(rq).shape == oq.shape and codes_np(rs).shape == os_.shape
+    assert np.array_equal(codes_np(rs), os_), "row scale bytes"
+    assert np.array_equal(codes_np(rq), oq), "row codes"
+    oq, os_ = Q.mx_quant_colwise(xf, fmt, two_d)
+    assert codes_np(cq).shape == oq.shape and codes_np(cs).shape == os_.shape
+    assert np.array_equal(codes_np(cs), os_), "col scale bytes"
+    assert np.array_equal(codes_np(cq), oq), "col codes"
+
+
+@pytest.mark.parametrize("fmt,dt", FMTS)
+@pytest.mark.parametrize("axis", [0, 1])
+def test_mx_single_direction_and_mixed_recipes(fmt, dt, axis):
+    """One direction equals the matching half of the dual call; the two directions of a dual
+    call may use different block shapes (1-D activations rows, 2-D columns)."""
+    x = bf16_randn((384, 256), seed=51).cuda()
+    q, s = _fn(fmt)(x, dt, axis, 32)
+    rq, rs, cq, cs = _fn(fmt)(x, dt, None, 32, with_trans=True)
+    want_q, want_s = (rq, rs) if axis == 1 else (cq, cs)
+    assert torch.equal(q.view(torch.uint8), want_q.view(torch.uint8)) and torch.equal(s.view(torch.uint8), want_s.view(torch.uint8))
+    rq, rs, cq, cs = _fn(fmt)(x, dt, None, 32, with_trans=True, scaling_recipe=ScalingRecipe(),
+                              scaling_recipe_for_trans=ScalingRecipe(use_2d_block=True))
+    xf = to_f32_np(x)
+    oq, os_ = Q.mx_quant_rowwise(xf, fmt, False)
+    assert np.array_equal(codes_np(rq), oq) and np.array_equal(codes_np(rs), os_)
+    oq, os_ = Q.mx_quant_colwise(xf, fmt, True)
+    assert np.array_equal(codes_np(cq), oq) and np.array_equal(codes_np(cs), os_)
+
+
+@pytest.mark.parametrize("fmt,dt", FMTS)
+def test_mx_batched_and_fp16(fmt, dt):
+    x = bf16_randn((3, 160, 192), seed=52, dtype=torch.float16)
+    rq, rs, cq, cs = _fn(fmt)(x.cuda(), dt, None, 32, with_trans=True)
+    assert rq.shape[0] == 3 and cq.shape[0] == 3
+    for b in range(3):
+        xf = to_f32_np(x[b])
+        oq, os_ = Q.mx_quant_rowwise(xf, fmt)
+        assert np.array_equal(codes_np(rq[b]), oq) and np.array_equal(codes_np(rs[b]), os_)
+        oq, os_ = Q.mx_quant_colwise(xf, fmt)
+        assert np.array_equal(codes_np(cq[b]), oq) and np.array_equal(codes_np(cs[b]), os_)
+
+
+@pytest.mark.parametrize("fmt,dt", FMTS)
+def test_mx_special_values(fmt, dt):
+    """All-zero blocks (scale byte 0), huge and tiny magnitudes, NaN and inf elements, exact
+    ties between representable codes."""
+    x = torch.zeros((128, 256), dtype=torch.float32)
+    x[0, :32] = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0] * 4)  # FP4 midpoints at scale 1
+    x[1, :32] = torch.linspace(-7, 7, 32)
+    x[2, 32:64] = 3.0e38
+    x[3, 64:96] = 1.0e-38
+    x[4, 5] = float("nan")
+    x[4, 6] = 2.0
+    x[5, 40] = float("inf")
+    x[5, 41] = -1.0
+    x[6, :] = torch.randn(256, generator=torch.Generator().manual_seed(53)) * 1e4
+    x[7, 96:128] = -0.0
+    xb = x.to(torch.bfloat16)
+    rq, rs, cq, cs = _fn(fmt)(xb.cuda(), dt, None, 32, with_trans=True)
+    xf = to_f32_np(xb)
+    oq, os_ = Q.mx_quant_rowwise(xf, fmt)
+    assert np.array_equal(codes_np(rs), os_) and np.array_equal(codes_np(rq), oq)
+    oq, os_ = Q.mx_quant_colwise(xf, fmt)
+    assert np.array_equal(codes_np(cs), os_) and np.array_equal(codes_np(cq), oq)
+    assert codes_np(rs)[8:, :].max() == 0  # untouched rows: all-zero blocks
+
+
+@pytest.mark.parametrize("fmt,dt", FMTS)
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_mx_dequant_matches_oracle(fmt, dt, out_dtype):
+    x = bf16_randn((200, 160), seed=54, outlier_frac=0.01).cuda()
+    rq, rs, cq, cs = _fn(fmt)(x, dt, None, 32, with_trans=True)
+    y = _dq(fmt)(rq, out_dtype, 1, 32, rs)
+    ref = torch.from_numpy(Q.mx_dequant(codes_np(rq), codes_np(rs), fmt)).to(out_dtype)
+    assert torch.equal(y.cpu(), ref)
+    yt = _dq(fmt)(cq, out_dtype, 0, 32, cs)  # transposed back: [M_pad, N]
+    ref_t = torch.from_numpy(np.ascontiguousarray(Q.mx_dequant(codes_np(cq), codes_np(cs), fmt).T)).to(out_dtype)
+    assert torch.equal(yt.cpu(), ref_t)
+    # round trip stays within half a code step of the block scale
+    err = (y[:, :160].float() - x.float()).abs().max().item()
+    # (relative code spacing: E2M1 1/2, E5M2 1/4, E4M3 1/8; the top sliver of a block saturates)
+    assert err <= x.float().abs().max().item() * {"e2m1": 0.26, "e5m2": 0.14, "e4m3": 0.07}[fmt]
+
+
+def test_mx_public_ops():
+    """The public quantize_fp8 / quantize_fp4 entry points route MX_BLOCKWISE to these kernels."""
+    x = bf16_randn((256, 256), seed=55).cuda()
+    q, s = turbo.ops.quantize_fp8(x, torch.float8_e4m3fn, G.MX_BLOCKWISE, block_size=32, axis=1)
+    oq, os_ = Q.mx_quant_rowwise(to_f32_np(x), "e4m3")
+    assert np.array_equal(codes_np(q), oq) and np.array_equal(codes_np(s), os_)
+    y = turbo.ops.dequantize_fp8(q, torch.bfloat16, G.MX_BLOCKWISE, block_size=32, axis=1, scale_inv=s)
+    assert torch.equal(y.cpu(), torch.from_numpy(Q.mx_dequant(oq, os_, "e4m3")).to(torch.bfloat16))
+    if FP4 is not None:
+        q, s = turbo.ops.quantize_fp4(x, FP4, G.MX_BLOCKWISE, block_size=32, axis=1)
+        oq, os_ = Q.mx_quant_rowwise(to_f32_np(x), "e2m1")
+        assert np.array_equal(codes_np(q), oq) and np.array_equal(codes_np(s), os_)
