@@ -237,6 +237,31 @@ PT_API int pt_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const v
                        int64_t sb_n, int64_t sb_k, int sa_block, int sb_block, int accumulate,
                        void *workspace, size_t workspace_bytes, int tile_cfg, void *stream);
 
+/* MX-scaled GEMM (MXFP8 / MXFP4), NT layout ----------------------------------
+ *
+ * Replaces primus_turbo::gemm_fp8_impl for the MX_BLOCKWISE granularity
+ * (primus_turbo/pytorch/kernels/gemm/gemm_fp8_impl.py:341-496, hipBLASLt / AITER / FlyDSL
+ * behind it) and primus_turbo::gemm_fp4_impl (kernels/gemm/gemm_fp4_impl.py:53-319,339-430):
+ *
+ *   C[m, n] = sum_kb 2^(a_scale[m, kb] - 127) * 2^(b_scale[n, kb] - 127)
+ *                    * sum_{k in block kb} A[m, k] * B[n, k],      32-wide K blocks,
+ *
+ * fp32 accumulation, the block scales applied by the matrix core. A is [M, K] and B is [N, K]
+ * (both K-contiguous) with row pitches lda / ldb in BYTES; ab_dtype PT_DTYPE_E4M3 / PT_DTYPE_E5M2
+ * selects MXFP8 (a_e5m2 / b_e5m2 give each operand's format), PT_DTYPE_E2M1X2 selects MXFP4 (two
+ * codes per byte, K counts codes). a_scale [M, >= K / 32] and b_scale [N, >= K / 32] are E8M0
+ * bytes with row pitches sa_ld / sb_ld. K % 32 == 0; bytes of a row behind K must be zero
+ * codes, as the MX quantizers leave them. Rows that are not whole 128-byte slabs (at least
+ * three) are first copied into `workspace` (pt_gemm_mx_workspace_bytes, 16-byte aligned).
+ * accumulate != 0 adds into C (beta = 1). tile_cfg as for pt_gemm_fp8. */
+PT_API size_t pt_gemm_mx_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                                         int fp4);
+PT_API int pt_gemm_mx(const void *a, const void *a_scale, const void *b, const void *b_scale,
+                      int ab_dtype, int a_e5m2, int b_e5m2, void *c, int c_dtype, int64_t M,
+                      int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t sa_ld, int64_t sb_ld,
+                      int accumulate, void *workspace, size_t workspace_bytes, int tile_cfg,
+                      void *stream);
+
 /* MoE grouped FP8 GEMM, 128-blockwise scales -------------------------------
  *
  * pt_grouped_gemm_fp8 replaces primus_turbo::grouped_gemm_fp8_impl

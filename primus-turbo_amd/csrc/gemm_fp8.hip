@@ -83,6 +83,23 @@ static int launch_gemm_vector(const GemmArgs &a, int fa, int fb, int tile_cfg, h
     return launch_vector_tiles<1, 1>(a, tile_cfg, stream);
 }
 
+// in[R, C] with row pitch ldi -> out[R, ldo], columns [C, ldo) zero-filled
+__global__ __launch_bounds__(256) void pad_rows2_u8_kernel(const uint8_t *__restrict__ in, uint8_t *__restrict__ out,
+                                                           const int64_t R, const int64_t C, const int64_t ldi,
+                                                           const int64_t ldo) {
+    const int64_t total  = R * ldo;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int64_t r = i / ldo, c = i % ldo;
+        out[i]          = c < C ? in[r * ldi + c] : 0;
+    }
+}
+
+void launch_pad_rows2(const uint8_t *in, uint8_t *out, int64_t R, int64_t C, int64_t ldi, int64_t ldo, hipStream_t st) {
+    if (R * ldo > 0)
+        pad_rows2_u8_kernel<<<static_cast<unsigned>(cdiv(R * ldo, 256 * 16)), 256, 0, st>>>(in, out, R, C, ldi, ldo);
+}
+
 void launch_pad_rows(const uint8_t *in, uint8_t *out, int64_t R, int64_t C, int64_t ldo, hipStream_t st) {
     pad_rows_u8_kernel<<<static_cast<unsigned>(cdiv(R * ldo, 256 * 16)), 256, 0, st>>>(in, out, R, C, ldo);
 }

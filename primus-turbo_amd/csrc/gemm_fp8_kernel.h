@@ -5,6 +5,9 @@
 //   VECTOR  C = (A.B^T) * sA[m] * sB[n]            tensorwise (stride 0) and rowwise
 //   BLOCK   C = sum_kb (A_kb.B_kb^T) * sA[m / bm, kb] * sB[n / bn, kb]   128-wide K blocks,
 //           bm, bn = 128 (2-D weight blocks) or 1 (1-D activation blocks)
+//   MX      C = sum_kb (A_kb.B_kb^T) * 2^(sA[m, kb] - 127) * 2^(sB[n, kb] - 127), 32-wide K
+//           blocks with E8M0 scale bytes applied by the matrix core itself (MXFP8, and MXFP4
+//           with two E2M1 codes per byte: gemm_fp8_impl.py:341-496, gemm_fp4_impl.py:53-319)
 //
 // Kernel structure (this library's own):
 //   * one workgroup = 4 wavefronts in a 2 x 2 grid; each wavefront owns a
@@ -35,7 +38,7 @@ namespace pt {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef int   i32x8 __attribute__((ext_vector_type(8)));
 
-enum : int { SCALE_VECTOR = 0, SCALE_BLOCK = 1 };
+enum : int { SCALE_VECTOR = 0, SCALE_BLOCK = 1, SCALE_MX = 2 };
 
 struct GemmArgs {
     const uint8_t *A; // [M, K] fp8, K contiguous
@@ -47,9 +50,10 @@ struct GemmArgs {
     int64_t        lda, ldb;    // row pitch of A and B in bytes (>= K)
     // VECTOR: sA[m * sa_m], sB[n * sb_n]                      (stride 0 = one scalar)
     // BLOCK : sA[(m >> sa_shift) * sa_m + kb * sa_k], sB[(n >> sb_shift) * sb_n + kb * sb_k]
+    // MX    : sA / sB point at E8M0 bytes, byte[m * sa_m + kb] and byte[n * sb_n + kb]
     int64_t sa_m, sa_k, sb_n, sb_k;
     int     sa_shift, sb_shift; // 0 (one scale per row) or 7 (one per 128 rows)
-    int     kb_valid;           // BLOCK: K blocks the scale arrays hold (K slabs beyond are zero padding)
+    int     kb_valid;           // BLOCK / MX: K blocks the scale arrays hold (slabs beyond are zero padding)
     int     out_dtype;
     int     accumulate; // C += result (beta = 1) instead of C = result
     int     tiles_m, tiles_n;
@@ -131,6 +135,14 @@ __device__ __forceinline__ f32x4 mfma_fp8(const i32x8 &rowop, const i32x8 &colop
     // rowop carries B-matrix rows (format FB), colop carries A-matrix rows (format FA)
     return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rowop, colop, c, FB, FA, 0, 0x7f7f7f7f,
                                                             0, 0x7f7f7f7f);
+}
+
+// The same instruction with E8M0 block scales: lane (r, g) supplies the scale byte of matrix
+// row r and 32-wide K block g of the 128 K values this instruction consumes.
+template <int FA, int FB>
+__device__ __forceinline__ f32x4 mfma_mx(const i32x8 &rowop, const i32x8 &colop, f32x4 c, uint32_t row_scale,
+                                         uint32_t col_scale) {
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rowop, colop, c, FB, FA, 0, row_scale, 0, col_scale);
 }
 
 // Tile coordinates of a workgroup: XCD-contiguous ids, then groups of GROUP_M tile rows
@@ -390,6 +402,11 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     constexpr int NL  = LA + LB;
     constexpr int JR  = TN - 2; // columns [0, JR) before the release point, [JR, TN) after
     constexpr int NSB = SB_VEC ? 4 : 1;
+    // MXFP4: a 128-byte slab row holds 256 E2M1 codes, i.e. two MFMAs' worth of K; a lane's two
+    // 16-byte fragment reads (chunks g and 4 + g) then feed one MFMA each instead of one together
+    constexpr bool F4 = FA == 4;
+    static_assert((FA == 4) == (FB == 4), "FP4 operands come in pairs");
+    constexpr int NH = F4 ? 2 : 1; // MFMAs per fragment pair
     // GROUP_K tiles have their own K extent (possibly none at all): they run the pipeline per
     // tile instead of across tile boundaries
     constexpr bool XPIPE = GMODE != GROUP_K;
@@ -533,6 +550,34 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         }
     };
 
+    // MX mode: the E8M0 bytes of the next slab are fetched the same way, one byte per lane,
+    // fragment and MFMA: lane (r, g) takes the byte of fragment row r and K block g.
+    [[maybe_unused]] uint32_t mxa_cur[TM][NH], mxa_nxt[TM][NH], mxb_cur[TN][NH], mxb_nxt[TN][NH];
+    auto fetch_mx = [&](int64_t m0, int64_t n0, const float *sAm, const float *sBm, int kt, uint32_t (&sa)[TM][NH],
+                        uint32_t (&sb)[TN][NH]) {
+        if constexpr (MODE == SCALE_MX) {
+            const uint8_t *pa = reinterpret_cast<const uint8_t *>(sAm), *pb = reinterpret_cast<const uint8_t *>(sBm);
+            const int64_t  wm_base = m0 + wm * (TM * 16), wn_base = n0 + wn * (TN * 16);
+#pragma unroll
+            for (int h = 0; h < NH; ++h) {
+                int kb = (kt * NH + h) * 4 + lg;
+                kb     = kb < a.kb_valid ? kb : a.kb_valid - 1; // zero-padded K: any finite scale will do
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    int64_t m = wm_base + i * 16 + lm;
+                    m         = m < a.M ? m : a.M - 1;
+                    sa[i][h]  = pa[m * a.sa_m + kb];
+                }
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    int64_t n = wn_base + j * 16 + lm;
+                    n         = n < a.N ? n : a.N - 1;
+                    sb[j][h]  = pb[n * a.sb_n + kb];
+                }
+            }
+        }
+    };
+
     f32x4 acc[TM][TN];
     // MFMA operand fragments (8 VGPRs each). Loop-carried: fa = the A fragments of the slab
     // about to be multiplied, fb[0] and fb[1] = its first two B fragments.
@@ -556,6 +601,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     auto start_pipeline = [&](const TileCtx &t) {
         loader_to(t);
         fetch_scales(t.m0, t.n0, t.sA, t.sB, 0, sa_nxt, sb_nxt);
+        fetch_mx(t.m0, t.n0, t.sA, t.sB, 0, mxa_nxt, mxb_nxt);
         static_for<0, NL>([&](auto l) { issue_copy(l, 0); });
         advance_loader();
         static_for<0, NL>([&](auto l) { issue_copy(l, 1); });
@@ -606,6 +652,17 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                     for (int e = 0; e < NSB; ++e)
                         sb_cur[j][e] = sb_nxt[j][e];
             }
+            if constexpr (MODE == SCALE_MX) {
+#pragma unroll
+                for (int h = 0; h < NH; ++h) {
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+                        mxa_cur[i][h] = mxa_nxt[i][h];
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        mxb_cur[j][h] = mxb_nxt[j][h];
+                }
+            }
 
             // BLOCK mode: MFMA t (in issue order) writes ring[t % RING]; DEPTH MFMAs later its
             // product is folded into the running sum with the block scales (VALU work in
@@ -633,6 +690,14 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                     ring[t % RING] = mfma_fp8<FA, FB>(bf, af, f32x4{0.f, 0.f, 0.f, 0.f});
                     if (t >= DEPTH)
                         fold(t - DEPTH);
+                } else if constexpr (MODE == SCALE_MX) {
+                    acc[i][j] = mfma_mx<FA, FB>(bf, af, acc[i][j], mxb_cur[j][0], mxa_cur[i][0]);
+                    if constexpr (F4) {
+                        // second half of the slab: the fragments' upper 16 bytes
+                        const i32x8 bh = __builtin_shufflevector(bf, bf, 4, 5, 6, 7, 4, 5, 6, 7);
+                        const i32x8 ah = __builtin_shufflevector(af, af, 4, 5, 6, 7, 4, 5, 6, 7);
+                        acc[i][j]      = mfma_mx<FA, FB>(bh, ah, acc[i][j], mxb_cur[j][1], mxa_cur[i][1]);
+                    }
                 } else {
                     acc[i][j] = mfma_fp8<FA, FB>(bf, af, acc[i][j]);
                 }
@@ -666,6 +731,12 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                     fetch_scales(cur_t.m0, cur_t.n0, cur_t.sA, cur_t.sB, kt + 1 < KT ? kt + 1 : kt, sa_nxt, sb_nxt);
                 }
             }
+            if constexpr (MODE == SCALE_MX) {
+                static_assert(MODE != SCALE_MX || XPIPE, "MX GEMMs are not grouped here");
+                const bool same = kt + 1 < KT;
+                fetch_mx(same ? cur_t.m0 : nxt_t.m0, same ? cur_t.n0 : nxt_t.n0, cur_t.sA, cur_t.sB, same ? kt + 1 : 0,
+                         mxa_nxt, mxb_nxt);
+            }
             fb[0] = ldfrag(nxt + b_part, 0);
             fb[1] = ldfrag(nxt + b_part, 1);
             __builtin_amdgcn_sched_barrier(0);
@@ -696,11 +767,11 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
 
         // the epilogue reads the accumulators with hand-written instructions the compiler's
         // hazard tracking does not see: let the last MFMA's write-back finish first
-        if constexpr (MODE == SCALE_VECTOR)
+        if constexpr (MODE != SCALE_BLOCK)
             asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
         PT_GEMM_TRACE_POINT(5);
         const int64_t wm_base = cur_t.m0 + wm * (TM * 16), wn_base = cur_t.n0 + wn * (TN * 16);
-        epilogue<TM, TN, MODE, MODE == SCALE_VECTOR>(a, acc, cur_t.C, cur_t.sA, cur_t.sB, cur_t.m_end, wm_base, wn_base,
+        epilogue<TM, TN, MODE, MODE != SCALE_BLOCK>(a, acc, cur_t.C, cur_t.sA, cur_t.sB, cur_t.m_end, wm_base, wn_base,
                                                      lane);
 
         PT_GEMM_TRACE_POINT(6);
@@ -769,6 +840,8 @@ void launch_transpose(const uint8_t *in, uint8_t *out, int64_t batch, int64_t R,
                       hipStream_t st);
 // in[R, C] -> out[R, ldo] (columns [C, ldo) zero-filled)
 void launch_pad_rows(const uint8_t *in, uint8_t *out, int64_t R, int64_t C, int64_t ldo, hipStream_t st);
+// in[R, C] with row pitch ldi -> out[R, ldo] (columns [C, ldo) zero-filled)
+void launch_pad_rows2(const uint8_t *in, uint8_t *out, int64_t R, int64_t C, int64_t ldi, int64_t ldo, hipStream_t st);
 int  launch_gemm_block(const GemmArgs &a, int fa, int fb, bool sb_vec, int tile_cfg, hipStream_t stream);
 
 } // namespace pt

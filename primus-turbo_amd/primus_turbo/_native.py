@@ -85,6 +85,12 @@ _SIGNATURES = {
          c_int, c_i64, c_i64, c_i64, c_i64, c_int, c_int, c_int, c_void_p, c_size_t, c_int, c_void_p],
     ),
     "pt_transpose_u8": (c_int, [c_void_p, c_void_p, c_i64, c_i64, c_i64, c_void_p]),
+    "pt_gemm_mx_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_i64, c_i64, c_int]),
+    "pt_gemm_mx": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_i64, c_i64, c_i64, c_i64, c_i64,
+         c_i64, c_i64, c_int, c_void_p, c_size_t, c_int, c_void_p],
+    ),
     "pt_quantize_mx": (
         c_int,
         [c_void_p, c_int, c_i64, c_i64, c_i64, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p],

@@ -63,7 +63,47 @@ def _scale_desc(granularity, a_scale_inv, b_scale_inv, trans_a, trans_b, M, Nn, 
     raise NotImplementedError(f"granularity {granularity} is handled by the MX GEMM entry points")
 
 
+def launch_mx(a, a_scale, b, b_scale, out, trans_c, accumulate):
+    """NT GEMM with E8M0 block scales on MX-quantized operands: ``a`` ``[M, K]`` and ``b`` ``[N, K]``
+    codes (fp8, or ``float4_e2m1fn_x2`` with two codes per byte), scales ``[rows, K / 32]``."""
+    N.require_cuda(a, b, a_scale, b_scale, out)
+    fp4 = hasattr(torch, "float4_e2m1fn_x2") and a.dtype == torch.float4_e2m1fn_x2
+    _check(a.dim() == 2 and b.dim() == 2, "MX GEMM expects 2-D operands")
+    _check(a.dtype == b.dtype if fp4 else (a.dtype in _FP8 and b.dtype in _FP8), "operands must both be fp8 or both fp4")
+    _check(out.dtype in _OUT, "out_dtype must be bfloat16, float16 or float32")
+    a, b, a_scale, b_scale = a.contiguous(), b.contiguous(), a_scale.contiguous(), b_scale.contiguous()
+    if trans_c:  # C^T = B . A^T
+        a, b, a_scale, b_scale = b, a, b_scale, a_scale
+    pack = 2 if fp4 else 1
+    M, Nn = a.shape[0], b.shape[0]
+    K = a.shape[1] * pack
+    _check(b.shape[1] * pack == K, f"reduction dims differ: {K} vs {b.shape[1] * pack}")
+    _check(K % 32 == 0, "K must be a multiple of 32")
+    _check(a_scale.shape[0] == M and b_scale.shape[0] == Nn, "scale rows must match operand rows")
+    _check(a_scale.shape[1] >= K // 32 and b_scale.shape[1] >= K // 32, "scales must hold K / 32 blocks per row")
+    _check(a_scale.element_size() == 1 and b_scale.element_size() == 1, "scales must be E8M0 bytes")
+    _check(tuple(out.shape) == (M, Nn) and out.is_contiguous(), f"out must be a contiguous {(M, Nn)} tensor")
+    lib = N.lib()
+    lda = ldb = K // pack
+    ws = None
+    ws_bytes = lib.pt_gemm_mx_workspace_bytes(M, Nn, K, lda, ldb, int(fp4))
+    if ws_bytes:
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
+    N.check(
+        lib.pt_gemm_mx(
+            N.ptr(a), N.ptr(a_scale), N.ptr(b), N.ptr(b_scale), N.dtype_code(a.dtype),
+            int(a.dtype == torch.float8_e5m2), int(b.dtype == torch.float8_e5m2),
+            N.ptr(out), N.dtype_code(out.dtype), M, Nn, K, lda, ldb, a_scale.shape[1], b_scale.shape[1],
+            int(accumulate), N.ptr(ws), ws_bytes, TILE_CFG, N.stream_of(a),
+        )
+    )
+    return out
+
+
 def _launch(a, a_scale_inv, trans_a, b, b_scale_inv, trans_b, out, trans_c, granularity, accumulate):
+    if granularity == ScalingGranularity.MX_BLOCKWISE:
+        _check(not trans_a and trans_b, "MX_BLOCKWISE GEMM supports the NT layout only (trans_a=False, trans_b=True)")
+        return launch_mx(a, a_scale_inv, b, b_scale_inv, out, trans_c, accumulate)
     N.require_cuda(a, b, a_scale_inv, b_scale_inv, out)
     _check(a.dtype in _FP8 and b.dtype in _FP8, "operands must be float8_e4m3fn / float8_e5m2")
     _check(out.dtype in _OUT, "out_dtype must be bfloat16, float16 or float32")
