@@ -217,7 +217,7 @@ PT_API int pt_dequantize_mx(const void *q, int q_dtype, const void *scale, int64
  * K as its row axis is transposed into `workspace` first, and when K is not a multiple
  * of 128 both operands are copied there with a zero-filled K tail
  * (pt_gemm_fp8_workspace_bytes(M, N, K, trans_a, trans_b) bytes, 16-byte aligned;
- * zero bytes, and `workspace` may be NULL, for trans_a == 0, trans_b != 0, K % 128 == 0).
+ * zero bytes, and `workspace` may be NULL, for trans_a == 0, trans_b != 0, K % 128 == 0, K >= 512).
  *
  * scale_mode 0 (vector):  C = (A.B) * a_scale[m * sa_m] * b_scale[n * sb_n]
  *     tensorwise: sa_m = sb_n = 0;  rowwise: sa_m = sb_n = 1.
@@ -252,7 +252,7 @@ PT_API int pt_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const v
  * codes per byte, K counts codes). a_scale [M, >= K / 32] and b_scale [N, >= K / 32] are E8M0
  * bytes with row pitches sa_ld / sb_ld. K % 32 == 0; bytes of a row behind K must be zero
  * codes, as the MX quantizers leave them. Rows that are not whole 128-byte slabs (at least
- * three) are first copied into `workspace` (pt_gemm_mx_workspace_bytes, 16-byte aligned).
+ * four) are first copied into `workspace` (pt_gemm_mx_workspace_bytes, 16-byte aligned).
  * accumulate != 0 adds into C (beta = 1). tile_cfg as for pt_gemm_fp8. */
 PT_API size_t pt_gemm_mx_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                                          int fp4);
@@ -278,7 +278,7 @@ PT_API int pt_gemm_mx(const void *a, const void *a_scale, const void *b, const v
  * [G, ceil(N/128), ceil(K/128)]; trans_b == 0: W is [G, K, N] with [G, ceil(K/128), ceil(N/128)].
  * group_offs: device int64 [G + 1] prefix sums of the per-group row counts (no host sync; groups
  * may be empty). The workspace (pt_grouped_gemm_fp8_workspace_bytes) holds the K-contiguous
- * copy of W when trans_b == 0 and zero-padded copies when K % 128 != 0 or K < 384.
+ * copy of W when trans_b == 0 and zero-padded copies when K % 128 != 0 or K < 512.
  *
  * pt_grouped_gemm_fp8_variable_k replaces primus_turbo::grouped_gemm_fp8_variable_k_impl and
  * ..._variable_k_accum_impl (grouped_gemm_fp8_impl.py:933-1022; Triton

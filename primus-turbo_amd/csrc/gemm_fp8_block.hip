@@ -9,11 +9,13 @@ namespace pt {
 
 template <bool SB_VEC, int FA, int FB>
 static int launch_block_tiles(const GemmArgs &a, int tile_cfg, hipStream_t stream) {
-    // tile_cfg: 0 = auto, 1 / 2 = 256x128, 3 = 128x128 (two workgroups per CU)
+    // tile_cfg: 0 = auto, 1 = 256x256, 2 = 256x128, 3 = 128x128 (two workgroups per CU)
     if (tile_cfg == 0)
         tile_cfg = 3;
     if (tile_cfg == 3)
         return launch_gemm_cfg<4, 4, SCALE_BLOCK, SB_VEC, FA, FB>(a, stream);
+    if (tile_cfg == 1)
+        return launch_gemm_cfg<8, 8, SCALE_BLOCK, SB_VEC, FA, FB>(a, stream);
     return launch_gemm_cfg<8, 4, SCALE_BLOCK, SB_VEC, FA, FB>(a, stream);
 }
 

@@ -74,6 +74,11 @@ enum : int { GROUP_NONE = 0, GROUP_ROWS = 1, GROUP_K = 2 };
 
 constexpr int KSTEP      = 128; // bytes of K per pipeline step (= one MFMA K)
 constexpr int GEMM_WAVES = 4;
+// pipeline depth of a tile configuration (see the kernel); K must span at least depth + 1 slabs
+constexpr int gemm_stages(int TM, int TN) {
+    return (TM == 8 && TN == 4) ? 3 : 2;
+}
+constexpr int GEMM_MIN_SLABS = 4;
 
 __device__ __forceinline__ int swz(int row) {
     return (row >> 1) & 7;
@@ -137,12 +142,35 @@ __device__ __forceinline__ f32x4 mfma_fp8(const i32x8 &rowop, const i32x8 &colop
                                                             0, 0x7f7f7f7f);
 }
 
-// The same instruction with E8M0 block scales: lane (r, g) supplies the scale byte of matrix
-// row r and 32-wide K block g of the 128 K values this instruction consumes.
+// E8M0 block scales of the instruction: lane (r, g) supplies, in the low byte of its scale
+// operand, the scale of matrix row r and 32-wide K block g of the 128 K values consumed.
+
+// The instruction written out by hand, accumulating in place in an AGPR tuple. The compiler's
+// own selection turns the tied accumulate form into "copy the accumulator tile, then write the
+// original registers" (four v_accvgpr_mov and a dozen wait states in front of every MFMA)
+// whenever it has registers to spare, which halves the matrix-core rate. Used by the modes
+// that accumulate inside the matrix core (VECTOR, MX). The compiler does not know this is an
+// MFMA, so the hazards are the caller's: the accumulators are only read (v_accvgpr_read in the
+// epilogue) after a padding of wait states, and two MFMAs on one accumulator are never issued
+// back to back.
+typedef int i32x4 __attribute__((ext_vector_type(4)));
 template <int FA, int FB>
-__device__ __forceinline__ f32x4 mfma_mx(const i32x8 &rowop, const i32x8 &colop, f32x4 c, uint32_t row_scale,
-                                         uint32_t col_scale) {
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rowop, colop, c, FB, FA, 0, row_scale, 0, col_scale);
+__device__ __forceinline__ void mfma_inplace(f32x4 &c, const i32x8 &rowop, const i32x8 &colop, uint32_t row_scale,
+                                             uint32_t col_scale) {
+#if defined(__HIP_DEVICE_COMPILE__) // the host pass cannot parse the AGPR constraint
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:%5 blgp:%6"
+                 : "+a"(c)
+                 : "v"(rowop), "v"(colop), "v"(row_scale), "v"(col_scale), "n"(FB), "n"(FA));
+#endif
+}
+// FP4 operands are 128 bits per lane
+__device__ __forceinline__ void mfma_inplace_f4(f32x4 &c, const i32x4 &rowop, const i32x4 &colop, uint32_t row_scale,
+                                                uint32_t col_scale) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4"
+                 : "+a"(c)
+                 : "v"(rowop), "v"(colop), "v"(row_scale), "v"(col_scale));
+#endif
 }
 
 // Tile coordinates of a workgroup: XCD-contiguous ids, then groups of GROUP_M tile rows
@@ -398,6 +426,10 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     static_assert(TN % 4 == 0, "the B fragment ring assumes TN = 4 or 8");
     constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
     constexpr int A_BYTES = BM * KSTEP, B_BYTES = BN * KSTEP, STAGE = A_BYTES + B_BYTES;
+    // LDS stages: two for the 256 x 256 tile (128 KB) and for the 128 x 128 tile (two workgroups
+    // per CU cover each other's waits); three where one workgroup per CU has the room, so that
+    // copies are requested three slabs ahead and survive an L2 miss without stalling the MFMAs
+    constexpr int NSTAGE = gemm_stages(TM, TN);
     constexpr int LA = BM / 8 / GEMM_WAVES, LB = BN / 8 / GEMM_WAVES; // copies per wave and slab
     constexpr int NL  = LA + LB;
     constexpr int JR  = TN - 2; // columns [0, JR) before the release point, [JR, TN) after
@@ -407,6 +439,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     constexpr bool F4 = FA == 4;
     static_assert((FA == 4) == (FB == 4), "FP4 operands come in pairs");
     constexpr int NH = F4 ? 2 : 1; // MFMAs per fragment pair
+    [[maybe_unused]] uint32_t unit_scale = 0x7f7f7f7fu; // E8M0 1.0 for all four K blocks
     // GROUP_K tiles have their own K extent (possibly none at all): they run the pipeline per
     // tile instead of across tile boundaries
     constexpr bool XPIPE = GMODE != GROUP_K;
@@ -423,7 +456,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     const uint32_t frag_off_hi = lm * KSTEP + (((4 + lg) ^ swz(lm)) << 4);
 
     // ---- tile list ----
-    int *prefix = reinterpret_cast<int *>(smem + 2 * STAGE); // GROUP_ROWS: tiles before group g
+    int *prefix = reinterpret_cast<int *>(smem + NSTAGE * STAGE); // GROUP_ROWS: tiles before group g
     int  total;
     if constexpr (GMODE == GROUP_ROWS) {
         for (int g = tid; g < a.G; g += 256) {
@@ -448,7 +481,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     }
     const int KT_ALL = static_cast<int>(a.K / KSTEP); // XPIPE: every tile has this many slabs (>= 3)
     int       tile   = blockIdx.x;
-    if (tile >= total || (XPIPE && KT_ALL < 3))
+    if (tile >= total || (XPIPE && KT_ALL <= NSTAGE))
         return;
     int     g_cur = 0, g_nxt = 0;
     TileCtx cur_t = make_tile<BM, BN, GMODE>(a, tile, prefix, g_cur);
@@ -460,7 +493,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     // descriptor, whose size makes rows beyond the tile's share of the matrix read as zero.
     // The loader therefore changes tile by swapping scalars -- no branch in the K loop, which
     // the compiler would use to sink MFMAs -- and it does so after requesting the tile's last
-    // slab, at step KT - 3 of the MFMAs (the host guarantees KT >= 3). Without cross-tile
+    // slab, NSTAGE + 1 steps before the MFMAs get there (the host guarantees KT > NSTAGE). Without cross-tile
     // pipelining it stops at the tile's last slab and keeps re-reading that one.
     uint32_t off[NL];
     {
@@ -602,11 +635,11 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         loader_to(t);
         fetch_scales(t.m0, t.n0, t.sA, t.sB, 0, sa_nxt, sb_nxt);
         fetch_mx(t.m0, t.n0, t.sA, t.sB, 0, mxa_nxt, mxb_nxt);
-        static_for<0, NL>([&](auto l) { issue_copy(l, 0); });
-        advance_loader();
-        static_for<0, NL>([&](auto l) { issue_copy(l, 1); });
-        advance_loader();
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
+        static_for<0, NSTAGE>([&](auto st) {
+            static_for<0, NL>([&](auto l) { issue_copy(l, st); });
+            advance_loader();
+        });
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NSTAGE - 1) * NL) : "memory");
         __builtin_amdgcn_s_barrier();
         buf   = 0;
         fb[0] = ldfrag(smem + b_part, 0);
@@ -640,8 +673,9 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         // one K slab per iteration; the body must stay a single basic block (no branches), or
         // the compiler sinks the MFMAs behind them
         for (int kt = 0; kt < KT; ++kt) {
-            const uint8_t *cur = smem + buf * STAGE;
-            const uint8_t *nxt = smem + (buf ^ 1) * STAGE;
+            const int      buf_n = buf + 1 == NSTAGE ? 0 : buf + 1;
+            const uint8_t *cur   = smem + buf * STAGE;
+            const uint8_t *nxt   = smem + buf_n * STAGE;
             if constexpr (MODE == SCALE_BLOCK) {
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
@@ -685,21 +719,20 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                         acc[i][j][e] = fmaf(p[e], sc, acc[i][j][e]);
                 }
             };
-            auto mma = [&](int t, int i, int j, const i32x8 &af, const i32x8 &bf) {
+            // h selects the half of an MXFP4 slab (always 0 otherwise)
+            auto mma = [&](int t, int i, int j, const i32x8 &af, const i32x8 &bf, int h) {
                 if constexpr (MODE == SCALE_BLOCK) {
                     ring[t % RING] = mfma_fp8<FA, FB>(bf, af, f32x4{0.f, 0.f, 0.f, 0.f});
                     if (t >= DEPTH)
                         fold(t - DEPTH);
+                } else if constexpr (F4) {
+                    const i32x4 bq = h ? __builtin_shufflevector(bf, bf, 4, 5, 6, 7) : __builtin_shufflevector(bf, bf, 0, 1, 2, 3);
+                    const i32x4 aq = h ? __builtin_shufflevector(af, af, 4, 5, 6, 7) : __builtin_shufflevector(af, af, 0, 1, 2, 3);
+                    mfma_inplace_f4(acc[i][j], bq, aq, mxb_cur[j][h ? NH - 1 : 0], mxa_cur[i][h ? NH - 1 : 0]);
                 } else if constexpr (MODE == SCALE_MX) {
-                    acc[i][j] = mfma_mx<FA, FB>(bf, af, acc[i][j], mxb_cur[j][0], mxa_cur[i][0]);
-                    if constexpr (F4) {
-                        // second half of the slab: the fragments' upper 16 bytes
-                        const i32x8 bh = __builtin_shufflevector(bf, bf, 4, 5, 6, 7, 4, 5, 6, 7);
-                        const i32x8 ah = __builtin_shufflevector(af, af, 4, 5, 6, 7, 4, 5, 6, 7);
-                        acc[i][j]      = mfma_mx<FA, FB>(bh, ah, acc[i][j], mxb_cur[j][1], mxa_cur[i][1]);
-                    }
+                    mfma_inplace<FA, FB>(acc[i][j], bf, af, mxb_cur[j][0], mxa_cur[i][0]);
                 } else {
-                    acc[i][j] = mfma_fp8<FA, FB>(bf, af, acc[i][j]);
+                    mfma_inplace<FA, FB>(acc[i][j], bf, af, unit_scale, unit_scale);
                 }
             };
 
@@ -710,14 +743,17 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                 // keep the instruction scheduler from moving MFMAs and LDS reads across each other
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int i = 0; i < TM; ++i)
-                    mma(j * TM + i, i, j, fa[i], fb[j % 4]);
+                for (int h = 0; h < NH; ++h)
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+                        mma(j * TM + i, i, j, fa[i], fb[j % 4], h);
                 __builtin_amdgcn_sched_barrier(0);
             }
 
             // ---- release point ----
-            // my reads of this stage are done and my copies of the next slab have landed
-            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            // my reads of this stage are done and my copies of the next slab have landed (the
+            // copies of the slabs after that, NSTAGE - 2 of them, may still be in flight)
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((NSTAGE - 2) * NL) : "memory");
             __builtin_amdgcn_s_barrier();
             PT_GEMM_TRACE_POINT(3);
             // (after a tile's last slab without a successor the following fetch and read leftovers:
@@ -743,8 +779,11 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             // ---- last two columns, row by row: A fragment i is refilled as soon as it is dead ----
             static_for<0, TM>([&](auto ic) {
                 constexpr int i = ic;
-                mma(JR * TM + 2 * i, i, JR, fa[i], fb[JR % 4]);
-                mma(JR * TM + 2 * i + 1, i, JR + 1, fa[i], fb[(JR + 1) % 4]);
+#pragma unroll
+                for (int h = 0; h < NH; ++h) {
+                    mma(JR * TM + 2 * i, i, JR, fa[i], fb[JR % 4], h);
+                    mma(JR * TM + 2 * i + 1, i, JR + 1, fa[i], fb[(JR + 1) % 4], h);
+                }
                 __builtin_amdgcn_sched_barrier(0);
                 fa[i] = ldfrag(nxt + a_part, i);
                 static_for<i * NL / TM, (i + 1) * NL / TM>([&](auto l) { issue_copy(l, buf); });
@@ -756,7 +795,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                     fold(t);
             }
             advance_loader();
-            buf ^= 1;
+            buf = buf_n;
         }
         if constexpr (!XPIPE) {
             // the re-read copies of the last slab must have landed everywhere before the next
@@ -789,8 +828,8 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
 template <int TM, int TN, int MODE, bool SB_VEC, int FA, int FB, int GMODE = GROUP_NONE>
 static int launch_gemm_cfg(const GemmArgs &args_in, hipStream_t stream) {
     constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
-    constexpr int STAGES  = 2 * (BM + BN) * KSTEP;
-    constexpr int MAX_G   = 4096;
+    constexpr int STAGES  = gemm_stages(TM, TN) * (BM + BN) * KSTEP;
+    constexpr int MAX_G   = 2048;
     constexpr int LDS_MAX = STAGES + (GMODE == GROUP_ROWS ? (MAX_G + 2) * 4 : 0);
     static_assert(LDS_MAX <= 160 * 1024, "tile configuration does not fit the LDS");
     GemmArgs a = args_in;
@@ -798,7 +837,7 @@ static int launch_gemm_cfg(const GemmArgs &args_in, hipStream_t stream) {
     a.tiles_m  = static_cast<int>(cdiv(a.M, BM));
     a.tiles_n  = static_cast<int>(cdiv(a.N, BN));
     if (GMODE != GROUP_NONE && a.G > MAX_G)
-        return fail(PT_ERR_INVALID_ARGUMENT, "grouped gemm: at most 4096 groups");
+        return fail(PT_ERR_INVALID_ARGUMENT, "grouped gemm: at most 2048 groups");
     auto kern            = gemm_fp8_nt_kernel<TM, TN, MODE, SB_VEC, FA, FB, GMODE>;
     static bool attr_set = false;
     if (!attr_set) {
@@ -830,10 +869,10 @@ static int launch_gemm_cfg(const GemmArgs &args_in, hipStream_t stream) {
 static inline int64_t round_up(int64_t x, int64_t m) {
     return (x + m - 1) / m * m;
 }
-// The kernel wants K as a multiple of 128 and at least three 128-byte slabs.
+// The kernel wants K as a multiple of 128 and at least GEMM_MIN_SLABS 128-byte slabs.
 static inline int64_t padded_k(int64_t K) {
     const int64_t kp = round_up(K, KSTEP);
-    return kp < 3 * KSTEP ? 3 * KSTEP : kp;
+    return kp < GEMM_MIN_SLABS * KSTEP ? GEMM_MIN_SLABS * KSTEP : kp;
 }
 // in[batch][R, C] -> out[batch][C, ldo] (columns [R, ldo) zero-filled), fp8 bytes
 void launch_transpose(const uint8_t *in, uint8_t *out, int64_t batch, int64_t R, int64_t C, int64_t ldo,

@@ -22,7 +22,7 @@ using namespace pt;
 
 extern "C" {
 
-// Bytes of one operand row as the kernel wants it: whole 128-byte slabs, at least three.
+// Bytes of one operand row as the kernel wants it: whole 128-byte slabs, at least four.
 static int64_t mx_row_bytes(int64_t K, bool fp4) {
     return padded_k(fp4 ? cdiv(K, 2) : K);
 }
@@ -56,7 +56,7 @@ int pt_gemm_mx(const void *a, const void *a_scale, const void *b, const void *b_
                "operands must be 16-byte aligned");
     auto st = static_cast<hipStream_t>(stream);
 
-    // the kernel reads whole 128-byte slabs (at least three): copy rows that are shorter, or
+    // the kernel reads whole 128-byte slabs (at least four): copy rows that are shorter, or
     // that carry anything but zeros behind K, into zero-padded rows
     const int64_t  need = mx_row_bytes(K, fp4);
     const uint8_t *A = static_cast<const uint8_t *>(a), *B = static_cast<const uint8_t *>(b);
