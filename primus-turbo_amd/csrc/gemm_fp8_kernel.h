@@ -753,6 +753,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             // ---- release point ----
             // my reads of this stage are done and my copies of the next slab have landed (the
             // copies of the slabs after that, NSTAGE - 2 of them, may still be in flight)
+            PT_GEMM_TRACE_POINT(2);
             asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((NSTAGE - 2) * NL) : "memory");
             __builtin_amdgcn_s_barrier();
             PT_GEMM_TRACE_POINT(3);
