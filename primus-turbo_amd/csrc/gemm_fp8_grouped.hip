@@ -16,7 +16,8 @@ namespace pt {
 template <int GMODE, bool SB_VEC, int FA, int FB>
 static int launch_grouped_tiles(const GemmArgs &a, int tile_cfg, hipStream_t stream) {
     // tile_cfg: 0 = auto, 1 / 2 = 256x128, 3 = 128x128 (two workgroups per CU)
-    if (tile_cfg == 0)
+    // (the 256x128 tile leaves LDS for the tile prefix sums of 1024 groups only)
+    if (tile_cfg == 0 || a.G > 1024)
         tile_cfg = 3;
     if (tile_cfg == 3)
         return launch_gemm_cfg<4, 4, SCALE_BLOCK, SB_VEC, FA, FB, GMODE>(a, stream);

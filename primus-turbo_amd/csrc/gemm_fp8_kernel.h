@@ -79,6 +79,14 @@ constexpr int gemm_stages(int TM, int TN) {
     return (TM == 8 && TN == 4) ? 3 : 2;
 }
 constexpr int GEMM_MIN_SLABS = 4;
+// BLOCK mode: the fp32 block scales of a slab travel with it through the LDS stages; every
+// wavefront keeps a private copy of the scales of its 16 * TM rows and 16 * TN columns.
+constexpr int gemm_scale_bytes(int TM, int TN, int MODE) {
+    return MODE == 1 ? GEMM_WAVES * (TM * 16 + TN * 16) * 4 : 0;
+}
+constexpr int gemm_stage_bytes(int TM, int TN, int MODE) {
+    return (2 * TM * 16 + 2 * TN * 16) * KSTEP + gemm_scale_bytes(TM, TN, MODE);
+}
 
 __device__ __forceinline__ int swz(int row) {
     return (row >> 1) & 7;
@@ -425,13 +433,20 @@ template <int TM, int TN, int MODE, bool SB_VEC, int FA, int FB, int GMODE>
 __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     static_assert(TN % 4 == 0, "the B fragment ring assumes TN = 4 or 8");
     constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
-    constexpr int A_BYTES = BM * KSTEP, B_BYTES = BN * KSTEP, STAGE = A_BYTES + B_BYTES;
+    constexpr int A_BYTES = BM * KSTEP, B_BYTES = BN * KSTEP, STAGE = gemm_stage_bytes(TM, TN, MODE);
     // LDS stages: two for the 256 x 256 tile (128 KB) and for the 128 x 128 tile (two workgroups
     // per CU cover each other's waits); three where one workgroup per CU has the room, so that
     // copies are requested three slabs ahead and survive an L2 miss without stalling the MFMAs
     constexpr int NSTAGE = gemm_stages(TM, TN);
     constexpr int LA = BM / 8 / GEMM_WAVES, LB = BN / 8 / GEMM_WAVES; // copies per wave and slab
-    constexpr int NL  = LA + LB;
+    constexpr int NLD = LA + LB;
+    // BLOCK mode: scale words of the wavefront's rows and columns, 64 per copy instruction
+    constexpr bool LDS_SC  = MODE == SCALE_BLOCK;
+    constexpr int  SC_A    = TM * 16, SC_B = TN * 16;
+    constexpr int  NSC     = LDS_SC ? (SC_A + SC_B) / 64 : 0;
+    constexpr int  SC_WAVE = (SC_A + SC_B) * 4; // bytes of a wavefront's scale area in a stage
+    constexpr int  NL      = NLD + NSC;         // copies per wave and slab, scales included
+    static_assert(!LDS_SC || SB_VEC || TN * 16 <= 128, "one B scale per wavefront and slab");
     constexpr int JR  = TN - 2; // columns [0, JR) before the release point, [JR, TN) after
     constexpr int NSB = SB_VEC ? 4 : 1;
     // MXFP4: a 128-byte slab row holds 256 E2M1 codes, i.e. two MFMAs' worth of K; a lane's two
@@ -499,15 +514,39 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     {
         const int lrow = lane >> 3, pchk = lane & 7;
 #pragma unroll
-        for (int j = 0; j < NL; ++j) {
+        for (int j = 0; j < NLD; ++j) {
             const bool isA = j < LA;
             const int  row = ((isA ? j : j - LA) * GEMM_WAVES + wave) * 8 + lrow;
             off[j] = static_cast<uint32_t>(row * (isA ? a.lda : a.ldb)) + ((pchk ^ swz(row)) << 4);
+        }
+        // scale copies: lane l of copy q fetches the scale of the wavefront's row (or column)
+        // 64 q + l; the offset is relative to the scale of the tile's first row / column, which
+        // is exact because tiles start on multiples of 128 wherever a scale spans 128 rows
+#pragma unroll
+        for (int q = 0; q < NSC; ++q) {
+            const int e = q * 64 + lane;
+            if (q * 64 < SC_A)
+                off[NLD + q] = static_cast<uint32_t>((wm * SC_A + e) >> a.sa_shift) * static_cast<uint32_t>(a.sa_m) * 4u;
+            else
+                off[NLD + q] = static_cast<uint32_t>((wn * SC_B + e - SC_A) >> a.sb_shift) * static_cast<uint32_t>(a.sb_n) * 4u;
         }
     }
     const uint8_t *ld_ga, *ld_gb; // slab the loader points at
     uint32_t       ld_na, ld_nb;  // bytes from there to the end of the tile's rows
     int            ld_kt;
+    // BLOCK mode: scales of the loader's slab for the tile's first row / column, and the end of
+    // the scale arrays (reads beyond return zero; they only ever meet zero-padded data)
+    [[maybe_unused]] const float *ld_sa = nullptr, *ld_sb = nullptr, *ld_sa_end = nullptr, *ld_sb_end = nullptr;
+    [[maybe_unused]] const int64_t sa_extent = ((a.M - 1) >> a.sa_shift) * a.sa_m + (a.kb_valid - 1) * a.sa_k + 1;
+    [[maybe_unused]] const int64_t sb_extent = ((a.N - 1) >> a.sb_shift) * a.sb_n + (a.kb_valid - 1) * a.sb_k + 1;
+    auto scales_to = [&](const TileCtx &t) {
+        if constexpr (LDS_SC) {
+            ld_sa     = t.sA + (t.m0 >> a.sa_shift) * a.sa_m;
+            ld_sb     = t.sB + (t.n0 >> a.sb_shift) * a.sb_n;
+            ld_sa_end = (GMODE == GROUP_K ? a.sA : t.sA) + sa_extent;
+            ld_sb_end = (GMODE == GROUP_K ? a.sB : t.sB) + sb_extent;
+        }
+    };
     TileCtx        nxt_t = cur_t; // tile after the MFMAs' tile (the same tile after the last one)
     auto           loader_to = [&](const TileCtx &t) {
         ld_ga = t.Ag;
@@ -515,6 +554,11 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         ld_na = t.rows_a * static_cast<uint32_t>(a.lda);
         ld_nb = t.rows_b * static_cast<uint32_t>(a.ldb);
         ld_kt = 0;
+        scales_to(t);
+    };
+    [[maybe_unused]] auto bytes_left = [](const float *p, const float *end) {
+        const int64_t n = end - p;
+        return n <= 0 ? 0u : (n > 0x3fffffff ? 0xfffffffcu : static_cast<uint32_t>(n) * 4u);
     };
     // copy number L of the loader's slab into stage `b`
     auto issue_copy = [&](auto lc, int b) {
@@ -522,7 +566,15 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         uint8_t      *dst = smem + b * STAGE;
 #if defined(__HIP_DEVICE_COMPILE__) // the buffer resource type only exists in the device pass
         constexpr uint32_t RSRC_FLAGS = 0x00020000; // raw buffer, 32-bit data format
-        if constexpr (L < LA) {
+        if constexpr (L >= NLD) {
+            constexpr int Q   = L - NLD;
+            const bool    isA = Q * 64 < SC_A;
+            __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<float *>(isA ? ld_sa : ld_sb), 0, isA ? bytes_left(ld_sa, ld_sa_end) : bytes_left(ld_sb, ld_sb_end),
+                RSRC_FLAGS);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr_t)(dst + A_BYTES + B_BYTES + wave * SC_WAVE + Q * 256), 4,
+                                                     off[L], 0, 0, 0);
+        } else if constexpr (L < LA) {
             __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(ld_ga), 0, ld_na, RSRC_FLAGS);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr_t)(dst + (L * GEMM_WAVES + wave) * 1024), 16, off[L], 0, 0, 0);
         } else {
@@ -539,6 +591,14 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             ld_gb = wrap ? nxt_t.Bg : ld_gb + KSTEP;
             ld_na = wrap ? nxt_t.rows_a * static_cast<uint32_t>(a.lda) : ld_na - KSTEP;
             ld_nb = wrap ? nxt_t.rows_b * static_cast<uint32_t>(a.ldb) : ld_nb - KSTEP;
+            if constexpr (LDS_SC) {
+                const float *na = nxt_t.sA + (nxt_t.m0 >> a.sa_shift) * a.sa_m;
+                const float *nb = nxt_t.sB + (nxt_t.n0 >> a.sb_shift) * a.sb_n;
+                ld_sa           = wrap ? na : ld_sa + a.sa_k;
+                ld_sb           = wrap ? nb : ld_sb + a.sb_k;
+                ld_sa_end       = wrap ? nxt_t.sA + sa_extent : ld_sa_end;
+                ld_sb_end       = wrap ? nxt_t.sB + sb_extent : ld_sb_end;
+            }
         } else {
             const int adv = ld_kt + 1 < cur_t.KT ? KSTEP : 0;
             ld_kt += adv / KSTEP;
@@ -546,39 +606,33 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             ld_gb += adv;
             ld_na -= adv;
             ld_nb -= adv;
+            if constexpr (LDS_SC) {
+                ld_sa += adv ? a.sa_k : 0;
+                ld_sb += adv ? a.sb_k : 0;
+            }
         }
     };
 
-    // BLOCK mode: the fp32 scales of a K block are fetched one slab ahead, at the release
-    // point and before that slab's tile copies are issued (so the copies stay the youngest
-    // entries of the vector-memory counter).
-    [[maybe_unused]] float sa_cur[TM], sa_nxt[TM], sb_cur[TN][NSB], sb_nxt[TN][NSB];
-    auto fetch_scales = [&](int64_t m0, int64_t n0, const float *sAm, const float *sBm, int kt, float (&sa)[TM],
-                            float (&sb)[TN][NSB]) {
-        if constexpr (MODE == SCALE_BLOCK) {
-            const int64_t wm_base = m0 + wm * (TM * 16), wn_base = n0 + wn * (TN * 16);
-            kt = kt < a.kb_valid ? kt : a.kb_valid - 1; // zero-padded slabs: any valid scale will do
+    // BLOCK mode: the fp32 scales of a slab are read from its stage at the release point of
+    // the slab before, next to its first fragments.
+    constexpr int NSBJ = SB_VEC ? TN : 1; // without per-column scales one value serves the wavefront
+    [[maybe_unused]] float sa_nxt[TM], sb_nxt[NSBJ][NSB], sc_cur[TM], sb_cur[NSBJ][NSB];
+    auto read_scales = [&](const uint8_t *stage) {
+        if constexpr (LDS_SC) {
+            const float *reg = reinterpret_cast<const float *>(stage + A_BYTES + B_BYTES + wave * SC_WAVE);
 #pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                int64_t m = wm_base + i * 16 + lm;
-                m         = m < a.M ? m : a.M - 1;
-                sa[i]     = sAm[(m >> a.sa_shift) * a.sa_m + kt * a.sa_k];
-            }
+            for (int i = 0; i < TM; ++i)
+                sa_nxt[i] = reg[i * 16 + lm];
+            if constexpr (SB_VEC) {
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                if constexpr (SB_VEC) {
+                for (int j = 0; j < TN; ++j) {
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(reg + SC_A + j * 16 + lg * 4);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        int64_t n = wn_base + j * 16 + lg * 4 + e;
-                        n         = n < a.N ? n : a.N - 1;
-                        sb[j][e]  = sBm[n * a.sb_n + kt * a.sb_k];
-                    }
-                } else {
-                    int64_t       nb    = (wn_base + j * 16) >> a.sb_shift;
-                    const int64_t nbmax = (a.N - 1) >> a.sb_shift;
-                    nb                  = nb < nbmax ? nb : nbmax;
-                    sb[j][0]            = sBm[nb * a.sb_n + kt * a.sb_k];
+                    for (int e = 0; e < 4; ++e)
+                        sb_nxt[j][e] = v[e];
                 }
+            } else {
+                sb_nxt[0][0] = reg[SC_A];
             }
         }
     };
@@ -633,7 +687,6 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     // pipeline start at tile t: slabs 0 and 1 requested, the first fragments of slab 0 on their way
     auto start_pipeline = [&](const TileCtx &t) {
         loader_to(t);
-        fetch_scales(t.m0, t.n0, t.sA, t.sB, 0, sa_nxt, sb_nxt);
         fetch_mx(t.m0, t.n0, t.sA, t.sB, 0, mxa_nxt, mxb_nxt);
         static_for<0, NSTAGE>([&](auto st) {
             static_for<0, NL>([&](auto l) { issue_copy(l, st); });
@@ -642,6 +695,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NSTAGE - 1) * NL) : "memory");
         __builtin_amdgcn_s_barrier();
         buf   = 0;
+        read_scales(smem);
         fb[0] = ldfrag(smem + b_part, 0);
         fb[1] = ldfrag(smem + b_part, 1);
 #pragma unroll
@@ -677,11 +731,12 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             const uint8_t *cur   = smem + buf * STAGE;
             const uint8_t *nxt   = smem + buf_n * STAGE;
             if constexpr (MODE == SCALE_BLOCK) {
+                // without per-column scales the two factors are combined once per row here
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
-                    sa_cur[i] = sa_nxt[i];
+                    sc_cur[i] = SB_VEC ? sa_nxt[i] : sa_nxt[i] * sb_nxt[0][0];
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
+                for (int j = 0; j < NSBJ; ++j)
 #pragma unroll
                     for (int e = 0; e < NSB; ++e)
                         sb_cur[j][e] = sb_nxt[j][e];
@@ -711,12 +766,11 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                 if constexpr (SB_VEC) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
-                        acc[i][j][e] = fmaf(p[e], sa_cur[i] * sb_cur[j][SB_VEC ? e : 0], acc[i][j][e]);
+                        acc[i][j][e] = fmaf(p[e], sc_cur[i] * sb_cur[SB_VEC ? j : 0][SB_VEC ? e : 0], acc[i][j][e]);
                 } else {
-                    const float sc = sa_cur[i] * sb_cur[j][0];
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
-                        acc[i][j][e] = fmaf(p[e], sc, acc[i][j][e]);
+                        acc[i][j][e] = fmaf(p[e], sc_cur[i], acc[i][j][e]);
                 }
             };
             // h selects the half of an MXFP4 slab (always 0 otherwise)
@@ -759,15 +813,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             PT_GEMM_TRACE_POINT(3);
             // (after a tile's last slab without a successor the following fetch and read leftovers:
             // harmless)
-            if constexpr (MODE == SCALE_BLOCK) {
-                if constexpr (XPIPE) {
-                    const bool same = kt + 1 < KT;
-                    fetch_scales(same ? cur_t.m0 : nxt_t.m0, same ? cur_t.n0 : nxt_t.n0, same ? cur_t.sA : nxt_t.sA,
-                                 same ? cur_t.sB : nxt_t.sB, same ? kt + 1 : 0, sa_nxt, sb_nxt);
-                } else {
-                    fetch_scales(cur_t.m0, cur_t.n0, cur_t.sA, cur_t.sB, kt + 1 < KT ? kt + 1 : kt, sa_nxt, sb_nxt);
-                }
-            }
+            read_scales(nxt);
             if constexpr (MODE == SCALE_MX) {
                 static_assert(MODE != SCALE_MX || XPIPE, "MX GEMMs are not grouped here");
                 const bool same = kt + 1 < KT;
@@ -829,8 +875,9 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
 template <int TM, int TN, int MODE, bool SB_VEC, int FA, int FB, int GMODE = GROUP_NONE>
 static int launch_gemm_cfg(const GemmArgs &args_in, hipStream_t stream) {
     constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
-    constexpr int STAGES  = gemm_stages(TM, TN) * (BM + BN) * KSTEP;
-    constexpr int MAX_G   = 2048;
+    constexpr int STAGES  = gemm_stages(TM, TN) * gemm_stage_bytes(TM, TN, MODE);
+    // groups whose tile prefix sums fit into the LDS next to the stages
+    constexpr int MAX_G   = (160 * 1024 - STAGES) / 4 - 2 < 2048 ? 1024 : 2048;
     constexpr int LDS_MAX = STAGES + (GMODE == GROUP_ROWS ? (MAX_G + 2) * 4 : 0);
     static_assert(LDS_MAX <= 160 * 1024, "tile configuration does not fit the LDS");
     GemmArgs a = args_in;
@@ -838,7 +885,9 @@ static int launch_gemm_cfg(const GemmArgs &args_in, hipStream_t stream) {
     a.tiles_m  = static_cast<int>(cdiv(a.M, BM));
     a.tiles_n  = static_cast<int>(cdiv(a.N, BN));
     if (GMODE != GROUP_NONE && a.G > MAX_G)
-        return fail(PT_ERR_INVALID_ARGUMENT, "grouped gemm: at most 2048 groups");
+        return fail(PT_ERR_INVALID_ARGUMENT, "grouped gemm: too many groups for this tile configuration");
+    if (MODE == SCALE_BLOCK && ((!SB_VEC && a.sb_shift != 7) || (GMODE == GROUP_ROWS && a.sa_shift != 0)))
+        return fail(PT_ERR_INVALID_ARGUMENT, "gemm_fp8: unsupported block-scale layout");
     auto kern            = gemm_fp8_nt_kernel<TM, TN, MODE, SB_VEC, FA, FB, GMODE>;
     static bool attr_set = false;
     if (!attr_set) {
