@@ -75,17 +75,18 @@ enum : int { GROUP_NONE = 0, GROUP_ROWS = 1, GROUP_K = 2 };
 constexpr int KSTEP      = 128; // bytes of K per pipeline step (= one MFMA K)
 constexpr int GEMM_WAVES = 4;
 // pipeline depth of a tile configuration (see the kernel); K must span at least depth + 1 slabs
-constexpr int gemm_stages(int TM, int TN) {
-    return (TM == 8 && TN == 4) ? 3 : 2;
+constexpr int gemm_stages(int TM, int TN, bool F4 = false) {
+    return (TM == 8 && TN == 4 && !F4) ? 3 : 2;
 }
 constexpr int GEMM_MIN_SLABS = 4;
-// BLOCK mode: the fp32 block scales of a slab travel with it through the LDS stages; every
-// wavefront keeps a private copy of the scales of its 16 * TM rows and 16 * TN columns.
-constexpr int gemm_scale_bytes(int TM, int TN, int MODE) {
-    return MODE == 1 ? GEMM_WAVES * (TM * 16 + TN * 16) * 4 : 0;
+// BLOCK and MX modes: the scales of a slab travel with it through the LDS stages; every
+// wavefront keeps a private copy of the scale words (one per slab, two for MXFP4) of its
+// 16 * TM rows and 16 * TN columns.
+constexpr int gemm_scale_bytes(int TM, int TN, int MODE, bool F4) {
+    return MODE == 0 ? 0 : GEMM_WAVES * (TM * 16 + TN * 16) * 4 * (F4 ? 2 : 1);
 }
-constexpr int gemm_stage_bytes(int TM, int TN, int MODE) {
-    return (2 * TM * 16 + 2 * TN * 16) * KSTEP + gemm_scale_bytes(TM, TN, MODE);
+constexpr int gemm_stage_bytes(int TM, int TN, int MODE, bool F4) {
+    return (2 * TM * 16 + 2 * TN * 16) * KSTEP + gemm_scale_bytes(TM, TN, MODE, F4);
 }
 
 __device__ __forceinline__ int swz(int row) {
@@ -415,45 +416,54 @@ __device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile, const 
 
 // Persistent kernel: the grid is sized to the machine and every workgroup walks tiles
 // blockIdx.x, blockIdx.x + gridDim.x, ... as one uninterrupted sequence of K steps
-// ("slabs" of 128 bytes of K, double-buffered in LDS stages s % 2). With one wavefront per
-// SIMD nothing hides a stall, so a slab is scheduled such that no MFMA ever waits for an
-// LDS round trip:
-//   * the A fragments of a wavefront's sub-tile live in one register set, the B fragments
-//     stream through a ring of four; every LDS read is issued at least one fragment
-//     (8 MFMAs) before its first use;
-//   * the MFMA tiles (i, j) are walked column by column up to column TN - 3; then the stage
-//     is released (barrier: everyone is done reading it and everyone's part of the next slab
-//     has landed), and the last two columns are walked row by row: after (i, TN-2), (i, TN-1)
-//     A fragment i is dead and is refilled at once from the next slab, together with a share
-//     of the copies that bring the slab after that into the stage just released;
+// ("slabs" of 128 bytes of K, rotating through the LDS stages). With one wavefront per SIMD
+// nothing hides a stall, and the path from L2 into the LDS moves about 64 bytes per clock and
+// CU -- more than half of what the MFMAs of a 256 x 256 tile consume per clock -- so a slab
+// is scheduled such that no MFMA waits for an LDS round trip and the copies are spread over
+// the whole slab instead of arriving at the copy unit in bursts:
+//   * all MFMA operand fragments of the slab being multiplied live in registers; the MFMA
+//     tiles (i, j) are walked column by column, and a fragment is refilled from the next
+//     slab's stage as soon as it is dead: B fragment j after column j, A fragment i after
+//     tile (i, TN - 1). Every LDS read is thus issued at least TM MFMAs before its first use;
+//   * the stage of the slab being multiplied is therefore only read during the slab before,
+//     and is free to receive the slab NSTAGE steps ahead during all of the current one: the B
+//     part (and the block scales) while columns 1 .. TN/2 - 1 are multiplied, the A part
+//     during the rest;
+//   * two barriers per slab: "X" after column 0 (everyone has finished reading the current
+//     stage; everyone's copies of the next slab's B part have landed) and "Y" after column
+//     TN/2 - 1 (the next slab's A part has landed). Both wait for copies requested at least
+//     half a slab earlier;
 //   * tile boundaries do not drain the pipeline: while a tile's result is written out, the
-//     first fragments of the next tile are already in registers and its second slab is in
-//     flight.
+//     fragments of the next tile's first slab are already in registers and its second slab is
+//     in flight.
 template <int TM, int TN, int MODE, bool SB_VEC, int FA, int FB, int GMODE>
 __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
-    static_assert(TN % 4 == 0, "the B fragment ring assumes TN = 4 or 8");
+    static_assert(TN % 4 == 0 && TM % 4 == 0, "sub-tiles are multiples of 64 x 64");
     constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
-    constexpr int A_BYTES = BM * KSTEP, B_BYTES = BN * KSTEP, STAGE = gemm_stage_bytes(TM, TN, MODE);
-    // LDS stages: two for the 256 x 256 tile (128 KB) and for the 128 x 128 tile (two workgroups
-    // per CU cover each other's waits); three where one workgroup per CU has the room, so that
-    // copies are requested three slabs ahead and survive an L2 miss without stalling the MFMAs
-    constexpr int NSTAGE = gemm_stages(TM, TN);
-    constexpr int LA = BM / 8 / GEMM_WAVES, LB = BN / 8 / GEMM_WAVES; // copies per wave and slab
+    constexpr int A_BYTES = BM * KSTEP, B_BYTES = BN * KSTEP, STAGE = gemm_stage_bytes(TM, TN, MODE, FA == 4);
+    constexpr int NSTAGE = gemm_stages(TM, TN, FA == 4);
+    constexpr int LA = BM / 8 / GEMM_WAVES, LB = BN / 8 / GEMM_WAVES; // data copies per wave and slab
     constexpr int NLD = LA + LB;
-    // BLOCK mode: scale words of the wavefront's rows and columns, 64 per copy instruction
-    constexpr bool LDS_SC  = MODE == SCALE_BLOCK;
-    constexpr int  SC_A    = TM * 16, SC_B = TN * 16;
-    constexpr int  NSC     = LDS_SC ? (SC_A + SC_B) / 64 : 0;
-    constexpr int  SC_WAVE = (SC_A + SC_B) * 4; // bytes of a wavefront's scale area in a stage
-    constexpr int  NL      = NLD + NSC;         // copies per wave and slab, scales included
-    static_assert(!LDS_SC || SB_VEC || TN * 16 <= 128, "one B scale per wavefront and slab");
-    constexpr int JR  = TN - 2; // columns [0, JR) before the release point, [JR, TN) after
-    constexpr int NSB = SB_VEC ? 4 : 1;
     // MXFP4: a 128-byte slab row holds 256 E2M1 codes, i.e. two MFMAs' worth of K; a lane's two
     // 16-byte fragment reads (chunks g and 4 + g) then feed one MFMA each instead of one together
     constexpr bool F4 = FA == 4;
     static_assert((FA == 4) == (FB == 4), "FP4 operands come in pairs");
     constexpr int NH = F4 ? 2 : 1; // MFMAs per fragment pair
+    // BLOCK and MX modes: the scales of a slab travel with it through the stages. Per row
+    // (column) of the wavefront's sub-tile and slab that is one 32-bit word -- an fp32 block
+    // scale, or the E8M0 bytes of four 32-wide K blocks (two words for MXFP4) -- fetched 64 rows
+    // per copy instruction into an area of the stage that is private to the wavefront.
+    constexpr bool LDS_SC  = MODE != SCALE_VECTOR;
+    constexpr int  SC_A    = TM * 16, SC_B = TN * 16, SC_ROWS = SC_A + SC_B;
+    constexpr int  NW      = MODE == SCALE_MX ? NH : 1;       // scale words per row and slab
+    constexpr int  NSC     = LDS_SC ? NW * SC_ROWS / 64 : 0;  // scale copies per wave and slab
+    constexpr int  SC_WAVE = NW * SC_ROWS * 4;                // bytes of a wavefront's scale area
+    constexpr int  SC_ELT  = MODE == SCALE_MX ? 1 : 4;        // bytes per scale array element
+    constexpr int  NB      = LB + NSC;                        // copies of the "B part" of a slab
+    constexpr int  NL      = NLD + NSC;                       // copies per wave and slab
+    constexpr int  JY      = TN / 2;                          // barrier Y follows column JY - 1
+    constexpr int  NSB     = SB_VEC ? 4 : 1;
+    static_assert(MODE != SCALE_BLOCK || SB_VEC || TN * 16 <= 128, "one B scale per wavefront and slab");
     [[maybe_unused]] uint32_t unit_scale = 0x7f7f7f7fu; // E8M0 1.0 for all four K blocks
     // GROUP_K tiles have their own K extent (possibly none at all): they run the pipeline per
     // tile instead of across tile boundaries
@@ -494,7 +504,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     } else {
         total = a.tiles_m * a.tiles_n;
     }
-    const int KT_ALL = static_cast<int>(a.K / KSTEP); // XPIPE: every tile has this many slabs (>= 3)
+    const int KT_ALL = static_cast<int>(a.K / KSTEP); // XPIPE: every tile has this many slabs (> NSTAGE)
     int       tile   = blockIdx.x;
     if (tile >= total || (XPIPE && KT_ALL <= NSTAGE))
         return;
@@ -502,14 +512,14 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     TileCtx cur_t = make_tile<BM, BN, GMODE>(a, tile, prefix, g_cur);
     g_nxt         = g_cur;
 
-    // ---- loader: two slabs ahead of the MFMAs ----
+    // ---- loader: NSTAGE slabs ahead of the MFMAs ----
     // Copies are buffer loads: a lane's offset inside a slab (row * pitch + swizzled chunk)
     // is the same for every tile; the tile and the K position live in the (uniform) buffer
     // descriptor, whose size makes rows beyond the tile's share of the matrix read as zero.
     // The loader therefore changes tile by swapping scalars -- no branch in the K loop, which
     // the compiler would use to sink MFMAs -- and it does so after requesting the tile's last
-    // slab, NSTAGE + 1 steps before the MFMAs get there (the host guarantees KT > NSTAGE). Without cross-tile
-    // pipelining it stops at the tile's last slab and keeps re-reading that one.
+    // slab, NSTAGE steps before the MFMAs get there (the host guarantees KT > NSTAGE). Without
+    // cross-tile pipelining it stops at the tile's last slab and keeps re-reading that one.
     uint32_t off[NL];
     {
         const int lrow = lane >> 3, pchk = lane & 7;
@@ -519,36 +529,44 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             const int  row = ((isA ? j : j - LA) * GEMM_WAVES + wave) * 8 + lrow;
             off[j] = static_cast<uint32_t>(row * (isA ? a.lda : a.ldb)) + ((pchk ^ swz(row)) << 4);
         }
-        // scale copies: lane l of copy q fetches the scale of the wavefront's row (or column)
-        // 64 q + l; the offset is relative to the scale of the tile's first row / column, which
-        // is exact because tiles start on multiples of 128 wherever a scale spans 128 rows
+        // scale copies: lane l of copy q fetches the word of the wavefront's row (or column)
+        // 64 q + l, at an offset relative to the scale of the tile's first row / column (exact,
+        // because tiles start on multiples of 128 wherever a scale spans 128 rows)
 #pragma unroll
         for (int q = 0; q < NSC; ++q) {
-            const int e = q * 64 + lane;
-            if (q * 64 < SC_A)
-                off[NLD + q] = static_cast<uint32_t>((wm * SC_A + e) >> a.sa_shift) * static_cast<uint32_t>(a.sa_m) * 4u;
+            const int e = (q % (SC_ROWS / 64)) * 64 + lane;
+            if (e < SC_A)
+                off[NLD + q] = static_cast<uint32_t>((wm * SC_A + e) >> a.sa_shift) * static_cast<uint32_t>(a.sa_m) * SC_ELT;
             else
-                off[NLD + q] = static_cast<uint32_t>((wn * SC_B + e - SC_A) >> a.sb_shift) * static_cast<uint32_t>(a.sb_n) * 4u;
+                off[NLD + q] = static_cast<uint32_t>((wn * SC_B + e - SC_A) >> a.sb_shift) * static_cast<uint32_t>(a.sb_n) * SC_ELT;
+            off[NLD + q] += (q / (SC_ROWS / 64)) * 4; // second scale word of an MXFP4 slab
         }
     }
     const uint8_t *ld_ga, *ld_gb; // slab the loader points at
     uint32_t       ld_na, ld_nb;  // bytes from there to the end of the tile's rows
     int            ld_kt;
-    // BLOCK mode: scales of the loader's slab for the tile's first row / column, and the end of
-    // the scale arrays (reads beyond return zero; they only ever meet zero-padded data)
-    [[maybe_unused]] const float *ld_sa = nullptr, *ld_sb = nullptr, *ld_sa_end = nullptr, *ld_sb_end = nullptr;
-    [[maybe_unused]] const int64_t sa_extent = ((a.M - 1) >> a.sa_shift) * a.sa_m + (a.kb_valid - 1) * a.sa_k + 1;
-    [[maybe_unused]] const int64_t sb_extent = ((a.N - 1) >> a.sb_shift) * a.sb_n + (a.kb_valid - 1) * a.sb_k + 1;
+    // scales of the loader's slab for the tile's first row / column, and the end of the scale
+    // arrays (reads beyond return zero; they only ever meet rows that are never stored)
+    [[maybe_unused]] const uint8_t *ld_sa = nullptr, *ld_sb = nullptr, *ld_sa_end = nullptr, *ld_sb_end = nullptr;
+    [[maybe_unused]] const int64_t  sa_extent =
+        MODE == SCALE_MX ? (a.M - 1) * a.sa_m + a.kb_valid
+                         : (((a.M - 1) >> a.sa_shift) * a.sa_m + (a.kb_valid - 1) * a.sa_k + 1) * 4;
+    [[maybe_unused]] const int64_t sb_extent =
+        MODE == SCALE_MX ? (a.N - 1) * a.sb_n + a.kb_valid
+                         : (((a.N - 1) >> a.sb_shift) * a.sb_n + (a.kb_valid - 1) * a.sb_k + 1) * 4;
+    [[maybe_unused]] const int64_t sa_step = MODE == SCALE_MX ? 4 * NW : a.sa_k * 4; // bytes per slab
+    [[maybe_unused]] const int64_t sb_step = MODE == SCALE_MX ? 4 * NW : a.sb_k * 4;
+    auto as_bytes = [](const float *p) { return reinterpret_cast<const uint8_t *>(p); };
     auto scales_to = [&](const TileCtx &t) {
         if constexpr (LDS_SC) {
-            ld_sa     = t.sA + (t.m0 >> a.sa_shift) * a.sa_m;
-            ld_sb     = t.sB + (t.n0 >> a.sb_shift) * a.sb_n;
-            ld_sa_end = (GMODE == GROUP_K ? a.sA : t.sA) + sa_extent;
-            ld_sb_end = (GMODE == GROUP_K ? a.sB : t.sB) + sb_extent;
+            ld_sa     = as_bytes(t.sA) + ((t.m0 >> a.sa_shift) * a.sa_m) * SC_ELT;
+            ld_sb     = as_bytes(t.sB) + ((t.n0 >> a.sb_shift) * a.sb_n) * SC_ELT;
+            ld_sa_end = as_bytes(GMODE == GROUP_K ? a.sA : t.sA) + sa_extent;
+            ld_sb_end = as_bytes(GMODE == GROUP_K ? a.sB : t.sB) + sb_extent;
         }
     };
-    TileCtx        nxt_t = cur_t; // tile after the MFMAs' tile (the same tile after the last one)
-    auto           loader_to = [&](const TileCtx &t) {
+    TileCtx nxt_t     = cur_t; // tile after the MFMAs' tile (the same tile after the last one)
+    auto    loader_to = [&](const TileCtx &t) {
         ld_ga = t.Ag;
         ld_gb = t.Bg;
         ld_na = t.rows_a * static_cast<uint32_t>(a.lda);
@@ -556,22 +574,26 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         ld_kt = 0;
         scales_to(t);
     };
-    [[maybe_unused]] auto bytes_left = [](const float *p, const float *end) {
-        const int64_t n = end - p;
-        return n <= 0 ? 0u : (n > 0x3fffffff ? 0xfffffffcu : static_cast<uint32_t>(n) * 4u);
+    // bytes a scale copy may read: none for a slab of zero padding beyond the K blocks the
+    // arrays hold (whatever lies there must not meet the matrix core: an E8M0 NaN would stick)
+    [[maybe_unused]] auto bytes_left = [&](const uint8_t *p, const uint8_t *end, int h) {
+        const int64_t n     = end - p;
+        const bool    valid = GMODE == GROUP_K || (MODE == SCALE_MX ? (ld_kt * NW + h) * 4 : ld_kt) < a.kb_valid;
+        return (n <= 0 || !valid) ? 0u : (n > 0x7fffffff ? 0x7fffffffu : static_cast<uint32_t>(n));
     };
-    // copy number L of the loader's slab into stage `b`
+    // copy number L of the loader's slab into stage `b`: [0, LA) A rows, [LA, NLD) B rows,
+    // [NLD, NL) scale words
     auto issue_copy = [&](auto lc, int b) {
         constexpr int L   = lc;
         uint8_t      *dst = smem + b * STAGE;
 #if defined(__HIP_DEVICE_COMPILE__) // the buffer resource type only exists in the device pass
         constexpr uint32_t RSRC_FLAGS = 0x00020000; // raw buffer, 32-bit data format
         if constexpr (L >= NLD) {
-            constexpr int Q   = L - NLD;
-            const bool    isA = Q * 64 < SC_A;
+            constexpr int  Q = L - NLD, H = Q / (SC_ROWS / 64), QQ = Q % (SC_ROWS / 64);
+            constexpr bool isA = QQ * 64 < SC_A;
             __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
-                const_cast<float *>(isA ? ld_sa : ld_sb), 0, isA ? bytes_left(ld_sa, ld_sa_end) : bytes_left(ld_sb, ld_sb_end),
-                RSRC_FLAGS);
+                const_cast<uint8_t *>(isA ? ld_sa : ld_sb), 0,
+                isA ? bytes_left(ld_sa, ld_sa_end, H) : bytes_left(ld_sb, ld_sb_end, H), RSRC_FLAGS);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr_t)(dst + A_BYTES + B_BYTES + wave * SC_WAVE + Q * 256), 4,
                                                      off[L], 0, 0, 0);
         } else if constexpr (L < LA) {
@@ -583,6 +605,11 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         }
 #endif
     };
+    // the copies of a slab in issue order: B part (B rows, then scales), then A part
+    auto issue_part_b = [&](auto cc, int b) {
+        constexpr int C = cc;
+        issue_copy(std::integral_constant<int, (C < LB ? LA + C : NLD + (C - LB))>{}, b);
+    };
     auto advance_loader = [&]() {
         if constexpr (XPIPE) {
             const bool wrap = ld_kt + 1 == KT_ALL;
@@ -592,12 +619,12 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             ld_na = wrap ? nxt_t.rows_a * static_cast<uint32_t>(a.lda) : ld_na - KSTEP;
             ld_nb = wrap ? nxt_t.rows_b * static_cast<uint32_t>(a.ldb) : ld_nb - KSTEP;
             if constexpr (LDS_SC) {
-                const float *na = nxt_t.sA + (nxt_t.m0 >> a.sa_shift) * a.sa_m;
-                const float *nb = nxt_t.sB + (nxt_t.n0 >> a.sb_shift) * a.sb_n;
-                ld_sa           = wrap ? na : ld_sa + a.sa_k;
-                ld_sb           = wrap ? nb : ld_sb + a.sb_k;
-                ld_sa_end       = wrap ? nxt_t.sA + sa_extent : ld_sa_end;
-                ld_sb_end       = wrap ? nxt_t.sB + sb_extent : ld_sb_end;
+                const uint8_t *na = as_bytes(nxt_t.sA) + ((nxt_t.m0 >> a.sa_shift) * a.sa_m) * SC_ELT;
+                const uint8_t *nb = as_bytes(nxt_t.sB) + ((nxt_t.n0 >> a.sb_shift) * a.sb_n) * SC_ELT;
+                ld_sa             = wrap ? na : ld_sa + sa_step;
+                ld_sb             = wrap ? nb : ld_sb + sb_step;
+                ld_sa_end         = wrap ? as_bytes(nxt_t.sA) + sa_extent : ld_sa_end;
+                ld_sb_end         = wrap ? as_bytes(nxt_t.sB) + sb_extent : ld_sb_end;
             }
         } else {
             const int adv = ld_kt + 1 < cur_t.KT ? KSTEP : 0;
@@ -607,18 +634,21 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             ld_na -= adv;
             ld_nb -= adv;
             if constexpr (LDS_SC) {
-                ld_sa += adv ? a.sa_k : 0;
-                ld_sb += adv ? a.sb_k : 0;
+                ld_sa += adv ? sa_step : 0;
+                ld_sb += adv ? sb_step : 0;
             }
         }
     };
 
-    // BLOCK mode: the fp32 scales of a slab are read from its stage at the release point of
-    // the slab before, next to its first fragments.
-    constexpr int NSBJ = SB_VEC ? TN : 1; // without per-column scales one value serves the wavefront
+    // BLOCK mode: the fp32 scales of a slab are read from its stage one slab ahead (after
+    // barrier X). Without per-column scales one B value serves the whole wavefront and is
+    // multiplied into the row scales once per slab.
+    constexpr int NSBJ = SB_VEC ? TN : 1;
     [[maybe_unused]] float sa_nxt[TM], sb_nxt[NSBJ][NSB], sc_cur[TM], sb_cur[NSBJ][NSB];
+    // MX mode: lane (r, g) takes the E8M0 byte of fragment row r and K block g
+    [[maybe_unused]] uint32_t mxa_cur[TM][NH], mxa_nxt[TM][NH], mxb_cur[TN][NH], mxb_nxt[TN][NH];
     auto read_scales = [&](const uint8_t *stage) {
-        if constexpr (LDS_SC) {
+        if constexpr (MODE == SCALE_BLOCK) {
             const float *reg = reinterpret_cast<const float *>(stage + A_BYTES + B_BYTES + wave * SC_WAVE);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
@@ -635,40 +665,23 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                 sb_nxt[0][0] = reg[SC_A];
             }
         }
-    };
-
-    // MX mode: the E8M0 bytes of the next slab are fetched the same way, one byte per lane,
-    // fragment and MFMA: lane (r, g) takes the byte of fragment row r and K block g.
-    [[maybe_unused]] uint32_t mxa_cur[TM][NH], mxa_nxt[TM][NH], mxb_cur[TN][NH], mxb_nxt[TN][NH];
-    auto fetch_mx = [&](int64_t m0, int64_t n0, const float *sAm, const float *sBm, int kt, uint32_t (&sa)[TM][NH],
-                        uint32_t (&sb)[TN][NH]) {
         if constexpr (MODE == SCALE_MX) {
-            const uint8_t *pa = reinterpret_cast<const uint8_t *>(sAm), *pb = reinterpret_cast<const uint8_t *>(sBm);
-            const int64_t  wm_base = m0 + wm * (TM * 16), wn_base = n0 + wn * (TN * 16);
+            const uint8_t *reg = stage + A_BYTES + B_BYTES + wave * SC_WAVE + lm * 4 + lg;
 #pragma unroll
             for (int h = 0; h < NH; ++h) {
-                int kb = (kt * NH + h) * 4 + lg;
-                kb     = kb < a.kb_valid ? kb : a.kb_valid - 1; // zero-padded K: any finite scale will do
 #pragma unroll
-                for (int i = 0; i < TM; ++i) {
-                    int64_t m = wm_base + i * 16 + lm;
-                    m         = m < a.M ? m : a.M - 1;
-                    sa[i][h]  = pa[m * a.sa_m + kb];
-                }
+                for (int i = 0; i < TM; ++i)
+                    mxa_nxt[i][h] = reg[(h * SC_ROWS + i * 16) * 4];
 #pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    int64_t n = wn_base + j * 16 + lm;
-                    n         = n < a.N ? n : a.N - 1;
-                    sb[j][h]  = pb[n * a.sb_n + kb];
-                }
+                for (int j = 0; j < TN; ++j)
+                    mxb_nxt[j][h] = reg[(h * SC_ROWS + SC_A + j * 16) * 4];
             }
         }
     };
 
     f32x4 acc[TM][TN];
-    // MFMA operand fragments (8 VGPRs each). Loop-carried: fa = the A fragments of the slab
-    // about to be multiplied, fb[0] and fb[1] = its first two B fragments.
-    i32x8 fa[TM], fb[4];
+    // MFMA operand fragments (8 VGPRs each) of the slab being multiplied
+    i32x8 fa[TM], fb[TN];
     int   buf = 0;
 
     // fragment f (16 rows) of the A or B part of a stage: two 16-byte LDS reads per lane
@@ -684,20 +697,21 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     const uint32_t a_part = wm * (TM * 16) * KSTEP;
     const uint32_t b_part = A_BYTES + wn * (TN * 16) * KSTEP;
 
-    // pipeline start at tile t: slabs 0 and 1 requested, the first fragments of slab 0 on their way
+    // pipeline start at tile t: NSTAGE slabs requested, the fragments of slab 0 on their way
     auto start_pipeline = [&](const TileCtx &t) {
         loader_to(t);
-        fetch_mx(t.m0, t.n0, t.sA, t.sB, 0, mxa_nxt, mxb_nxt);
         static_for<0, NSTAGE>([&](auto st) {
-            static_for<0, NL>([&](auto l) { issue_copy(l, st); });
+            static_for<0, NB>([&](auto c) { issue_part_b(c, st); });
+            static_for<0, LA>([&](auto c) { issue_copy(c, st); });
             advance_loader();
         });
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NSTAGE - 1) * NL) : "memory");
         __builtin_amdgcn_s_barrier();
-        buf   = 0;
+        buf = 0;
         read_scales(smem);
-        fb[0] = ldfrag(smem + b_part, 0);
-        fb[1] = ldfrag(smem + b_part, 1);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            fb[j] = ldfrag(smem + b_part, j);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
             fa[i] = ldfrag(smem + a_part, i);
@@ -728,10 +742,8 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         // the compiler sinks the MFMAs behind them
         for (int kt = 0; kt < KT; ++kt) {
             const int      buf_n = buf + 1 == NSTAGE ? 0 : buf + 1;
-            const uint8_t *cur   = smem + buf * STAGE;
             const uint8_t *nxt   = smem + buf_n * STAGE;
             if constexpr (MODE == SCALE_BLOCK) {
-                // without per-column scales the two factors are combined once per row here
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
                     sc_cur[i] = SB_VEC ? sa_nxt[i] : sa_nxt[i] * sb_nxt[0][0];
@@ -753,15 +765,13 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                 }
             }
 
-            // BLOCK mode: MFMA t (in issue order) writes ring[t % RING]; DEPTH MFMAs later its
-            // product is folded into the running sum with the block scales (VALU work in
-            // the shadow of later MFMAs).
+            // BLOCK mode: MFMA t (in issue order, t = j TM + i) writes ring[t % RING]; DEPTH
+            // MFMAs later its product is folded into the running sum with the block scales
+            // (VALU work in the shadow of later MFMAs).
             [[maybe_unused]] constexpr int DEPTH = 2, RING = DEPTH + 1, TILES = TM * TN;
             [[maybe_unused]] f32x4 ring[RING];
-            // issue order -> tile: columns [0, JR) column-major, then rows of the last two columns
             [[maybe_unused]] auto  fold = [&](int t) {
-                const int    i = t < JR * TM ? t % TM : (t - JR * TM) / 2;
-                const int    j = t < JR * TM ? t / TM : JR + (t - JR * TM) % 2;
+                const int    i = t % TM, j = t / TM;
                 const f32x4 &p = ring[t % RING];
                 if constexpr (SB_VEC) {
 #pragma unroll
@@ -774,8 +784,10 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                 }
             };
             // h selects the half of an MXFP4 slab (always 0 otherwise)
-            auto mma = [&](int t, int i, int j, const i32x8 &af, const i32x8 &bf, int h) {
+            auto mma = [&](int i, int j, int h) {
+                const i32x8 &af = fa[i], &bf = fb[j];
                 if constexpr (MODE == SCALE_BLOCK) {
+                    const int t    = j * TM + i;
                     ring[t % RING] = mfma_fp8<FA, FB>(bf, af, f32x4{0.f, 0.f, 0.f, 0.f});
                     if (t >= DEPTH)
                         fold(t - DEPTH);
@@ -790,50 +802,41 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                 }
             };
 
-            // ---- columns 0 .. JR-1: B fragment j + 2 is requested before column j is multiplied ----
-#pragma unroll
-            for (int j = 0; j < JR; ++j) {
-                fb[(j + 2) % 4] = ldfrag(cur + b_part, j + 2);
-                // keep the instruction scheduler from moving MFMAs and LDS reads across each other
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int h = 0; h < NH; ++h)
-#pragma unroll
-                    for (int i = 0; i < TM; ++i)
-                        mma(j * TM + i, i, j, fa[i], fb[j % 4], h);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-
-            // ---- release point ----
-            // my reads of this stage are done and my copies of the next slab have landed (the
-            // copies of the slabs after that, NSTAGE - 2 of them, may still be in flight)
-            PT_GEMM_TRACE_POINT(2);
-            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((NSTAGE - 2) * NL) : "memory");
-            __builtin_amdgcn_s_barrier();
-            PT_GEMM_TRACE_POINT(3);
-            // (after a tile's last slab without a successor the following fetch and read leftovers:
-            // harmless)
-            read_scales(nxt);
-            if constexpr (MODE == SCALE_MX) {
-                static_assert(MODE != SCALE_MX || XPIPE, "MX GEMMs are not grouped here");
-                const bool same = kt + 1 < KT;
-                fetch_mx(same ? cur_t.m0 : nxt_t.m0, same ? cur_t.n0 : nxt_t.n0, cur_t.sA, cur_t.sB, same ? kt + 1 : 0,
-                         mxa_nxt, mxb_nxt);
-            }
-            fb[0] = ldfrag(nxt + b_part, 0);
-            fb[1] = ldfrag(nxt + b_part, 1);
-            __builtin_amdgcn_sched_barrier(0);
-            // ---- last two columns, row by row: A fragment i is refilled as soon as it is dead ----
-            static_for<0, TM>([&](auto ic) {
-                constexpr int i = ic;
-#pragma unroll
-                for (int h = 0; h < NH; ++h) {
-                    mma(JR * TM + 2 * i, i, JR, fa[i], fb[JR % 4], h);
-                    mma(JR * TM + 2 * i + 1, i, JR + 1, fa[i], fb[(JR + 1) % 4], h);
+            // MFMA slots of a slab: s = (j NH + h) TM + i. B-part copies are spread over the
+            // slots of columns [1, JY), A-part copies over those of columns [JY, TN).
+            constexpr int COL = NH * TM, S_B0 = COL, S_B1 = JY * COL, S_A0 = JY * COL, S_A1 = TN * COL;
+            static_for<0, TN>([&](auto jc) {
+                constexpr int j = jc;
+                static_for<0, COL>([&](auto sc) {
+                    constexpr int h = sc / TM, i = sc % TM, s = j * COL + sc;
+                    mma(i, j, h);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (j == TN - 1 && h == NH - 1)
+                        fa[i] = ldfrag(nxt + a_part, i); // dead from here on: refill from the next slab
+                    if constexpr (s >= S_B0 && s < S_B1)
+                        static_for<(s - S_B0) * NB / (S_B1 - S_B0), (s + 1 - S_B0) * NB / (S_B1 - S_B0)>(
+                            [&](auto c) { issue_part_b(c, buf); });
+                    if constexpr (s >= S_A0 && s < S_A1)
+                        static_for<(s - S_A0) * LA / (S_A1 - S_A0), (s + 1 - S_A0) * LA / (S_A1 - S_A0)>(
+                            [&](auto c) { issue_copy(c, buf); });
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+                if constexpr (j == 0) {
+                    // ---- barrier X ----
+                    // my reads of the current stage are done (they were issued a column ago) and my
+                    // copies of the next slab's B part have landed; younger copies may be in flight
+                    PT_GEMM_TRACE_POINT(2);
+                    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LA + (NSTAGE - 2) * NL) : "memory");
+                    __builtin_amdgcn_s_barrier();
+                    PT_GEMM_TRACE_POINT(3);
+                    read_scales(nxt);
                 }
-                __builtin_amdgcn_sched_barrier(0);
-                fa[i] = ldfrag(nxt + a_part, i);
-                static_for<i * NL / TM, (i + 1) * NL / TM>([&](auto l) { issue_copy(l, buf); });
+                if constexpr (j == JY - 1) {
+                    // ---- barrier Y: the next slab's A part has landed ----
+                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NB + (NSTAGE - 2) * NL) : "memory");
+                    __builtin_amdgcn_s_barrier();
+                }
+                fb[j] = ldfrag(nxt + b_part, j); // column j is done: refill from the next slab
                 __builtin_amdgcn_sched_barrier(0);
             });
             if constexpr (MODE == SCALE_BLOCK) {
@@ -845,9 +848,9 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             buf = buf_n;
         }
         if constexpr (!XPIPE) {
-            // the re-read copies of the last slab must have landed everywhere before the next
-            // tile's first copies go into the same stages
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            // the re-read copies of the last slab must have landed everywhere, and everyone must be
+            // done reading the stages, before the next tile's first copies go into them
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_s_barrier();
         }
 
@@ -875,7 +878,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
 template <int TM, int TN, int MODE, bool SB_VEC, int FA, int FB, int GMODE = GROUP_NONE>
 static int launch_gemm_cfg(const GemmArgs &args_in, hipStream_t stream) {
     constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
-    constexpr int STAGES  = gemm_stages(TM, TN) * gemm_stage_bytes(TM, TN, MODE);
+    constexpr int STAGES  = gemm_stages(TM, TN, FA == 4) * gemm_stage_bytes(TM, TN, MODE, FA == 4);
     // groups whose tile prefix sums fit into the LDS next to the stages
     constexpr int MAX_G   = (160 * 1024 - STAGES) / 4 - 2 < 2048 ? 1024 : 2048;
     constexpr int LDS_MAX = STAGES + (GMODE == GROUP_ROWS ? (MAX_G + 2) * 4 : 0);
@@ -888,6 +891,10 @@ static int launch_gemm_cfg(const GemmArgs &args_in, hipStream_t stream) {
         return fail(PT_ERR_INVALID_ARGUMENT, "grouped gemm: too many groups for this tile configuration");
     if (MODE == SCALE_BLOCK && ((!SB_VEC && a.sb_shift != 7) || (GMODE == GROUP_ROWS && a.sa_shift != 0)))
         return fail(PT_ERR_INVALID_ARGUMENT, "gemm_fp8: unsupported block-scale layout");
+    // MX scale words are fetched as aligned 32-bit units
+    if (MODE == SCALE_MX && (a.sa_shift != 0 || a.sb_shift != 0 || a.sa_m % 4 != 0 || a.sb_n % 4 != 0 ||
+                             reinterpret_cast<uintptr_t>(a.sA) % 4 != 0 || reinterpret_cast<uintptr_t>(a.sB) % 4 != 0))
+        return fail(PT_ERR_INVALID_ARGUMENT, "gemm_mx: scale rows must be 4-byte aligned");
     auto kern            = gemm_fp8_nt_kernel<TM, TN, MODE, SB_VEC, FA, FB, GMODE>;
     static bool attr_set = false;
     if (!attr_set) {
