@@ -53,9 +53,68 @@ __global__ __launch_bounds__(256) void pad_rows_u8_kernel(const uint8_t *__restr
     }
 }
 
+// The same for 16-byte aligned shapes: a workgroup moves a 128 x 128 byte tile. A thread loads
+// 16 bytes from each of four consecutive rows, transposes the four 4 x 4 byte blocks in
+// registers (v_perm_b32) and writes 16 words "four rows of one column" into the LDS tile, which
+// is then written out as full 128-byte rows.
+__global__ __launch_bounds__(256) void transpose_u8_tile128_kernel(const uint8_t *__restrict__ in,
+                                                                   uint8_t *__restrict__ out, const int64_t R,
+                                                                   const int64_t C, const int64_t ldo) {
+    constexpr int  P = 33; // words per LDS row: conflict-free 16-byte row reads, 2-way column writes
+    __shared__ uint32_t t[128 * P];
+    const int64_t  r0 = static_cast<int64_t>(blockIdx.y) * 128, c0 = static_cast<int64_t>(blockIdx.x) * 128;
+    const int64_t  bi = static_cast<int64_t>(blockIdx.z) * R * C, bo = static_cast<int64_t>(blockIdx.z) * C * ldo;
+    const int      tid = threadIdx.x;
+    {
+        const int     cc = tid & 7, rg = tid >> 3; // 16-byte column chunk, group of four rows
+        const int64_t gc = c0 + cc * 16;
+        u32x4         a[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int64_t gr = r0 + rg * 4 + e;
+            a[e] = (gr < R && gc < C) ? *reinterpret_cast<const u32x4 *>(in + bi + gr * C + gc) : u32x4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int w = 0; w < 4; ++w) { // word w of the four rows = columns 4w .. 4w+3
+            const uint32_t t0 = __builtin_amdgcn_perm(a[1][w], a[0][w], 0x05010400u);
+            const uint32_t t1 = __builtin_amdgcn_perm(a[1][w], a[0][w], 0x07030602u);
+            const uint32_t t2 = __builtin_amdgcn_perm(a[3][w], a[2][w], 0x05010400u);
+            const uint32_t t3 = __builtin_amdgcn_perm(a[3][w], a[2][w], 0x07030602u);
+            const int      c  = cc * 16 + w * 4;
+            t[(c + 0) * P + rg] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+            t[(c + 1) * P + rg] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+            t[(c + 2) * P + rg] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+            t[(c + 3) * P + rg] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+        }
+    }
+    __syncthreads();
+    const int j = tid & 7; // 16-byte chunk of an output row
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int     c  = (tid >> 3) + 32 * p; // output row = input column
+        const int64_t gc = c0 + c, gr = r0 + j * 16;
+        if (gc < C && gr < ldo) {
+            u32x4 v;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                v[k] = t[c * P + j * 4 + k];
+            *reinterpret_cast<u32x4 *>(out + bo + gc * ldo + gr) = v; // rows >= R were loaded as 0
+        }
+    }
+}
+
 void launch_transpose(const uint8_t *in, uint8_t *out, int64_t batch, int64_t R, int64_t C,
                       int64_t ldo, hipStream_t st) {
-    // the grid covers ldo (>= R) input-row positions so that the zero tail gets written too
+    if (batch <= 0 || C <= 0 || ldo <= 0)
+        return;
+    // the grids cover ldo (>= R) input-row positions so that the zero tail gets written too
+    const bool aligned = C % 16 == 0 && ldo % 16 == 0 && reinterpret_cast<uintptr_t>(in) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    if (aligned) {
+        dim3 g(static_cast<unsigned>(cdiv(C, 128)), static_cast<unsigned>(cdiv(ldo, 128)), static_cast<unsigned>(batch));
+        transpose_u8_tile128_kernel<<<g, 256, 0, st>>>(in, out, R, C, ldo);
+        return;
+    }
     dim3 g(static_cast<unsigned>(cdiv(C, 64)), static_cast<unsigned>(cdiv(ldo, 64)),
            static_cast<unsigned>(batch));
     transpose_u8_kernel<<<g, 256, 0, st>>>(in, out, R, C, ldo);

@@ -768,7 +768,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             // BLOCK mode: MFMA t (in issue order, t = j TM + i) writes ring[t % RING]; DEPTH
             // MFMAs later its product is folded into the running sum with the block scales
             // (VALU work in the shadow of later MFMAs).
-            [[maybe_unused]] constexpr int DEPTH = 2, RING = DEPTH + 1, TILES = TM * TN;
+            [[maybe_unused]] constexpr int DEPTH = 3, RING = DEPTH + 1, TILES = TM * TN; // depth 2 costs a dozen wait states per fold
             [[maybe_unused]] f32x4 ring[RING];
             [[maybe_unused]] auto  fold = [&](int t) {
                 const int    i = t % TM, j = t / TM;
