@@ -196,8 +196,223 @@ class GemmFp8Blockwise(_GemmBase):
         )
 
 
+class GemmMx(_GemmBase):
+    """BASELINE config 4: MX-scaled GEMM (E8M0 scale per 32 elements of K, applied by the matrix
+    core): MXFP4 (E2M1) or its MXFP8 (E4M3) fallback, bf16 source ~N(0, 1), bf16 output."""
+
+    def __init__(self, dev, fp4=True, M=16384, N=16384, K=16384):
+        import primus_turbo.pytorch as turbo
+        from primus_turbo.pytorch.core.low_precision import (
+            Float4QuantConfig,
+            Float8QuantConfig,
+            Format,
+            ScaleDtype,
+            ScalingGranularity,
+            ScalingRecipe,
+        )
+        from primus_turbo.pytorch.kernels.gemm import gemm_fp4_impl, gemm_fp8_impl
+        from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+        self.turbo, self.G, self.fp4 = turbo, ScalingGranularity, fp4
+        self.M, self.N, self.K = M, N, K
+        kind = "mxfp4_e2m1" if fp4 else "mxfp8_e4m3"
+        self.name = f"{kind}_gemm_{M}x{N}x{K}_bf16_out (quantize A 1x32, quantize B 32x32, multiply)"
+        self.dtype = ("fp4_e2m1" if fp4 else "fp8_e4m3") + " with E8M0 block scales (fp32 accumulate)"
+        self.peak = 10100.0 if fp4 else FP8_PEAK_TFLOPS
+        self.dominant_name = "gemm_fp8_nt_kernel<256x256 tile, E8M0 block scales in the MFMA>"
+        self.fmt = "e2m1" if fp4 else "e4m3"
+        if fp4:
+            self.cfg = Float4QuantConfig()
+            self.qdt = torch.float4_e2m1fn_x2
+            self._quant, self._impl = qi.quantize_mxfp4_impl, gemm_fp4_impl.gemm_fp4_impl
+        else:
+            self.cfg = Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.MX_BLOCKWISE,
+                                         block_size=32, scale_dtype=ScaleDtype.E8M0)
+            self.qdt = torch.float8_e4m3fn
+            self._quant, self._impl = qi.quantize_mxfp8_impl, gemm_fp8_impl.gemm_fp8_impl
+        self.a_cpu = _randn_bf16((M, K), 5, 1.0)
+        self.b_cpu = _randn_bf16((N, K), 6, 1.0)
+        self.a, self.b = self.a_cpu.to(dev), self.b_cpu.to(dev)
+        self.aq, self.as_ = self._quant(self.a, self.qdt, 1, 32)
+        self.bq, self.bs = self._quant(self.b, self.qdt, 1, 32, scaling_recipe=ScalingRecipe(use_2d_block=True))
+
+    def step(self):
+        op = self.turbo.ops.gemm_fp4 if self.fp4 else self.turbo.ops.gemm_fp8
+        return op(self.a, self.b, trans_a=False, trans_b=True, out_dtype=torch.bfloat16, config=self.cfg)
+
+    def dominant(self):
+        return self._impl(self.aq, self.as_, False, self.bq, self.bs, True, torch.bfloat16, False,
+                          self.G.MX_BLOCKWISE.value, 0)
+
+    def check(self):
+        """Quantized codes and E8M0 bytes of 128 rows of A and the first 128 rows of B bit-exact
+        with the oracle; the product of those A rows against the oracle's de-quantized matmul."""
+        import numpy as np
+
+        from oracle import gemm as OG
+        from oracle import quantize as Q
+
+        def u8(t):
+            return t.contiguous().view(torch.uint8).cpu().numpy()
+
+        out = self.dominant().float().cpu().numpy()
+        rows = np.r_[0:64, self.M - 64 : self.M]
+        a = self.a_cpu.float().numpy()[rows]
+        aq, asc = Q.mx_quant_rowwise(a, self.fmt)
+        bq, bsc = Q.mx_quant_rowwise(self.b_cpu.float().numpy()[:128], self.fmt, use_2d_block=True)
+        kb = self.K // 32
+        same = np.array_equal(u8(self.aq)[rows], aq) and np.array_equal(u8(self.as_)[rows][:, :kb], asc[:, :kb])
+        same = same and np.array_equal(u8(self.bq)[:128], bq) and np.array_equal(u8(self.bs)[:128, :kb], bsc[:, :kb])
+        nb = min(self.N, 2048)  # output columns checked
+        b_deq = Q.mx_dequant(u8(self.bq)[:nb], u8(self.bs)[:nb], self.fmt)
+        ref = OG.gemm_dequantized(Q.mx_dequant(aq, asc, self.fmt), b_deq, trans_b=True)
+        ref_t = torch.from_numpy(np.ascontiguousarray(ref, dtype=np.float32)).to(torch.bfloat16).float().numpy()
+        rel = OG.max_rel_err(ref_t, out[rows][:, :nb])
+        cos = OG.cosine(out[rows][:, :nb], ref_t)
+        ok = bool(same and rel <= 1e-2 and cos >= 0.9999)
+        return ok, f"codes and E8M0 bytes bit-exact: {same}; 128 x 2048 outputs vs oracle: max_rel_err={rel:.2e}, cosine={cos:.6f}"
+
+    def cpu_baseline(self):
+        """The oracle (numpy restatement of the reference's MX quantizer) plus an fp32 matmul on a
+        slice: 256 rows of A against 2048 rows of B."""
+        import numpy as np
+
+        from oracle import quantize as Q
+
+        ra, rb = 256, 2048
+        a = self.a_cpu[:ra].float().numpy()
+        b = self.b_cpu[:rb].float().numpy()
+        t0 = time.perf_counter()
+        aq, asc = Q.mx_quant_rowwise(a, self.fmt)
+        bq, bsc = Q.mx_quant_rowwise(b, self.fmt, use_2d_block=True)
+        y = Q.mx_dequant(aq, asc, self.fmt) @ Q.mx_dequant(bq, bsc, self.fmt).T
+        dt = time.perf_counter() - t0
+        del y
+        return dict(
+            value=round(2.0 * ra * rb * self.K / dt / 1e12, 5),
+            unit="TFLOP/s",
+            cores=torch.get_num_threads(),
+            kind="port",
+            sample=f"{ra} rows of A against {rb} rows of B (MX quantize both, dequantize, fp32 matmul), {dt:.1f} s, "
+            f"{os.cpu_count()} logical CPUs visible",
+        )
+
+
+def _zipf_group_lens(groups, total, seed):
+    """Per-expert token counts ~ Zipf(1.2) over a random expert order, two experts empty."""
+    import numpy as np
+
+    rng = np.random.default_rng(seed)
+    w = rng.permutation((1.0 + np.arange(groups)) ** -1.2)
+    w[rng.choice(groups, 2, replace=False)] = 0
+    lens = np.floor(w / w.sum() * total).astype(np.int64)
+    lens[np.argmax(lens)] += total - lens.sum()
+    return lens
+
+
+class GroupedGemmFp8(_GemmBase):
+    """BASELINE config 3: MoE grouped GEMM of one GPU's experts (32 experts, 32768 routed tokens,
+    Zipf(1.2) counts with empty experts), blockwise 128 scales; a step is forward + dgrad + wgrad
+    of one expert layer through the autograd op."""
+
+    dominant_name = "gemm_fp8_nt_kernel<128x128 tile, row groups, 1x128 * 128x128 block scales> (forward)"
+
+    def __init__(self, dev, N=4096, K=7168, groups=32, tokens=32768):
+        import primus_turbo.pytorch as turbo
+        from primus_turbo.pytorch.core.low_precision import Float8QuantConfig, Format, ScalingGranularity
+        from primus_turbo.pytorch.kernels.grouped_gemm import grouped_gemm_fp8_impl as gg
+        from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+        self.turbo, self.G, self.gg, self.qi = turbo, ScalingGranularity, gg, qi
+        self.M, self.N, self.K, self.groups = tokens, N, K, groups
+        self.name = (f"moe_grouped_gemm_fp8_blockwise_{groups}experts_{tokens}tokens_zipf1.2_k{K}_n{N} "
+                     "(forward + dgrad + wgrad, quantizers included)")
+        self.cfg = Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.BLOCKWISE, block_size=128)
+        self.lens = _zipf_group_lens(groups, tokens, 7)
+        self.gl = torch.from_numpy(self.lens).to(dev)
+        self.offs = torch.ops.primus_turbo_cpp_extension.grouped_gemm_compute_offs(self.gl)
+        self.x_cpu = _randn_bf16((tokens, K), 7, 1.0)
+        self.w_cpu = _randn_bf16((groups, N, K), 8, 1.0)
+        self.x = self.x_cpu.to(dev).requires_grad_(True)
+        self.w = self.w_cpu.to(dev).requires_grad_(True)
+        self.dy = _randn_bf16((tokens, N), 9, 1.0).to(dev)
+        self.qr, _, self.sr, _, _, _ = qi.quant_fp8_blockwise_segment_m_row_col_impl(
+            self.x.detach(), torch.float8_e4m3fn, 128, self.gl, self.offs, N)
+        self.wq, self.ws = qi.quant_fp8_blockwise_for_weight_impl(self.w.detach(), torch.float8_e4m3fn, 128)
+
+    def step_work(self):
+        return 3 * 2.0 * self.M * self.N * self.K
+
+    def step(self):
+        self.x.grad = None
+        self.w.grad = None
+        y = self.turbo.ops.grouped_gemm_fp8(self.x, self.w, self.gl, self.offs, trans_b=True, config=self.cfg)
+        y.backward(self.dy)
+        return y
+
+    def dominant(self):
+        return self.gg.grouped_gemm_fp8_impl(self.qr, self.wq, self.sr, self.ws, self.gl, self.offs, False, True,
+                                             torch.bfloat16, self.G.BLOCKWISE.value, None, 0)
+
+    def check(self):
+        """Forward rows of the first and of the last non-empty expert (up to 64 each) against the
+        oracle's de-quantized matmul; their quantized bytes bit-exact."""
+        import numpy as np
+
+        from oracle import gemm as OG
+        from oracle import quantize as Q
+
+        out = self.dominant().float().cpu().numpy()
+        offs = np.concatenate([[0], np.cumsum(self.lens)])
+        live = [g for g in range(self.groups) if self.lens[g] > 0]
+        same, rel, cos = True, 0.0, 1.0
+        for g in (live[0], live[-1]):
+            r0, r1 = int(offs[g]), int(min(offs[g] + 64, offs[g + 1]))
+            aq, asi = Q.fp8_blockwise(self.x_cpu.float().numpy()[r0:r1], 1, "e4m3", 128)
+            bq, bsi = Q.fp8_blockwise_weight(self.w_cpu[g].float().numpy(), "e4m3", 128)
+            same = same and np.array_equal(self.qr[r0:r1].view(torch.uint8).cpu().numpy(), aq)
+            same = same and np.array_equal(self.wq[g].view(torch.uint8).cpu().numpy(), bq)
+            ref = OG.gemm_dequantized(Q.fp8_blockwise_dequant(aq, asi, 1, "e4m3", 128),
+                                      Q.fp8_blockwise_weight_dequant(bq, bsi, "e4m3", 128), trans_b=True)
+            ref_t = torch.from_numpy(np.ascontiguousarray(ref, dtype=np.float32)).to(torch.bfloat16).float().numpy()
+            rel = max(rel, OG.max_rel_err(ref_t, out[r0:r1]))
+            cos = min(cos, OG.cosine(out[r0:r1], ref_t))
+        ok = bool(same and rel <= 1e-2 and cos >= 0.9999)
+        return ok, f"quantized bytes bit-exact: {same}; rows of two experts vs oracle: max_rel_err={rel:.2e}, cosine={cos:.6f}"
+
+    def cpu_baseline(self):
+        """The reference's CPU formulas (blockwise quantize, dequantize, per-expert fp32 matmul) for
+        the forward product of the four experts with the most tokens."""
+        from oracle import cpu_reference as R
+
+        import numpy as np
+
+        offs = np.concatenate([[0], np.cumsum(self.lens)])
+        top = np.argsort(-self.lens)[:4]
+        rows = int(self.lens[top].sum())
+        t0 = time.perf_counter()
+        for g in top:
+            y = R.gemm_fp8_blockwise_ref(self.x_cpu[int(offs[g]) : int(offs[g + 1])], self.w_cpu[g], torch.float8_e4m3fn, 128)
+        dt = time.perf_counter() - t0
+        del y
+        return dict(
+            value=round(2.0 * rows * self.N * self.K / dt / 1e12, 4),
+            unit="TFLOP/s",
+            cores=torch.get_num_threads(),
+            kind="port",
+            sample=f"forward product of the 4 largest experts ({rows} of {self.M} tokens: blockwise quantize, "
+            f"dequantize, fp32 matmul), {dt:.1f} s, {os.cpu_count()} logical CPUs visible",
+        )
+
+
 def register(workloads):
     workloads["gemm_fp8_rowwise"] = GemmFp8Rowwise
     workloads["gemm_fp8_blockwise"] = GemmFp8Blockwise
     workloads["gemm_fp8_blockwise_k7168"] = lambda dev: GemmFp8Blockwise(dev, 16384, 4096, 7168)
     workloads["gemm_fp8_blockwise_8192"] = lambda dev: GemmFp8Blockwise(dev, 8192, 8192, 8192)
+    workloads["gemm_mxfp4"] = lambda dev: GemmMx(dev, True, 16384, 16384, 16384)
+    workloads["gemm_mxfp4_n28672"] = lambda dev: GemmMx(dev, True, 8192, 28672, 8192)
+    workloads["gemm_mxfp8"] = lambda dev: GemmMx(dev, False, 16384, 16384, 16384)
+    workloads["gemm_mxfp8_n28672"] = lambda dev: GemmMx(dev, False, 8192, 28672, 8192)
+    workloads["grouped_gemm_fp8"] = lambda dev: GroupedGemmFp8(dev, 4096, 7168)
+    workloads["grouped_gemm_fp8_down"] = lambda dev: GroupedGemmFp8(dev, 7168, 2048)
