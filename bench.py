@@ -145,6 +145,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="auto", help="one of: auto, " + ", ".join(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also launch one plain elementwise copy of 256 MiB (fp32 x + 0 -> y): the known-size "
+                    "kernel that HBM traffic counters of a profiled run are scaled by")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -164,6 +167,13 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     wl = WORKLOADS[name](dev)
+
+    if args.calib_copy:
+        src = torch.ones(64 << 20, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        torch.add(src, 0.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
 
     ok, what = wl.check()
     for _ in range(args.warmup):

@@ -185,18 +185,18 @@ __device__ __forceinline__ void mfma_inplace_f4(f32x4 &c, const i32x4 &rowop, co
 // Tile coordinates of a workgroup: XCD-contiguous ids, then groups of GROUP_M tile rows
 // walked column-major so that concurrently running tiles share A and B panels in L2.
 __device__ __forceinline__ void tile_coords_local(int lid, int tiles_m, int tiles_n, int &tm, int &tn);
+__device__ __forceinline__ int xcd_contiguous_id(int pid, int total) {
+    constexpr int NXCD = 8;
+    if (total < NXCD * 4)
+        return pid;
+    // workgroup i runs on XCD i % 8: give each XCD one contiguous id range
+    const int per = total / NXCD, rem = total % NXCD;
+    const int xcd = pid % NXCD, slot = pid / NXCD;
+    // XCDs [0, rem) own per + 1 ids
+    return xcd * per + (xcd < rem ? xcd : rem) + slot;
+}
 __device__ __forceinline__ void tile_coords(int pid, int tiles_m, int tiles_n, int &tm, int &tn) {
-    constexpr int NXCD  = 8;
-    const int     total = tiles_m * tiles_n;
-    int           lid   = pid;
-    if (total >= NXCD * 4) {
-        // workgroup i runs on XCD i % 8: give each XCD one contiguous id range
-        const int per  = total / NXCD, rem = total % NXCD;
-        const int xcd  = pid % NXCD, slot = pid / NXCD;
-        // XCDs [0, rem) own per + 1 ids
-        lid = xcd * per + (xcd < rem ? xcd : rem) + slot;
-    }
-    tile_coords_local(lid, tiles_m, tiles_n, tm, tn);
+    tile_coords_local(xcd_contiguous_id(pid, tiles_m * tiles_n), tiles_m, tiles_n, tm, tn);
 }
 __device__ __forceinline__ void tile_coords_local(int lid, int tiles_m, int tiles_n, int &tm, int &tn) {
     constexpr int GROUP_M  = 8;
@@ -235,40 +235,72 @@ template <bool ACC_IN_AGPR> __device__ __forceinline__ f32x4 read_acc(const f32x
     return v;
 }
 
+// 16-bit outputs are written by pairs of MFMA tiles (i, j), (i, j + 1): the odd 16-lane rows of
+// tile j are swapped with the even rows of tile j + 1 (v_permlane16_swap), after which a lane
+// holds eight consecutive n of one m -- one 16-byte store, and 64 contiguous bytes per matrix
+// row and store instruction, so that no partially written 64-byte unit ever leaves the L2.
+// `row` points at C[m][wn_base + 16 (lg & 1) + 8 (lg >> 1)] for 16-bit outputs and at
+// C[m][wn_base + 4 lg] for fp32.
 template <typename T, int TM, int TN, int MODE, bool ACC_IN_AGPR>
 __device__ __forceinline__ void epilogue_inner(T *row, int64_t step, bool accu, const f32x4 (&acc)[TM][TN],
                                                const float (&sa)[TM], const f32x4 (&sb)[TN]) {
     static_for<0, TM>([&](auto ic) {
         constexpr int i = ic;
-        static_for<0, TN>([&](auto jc) {
-            constexpr int j = jc;
-            f32x4         v = read_acc<ACC_IN_AGPR>(acc[i][j]);
-            if constexpr (MODE == SCALE_VECTOR) {
+        if constexpr (sizeof(T) == 4) {
+            static_for<0, TN>([&](auto jc) {
+                constexpr int j = jc;
+                f32x4         v = read_acc<ACC_IN_AGPR>(acc[i][j]);
+                if constexpr (MODE == SCALE_VECTOR) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    v[e] = v[e] * sa[i] * sb[j][e];
-            }
-            T *q = row + j * 16;
-            if constexpr (sizeof(T) == 4) {
+                    for (int e = 0; e < 4; ++e)
+                        v[e] = v[e] * sa[i] * sb[j][e];
+                }
+                T *q = row + j * 16;
                 if (accu)
                     v += *reinterpret_cast<const f32x4 *>(q);
                 *reinterpret_cast<f32x4 *>(q) = v;
-            } else {
-                if (accu) {
-                    const u32x2 old = *reinterpret_cast<const u32x2 *>(q);
-                    float       o0, o1, o2, o3;
-                    unpack2<T>(old.x, o0, o1);
-                    unpack2<T>(old.y, o2, o3);
-                    v[0] += o0; v[1] += o1; v[2] += o2; v[3] += o3;
+                // keep each accumulator's read next to its store (register pressure)
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        } else {
+            static_for<0, TN / 2>([&](auto jc) {
+                constexpr int j = 2 * jc;
+                f32x4         x = read_acc<ACC_IN_AGPR>(acc[i][j]), y = read_acc<ACC_IN_AGPR>(acc[i][j + 1]);
+                if constexpr (MODE == SCALE_VECTOR) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        x[e] = x[e] * sa[i] * sb[j][e];
+                        y[e] = y[e] * sa[i] * sb[j + 1][e];
+                    }
                 }
-                u32x2 w;
-                w.x = pack2<T>(v[0], v[1]);
-                w.y = pack2<T>(v[2], v[3]);
-                *reinterpret_cast<u32x2 *>(q) = w;
-            }
-            // keep each accumulator's read next to its store (register pressure)
-            __builtin_amdgcn_sched_barrier(0);
-        });
+                // (written out by hand: the compiler's builtin for this instruction loses track of
+                // vector elements; the wait states cover the VALU writes just before)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float xe = x[e], ye = y[e];
+                    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(xe), "+v"(ye));
+                    x[e] = xe;
+                    y[e] = ye;
+                }
+                asm volatile("s_nop 1" ::: "memory");
+                T *q = row + j * 16;
+                if (accu) {
+                    const u32x4 old = *reinterpret_cast<const u32x4 *>(q);
+                    float       o0, o1;
+                    unpack2<T>(old.x, o0, o1); x[0] += o0; x[1] += o1;
+                    unpack2<T>(old.y, o0, o1); x[2] += o0; x[3] += o1;
+                    unpack2<T>(old.z, o0, o1); y[0] += o0; y[1] += o1;
+                    unpack2<T>(old.w, o0, o1); y[2] += o0; y[3] += o1;
+                }
+                u32x4 w;
+                w.x = pack2<T>(x[0], x[1]);
+                w.y = pack2<T>(x[2], x[3]);
+                w.z = pack2<T>(y[0], y[1]);
+                w.w = pack2<T>(y[2], y[3]);
+                *reinterpret_cast<u32x4 *>(q) = w;
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        }
         row += step;
     });
 }
@@ -314,16 +346,18 @@ __device__ __forceinline__ void epilogue(const GemmArgs &a, const f32x4 (&acc)[T
                 sb[j][e]        = sBm[(n < a.N ? n : a.N - 1) * a.sb_n];
             }
     }
-    // whole sub-tile inside the matrix and every 4-element group aligned: no per-element checks
-    const bool fast = wm_base + TM * 16 <= m_end && wn_base + TN * 16 <= a.N && (a.N & 3) == 0 &&
+    // whole sub-tile inside the matrix and every 16-byte group aligned: no per-element checks
+    const bool fast = wm_base + TM * 16 <= m_end && wn_base + TN * 16 <= a.N && (a.N & 7) == 0 &&
                       (reinterpret_cast<uintptr_t>(C) & 15) == 0;
     uint8_t      *row  = C + (m0 * a.N + n0) * ES;
     const int64_t step = 16 * a.N;
     if (fast) {
+        // 16-bit outputs: the lane's eight columns after the exchange between tile pairs
+        uint8_t *rowp = C + (m0 * a.N + wn_base + 16 * (lg & 1) + 8 * (lg >> 1)) * 2;
         if (a.out_dtype == PT_DTYPE_BF16)
-            epilogue_inner<bf16_t, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<bf16_t *>(row), step, accu, acc, sa, sb);
+            epilogue_inner<bf16_t, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<bf16_t *>(rowp), step, accu, acc, sa, sb);
         else if (a.out_dtype == PT_DTYPE_F16)
-            epilogue_inner<f16_t, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<f16_t *>(row), step, accu, acc, sa, sb);
+            epilogue_inner<f16_t, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<f16_t *>(rowp), step, accu, acc, sa, sb);
         else
             epilogue_inner<float, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<float *>(row), step, accu, acc, sa, sb);
     } else {
@@ -379,6 +413,8 @@ __device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile, const 
         t.C     = static_cast<uint8_t *>(a.C);
         t.KT    = static_cast<int>(a.K / KSTEP);
     } else if constexpr (GMODE == GROUP_ROWS) {
+        // (tile ids stay round-robin over the XCDs here: the XCD-contiguous renumbering of the
+        // dense case measured 3-15% slower on Zipf-distributed groups)
         while (g + 1 < a.G && tile >= __builtin_amdgcn_readfirstlane(prefix[g + 1]))
             ++g;
         const int     local = tile - __builtin_amdgcn_readfirstlane(prefix[g]);
