@@ -96,6 +96,7 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
     constexpr bool ANY2D = (ROW && ROW2D) || (COL && COL2D);
     __shared__ __attribute__((aligned(16))) uint16_t tile[MX_TILE * MX_PITCH];
     __shared__ float                                 amax_rc[ANY2D ? MX_TILE * 4 : 1]; // [row][32-col block]
+    __shared__ __attribute__((aligned(4))) uint8_t   sbytes[MX_TILE * 4]; // E8M0 bytes of the tile, [row or column][block]
     const int     tid = threadIdx.x;
     const int64_t n0 = static_cast<int64_t>(blockIdx.x) * MX_TILE, m0 = static_cast<int64_t>(blockIdx.y) * MX_TILE;
     const int64_t b  = blockIdx.z;
@@ -173,9 +174,9 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
             const int e = mx_exponent<FMT>(am);
             uint32_t  code[8];
             mx_encode32<FMT>(rv[p], mx_inv_scale(e), code);
+            sbytes[r * 4 + c] = static_cast<uint8_t>(e + 127);
             if (m < a.M) {
                 const int64_t nb = (n0 >> 5) + c; // 32-column block index in the padded row
-                a.row_s[(b * a.M + m) * (a.Npad >> 5) + nb] = static_cast<uint8_t>(e + 127);
                 if constexpr (FMT == MX_E2M1) {
                     uint8_t *q = a.row_q + (b * a.M + m) * (a.Npad >> 1) + nb * 16;
                     st128(q, u32x4{code[0], code[1], code[2], code[3]});
@@ -186,16 +187,29 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
                 }
             }
         }
+        __syncthreads();
+        // the four scale bytes of a tile row leave as one word (Npad / 32 is a multiple of 4)
+        if (tid < MX_TILE && m0 + tid < a.M)
+            *reinterpret_cast<uint32_t *>(a.row_s + (b * a.M + m0 + tid) * (a.Npad >> 5) + (n0 >> 5)) =
+                *reinterpret_cast<const uint32_t *>(&sbytes[tid * 4]);
     }
 
     // ---- column direction: task = (column n, 32-row block rb); output transposed ----
+    // The codes go back through the LDS (over the input tile, once everybody has read it) so that
+    // they leave as whole 128-byte (FP4: 64-byte) rows of the transposed output.
     if constexpr (COL) {
+        constexpr int CB    = FMT == MX_E2M1 ? 16 : 32;   // code bytes per 32-row block
+        constexpr int CROW  = 4 * CB;                     // code bytes per output row of the tile
+        constexpr int CPITCH = CROW + 16;                 // LDS pitch of an output row
+        static_assert(MX_TILE * CPITCH <= MX_TILE * MX_PITCH * 2, "the staged codes fit over the input tile");
+        uint32_t code[2][8];
+        if constexpr (ROW)
+            __syncthreads(); // the row pass's scale bytes have been read
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
-            const int     t = tid + 256 * p, c = t & 127, rb = t >> 7;
-            const int64_t n = n0 + c;
-            float         v[32];
-            float         am = 0.f;
+            const int t = tid + 256 * p, c = t & 127, rb = t >> 7;
+            float     v[32];
+            float     am = 0.f;
 #pragma unroll
             for (int i = 0; i < 32; ++i) {
                 v[i] = elem(tile[(rb * 32 + i) * MX_PITCH + c]);
@@ -208,21 +222,34 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
                     am = fmaxf(am, amax_rc[(rb * 32 + i) * 4 + (c >> 5)]);
             }
             const int e = mx_exponent<FMT>(am);
-            uint32_t  code[8];
-            mx_encode32<FMT>(v, mx_inv_scale(e), code);
+            mx_encode32<FMT>(v, mx_inv_scale(e), code[p]);
+            sbytes[c * 4 + rb] = static_cast<uint8_t>(e + 127);
+        }
+        __syncthreads(); // everybody is done with the input tile
+        uint8_t *stage = reinterpret_cast<uint8_t *>(tile);
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const int t = tid + 256 * p, c = t & 127, rb = t >> 7;
+            uint8_t  *d = stage + c * CPITCH + rb * CB;
+            *reinterpret_cast<u32x4 *>(d) = u32x4{code[p][0], code[p][1], code[p][2], code[p][3]};
+            if constexpr (FMT != MX_E2M1)
+                *reinterpret_cast<u32x4 *>(d + 16) = u32x4{code[p][4], code[p][5], code[p][6], code[p][7]};
+        }
+        __syncthreads();
+        constexpr int CHUNKS = CROW / 16; // 16-byte chunks per output row
+#pragma unroll
+        for (int p = 0; p < MX_TILE * CHUNKS / 256; ++p) {
+            const int     k = tid + 256 * p, c = k / CHUNKS, ch = k % CHUNKS;
+            const int64_t n = n0 + c;
             if (n < a.N) {
-                const int64_t mb = (m0 >> 5) + rb;
-                a.col_s[(b * a.N + n) * (a.Mpad >> 5) + mb] = static_cast<uint8_t>(e + 127);
-                if constexpr (FMT == MX_E2M1) {
-                    uint8_t *q = a.col_q + (b * a.N + n) * (a.Mpad >> 1) + mb * 16;
-                    st128(q, u32x4{code[0], code[1], code[2], code[3]});
-                } else {
-                    uint8_t *q = a.col_q + (b * a.N + n) * a.Mpad + mb * 32;
-                    st128(q, u32x4{code[0], code[1], code[2], code[3]});
-                    st128(q + 16, u32x4{code[4], code[5], code[6], code[7]});
-                }
+                const u32x4 w = *reinterpret_cast<const u32x4 *>(stage + c * CPITCH + ch * 16);
+                uint8_t    *q = a.col_q + (b * a.N + n) * (FMT == MX_E2M1 ? a.Mpad >> 1 : a.Mpad) + (m0 >> 5) * CB + ch * 16;
+                st128(q, w);
             }
         }
+        if (tid < MX_TILE && n0 + tid < a.N)
+            *reinterpret_cast<uint32_t *>(a.col_s + (b * a.N + n0 + tid) * (a.Mpad >> 5) + (m0 >> 5)) =
+                *reinterpret_cast<const uint32_t *>(&sbytes[tid * 4]);
     }
 }
 
@@ -352,6 +379,7 @@ int pt_quantize_mx(const void *x, int x_dtype, int64_t B, int64_t M, int64_t N, 
         return PT_OK;
     PT_REQUIRE(x, "NULL input");
     PT_REQUIRE(aligned_to(row_q, 16) && aligned_to(col_q, 16), "outputs must be 16-byte aligned");
+    PT_REQUIRE(aligned_to(row_scale, 4) && aligned_to(col_scale, 4), "scale outputs must be 4-byte aligned");
     MxArgs a;
     a.x     = x;
     a.B     = B;
