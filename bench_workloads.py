@@ -16,6 +16,26 @@ import torch
 
 FP8_PEAK_TFLOPS = 5000.0
 
+# HBM-side bytes per launch of each workload's dominant kernel: rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a plain copy of
+# 256 MiB launched in the same run (`bench.py --calib-copy`; factors 2.000 and 1.000); the runs are
+# summarised under profiles/. (fetched, written) in MiB.
+TRAFFIC_MIB = {
+    "gemm_fp8_rowwise": (779.1, 151.6),
+    "gemm_fp8_blockwise": (493.5, 224.0),
+    "gemm_fp8_blockwise_k7168": (1434.1, 128.0),
+    "gemm_fp8_blockwise_8192": (1482.7, 128.0),
+    "gemm_mxfp4": (3332.6, 754.7),
+    "gemm_mxfp8": (6488.6, 700.2),
+    "grouped_gemm_fp8": (8922.6, 256.1),  # forward launches only
+    "grouped_gemm_fp8_down": (4180.1, 448.2),
+}
+
+
+def _traffic(key):
+    t = TRAFFIC_MIB.get(key)
+    return None if t is None else int((t[0] + t[1]) * 1024 * 1024)
+
 
 def _randn_bf16(shape, seed, std):
     g = torch.Generator().manual_seed(seed)
@@ -405,6 +425,15 @@ class GroupedGemmFp8(_GemmBase):
         )
 
 
+def _keyed(key, make):
+    def build(dev):
+        wl = make(dev)
+        wl.traffic = _traffic(key)
+        return wl
+
+    return build
+
+
 def register(workloads):
     workloads["gemm_fp8_rowwise"] = GemmFp8Rowwise
     workloads["gemm_fp8_blockwise"] = GemmFp8Blockwise
@@ -416,3 +445,6 @@ def register(workloads):
     workloads["gemm_mxfp8_n28672"] = lambda dev: GemmMx(dev, False, 8192, 28672, 8192)
     workloads["grouped_gemm_fp8"] = lambda dev: GroupedGemmFp8(dev, 4096, 7168)
     workloads["grouped_gemm_fp8_down"] = lambda dev: GroupedGemmFp8(dev, 7168, 2048)
+    for key in list(workloads):
+        if key in TRAFFIC_MIB:
+            workloads[key] = _keyed(key, workloads[key])

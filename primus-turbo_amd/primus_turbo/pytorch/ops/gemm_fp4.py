@@ -29,6 +29,7 @@ from primus_turbo.pytorch.core.quantized_tensor import (
     check_quantized_tensor,
 )
 from primus_turbo.pytorch.kernels.gemm.gemm_fp4_impl import gemm_fp4_accum_impl, gemm_fp4_impl
+from primus_turbo.pytorch.kernels.quantization.quantization_impl import quantize_mxfp4_impl
 from primus_turbo.pytorch.ops.quantization import quantize_fp4_with_trans
 from primus_turbo.pytorch.ops.utils import _get_dummy_wgrad, _setup_fused_grad_accum
 
@@ -65,6 +66,8 @@ class FP4GemmMXFunction(torch.autograd.Function):
         dt = FP4GemmMXFunction.get_fp4_dtype(config.format)
         gran, bs = config.granularity, config.block_size
 
+        need_bwd = any(ctx.needs_input_grad[:2])
+
         def both_ways(x, x_t, recipe):
             if isinstance(x, QuantizedTensor):
                 check_quantized_tensor(x, config, scaling_recipe=recipe)
@@ -72,6 +75,10 @@ class FP4GemmMXFunction(torch.autograd.Function):
                     x_t = QuantizedTensor.quantize(x.dequantize(), x.real_dtype, gran, axis=-2, block_size=bs,
                                                    scaling_recipe=recipe)
                 return x.qdata, x.scale_inv, x_t.qdata, x_t.scale_inv
+            if not need_bwd:
+                # the transposed copies only feed backward: skip them when nothing asks for a gradient
+                q, sc = quantize_mxfp4_impl(x, dt, x.dim() - 1, bs, scaling_recipe=recipe)
+                return q, sc, q, sc
             return quantize_fp4_with_trans(x, dt, gran, block_size=bs, scaling_recipe=recipe,
                                            scaling_recipe_for_trans=recipe)
 

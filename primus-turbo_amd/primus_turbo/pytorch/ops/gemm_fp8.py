@@ -154,8 +154,12 @@ class FP8GemmBlockFunction(torch.autograd.Function):
             if a_t is None:
                 a_t = QuantizedTensor.quantize(a.dequantize(), fdt, gran, axis=-2, block_size=bs)
             a_col, a_col_s = a_t.qdata, a_t.scale_inv
-        else:
+        elif any(ctx.needs_input_grad[:2]):
             a_row, a_row_s, a_col, a_col_s = quantize_fp8_with_trans(a, fdt, gran, block_size=bs)
+        else:
+            # the column-direction copy of `a` only feeds wgrad: skip it when nothing asks for a gradient
+            a_row, a_row_s = quantize_fp8(a, fdt, gran, axis=-1, block_size=bs)
+            a_col, a_col_s = a_row, a_row_s
         w_recipe = ScalingRecipe(use_2d_block=True)  # weight tiles serve forward and backward unchanged
         if isinstance(b, QuantizedTensor):
             check_quantized_tensor(b, config, scaling_recipe=w_recipe)
@@ -192,6 +196,8 @@ class FP8GemmMXFunction(torch.autograd.Function):
         fdt = _get_fp8_dtype(config.format, True)
         gran, bs = config.granularity, config.block_size
 
+        need_bwd = any(ctx.needs_input_grad[:2])
+
         def both_ways(x, x_t, recipe):
             if isinstance(x, QuantizedTensor):
                 check_quantized_tensor(x, config, axis=-1, scaling_recipe=recipe)
@@ -199,6 +205,10 @@ class FP8GemmMXFunction(torch.autograd.Function):
                     x_t = QuantizedTensor.quantize(x.dequantize(), x.real_dtype, gran, axis=-2, block_size=bs,
                                                    scaling_recipe=recipe)
                 return x.qdata, x.scale_inv, x_t.qdata, x_t.scale_inv
+            if not need_bwd:
+                # the transposed copies only feed backward: skip them when nothing asks for a gradient
+                q, sc = quantize_mxfp8_impl(x, fdt, x.dim() - 1, bs, scaling_recipe=recipe)
+                return q, sc, q, sc
             return quantize_mxfp8_impl(x, fdt, None, bs, with_trans=True, scaling_recipe=recipe,
                                        scaling_recipe_for_trans=recipe)
 
