@@ -11,15 +11,18 @@
 //
 // Kernel structure (this library's own):
 //   * one workgroup = 4 wavefronts in a 2 x 2 grid; each wavefront owns a
-//     (16 TM) x (16 TN) sub-tile built from v_mfma_f32_16x16x128_f8f6f4;
-//   * K advances 128 bytes per step; A and B tiles go HBM/L2 -> LDS directly
-//     (global_load_lds_dwordx4, no VGPR staging) into a double buffer, requested two steps
-//     ahead; the MFMA operand fragments of step k+1 are read from LDS into a second
-//     register set while the last MFMAs of step k run; one barrier per step;
+//     (16 TM) x (16 TN) sub-tile built from v_mfma_scale_f32_16x16x128_f8f6f4;
+//   * K advances 128 bytes per step ("slab"); A and B tiles go HBM/L2 -> LDS directly
+//     (buffer_load_dwordx4 ... lds, no VGPR staging) into two or three LDS stages; the MFMA
+//     operand fragments of a slab all live in registers and are refilled from the next slab's
+//     stage one by one as they die, so the copies of the slab after that can be spread over the
+//     whole slab; two barriers per slab (see the kernel);
 //   * LDS rows are 128 B; the 16-byte chunk c of row r sits at chunk c ^ ((r >> 1) & 7),
 //     which makes the 16 lanes of an MFMA operand read hit 16 different bank groups;
+//   * BLOCK and MX scales travel through the LDS stages with the slab they belong to;
 //   * the MFMA is issued with B as the "row" operand, so a lane ends up holding four
-//     consecutive n for one m and stores them without any exchange between lanes;
+//     consecutive n for one m; 16-bit outputs exchange 16-lane rows between neighbouring tiles
+//     so that a lane stores eight consecutive n;
 //   * workgroup ids are remapped so that the 8 XCDs (one L2 each) work on compact
 //     neighbourhoods of the tile grid.
 #pragma once
@@ -98,44 +101,15 @@ typedef const __attribute__((address_space(1))) void *glb_ptr_t;
 
 // Direct-to-LDS copies: each wave instruction moves 8 tile rows x 128 B = 1 KB to
 // contiguous LDS; lane l fills physical chunk l % 8 of row l / 8, reading the logical chunk
-// that the swizzle maps there. Rows at or beyond the matrix edge re-read the last valid
-// row (their products are never stored).
-
+// that the swizzle maps there. Rows at or beyond the end of the tile's share of the matrix
+// read as zero (buffer descriptor bounds); their products are never stored.
+//
 // MFMA operand fragment of 16 tile rows: lane (r = lane % 16, g = lane / 16) takes K bytes
 // [16g, 16g+16) and [64+16g, 64+16g+16) of row r, i.e. two 16-byte LDS reads. The swizzle
 // term of a row depends only on r (16 rows = 2 swizzle periods), so every fragment of a
-// wavefront's sub-tile uses the same two lane addresses plus an immediate offset.
-//
-// The reads are inline assembly on purpose: the compiler's wait-count pass has to assume
-// that an outstanding direct-to-LDS load may alias any LDS read it can see and would drain
-// the prefetch (vmcnt(0)) before every one of them. Completion is awaited explicitly with
-// frag_wait<N>() -- LDS returns data in order, so "at most N operations outstanding" means
-// everything but the N youngest reads has landed -- and a fragment must pass through
-// frag_ready() before its first use so that no consumer can be scheduled above the wait.
-struct Frag {
-    u32x4 lo, hi;
-};
-
-__device__ __forceinline__ uint32_t lds_addr(const void *p) {
-    return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((lds_ptr_t)p));
-}
-
-template <int OFF> __device__ __forceinline__ void frag_issue(Frag &f, uint32_t addr_lo, uint32_t addr_hi) {
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.lo) : "v"(addr_lo), "n"(OFF));
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.hi) : "v"(addr_hi), "n"(OFF));
-}
-
-template <int N> __device__ __forceinline__ void frag_wait() {
-    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
-}
-
-__device__ __forceinline__ i32x8 frag_ready(Frag &f) {
-    asm volatile("" : "+v"(f.lo), "+v"(f.hi));
-    i32x8 r;
-    r[0] = f.lo.x; r[1] = f.lo.y; r[2] = f.lo.z; r[3] = f.lo.w;
-    r[4] = f.hi.x; r[5] = f.hi.y; r[6] = f.hi.z; r[7] = f.hi.w;
-    return r;
-}
+// wavefront's sub-tile uses the same two lane addresses plus an immediate offset. The reads
+// are ordinary loads: with buffer-load copies the compiler's wait-count pass does not treat an
+// outstanding direct-to-LDS copy as aliasing them.
 
 template <int I, int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
     if constexpr (I < N) {
