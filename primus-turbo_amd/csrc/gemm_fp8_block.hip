@@ -11,7 +11,7 @@ template <bool SB_VEC, int FA, int FB>
 static int launch_block_tiles(const GemmArgs &a, int tile_cfg, hipStream_t stream) {
     // tile_cfg: 0 = auto, 1 = 256x256, 2 = 256x128, 3 = 128x128 (two workgroups per CU)
     if (tile_cfg == 0)
-        tile_cfg = 3;
+        tile_cfg = (a.M >= 2048 && a.N >= 1024) ? 2 : 3;
     if (tile_cfg == 3)
         return launch_gemm_cfg<4, 4, SCALE_BLOCK, SB_VEC, FA, FB>(a, stream);
     if (tile_cfg == 1)

@@ -17,7 +17,9 @@ template <int GMODE, bool SB_VEC, int FA, int FB>
 static int launch_grouped_tiles(const GemmArgs &a, int tile_cfg, hipStream_t stream) {
     // tile_cfg: 0 = auto, 1 / 2 = 256x128, 3 = 128x128 (two workgroups per CU)
     // (the 256x128 tile leaves LDS for the tile prefix sums of 1024 groups only)
-    if (tile_cfg == 0 || a.G > 1024)
+    if (tile_cfg == 0) // 256-row tiles once the average group fills a couple of them
+        tile_cfg = ((GMODE == GROUP_K ? a.M >= 1024 : (a.G > 0 && a.M / a.G >= 512)) && a.N >= 1024) ? 2 : 3;
+    if (a.G > 1024)
         tile_cfg = 3;
     if (tile_cfg == 3)
         return launch_gemm_cfg<4, 4, SCALE_BLOCK, SB_VEC, FA, FB, GMODE>(a, stream);

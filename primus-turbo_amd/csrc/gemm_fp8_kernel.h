@@ -436,9 +436,10 @@ __device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile, const 
 //     slab's stage as soon as it is dead: B fragment j after column j, A fragment i after
 //     tile (i, TN - 1). Every LDS read is thus issued at least TM MFMAs before its first use;
 //   * the stage of the slab being multiplied is therefore only read during the slab before,
-//     and is free to receive the slab NSTAGE steps ahead during all of the current one: the B
-//     part (and the block scales) while columns 1 .. TN/2 - 1 are multiplied, the A part
-//     during the rest;
+//     and receives the slab two steps ahead during the current one: the B part (and the block
+//     scales) while columns 1 .. TN/2 - 1 are multiplied, the A part during the rest. Where
+//     three stages fit, that slab goes into the stage freed one slab ago instead, and its
+//     copies are spread over all of the current slab's MFMAs;
 //   * two barriers per slab: "X" after column 0 (everyone has finished reading the current
 //     stage; everyone's copies of the next slab's B part have landed) and "Y" after column
 //     TN/2 - 1 (the next slab's A part has landed). Both wait for copies requested at least
@@ -514,21 +515,21 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     } else {
         total = a.tiles_m * a.tiles_n;
     }
-    const int KT_ALL = static_cast<int>(a.K / KSTEP); // XPIPE: every tile has this many slabs (> NSTAGE)
+    const int KT_ALL = static_cast<int>(a.K / KSTEP); // XPIPE: every tile has this many slabs (> 2)
     int       tile   = blockIdx.x;
-    if (tile >= total || (XPIPE && KT_ALL <= NSTAGE))
+    if (tile >= total || (XPIPE && KT_ALL <= 2))
         return;
     int     g_cur = 0, g_nxt = 0;
     TileCtx cur_t = make_tile<BM, BN, GMODE>(a, tile, prefix, g_cur);
     g_nxt         = g_cur;
 
-    // ---- loader: NSTAGE slabs ahead of the MFMAs ----
+    // ---- loader: two slabs ahead of the MFMAs ----
     // Copies are buffer loads: a lane's offset inside a slab (row * pitch + swizzled chunk)
     // is the same for every tile; the tile and the K position live in the (uniform) buffer
     // descriptor, whose size makes rows beyond the tile's share of the matrix read as zero.
     // The loader therefore changes tile by swapping scalars -- no branch in the K loop, which
     // the compiler would use to sink MFMAs -- and it does so after requesting the tile's last
-    // slab, NSTAGE steps before the MFMAs get there (the host guarantees KT > NSTAGE). Without
+    // slab, two steps before the MFMAs get there (the host guarantees KT > 2). Without
     // cross-tile pipelining it stops at the tile's last slab and keeps re-reading that one.
     uint32_t off[NL];
     {
@@ -707,15 +708,15 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     const uint32_t a_part = wm * (TM * 16) * KSTEP;
     const uint32_t b_part = A_BYTES + wn * (TN * 16) * KSTEP;
 
-    // pipeline start at tile t: NSTAGE slabs requested, the fragments of slab 0 on their way
+    // pipeline start at tile t: two slabs requested, the fragments of slab 0 on their way
     auto start_pipeline = [&](const TileCtx &t) {
         loader_to(t);
-        static_for<0, NSTAGE>([&](auto st) {
+        static_for<0, 2>([&](auto st) {
             static_for<0, NB>([&](auto c) { issue_part_b(c, st); });
             static_for<0, LA>([&](auto c) { issue_copy(c, st); });
             advance_loader();
         });
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NSTAGE - 1) * NL) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
         __builtin_amdgcn_s_barrier();
         buf = 0;
         read_scales(smem);
@@ -753,6 +754,9 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         for (int kt = 0; kt < KT; ++kt) {
             const int      buf_n = buf + 1 == NSTAGE ? 0 : buf + 1;
             const uint8_t *nxt   = smem + buf_n * STAGE;
+            // where the slab two steps ahead goes: the current stage (after barrier X), or with
+            // three stages the one that was current a slab ago
+            const int      buf_w = NSTAGE == 2 ? buf : (buf == 0 ? NSTAGE - 1 : buf - 1);
             if constexpr (MODE == SCALE_BLOCK) {
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
@@ -814,7 +818,16 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
 
             // MFMA slots of a slab: s = (j NH + h) TM + i. B-part copies are spread over the
             // slots of columns [1, JY), A-part copies over those of columns [JY, TN).
-            constexpr int COL = NH * TM, S_B0 = COL, S_B1 = JY * COL, S_A0 = JY * COL, S_A1 = TN * COL;
+            // (Three stages: both parts spread over all slots in proportion to their copy counts.)
+            constexpr int COL = NH * TM, SLOTS = TN * COL;
+            constexpr int S_B0 = NSTAGE == 2 ? COL : 0, S_B1 = NSTAGE == 2 ? JY * COL : SLOTS * NB / NL;
+            constexpr int S_A0 = S_B1, S_A1 = SLOTS;
+            // copies of this slab's schedule issued before slot s
+            constexpr auto issued_before = [](int s) {
+                const int b = s <= S_B0 ? 0 : (s >= S_B1 ? NB : (s - S_B0) * NB / (S_B1 - S_B0));
+                const int a = s <= S_A0 ? 0 : (s >= S_A1 ? LA : (s - S_A0) * LA / (S_A1 - S_A0));
+                return b + a;
+            };
             static_for<0, TN>([&](auto jc) {
                 constexpr int j = jc;
                 static_for<0, COL>([&](auto sc) {
@@ -825,10 +838,10 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                         fa[i] = ldfrag(nxt + a_part, i); // dead from here on: refill from the next slab
                     if constexpr (s >= S_B0 && s < S_B1)
                         static_for<(s - S_B0) * NB / (S_B1 - S_B0), (s + 1 - S_B0) * NB / (S_B1 - S_B0)>(
-                            [&](auto c) { issue_part_b(c, buf); });
+                            [&](auto c) { issue_part_b(c, buf_w); });
                     if constexpr (s >= S_A0 && s < S_A1)
                         static_for<(s - S_A0) * LA / (S_A1 - S_A0), (s + 1 - S_A0) * LA / (S_A1 - S_A0)>(
-                            [&](auto c) { issue_copy(c, buf); });
+                            [&](auto c) { issue_copy(c, buf_w); });
                     __builtin_amdgcn_sched_barrier(0);
                 });
                 if constexpr (j == 0) {
@@ -836,14 +849,14 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                     // my reads of the current stage are done (they were issued a column ago) and my
                     // copies of the next slab's B part have landed; younger copies may be in flight
                     PT_GEMM_TRACE_POINT(2);
-                    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LA + (NSTAGE - 2) * NL) : "memory");
+                    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LA + issued_before(COL)) : "memory");
                     __builtin_amdgcn_s_barrier();
                     PT_GEMM_TRACE_POINT(3);
                     read_scales(nxt);
                 }
                 if constexpr (j == JY - 1) {
                     // ---- barrier Y: the next slab's A part has landed ----
-                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NB + (NSTAGE - 2) * NL) : "memory");
+                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(issued_before(JY * COL)) : "memory");
                     __builtin_amdgcn_s_barrier();
                 }
                 fb[j] = ldfrag(nxt + b_part, j); // column j is done: refill from the next slab
