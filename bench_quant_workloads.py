@@ -1,0 +1,352 @@
+"""Quantizer workloads of bench.py: one per quantizer family of the hot path, at the operand shapes
+of the GEMM configurations they feed.
+
+A step quantizes (and, where the reference has the inverse op, de-quantizes) one tensor that is
+resident in HBM; ``value`` is algorithmic bytes per second: every input element read once, every
+output element written once, scales included. ``dominant()`` is the quantizer kernel alone. Every
+workload checks the bytes and scales of a slice against the CPU oracle, bit for bit, and times the
+reference's CPU formulas (torch for FP8, the numpy oracle for MX) on a bounded slice.
+"""
+
+from __future__ import annotations
+
+import os
+import time
+
+import numpy as np
+import torch
+
+HBM_PEAK_GBS = 8000.0
+
+
+def _randn_bf16(shape, seed, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g, dtype=torch.float32) * std).to(torch.bfloat16)
+
+
+def _u8(t):
+    return t.contiguous().view(torch.uint8).cpu().numpy()
+
+
+def _f32(t):
+    return t.float().cpu().numpy()
+
+
+class _QuantBase:
+    unit = "GB/s"
+    bound = "hbm"
+    dtype = "f32"
+    metric = "quantize GB/s (algorithmic bytes) & fraction of HBM peak"
+    graph_dominant = True  # kernels of tens of microseconds: time replays of a captured batch
+
+    def _cpu(self, fn, nbytes, what):
+        fn()
+        times = []
+        t_end = time.perf_counter() + 10.0
+        while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 20):
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+        med = sorted(times)[len(times) // 2]
+        return dict(value=round(nbytes / med / 1e9, 3), unit="GB/s", cores=torch.get_num_threads(), kind="port",
+                    sample=f"{what}, median of {len(times)} runs, {os.cpu_count()} logical CPUs visible")
+
+
+class QuantRowwise(_QuantBase):
+    """Rowwise FP8 quantize (last axis) + dequantize of an 8192 x 8192 bf16 GEMM operand."""
+
+    name = "fp8_e4m3_rowwise_quant_dequant_8192x8192_bf16 (axis -1)"
+    dominant_name = "quant_rowwise_inner_kernel (row parked in registers between amax and cast)"
+
+    def __init__(self, dev, M=8192, N=8192):
+        import primus_turbo.pytorch as turbo
+        from primus_turbo.pytorch.core.low_precision import ScalingGranularity as G
+
+        self.turbo, self.G, self.M, self.N = turbo, G, M, N
+        self.x_cpu = _randn_bf16((M, N), 11, 0.02)
+        self.x = self.x_cpu.to(dev)
+
+    def step_work(self):
+        return 6.0 * self.M * self.N + 8.0 * self.M
+
+    def dominant_work(self):
+        return 3.0 * self.M * self.N + 4.0 * self.M
+
+    def dominant(self):
+        return self.turbo.ops.quantize_fp8(self.x, self.turbo.float8_e4m3, self.G.ROWWISE, axis=-1)
+
+    def step(self):
+        q, s = self.dominant()
+        return self.turbo.ops.dequantize_fp8(q, torch.bfloat16, self.G.ROWWISE, axis=-1, scale_inv=s)
+
+    def check(self):
+        from oracle import quantize as Q
+
+        q, s = self.dominant()
+        y = self.turbo.ops.dequantize_fp8(q, torch.bfloat16, self.G.ROWWISE, axis=-1, scale_inv=s)
+        rows = np.r_[0:128, self.M - 128 : self.M]
+        oq, os_ = Q.fp8_rowwise(self.x_cpu.float().numpy()[rows], -1, "e4m3")
+        same = np.array_equal(_u8(q)[rows], oq) and np.array_equal(_f32(s)[rows].view(np.int32), os_.view(np.int32))
+        oy = torch.from_numpy(Q.fp8_dequant(oq, os_, "e4m3")).to(torch.bfloat16)
+        same = same and torch.equal(y.cpu()[rows], oy)
+        return bool(same), "256 rows: bytes, scale_inv and de-quantized bf16 bit-exact vs oracle"
+
+    def cpu_baseline(self):
+        from oracle import cpu_reference as R
+
+        def fn():
+            q, _, sinv = R.quantize_fp8_rowwise_ref(self.x_cpu, torch.float8_e4m3fn, axis=-1)
+            R.dequantize_fp8_ref(q, torch.bfloat16, sinv)
+
+        return self._cpu(fn, self.step_work(), "full 8192x8192 quantize + dequantize")
+
+
+class QuantBlockwise(_QuantBase):
+    """1x128 (and 128x1) blockwise FP8 quantize of a [16384, 7168] activation."""
+
+    def __init__(self, dev, dual=False, M=16384, N=7168):
+        from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+        self.qi, self.dual, self.M, self.N = qi, dual, M, N
+        self.name = f"fp8_e4m3_blockwise_{'1x128+128x1_dual' if dual else '1x128'}_quant_{M}x{N}_bf16"
+        self.dominant_name = "quant_block128_kernel (one 128x128 tile per workgroup, " + ("row and column blocks)" if dual else "row blocks)")
+        self.x_cpu = _randn_bf16((M, N), 12)
+        self.x = self.x_cpu.to(dev)
+
+    def step_work(self):
+        n = self.M * self.N
+        return (4.0 if self.dual else 3.0) * n + 4.0 * n / 128 * (2 if self.dual else 1)
+
+    dominant_work = step_work
+
+    def dominant(self):
+        if self.dual:
+            return self.qi.quant_fp8_blockwise_dual_impl(self.x, torch.float8_e4m3fn, 128)
+        return self.qi.quant_fp8_blockwise_impl(self.x, torch.float8_e4m3fn, -1, 128)
+
+    step = dominant
+
+    def check(self):
+        from oracle import quantize as Q
+
+        out = self.dominant()
+        x = self.x_cpu.float().numpy()[:256]
+        oq, os_ = Q.fp8_blockwise(x, 1, "e4m3", 128)
+        same = np.array_equal(_u8(out[0])[:256], oq) and np.array_equal(_f32(out[1])[:256].view(np.int32), os_.view(np.int32))
+        if self.dual:
+            cq, cs = Q.fp8_blockwise(x, 0, "e4m3", 128)
+            same = same and np.array_equal(_u8(out[2])[:256], cq) and np.array_equal(_f32(out[3])[:2].view(np.int32), cs.view(np.int32))
+        return bool(same), "first 256 rows: bytes and scale_inv bit-exact vs oracle"
+
+    def cpu_baseline(self):
+        from oracle import cpu_reference as R
+
+        rows = 4096
+        x = self.x_cpu[:rows]
+
+        def fn():
+            R.quantize_fp8_blockwise_ref(x, torch.float8_e4m3fn, 1, 128)
+            if self.dual:
+                R.quantize_fp8_blockwise_ref(x, torch.float8_e4m3fn, 128, 1)
+
+        return self._cpu(fn, self.step_work() * rows / self.M, f"first {rows} rows")
+
+
+class QuantBlockwiseWeight(_QuantBase):
+    """128x128-tile FP8 quantize of the expert weights [32, 4096, 7168]."""
+
+    name = "fp8_e4m3_blockwise_128x128_weight_quant_32x4096x7168_bf16"
+    dominant_name = "quant_block128_kernel (one 128x128 tile per workgroup, tile scale)"
+    graph_dominant = False
+
+    def __init__(self, dev, B=32, M=4096, N=7168):
+        from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+        self.qi, self.B, self.M, self.N = qi, B, M, N
+        self.w_cpu = _randn_bf16((B, M, N), 13)
+        self.w = self.w_cpu.to(dev)
+
+    def step_work(self):
+        n = self.B * self.M * self.N
+        return 3.0 * n + 4.0 * n / (128 * 128)
+
+    dominant_work = step_work
+
+    def dominant(self):
+        return self.qi.quant_fp8_blockwise_for_weight_impl(self.w, torch.float8_e4m3fn, 128)
+
+    step = dominant
+
+    def check(self):
+        from oracle import quantize as Q
+
+        q, s = self.dominant()
+        same = True
+        for b in (0, self.B - 1):
+            oq, os_ = Q.fp8_blockwise_weight(self.w_cpu[b].float().numpy(), "e4m3", 128)
+            same = same and np.array_equal(_u8(q[b]), oq) and np.array_equal(_f32(s[b]).view(np.int32), os_.view(np.int32))
+        return bool(same), "experts 0 and 31: bytes and scale_inv bit-exact vs oracle"
+
+    def cpu_baseline(self):
+        from oracle import cpu_reference as R
+
+        w = self.w_cpu[0]
+        return self._cpu(lambda: R.quantize_fp8_blockwise_ref(w, torch.float8_e4m3fn, 128, 128), self.step_work() / self.B,
+                         "one expert's weight of 32")
+
+
+class QuantGrouped(_QuantBase):
+    """Fused grouped row + column blockwise quantize of the routed tokens [32768, 7168], 32 experts."""
+
+    name = "fp8_e4m3_grouped_row+col_blockwise_quant_32768x7168_bf16_32experts_zipf1.2"
+    dominant_name = "quant_block128_kernel (grouped: row blocks + segment-padded column blocks from one read)"
+    graph_dominant = False
+
+    def __init__(self, dev, M=32768, N=7168, groups=32):
+        from bench_workloads import _zipf_group_lens
+        from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+        self.qi, self.M, self.N, self.groups = qi, M, N, groups
+        self.lens = _zipf_group_lens(groups, M, 7)
+        self.gl = torch.from_numpy(self.lens).to(dev)
+        self.offs = torch.ops.primus_turbo_cpp_extension.grouped_gemm_compute_offs(self.gl)
+        self.x_cpu = _randn_bf16((M, N), 14)
+        self.x = self.x_cpu.to(dev)
+
+    def step_work(self):
+        n = self.M * self.N
+        return 4.0 * n + 8.0 * n / 128
+
+    dominant_work = step_work
+
+    def dominant(self):
+        return self.qi.quant_fp8_blockwise_segment_m_row_col_impl(self.x, torch.float8_e4m3fn, 128, self.gl, self.offs, 4096)
+
+    step = dominant
+
+    def check(self):
+        """Experts that are small enough for the oracle to finish in seconds: all outputs of the
+        whole call would need the full tensor, so the oracle runs on the rows of the first three
+        non-empty experts re-based to a three-expert problem."""
+        from oracle import quantize as Q
+
+        qr, qc, sr, sc, plens, poffs = self.dominant()
+        live = [g for g in range(self.groups) if self.lens[g] > 0][:3]
+        offs = np.concatenate([[0], np.cumsum(self.lens)])
+        poff = poffs.cpu().numpy()
+        same = True
+        for g in live:
+            r0, r1 = int(offs[g]), int(offs[g + 1])
+            x = self.x_cpu[r0:r1].float().numpy()
+            o = Q.fp8_blockwise_segment_m_row_col(x, np.array([r1 - r0], dtype=np.int64), "e4m3", 128)
+            rows_p = o["written_rows"]
+            oqr, oqc, osr, osc = o["row"], o["col"][:rows_p], o["row_scale"], o["col_scale"][: rows_p // 128]
+            p0 = int(poff[g])
+            same = same and np.array_equal(_u8(qr[r0:r1]), oqr)
+            same = same and np.array_equal(_f32(sr[:, r0:r1]).view(np.int32), osr.view(np.int32))
+            same = same and np.array_equal(_u8(qc[p0 : p0 + rows_p]), oqc)
+            same = same and np.array_equal(_f32(sc[p0 // 128 : (p0 + rows_p) // 128]).view(np.int32), osc.view(np.int32))
+        return bool(same), f"experts {live}: row / column bytes and scales bit-exact vs oracle"
+
+    def cpu_baseline(self):
+        from oracle import cpu_reference as R
+
+        rows = 4096
+        x = self.x_cpu[:rows]
+
+        def fn():
+            R.quantize_fp8_blockwise_ref(x, torch.float8_e4m3fn, 1, 128)
+            R.quantize_fp8_blockwise_ref(x, torch.float8_e4m3fn, 128, 1)
+
+        return self._cpu(fn, self.step_work() * rows / self.M, f"row and column blocks of the first {rows} rows")
+
+
+class QuantMx(_QuantBase):
+    """MXFP8 / MXFP4 quantize (1x32 blocks, optionally also the transposed column direction) of a
+    16384 x 16384 bf16 operand, plus the de-quantizer of the row output."""
+
+    graph_dominant = False
+
+    def __init__(self, dev, fp4=False, dual=False, M=16384, N=16384):
+        from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+        self.qi, self.fp4, self.dual, self.M, self.N = qi, fp4, dual, M, N
+        kind = "mxfp4_e2m1" if fp4 else "mxfp8_e4m3"
+        self.fmt = "e2m1" if fp4 else "e4m3"
+        self.name = f"{kind}_{'row+col_dual' if dual else 'row'}_quant_{M}x{N}_bf16" + ("" if dual else " (+ dequantize)")
+        self.dominant_name = "mx_quant_kernel (128x128 tile through LDS, E8M0 exponent from the amax bits)"
+        self.qdt = torch.float4_e2m1fn_x2 if fp4 else torch.float8_e4m3fn
+        self._q = qi.quantize_mxfp4_impl if fp4 else qi.quantize_mxfp8_impl
+        self._dq = qi.dequantize_mxfp4_impl if fp4 else qi.dequantize_mxfp8_impl
+        self.x_cpu = _randn_bf16((M, N), 15)
+        self.x = self.x_cpu.to(dev)
+
+    def _qbytes(self):
+        code = 0.5 if self.fp4 else 1.0
+        n = self.M * self.N
+        return (2.0 + (2 if self.dual else 1) * (code + 1.0 / 32)) * n
+
+    def dominant_work(self):
+        return self._qbytes()
+
+    def step_work(self):
+        code = 0.5 if self.fp4 else 1.0
+        return self._qbytes() + (0.0 if self.dual else (code + 1.0 / 32 + 2.0) * self.M * self.N)
+
+    def dominant(self):
+        if self.dual:
+            return self._q(self.x, self.qdt, None, 32, with_trans=True)
+        return self._q(self.x, self.qdt, 1, 32)
+
+    def step(self):
+        out = self.dominant()
+        if self.dual:
+            return out
+        return self._dq(out[0], torch.bfloat16, 1, 32, out[1])
+
+    def check(self):
+        from oracle import quantize as Q
+
+        out = self.dominant()
+        x = self.x_cpu.float().numpy()[:128]
+        oq, os_ = Q.mx_quant_rowwise(x, self.fmt)
+        same = np.array_equal(_u8(out[0])[:128], oq) and np.array_equal(_u8(out[1])[:128], os_)
+        what = "first 128 rows: codes and E8M0 bytes bit-exact vs oracle"
+        if self.dual:
+            cq, cs = Q.mx_quant_colwise(x, self.fmt)
+            cb = 64 if self.fp4 else 128  # code bytes of the first 128 rows in a transposed row
+            same = same and np.array_equal(_u8(out[2])[:, :cb], cq[:, :cb]) and np.array_equal(_u8(out[3])[:, :4], cs[:, :4])
+            what += " (row and transposed column outputs)"
+        else:
+            y = self._dq(out[0], torch.bfloat16, 1, 32, out[1])
+            oy = torch.from_numpy(Q.mx_dequant(oq, os_, self.fmt)[:, : self.N].astype(np.float32)).to(torch.bfloat16)
+            same = same and torch.equal(y.cpu()[:128], oy)
+            what += "; de-quantized bf16 bit-exact"
+        return bool(same), what
+
+    def cpu_baseline(self):
+        from oracle import quantize as Q
+
+        rows = 512
+        x = self.x_cpu[:rows].float().numpy()
+
+        def fn():
+            q, s = Q.mx_quant_rowwise(x, self.fmt)
+            if self.dual:
+                Q.mx_quant_colwise(x, self.fmt)
+            else:
+                Q.mx_dequant(q, s, self.fmt)
+
+        return self._cpu(fn, self.step_work() * rows / self.M, f"numpy oracle on the first {rows} rows")
+
+
+def register(workloads):
+    workloads["quant_rowwise"] = QuantRowwise
+    workloads["quant_blockwise"] = lambda dev: QuantBlockwise(dev, False)
+    workloads["quant_blockwise_dual"] = lambda dev: QuantBlockwise(dev, True)
+    workloads["quant_blockwise_weight"] = QuantBlockwiseWeight
+    workloads["quant_grouped"] = QuantGrouped
+    workloads["quant_mxfp8"] = lambda dev: QuantMx(dev, False, False)
+    workloads["quant_mxfp8_dual"] = lambda dev: QuantMx(dev, False, True)
+    workloads["quant_mxfp4"] = lambda dev: QuantMx(dev, True, False)
+    workloads["quant_mxfp4_dual"] = lambda dev: QuantMx(dev, True, True)
