@@ -290,6 +290,13 @@ template <typename T> static void launch_mx_fmt(const MxArgs &a, int fmt, bool r
 //   -> y [rows, cols], or y [cols, rows] when `transpose` (column-direction data)
 // One workgroup per 64 x 64 tile through LDS so that both layouts store whole lines.
 // ---------------------------------------------------------------------------
+__device__ __forceinline__ float e2m1_to_f32(uint32_t nib) {
+    // E2M1: 1 sign, 2 exponent, 1 mantissa bits: {0, .5, 1, 1.5, 2, 3, 4, 6}
+    const uint32_t mag = nib & 7u;
+    const float    f   = mag < 2 ? 0.5f * mag : __uint_as_float(((126u + (mag >> 1)) << 23) | ((mag & 1u) << 22));
+    return nib & 8u ? -f : f;
+}
+
 template <typename T, int FMT>
 __global__ __launch_bounds__(256) void mx_dequant_kernel(const uint8_t *__restrict__ q, const uint8_t *__restrict__ s,
                                                          T *__restrict__ y, const int64_t rows, const int64_t cols,
@@ -308,11 +315,7 @@ __global__ __launch_bounds__(256) void mx_dequant_kernel(const uint8_t *__restri
                 const uint16_t w = *reinterpret_cast<const uint16_t *>(q + gr * (cols >> 1) + (gc >> 1));
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    const uint32_t nib = (w >> (4 * k)) & 0xFu;
-                    // E2M1: 1 sign, 2 exponent, 1 mantissa bits: {0, .5, 1, 1.5, 2, 3, 4, 6}
-                    const uint32_t mag = nib & 7u;
-                    const float    f   = mag < 2 ? 0.5f * mag : __uint_as_float(((126u + (mag >> 1)) << 23) | ((mag & 1u) << 22));
-                    v[k]               = (nib & 8u ? -f : f) * sc;
+                    v[k] = e2m1_to_f32((w >> (4 * k)) & 0xFu) * sc;
                 }
             } else {
                 const uint32_t w = *reinterpret_cast<const uint32_t *>(q + gr * cols + gc);
@@ -344,16 +347,74 @@ __global__ __launch_bounds__(256) void mx_dequant_kernel(const uint8_t *__restri
     }
 }
 
+// Row-direction data with 16-byte aligned pointers: a plain stream. A thread takes 16 consecutive
+// elements of a row (half a 32-element block, one scale byte): 16 (FP4: 8) code bytes in, 32 or
+// 64 bytes out, whole lines per wavefront on both sides.
+template <typename T, int FMT>
+__global__ __launch_bounds__(256) void mx_dequant_stream_kernel(const uint8_t *__restrict__ q, const uint8_t *__restrict__ s,
+                                                                T *__restrict__ y, const int64_t rows, const int64_t cols) {
+    const int64_t per_row = cols >> 4, units = rows * per_row;
+    const int64_t stride  = static_cast<int64_t>(gridDim.x) * 256;
+    for (int64_t u = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; u < units; u += stride) {
+        const int64_t r = u / per_row, c = u - r * per_row;
+        const float   sc = __uint_as_float(static_cast<uint32_t>(s[r * (cols >> 5) + (c >> 1)]) << 23);
+        float         f[16];
+        if constexpr (FMT == MX_E2M1) {
+            const u32x2    w     = *reinterpret_cast<const u32x2 *>(q + (u << 3));
+            const uint32_t ww[2] = {w.x, w.y};
+#pragma unroll
+            for (int k = 0; k < 16; ++k)
+                f[k] = e2m1_to_f32(ww[k >> 3] >> (4 * (k & 7))) * sc;
+        } else {
+            const u32x4    w     = ld128(q + (u << 4));
+            const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                f[4 * k + 0] = fp8_to_f32<FMT == MX_E5M2>(ww[k], 0) * sc;
+                f[4 * k + 1] = fp8_to_f32<FMT == MX_E5M2>(ww[k], 1) * sc;
+                f[4 * k + 2] = fp8_to_f32<FMT == MX_E5M2>(ww[k], 2) * sc;
+                f[4 * k + 3] = fp8_to_f32<FMT == MX_E5M2>(ww[k], 3) * sc;
+            }
+        }
+        char *dst = reinterpret_cast<char *>(y + (u << 4));
+        if constexpr (sizeof(T) == 4) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                st128(dst + 16 * k, u32x4{__float_as_uint(f[4 * k]), __float_as_uint(f[4 * k + 1]),
+                                          __float_as_uint(f[4 * k + 2]), __float_as_uint(f[4 * k + 3])});
+        } else {
+#pragma unroll
+            for (int k = 0; k < 2; ++k)
+                st128(dst + 16 * k, u32x4{pack2<T>(f[8 * k], f[8 * k + 1]), pack2<T>(f[8 * k + 2], f[8 * k + 3]),
+                                          pack2<T>(f[8 * k + 4], f[8 * k + 5]), pack2<T>(f[8 * k + 6], f[8 * k + 7])});
+        }
+    }
+}
+
+template <typename T, int FMT>
+static void launch_mx_dequant_t(const uint8_t *q, const uint8_t *s, T *y, int64_t rows, int64_t cols, int transpose,
+                                hipStream_t st) {
+    if (!transpose && aligned_to(q, 16) && aligned_to(y, 16)) {
+        const int64_t units = rows * (cols >> 4);
+        int64_t       grid  = cdiv(units, 256);
+        const int64_t cap   = 32L * device_cu_count();
+        grid                = grid > cap ? cap : grid;
+        mx_dequant_stream_kernel<T, FMT><<<static_cast<unsigned>(grid), 256, 0, st>>>(q, s, y, rows, cols);
+        return;
+    }
+    dim3 grid(static_cast<unsigned>(cdiv(cols, 64)), static_cast<unsigned>(cdiv(rows, 64)));
+    mx_dequant_kernel<T, FMT><<<grid, 256, 0, st>>>(q, s, y, rows, cols, transpose);
+}
+
 template <int FMT>
 static void launch_mx_dequant(const uint8_t *q, const uint8_t *s, void *y, int ydtype, int64_t rows, int64_t cols,
                               int transpose, hipStream_t st) {
-    dim3 grid(static_cast<unsigned>(cdiv(cols, 64)), static_cast<unsigned>(cdiv(rows, 64)));
     if (ydtype == PT_DTYPE_BF16)
-        mx_dequant_kernel<bf16_t, FMT><<<grid, 256, 0, st>>>(q, s, static_cast<bf16_t *>(y), rows, cols, transpose);
+        launch_mx_dequant_t<bf16_t, FMT>(q, s, static_cast<bf16_t *>(y), rows, cols, transpose, st);
     else if (ydtype == PT_DTYPE_F16)
-        mx_dequant_kernel<f16_t, FMT><<<grid, 256, 0, st>>>(q, s, static_cast<f16_t *>(y), rows, cols, transpose);
+        launch_mx_dequant_t<f16_t, FMT>(q, s, static_cast<f16_t *>(y), rows, cols, transpose, st);
     else
-        mx_dequant_kernel<float, FMT><<<grid, 256, 0, st>>>(q, s, static_cast<float *>(y), rows, cols, transpose);
+        launch_mx_dequant_t<float, FMT>(q, s, static_cast<float *>(y), rows, cols, transpose, st);
 }
 
 static int mx_fmt_of(int dtype) {
