@@ -40,21 +40,57 @@ struct BlockQuantArgs {
     float          qmax;
 };
 
-template <typename T> __device__ __forceinline__ void load8(const T *p, float (&f)[8]) {
-    if constexpr (sizeof(T) == 4) {
-        const u32x4 a = ld128(p), b = ld128(p + 4);
-        f[0] = __uint_as_float(a.x); f[1] = __uint_as_float(a.y);
-        f[2] = __uint_as_float(a.z); f[3] = __uint_as_float(a.w);
-        f[4] = __uint_as_float(b.x); f[5] = __uint_as_float(b.y);
-        f[6] = __uint_as_float(b.z); f[7] = __uint_as_float(b.w);
-    } else {
+// Eight consecutive elements of a tile row as they come from memory (16-bit inputs stay packed:
+// four registers instead of eight between the phases of the kernel).
+template <typename T> struct Held8 {
+    static constexpr int WORDS = sizeof(T) == 4 ? 8 : 4;
+    uint32_t             w[WORDS];
+    __device__ __forceinline__ void load(const T *p) {
         const u32x4 a = ld128(p);
-        unpack2<T>(a.x, f[0], f[1]);
-        unpack2<T>(a.y, f[2], f[3]);
-        unpack2<T>(a.z, f[4], f[5]);
-        unpack2<T>(a.w, f[6], f[7]);
+        w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w;
+        if constexpr (sizeof(T) == 4) {
+            const u32x4 b = ld128(p + 4);
+            w[4] = b.x; w[5] = b.y; w[6] = b.z; w[7] = b.w;
+        }
     }
-}
+    // element by element, zeros where `ok` says so (tile edges, rows of other groups)
+    template <typename OK> __device__ __forceinline__ void load_checked(const T *p, OK ok) {
+        uint32_t e[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            e[i] = 0;
+            if (ok(i)) {
+                if constexpr (sizeof(T) == 4) {
+                    e[i] = __float_as_uint(p[i]);
+                } else {
+                    uint16_t b;
+                    __builtin_memcpy(&b, p + i, 2);
+                    e[i] = b;
+                }
+            }
+        }
+        if constexpr (sizeof(T) == 4) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                w[i] = e[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                w[i] = e[2 * i] | (e[2 * i + 1] << 16);
+        }
+    }
+    __device__ __forceinline__ void get(float (&f)[8]) const {
+        if constexpr (sizeof(T) == 4) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                f[i] = __uint_as_float(w[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                unpack2<T>(w[i], f[2 * i], f[2 * i + 1]);
+        }
+    }
+};
 
 template <bool E5M2>
 __device__ __forceinline__ u32x2 quant8(const float (&f)[8], const float (&s)[8], float qmax) {
@@ -111,7 +147,18 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
     const int64_t gn   = tn * BQ + cseg * BQ_PACK;
     const bool    full = VEC8 && (gn + BQ_PACK <= N);
 
-    float vals[BQ_ROUNDS][BQ_PACK];
+    // phase 1: the whole tile share of this thread is requested before anything is used
+    Held8<T> held[BQ_ROUNDS];
+#pragma unroll
+    for (int r = 0; r < BQ_ROUNDS; ++r) {
+        const int64_t in_m  = in_m0 + rslot + 16 * r;
+        const bool    valid = in_m < in_end;
+        if (valid && full)
+            held[r].load(x + in_m * N + gn);
+        else
+            held[r].load_checked(x + in_m * N + gn, [&](int i) { return valid && gn + i < N; });
+    }
+
     float col_amax[BQ_PACK];
     float tile_amax = 0.f;
 #pragma unroll
@@ -123,17 +170,12 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
         const int     lm    = rslot + 16 * r;
         const int64_t in_m  = in_m0 + lm;
         const bool    valid = in_m < in_end;
-        if (valid && full) {
-            load8<T>(x + in_m * N + gn, vals[r]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < BQ_PACK; ++i)
-                vals[r][i] = (valid && gn + i < N) ? HP<T>::to_f32(x[in_m * N + gn + i]) : 0.f;
-        }
+        float         vals[BQ_PACK];
+        held[r].get(vals);
         float amax = 0.f;
 #pragma unroll
         for (int i = 0; i < BQ_PACK; ++i) {
-            const float av = fabsf(vals[r][i]);
+            const float av = fabsf(vals[i]);
             amax           = fmaxf(amax, av);
             if constexpr (MODE & MODE_COL)
                 col_amax[i] = fmaxf(col_amax[i], av);
@@ -145,7 +187,7 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
             const float scale = qmax / fmaxf(amax, BQ_EPS);
             if (valid) {
                 const float s[8] = {scale, scale, scale, scale, scale, scale, scale, scale};
-                store8(a.q_row + batch * M * N + in_m * N + gn, quant8<E5M2>(vals[r], s, qmax),
+                store8(a.q_row + batch * M * N + in_m * N + gn, quant8<E5M2>(vals, s, qmax),
                        full, gn, N);
                 if (cseg == 0)
                     a.s_row[in_m * a.rs_m + tn * a.rs_n] = 1.0f / scale;
@@ -163,9 +205,11 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
 #pragma unroll
         for (int r = 0; r < BQ_ROUNDS; ++r) {
             const int64_t in_m = in_m0 + rslot + 16 * r;
-            if (in_m < in_end)
-                store8(a.q_row + batch * M * N + in_m * N + gn, quant8<E5M2>(vals[r], s, qmax),
-                       full, gn, N);
+            if (in_m < in_end) {
+                float vals[BQ_PACK];
+                held[r].get(vals);
+                store8(a.q_row + batch * M * N + in_m * N + gn, quant8<E5M2>(vals, s, qmax), full, gn, N);
+            }
         }
     }
 
@@ -195,8 +239,11 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
 #pragma unroll
         for (int r = 0; r < BQ_ROUNDS; ++r) {
             const int64_t out_m = tm * BQ + rslot + 16 * r;
-            if (out_m < M_out) // grouped: pad rows carry zeros -> code 0
-                store8(a.q_col + out_m * N + gn, quant8<E5M2>(vals[r], s, qmax), full, gn, N);
+            if (out_m < M_out) { // grouped: pad rows carry zeros -> code 0
+                float vals[BQ_PACK];
+                held[r].get(vals);
+                store8(a.q_col + out_m * N + gn, quant8<E5M2>(vals, s, qmax), full, gn, N);
+            }
         }
     }
 }
