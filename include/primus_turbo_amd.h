@@ -306,6 +306,54 @@ PT_API int pt_grouped_gemm_fp8_variable_k(const void *lhs, int lhs_dtype, const 
                                           int accumulate, void *workspace, size_t workspace_bytes,
                                           int tile_cfg, void *stream);
 
+/* Grouped MXFP8 path (MoE experts with E8M0 block scales) ------------------------------
+ *
+ * pt_grouped_quantize_mx replaces the dispatcher ops grouped_quantize_mxfp8 /
+ * grouped_quantize_mxfp8_dual (csrc/pytorch/quantization/quantization.cpp:971-1378; Python
+ * quantization_impl.py:572-700, FlyDSL mxfp8_quant_flydsl.py:982-1045) for round-to-nearest-even
+ * without output shuffling: x [M, N] bf16 / fp16 holds the rows of G groups (group_offs, device
+ * int64 [G + 1]); numerics per 32-element block as pt_quantize_mx.
+ *   Row direction: row_q [*, Npad] codes and row_scale [*, Npad / 32] with the rows of group g
+ *   at row_offs_padded[g] (every group padded to a multiple of 32 rows; pad rows are not
+ *   written); row_offs_padded == NULL keeps the rows where they are in x.
+ *   Column direction, emitted transposed: col_q [N, col_ld], col_scale [N, col_ld / 32] with
+ *   the rows of group g at columns col_offs_padded[g] ... (every group padded to a multiple of
+ *   128 rows with zero data, scale byte 0); col_ld is a multiple of 128 >= col_offs_padded[G];
+ *   columns from col_offs_padded[G] on are not written.
+ * Either pair may be NULL. The padded offsets come from pt_compute_group_offs (align 32 / 128).
+ *
+ * pt_grouped_gemm_mx replaces primus_turbo::grouped_gemm_fp8_impl for MX_BLOCKWISE
+ * (kernels/grouped_gemm/grouped_gemm_fp8_impl.py:888-930 with group_offs_out; caller
+ * ops/grouped_gemm_fp8.py:726-741,786-801), forward and dgrad:
+ *   out[oo[g] : oo[g] + len_g, :] = A[o[g] : o[g] + len_g, :] . B[g]^T,   out[oo[G] : out_rows] = 0
+ * A [a_rows, K] MXFP8 codes with scale bytes [a_rows, sa_ld], B [G, N, K] with [G, N, sb_ld];
+ * o = group_offs (rows of A, e.g. the padded row layout above), oo = group_offs_out (rows of the
+ * output, packed tight; NULL = the same as o); len_g = oo[g + 1] - oo[g] when oo is given.
+ * K is a multiple of 128 and at least 512.
+ *
+ * pt_grouped_gemm_mx_variable_k replaces primus_turbo::grouped_gemm_fp8_variable_k_impl for
+ * MX_BLOCKWISE (grouped_gemm_fp8_impl.py:933-974; caller ops/grouped_gemm_fp8.py:809-825), wgrad:
+ *   C[g] (+)= L[:, p[g] : p[g+1]] . R[:, p[g] : p[g+1]]^T      C is [G, Ml, Nr]
+ * L [Ml, ld] and R [Nr, ld] are transposed column-direction outputs of pt_grouped_quantize_mx
+ * with scale bytes [rows, ld / 32]; p = the 128-padded group offsets. An empty group yields
+ * C[g] = 0 (or leaves it unchanged when accumulating). No workspace: both operands are read in
+ * place. */
+PT_API int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype,
+                                  const int64_t *group_offs, const int64_t *row_offs_padded,
+                                  const int64_t *col_offs_padded, int64_t G, void *row_q,
+                                  void *row_scale, void *col_q, void *col_scale, int64_t col_ld,
+                                  void *stream);
+PT_API int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, int64_t sa_ld,
+                              const void *b, int b_dtype, const void *b_scale, int64_t sb_ld, void *c,
+                              int c_dtype, const int64_t *group_offs, const int64_t *group_offs_out,
+                              int64_t G, int64_t a_rows, int64_t out_rows, int64_t N, int64_t K,
+                              int tile_cfg, void *stream);
+PT_API int pt_grouped_gemm_mx_variable_k(const void *lhs, int lhs_dtype, const void *lhs_scale,
+                                         const void *rhs, int rhs_dtype, const void *rhs_scale, void *c,
+                                         int c_dtype, const int64_t *group_offs, int64_t G, int64_t Ml,
+                                         int64_t Nr, int64_t ld, int accumulate, int tile_cfg,
+                                         void *stream);
+
 /* Byte-matrix transpose out[b, c, r] = in[b, r, c] (fp8 payloads; replaces the 2-D
  * transpose used for tensorwise `.t()` copies, csrc/kernels/transpose/). */
 PT_API int pt_transpose_u8(const void *in, void *out, int64_t batch, int64_t R, int64_t C,

@@ -33,6 +33,11 @@ What each function follows, and what pins it (tests/test_oracle_*.py):
   brute force over every bf16 amax, the saturation invariant, 2-D blocks constant
   over 32x32 tiles, round trips through the de-quantizer. Random Hadamard transform
   and stochastic rounding recipes are not restated (unpinned, not implemented).
+* ``mx_grouped_quant`` — per-group composition of the two above in the padded layouts of
+  /root/reference/csrc/pytorch/quantization/quantization.cpp:971-1100 (rows of a group padded
+  to 32 / 128 with zero data); pinned by the group-by-group round trip against the dense
+  quantizer and by the zero-pad invariants (same PARITY UNPINNED remark for bit-identity
+  with the reference's own kernels).
 """
 
 from __future__ import annotations
@@ -331,6 +336,51 @@ def mx_quant_colwise(x: np.ndarray, fmt, use_2d_block: bool = False, pad: int = 
     codes [K, M_pad] (FP4 packed [K, M_pad/2]) and bytes [K, M_pad/32]."""
     x = np.asarray(x, dtype=F32)
     return mx_quant_rowwise(np.ascontiguousarray(x.T), fmt, use_2d_block, pad)
+
+
+def mx_grouped_quant(x: np.ndarray, group_lens: np.ndarray, fmt, row_align: int = 32, col_align: int = 128):
+    """Grouped MX quantizer of a packed-M activation ``x [M, N]`` (layout rules of
+    /root/reference/csrc/pytorch/quantization/quantization.cpp:971-1100 and
+    /root/reference/primus_turbo/pytorch/kernels/quantization/quantization_impl.py:572-700:
+    every group is virtually zero-padded along M, to ``row_align`` rows for the row direction
+    and to ``col_align`` rows for the column direction; per-block numerics are those of the
+    dense MX quantizer). Composition of ``mx_quant_rowwise`` / ``mx_quant_colwise`` per group
+    (pinned there); the padded placement is pinned by the round trip through ``mx_dequant``
+    against the dense quantizer of each group.
+
+    Returns a dict with
+      row [Mr, N_pad] codes, row_scale [Mr, N_pad/32]     group g at rows row_offs[g] ...,
+                                                          Mr = row_offs[G]; pad rows zero
+      col [N, Mc] codes, col_scale [N, Mc/32]             transposed; group g at columns
+                                                          col_offs[g] ..., Mc = col_offs[G]
+      row_lens / row_offs, col_lens / col_offs            int64 padded lengths and offsets
+    (FP4: code arrays packed two per byte along their last axis)."""
+    fmt = _fmt(fmt)
+    x = np.asarray(x, dtype=F32)
+    M, N = x.shape
+    gl = np.asarray(group_lens, dtype=np.int64)
+    offs = group_offs(gl)
+    rl, ro = padded_group_offs(gl, row_align)
+    cl, co = padded_group_offs(gl, col_align)
+    n_pad = _cdiv(N, 128) * 128
+    cpb = 2 if fmt is E2M1 else 1  # codes per byte
+    row = np.zeros((int(ro[-1]), n_pad // cpb), dtype=np.uint8)
+    row_scale = np.zeros((int(ro[-1]), n_pad // 32), dtype=np.uint8)
+    col = np.zeros((N, int(co[-1]) // cpb), dtype=np.uint8)
+    col_scale = np.zeros((N, int(co[-1]) // 32), dtype=np.uint8)
+    for g in range(len(gl)):
+        n = int(gl[g])
+        if n == 0:
+            continue
+        seg = x[offs[g] : offs[g] + n]
+        q, sc = mx_quant_rowwise(seg, fmt)
+        row[ro[g] : ro[g] + n] = q
+        row_scale[ro[g] : ro[g] + n] = sc
+        q, sc = mx_quant_colwise(seg, fmt, pad=col_align)
+        col[:, co[g] // cpb : co[g + 1] // cpb] = q
+        col_scale[:, co[g] // 32 : co[g + 1] // 32] = sc
+    return dict(row=row, row_scale=row_scale, col=col, col_scale=col_scale, row_lens=rl, row_offs=ro, col_lens=cl,
+                col_offs=co)
 
 
 def mx_dequant(codes: np.ndarray, scale_bytes: np.ndarray, fmt) -> np.ndarray:

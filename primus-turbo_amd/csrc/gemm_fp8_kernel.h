@@ -68,6 +68,9 @@ struct GemmArgs {
     int            gmode;
     int            G;
     const int64_t *group_offs;
+    // GROUP_ROWS only, optional: row offsets of the groups in C when they differ from those in A
+    // (A in a per-group padded layout, C packed tight); NULL = the same offsets
+    const int64_t *group_offs_out;
     int64_t        b_gstride;  // bytes
     int64_t        sb_gstride; // floats
     int64_t        c_gstride;  // elements
@@ -392,7 +395,10 @@ __device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile, const 
         while (g + 1 < a.G && tile >= __builtin_amdgcn_readfirstlane(prefix[g + 1]))
             ++g;
         const int     local = tile - __builtin_amdgcn_readfirstlane(prefix[g]);
-        const int64_t lo = a.group_offs[g], hi = a.group_offs[g + 1];
+        const int64_t lo = a.group_offs[g];
+        // with separate output offsets the group's row count is theirs (A may be padded per group)
+        const int64_t hi = a.group_offs_out != nullptr ? lo + (a.group_offs_out[g + 1] - a.group_offs_out[g])
+                                                       : a.group_offs[g + 1];
         const int     gtm = static_cast<int>((hi - lo + BM - 1) / BM);
         tile_coords_local(local, gtm, a.tiles_n, tm, tn);
         t.m0    = lo + static_cast<int64_t>(tm) * BM;
@@ -402,6 +408,8 @@ __device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile, const 
         t.sA    = a.sA;
         t.sB    = a.sB + g * a.sb_gstride;
         t.C     = static_cast<uint8_t *>(a.C);
+        if (a.group_offs_out != nullptr) // the tile's rows keep their A numbering; C moves instead
+            t.C += (a.group_offs_out[g] - lo) * a.N * (a.out_dtype == PT_DTYPE_F32 ? 4 : 2);
         t.KT    = static_cast<int>(a.K / KSTEP);
     } else {
         const int per = a.tiles_m * a.tiles_n;
@@ -496,7 +504,8 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     int  total;
     if constexpr (GMODE == GROUP_ROWS) {
         for (int g = tid; g < a.G; g += 256) {
-            const int64_t rows = a.group_offs[g + 1] - a.group_offs[g];
+            const int64_t *o   = a.group_offs_out != nullptr ? a.group_offs_out : a.group_offs;
+            const int64_t rows = o[g + 1] - o[g];
             prefix[g + 1]      = static_cast<int>((rows + BM - 1) / BM) * a.tiles_n;
         }
         __syncthreads();

@@ -83,6 +83,15 @@ struct MxArgs {
     uint8_t    *row_s; // [B, M, Npad / 32] or NULL
     uint8_t    *col_q; // [B, N, Mpad] (FP4: Mpad / 2) or NULL
     uint8_t    *col_s; // [B, N, Mpad / 32] or NULL
+    // Grouped mode (B = 1, group_offs != NULL): the rows of x belong to G groups; the tile grid
+    // runs over the row space in which every group is padded to a multiple of 128 rows
+    // (col_offs_pad, Mpad = its allocated extent): the column-direction output lives there, pad
+    // rows are zero data. The row-direction output puts the rows of group g at row_offs_pad[g]
+    // (NULL: at their place in x); its pad rows are not written.
+    const int64_t *group_offs;   // [G + 1]
+    const int64_t *row_offs_pad; // [G + 1] or NULL
+    const int64_t *col_offs_pad; // [G + 1]
+    int            G;
 };
 
 // fabsf(x) with NaN mapped to 0 (fmaxf-style abs-max ignores NaN)
@@ -101,15 +110,32 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
     const int64_t n0 = static_cast<int64_t>(blockIdx.x) * MX_TILE, m0 = static_cast<int64_t>(blockIdx.y) * MX_TILE;
     const int64_t b  = blockIdx.z;
     const uint16_t *x = static_cast<const uint16_t *>(a.x) + b * a.M * a.N;
+    // tile row r holds input row in_m0 + r (while below in_end) and goes to row row_dst0 + r of
+    // the row-direction output (while r < row_cnt: in the padded layout that includes the zero
+    // rows that round the group up to a multiple of 32)
+    int64_t in_m0 = m0, in_end = a.M, row_dst0 = b * a.M + m0, row_cnt = a.M - m0;
+    if (a.group_offs != nullptr) {
+        if (m0 >= a.col_offs_pad[a.G])
+            return;
+        int g = 0;
+        for (int i = 0; i < a.G; ++i)
+            if (m0 >= a.col_offs_pad[i] && m0 < a.col_offs_pad[i + 1])
+                g = i;
+        in_m0    = a.group_offs[g] + (m0 - a.col_offs_pad[g]);
+        in_end   = a.group_offs[g + 1];
+        const int64_t done = in_m0 - a.group_offs[g]; // rows of the group in earlier tiles
+        row_dst0 = a.row_offs_pad != nullptr ? a.row_offs_pad[g] + done : in_m0;
+        row_cnt  = (a.row_offs_pad != nullptr ? a.row_offs_pad[g + 1] - a.row_offs_pad[g] : in_end - a.group_offs[g]) - done;
+    }
 
     // ---- tile -> LDS (zeros outside the matrix) ----
     const bool vec = (a.N & 7) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
 #pragma unroll
     for (int p = 0; p < 8; ++p) {
         const int     r = p * 16 + (tid >> 4), c = (tid & 15) * 8;
-        const int64_t m = m0 + r, n = n0 + c;
+        const int64_t m = in_m0 + r, n = n0 + c;
         u32x4         v = u32x4{0u, 0u, 0u, 0u};
-        if (m < a.M && n < a.N) {
+        if (m < in_end && n < a.N) {
             if (vec) {
                 v = ld128(x + m * a.N + n);
             } else {
@@ -162,7 +188,6 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
             const int     t = tid + 256 * p, r = t >> 2, c = t & 3;
-            const int64_t m = m0 + r;
             float         am = ram[p];
             if constexpr (ROW2D) {
                 const int rb = r & ~31;
@@ -175,13 +200,13 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
             uint32_t  code[8];
             mx_encode32<FMT>(rv[p], mx_inv_scale(e), code);
             sbytes[r * 4 + c] = static_cast<uint8_t>(e + 127);
-            if (m < a.M) {
+            if (r < row_cnt) {
                 const int64_t nb = (n0 >> 5) + c; // 32-column block index in the padded row
                 if constexpr (FMT == MX_E2M1) {
-                    uint8_t *q = a.row_q + (b * a.M + m) * (a.Npad >> 1) + nb * 16;
+                    uint8_t *q = a.row_q + (row_dst0 + r) * (a.Npad >> 1) + nb * 16;
                     st128(q, u32x4{code[0], code[1], code[2], code[3]});
                 } else {
-                    uint8_t *q = a.row_q + (b * a.M + m) * a.Npad + nb * 32;
+                    uint8_t *q = a.row_q + (row_dst0 + r) * a.Npad + nb * 32;
                     st128(q, u32x4{code[0], code[1], code[2], code[3]});
                     st128(q + 16, u32x4{code[4], code[5], code[6], code[7]});
                 }
@@ -189,8 +214,8 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
         }
         __syncthreads();
         // the four scale bytes of a tile row leave as one word (Npad / 32 is a multiple of 4)
-        if (tid < MX_TILE && m0 + tid < a.M)
-            *reinterpret_cast<uint32_t *>(a.row_s + (b * a.M + m0 + tid) * (a.Npad >> 5) + (n0 >> 5)) =
+        if (tid < MX_TILE && tid < row_cnt)
+            *reinterpret_cast<uint32_t *>(a.row_s + (row_dst0 + tid) * (a.Npad >> 5) + (n0 >> 5)) =
                 *reinterpret_cast<const uint32_t *>(&sbytes[tid * 4]);
     }
 
@@ -452,6 +477,8 @@ int pt_quantize_mx(const void *x, int x_dtype, int64_t B, int64_t M, int64_t N, 
     a.row_s = static_cast<uint8_t *>(row_scale);
     a.col_q = static_cast<uint8_t *>(col_q);
     a.col_s = static_cast<uint8_t *>(col_scale);
+    a.group_offs = a.row_offs_pad = a.col_offs_pad = nullptr;
+    a.G          = 0;
     PT_REQUIRE(a.Mpad / 128 < 65536 && B < 65536, "grid dimension out of range");
     dim3 grid(static_cast<unsigned>(a.Npad / 128), static_cast<unsigned>(a.Mpad / 128), static_cast<unsigned>(B));
     auto st = static_cast<hipStream_t>(stream);
@@ -459,6 +486,47 @@ int pt_quantize_mx(const void *x, int x_dtype, int64_t B, int64_t M, int64_t N, 
         launch_mx_fmt<bf16_t>(a, fmt, row_2d != 0, col_2d != 0, grid, st);
     else
         launch_mx_fmt<f16_t>(a, fmt, row_2d != 0, col_2d != 0, grid, st);
+    return check_launch("mx_quant_kernel");
+}
+
+int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype, const int64_t *group_offs,
+                           const int64_t *row_offs_padded, const int64_t *col_offs_padded, int64_t G, void *row_q,
+                           void *row_scale, void *col_q, void *col_scale, int64_t col_ld, void *stream) {
+    PT_REQUIRE(x_dtype == PT_DTYPE_BF16 || x_dtype == PT_DTYPE_F16, "input must be bf16 or fp16");
+    const int fmt = mx_fmt_of(q_dtype);
+    PT_REQUIRE(fmt >= 0, "q_dtype must be e4m3, e5m2 or e2m1x2");
+    PT_REQUIRE(M >= 0 && N >= 0 && G >= 1 && G <= 65535, "bad dimensions");
+    PT_REQUIRE((row_q != nullptr) == (row_scale != nullptr) && (col_q != nullptr) == (col_scale != nullptr),
+               "codes and scales come in pairs");
+    PT_REQUIRE(row_q || col_q, "nothing to produce");
+    PT_REQUIRE(col_ld % 128 == 0 && col_ld >= M, "col_ld must be a multiple of 128 that holds every padded group");
+    if (M == 0 || N == 0)
+        return PT_OK;
+    PT_REQUIRE(x && group_offs && col_offs_padded, "NULL pointer");
+    PT_REQUIRE(aligned_to(row_q, 16) && aligned_to(col_q, 16), "outputs must be 16-byte aligned");
+    PT_REQUIRE(aligned_to(row_scale, 4) && aligned_to(col_scale, 4), "scale outputs must be 4-byte aligned");
+    MxArgs a;
+    a.x            = x;
+    a.B            = 1;
+    a.M            = M;
+    a.N            = N;
+    a.Mpad         = col_ld;
+    a.Npad         = cdiv(N, 128) * 128;
+    a.row_q        = static_cast<uint8_t *>(row_q);
+    a.row_s        = static_cast<uint8_t *>(row_scale);
+    a.col_q        = static_cast<uint8_t *>(col_q);
+    a.col_s        = static_cast<uint8_t *>(col_scale);
+    a.group_offs   = group_offs;
+    a.row_offs_pad = row_offs_padded;
+    a.col_offs_pad = col_offs_padded;
+    a.G            = static_cast<int>(G);
+    PT_REQUIRE(col_ld / 128 < 65536, "grid dimension out of range");
+    dim3 grid(static_cast<unsigned>(a.Npad / 128), static_cast<unsigned>(col_ld / 128), 1);
+    auto st = static_cast<hipStream_t>(stream);
+    if (x_dtype == PT_DTYPE_BF16)
+        launch_mx_fmt<bf16_t>(a, fmt, false, false, grid, st);
+    else
+        launch_mx_fmt<f16_t>(a, fmt, false, false, grid, st);
     return check_launch("mx_quant_kernel");
 }
 

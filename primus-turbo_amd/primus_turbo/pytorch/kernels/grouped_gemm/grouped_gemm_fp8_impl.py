@@ -5,7 +5,8 @@ on top of ``pt_grouped_gemm_fp8`` and ``pt_grouped_gemm_fp8_variable_k``.
 
 One backend exists here, so ``default_backend``, ``num_cu`` and ``maybe_pre_sync`` are accepted
 and ignored (the kernel is persistent over all CUs and never needs the group sizes on the
-host). BLOCKWISE is the granularity these kernels implement.
+host). BLOCKWISE (fp32 scales per 128 block) and MX_BLOCKWISE (E8M0 bytes per 32 elements,
+MXFP8) are the granularities these kernels implement.
 """
 
 from __future__ import annotations
@@ -20,6 +21,7 @@ from primus_turbo.pytorch.core.low_precision import ScalingGranularity
 _FP8 = (torch.float8_e4m3fn, torch.float8_e5m2)
 
 TILE_CFG = 0  # 0 = automatic; tests and the benchmark may pin 2 (256x128) or 3 (128x128)
+MX_TILE_CFG = 0  # MX path: 0 = automatic, 1 = 256x256, 3 = 128x128
 
 
 def _check(cond, msg):
@@ -30,8 +32,73 @@ def _check(cond, msg):
 def _require_blockwise(granularity: int):
     if ScalingGranularity(granularity) != ScalingGranularity.BLOCKWISE:
         raise NotImplementedError(
-            f"grouped FP8 GEMM: only BLOCKWISE scaling is implemented, got {ScalingGranularity(granularity)}"
+            f"grouped FP8 GEMM: only BLOCKWISE and MX_BLOCKWISE scaling are implemented, got {ScalingGranularity(granularity)}"
         )
+
+
+def _is_mx(granularity: int) -> bool:
+    return ScalingGranularity(granularity) == ScalingGranularity.MX_BLOCKWISE
+
+
+def _u8(t: torch.Tensor) -> torch.Tensor:
+    return t.contiguous().view(torch.uint8)
+
+
+def _grouped_mx(a, b, a_scales, b_scales, group_offs, group_offs_out, trans_a, trans_b, out_dtype):
+    """MXFP8 row groups: ``out[oo[g] : oo[g+1]] = a[o[g] : o[g] + len_g] @ b[g]^T`` with ``a`` in
+    the (possibly per-group padded) row layout of the grouped quantizer and the output packed
+    by ``group_offs_out`` (over-allocated to the rows of ``a``; the tail is zero)."""
+    _check(not trans_a and trans_b, "MXFP8 grouped GEMM only supports trans_a=False, trans_b=True (NT layout).")
+    N.require_cuda(a, b, a_scales, b_scales, group_offs)
+    _check(a.dim() == 2 and b.dim() == 3, "a must be 2-D and b 3-D")
+    _check(a.dtype in _FP8 and b.dtype in _FP8, "operands must be float8_e4m3fn / float8_e5m2")
+    _check(out_dtype in (torch.float16, torch.bfloat16, torch.float32), "out_dtype must be float16, bfloat16 or float32")
+    G, Nn, K = b.shape
+    rows = a.shape[0]
+    _check(a.shape[1] == K, f"reduction dims differ: {a.shape[1]} vs {K}")
+    _check(K % 128 == 0 and K >= 512, "grouped MXFP8 GEMM needs K to be a multiple of 128 and at least 512")
+    _check(group_offs.dtype == torch.int64 and group_offs.numel() == G + 1, "group_offs must be int64 [G + 1]")
+    a_s, b_s = _u8(a_scales), _u8(b_scales)
+    _check(a_s.dim() == 2 and a_s.shape[0] == rows and a_s.shape[1] >= K // 32, "a_scales must be [rows, K/32]")
+    _check(b_s.dim() == 3 and tuple(b_s.shape[:2]) == (G, Nn) and b_s.shape[2] >= K // 32, "b_scales must be [G, N, K/32]")
+    a, b = a.contiguous(), b.contiguous()
+    out = torch.empty((rows, Nn), dtype=out_dtype, device=a.device)
+    oo = None if group_offs_out is None else group_offs_out.contiguous()
+    N.check(
+        N.lib().pt_grouped_gemm_mx(
+            N.ptr(a), N.dtype_code(a.dtype), N.ptr(a_s), a_s.shape[1], N.ptr(b), N.dtype_code(b.dtype), N.ptr(b_s),
+            b_s.shape[2], N.ptr(out), N.dtype_code(out.dtype), N.ptr(group_offs.contiguous()), N.ptr(oo), G, rows, rows,
+            Nn, K, MX_TILE_CFG, N.stream_of(a),
+        )
+    )
+    return out
+
+
+def _variable_k_mx(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, accumulate):
+    """MXFP8 variable K: ``out[g] = a[:, p[g]:p[g+1]] @ b[:, p[g]:p[g+1]]^T`` over the transposed
+    column-direction outputs of the grouped quantizer (both K-contiguous already)."""
+    _check(not trans_a and not trans_b, "MXFP8 variable-K grouped GEMM takes both operands transposed already")
+    N.require_cuda(a, b, a_scales, b_scales, group_offs, out)
+    _check(a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[1], "a and b must be 2-D with the same padded length")
+    _check(a.dtype in _FP8 and b.dtype in _FP8, "operands must be float8_e4m3fn / float8_e5m2")
+    if trans_c:
+        a, b, a_scales, b_scales = b, a, b_scales, a_scales
+    Ml, ld = a.shape
+    Nr = b.shape[0]
+    G = group_offs.numel() - 1
+    _check(ld % 128 == 0, "the padded length must be a multiple of 128")
+    a_s, b_s = _u8(a_scales), _u8(b_scales)
+    _check(tuple(a_s.shape) == (Ml, ld // 32) and tuple(b_s.shape) == (Nr, ld // 32), "scales must be [rows, padded length / 32]")
+    _check(tuple(out.shape) == (G, Ml, Nr) and out.is_contiguous(), f"out must be a contiguous {(G, Ml, Nr)} tensor")
+    a, b = a.contiguous(), b.contiguous()
+    N.check(
+        N.lib().pt_grouped_gemm_mx_variable_k(
+            N.ptr(a), N.dtype_code(a.dtype), N.ptr(a_s), N.ptr(b), N.dtype_code(b.dtype), N.ptr(b_s), N.ptr(out),
+            N.dtype_code(out.dtype), N.ptr(group_offs.contiguous()), G, Ml, Nr, ld, int(accumulate), MX_TILE_CFG,
+            N.stream_of(a),
+        )
+    )
+    return out
 
 
 @torch.library.custom_op("primus_turbo::grouped_gemm_fp8_impl", mutates_args=(), device_types="cuda")
@@ -55,6 +122,8 @@ def grouped_gemm_fp8_impl(
 
     ``a`` ``[M, K]`` fp8 with row scales stored ``[K/128, M]``; ``b`` ``[G, N, K]`` (``trans_b``)
     or ``[G, K, N]`` fp8 with 128 x 128 tile scales."""
+    if _is_mx(granularity):
+        return _grouped_mx(a, b, a_scales, b_scales, group_offs, group_offs_out, trans_a, trans_b, out_dtype)
     _require_blockwise(granularity)
     _check(not trans_a, "Only trans_a=False is supported.")
     _check(group_offs_out is None, "group_offs_out belongs to the MX grouped path")
@@ -145,8 +214,12 @@ def grouped_gemm_fp8_variable_k_impl(
 ) -> torch.Tensor:
     """``out[g] = a[p[g]:p[g+1]]^T @ b[p[g]:p[g+1]]`` (transposed when ``trans_c``) over the
     segment-padded column quantizations; ``group_offs`` holds the padded offsets ``p``."""
-    _require_blockwise(granularity)
     G = group_offs.numel() - 1
+    if _is_mx(granularity):
+        shape = (G, b.shape[0], a.shape[0]) if trans_c else (G, a.shape[0], b.shape[0])
+        out = torch.empty(shape, dtype=out_dtype, device=a.device)
+        return _variable_k_mx(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, False)
+    _require_blockwise(granularity)
     shape = (G, b.shape[1], a.shape[1]) if trans_c else (G, a.shape[1], b.shape[1])
     out = torch.empty(shape, dtype=out_dtype, device=a.device)
     return _variable_k(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, False)
@@ -157,7 +230,10 @@ def _grouped_gemm_fp8_variable_k_impl_fake(a, b, a_scales, b_scales, group_lens,
                                            trans_c, out_dtype, granularity, num_cu, default_backend,
                                            maybe_pre_sync=False):
     G = group_offs.numel() - 1
-    shape = (G, b.shape[1], a.shape[1]) if trans_c else (G, a.shape[1], b.shape[1])
+    if _is_mx(granularity):
+        shape = (G, b.shape[0], a.shape[0]) if trans_c else (G, a.shape[0], b.shape[0])
+    else:
+        shape = (G, b.shape[1], a.shape[1]) if trans_c else (G, a.shape[1], b.shape[1])
     return torch.empty(shape, dtype=out_dtype, device=a.device)
 
 
@@ -180,6 +256,9 @@ def grouped_gemm_fp8_variable_k_accum_impl(
     maybe_pre_sync: bool = False,
 ) -> None:
     """Same product, added into ``out`` in the GEMM epilogue (beta = 1)."""
+    if _is_mx(granularity):
+        _variable_k_mx(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, True)
+        return
     _require_blockwise(granularity)
     _variable_k(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, True)
 

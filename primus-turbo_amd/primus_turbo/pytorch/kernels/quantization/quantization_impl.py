@@ -701,3 +701,89 @@ def dequantize_mxfp8_impl(x, out_dtype, axis, block_size, scale_inv):
 
 def dequantize_mxfp4_impl(x, out_dtype, axis, block_size, scale_inv):
     return _dequantize_mx(x, out_dtype, axis, block_size, scale_inv, fp4=True)
+
+
+# ===========================================================================
+# Grouped MXFP8 quantizers (MoE experts): per-group zero padding along M, 32 rows for the row
+# direction and 128 for the transposed column direction
+# ===========================================================================
+MXFP8_GROUP_M_PADDING_ALIGN_SIZE = 32
+MXFP8_K_DIM_PADDING_ALIGN_SIZE = 128
+
+
+def _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, want_row: bool, want_col: bool):
+    N.require_cuda(x, group_lens, group_offs)
+    if x.dtype not in (torch.bfloat16, torch.float16):
+        raise RuntimeError("Input must be BFloat16 or Half")
+    _check(x.dim() == 2 and x.is_contiguous(), "Input must be 2D and contiguous")
+    _check(group_lens.dtype == torch.int64 and group_offs.dtype == torch.int64, "group_lens / group_offs must be int64")
+    _check(group_lens.dim() == 1 and group_offs.dim() == 1 and group_offs.numel() == group_lens.numel() + 1,
+           "group_offs.size(0) must equal group_lens.size(0) + 1")
+    _check(group_lens.numel() >= 1, "must have at least one group")
+    _check(out_dtype in (torch.float8_e4m3fn, torch.float8_e5m2), "Output must be Float8_e4m3fn or Float8_e5m2")
+    M, Nn = x.shape
+    _check(Nn % 32 == 0, f"N must be divisible by 32, got N={Nn}")
+    G = group_lens.numel()
+    ra, ca = MXFP8_GROUP_M_PADDING_ALIGN_SIZE, MXFP8_K_DIM_PADDING_ALIGN_SIZE
+    m_pad_row = -(-(M + G * ra) // ra) * ra
+    m_pad_col = -(-(M + G * ca) // ca) * ca
+    n_pad = -(-Nn // _MX_PAD) * _MX_PAD
+    dev = x.device
+    lens_row, offs_row = _group_offs(group_lens, ra, True)
+    lens_col, offs_col = _group_offs(group_lens, ca, True)
+    row_q = row_s = col_q = col_s = None
+    if want_row:
+        row_q = torch.empty((m_pad_row, n_pad), dtype=torch.uint8, device=dev)
+        row_s = torch.empty((m_pad_row, n_pad // 32), dtype=torch.uint8, device=dev)
+    if want_col:
+        col_q = torch.empty((Nn, m_pad_col), dtype=torch.uint8, device=dev)
+        col_s = torch.empty((Nn, m_pad_col // 32), dtype=torch.uint8, device=dev)
+    N.check(
+        N.lib().pt_grouped_quantize_mx(
+            N.ptr(x), N.dtype_code(x.dtype), M, Nn, N.dtype_code(out_dtype), N.ptr(group_offs.contiguous()),
+            N.ptr(offs_row), N.ptr(offs_col), G, N.ptr(row_q), N.ptr(row_s), N.ptr(col_q), N.ptr(col_s), m_pad_col,
+            N.stream_of(x),
+        )
+    )
+    view = lambda t, dt: None if t is None else t.view(dt)  # noqa: E731
+    return (view(row_q, out_dtype), view(row_s, _E8M0), view(col_q, out_dtype), view(col_s, _E8M0),
+            lens_row, offs_row, lens_col, offs_col)
+
+
+def grouped_quantize_mxfp8_impl(x, out_dtype, axis, block_size, group_lens, group_offs, with_trans=False,
+                                scaling_recipe=None, scaling_recipe_for_trans=None):
+    """MXFP8 quantization of the packed rows of G groups, each virtually zero-padded along M.
+
+    ``with_trans`` -> ``(row_q [M_pad_row, N_pad], row_scale [M_pad_row, N_pad/32], col_q [N, M_pad_col],
+    col_scale [N, M_pad_col/32], lens_padded_row, offs_padded_row, lens_padded_col, offs_padded_col)``;
+    otherwise ``(q, scale, group_lens_padded, group_offs_padded)`` of the direction ``axis`` asks
+    for (1 = rows padded to 32 per group, 0 = transposed columns padded to 128 per group).
+    ``M_pad_row`` / ``M_pad_col`` = ``total_M + G * align`` rounded up to ``align``; what lies
+    beyond ``offs_padded[G]`` is unspecified."""
+    assert block_size == 32, "The block size must be 32 for MXFP8 quantization"
+    for r in (scaling_recipe, scaling_recipe_for_trans):
+        if r is not None and (r.use_2d_block or getattr(r, "shuffle_scale", False) or getattr(r, "shuffle_out", False)):
+            raise NotImplementedError("grouped MXFP8 quantization: 2-D blocks and shuffled layouts are not implemented")
+    if with_trans:
+        return _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, True, True)
+    assert axis in (0, 1), "The axis must be 0 or 1"
+    rq, rs, cq, cs, lr, orow, lc, ocol = _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, axis == 1, axis == 0)
+    return (rq, rs, lr, orow) if axis == 1 else (cq, cs, lc, ocol)
+
+
+def grouped_dequantize_mxfp8_impl(x, out_dtype, axis, block_size, scale_inv, group_offs, group_offs_padded,
+                                  total_M=None):
+    """Inverse of the grouped quantizer: the padded layout is de-quantized as a whole and the
+    rows of every group are gathered back to their packed place (``[total_M, N]``). ``axis`` 1:
+    ``x [M_pad_row, N_pad]``; 0: the transposed ``x [N, M_pad_col]``."""
+    assert x.is_contiguous() and x.dim() == 2, "The x must be a contiguous 2D tensor."
+    assert scale_inv.dim() == 2 and scale_inv.is_contiguous(), "The scale_inv must be a contiguous 2D tensor."
+    assert axis in (0, 1), "The axis must be 0 or 1."
+    full = _dequantize_mx(x, out_dtype, axis, block_size, scale_inv, fp4=False)  # [M_pad, N_pad]
+    if total_M is None:
+        total_M = int(group_offs[-1].item())
+    # packed row i of group g sits at padded row i + (offs_padded[g] - offs[g])
+    rows = torch.arange(total_M, device=x.device, dtype=torch.int64)
+    g = torch.searchsorted(group_offs[1:].contiguous(), rows, right=True)
+    src = rows + (group_offs_padded[:-1] - group_offs[:-1])[g]
+    return full.index_select(0, src)

@@ -1,0 +1,141 @@
+"""GPU parity of the grouped MXFP8 path (MoE experts with E8M0 block scales): the grouped quantizer
+(rows of every group padded to 32 for the row direction, to 128 for the transposed column
+direction) bit for bit against the oracle, the row-group GEMM (padded A rows, tightly packed
+output) and the variable-K wgrad GEMM against the fp32 matmul of the de-quantized operands
+(max |err| / max |ref| <= 1e-2, cosine >= 0.9999), and the autograd op at the reference's SNR gate
+(tests/pytorch/ops/test_grouped_gemm_fp8.py of the reference: 25 dB E4M3, 20 dB E5M2 / HYBRID)."""
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import bf16_randn, codes_np, group_lens, to_f32_np
+from oracle import gemm as OG
+from oracle import quantize as Q
+
+pytestmark = pytest.mark.gpu
+
+FMT = {torch.float8_e4m3fn: "e4m3", torch.float8_e5m2: "e5m2"}
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _turbo(native_lib):
+    global turbo, G, Float8QuantConfig, Format, ScaleDtype, ScalingRecipe, gimpl, qimpl
+    import primus_turbo.pytorch as turbo
+    from primus_turbo.pytorch.core.low_precision import Float8QuantConfig, Format, ScaleDtype, ScalingRecipe
+    from primus_turbo.pytorch.core.low_precision import ScalingGranularity as G
+    from primus_turbo.pytorch.kernels.grouped_gemm import grouped_gemm_fp8_impl as gimpl
+    from primus_turbo.pytorch.kernels.quantization import quantization_impl as qimpl
+
+
+def _gate(ref, got, what=""):
+    cos, rel = OG.cosine(ref, got), OG.max_rel_err(ref, got)
+    assert cos >= 0.9999 and rel <= 1e-2, f"{what}: cosine {cos:.6f}, max rel err {rel:.3e}"
+
+
+def _offs(lens):
+    gl = torch.from_numpy(lens).cuda()
+    return gl, torch.ops.primus_turbo_cpp_extension.grouped_gemm_compute_offs(gl)
+
+
+QCASES = [("balanced", 4, 512, 256), ("ragged", 8, 1000, 384), ("zeros", 8, 640, 128), ("zipf", 32, 4096, 512),
+          ("ragged", 3, 77, 96), ("balanced", 1, 200, 160)]
+
+
+@pytest.mark.parametrize("kind,G_,M,N", QCASES)
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+def test_grouped_mx_quantizer_bit_exact(kind, G_, M, N, dtype):
+    lens = group_lens(kind, G_, M, 41)
+    gl, offs = _offs(lens)
+    x = bf16_randn((M, N), seed=42, outlier_frac=0.002)
+    rq, rs, cq, cs, lr, orow, lc, ocol = qimpl.grouped_quantize_mxfp8_impl(x.cuda(), dtype, None, 32, gl, offs, with_trans=True)
+    o = Q.mx_grouped_quant(x.float().numpy(), lens, FMT[dtype])
+    G1 = G_ * 32, G_ * 128
+    assert rq.shape == (-(-(M + G1[0]) // 32) * 32, -(-N // 128) * 128) and cq.shape == (N, -(-(M + G1[1]) // 128) * 128)
+    assert np.array_equal(lr.cpu().numpy(), o["row_lens"]) and np.array_equal(orow.cpu().numpy(), o["row_offs"])
+    assert np.array_equal(lc.cpu().numpy(), o["col_lens"]) and np.array_equal(ocol.cpu().numpy(), o["col_offs"])
+    mr, mc = int(o["row_offs"][-1]), int(o["col_offs"][-1])
+    assert np.array_equal(codes_np(rq)[:mr], o["row"]) and np.array_equal(codes_np(rs)[:mr], o["row_scale"])
+    assert np.array_equal(codes_np(cq)[:, :mc], o["col"]) and np.array_equal(codes_np(cs)[:, : mc // 32], o["col_scale"])
+    # one direction at a time gives the same tensors
+    q1, s1, l1, o1 = qimpl.grouped_quantize_mxfp8_impl(x.cuda(), dtype, 1, 32, gl, offs)
+    q0, s0, l0, o0 = qimpl.grouped_quantize_mxfp8_impl(x.cuda(), dtype, 0, 32, gl, offs)
+    assert np.array_equal(codes_np(q1)[:mr], o["row"]) and np.array_equal(codes_np(s1)[:mr], o["row_scale"])
+    assert np.array_equal(codes_np(q0)[:, :mc], o["col"]) and np.array_equal(codes_np(s0)[:, : mc // 32], o["col_scale"])
+    assert torch.equal(o1, orow) and torch.equal(o0, ocol) and torch.equal(l1, lr) and torch.equal(l0, lc)
+    # the de-quantizer gathers the packed rows back
+    for axis, (q, s, op) in ((1, (rq, rs, orow)), (0, (cq, cs, ocol))):
+        y = qimpl.grouped_dequantize_mxfp8_impl(q, torch.float32, axis, 32, s, offs, op, total_M=M)
+        if axis == 1:
+            ref = Q.mx_dequant(o["row"], o["row_scale"], FMT[dtype])
+            pad_offs = o["row_offs"]
+        else:
+            ref = Q.mx_dequant(o["col"], o["col_scale"], FMT[dtype]).T
+            pad_offs = o["col_offs"]
+        starts = np.concatenate([[0], np.cumsum(lens)])
+        want = np.concatenate([ref[pad_offs[g] : pad_offs[g] + lens[g]] for g in range(G_)], axis=0)
+        assert y.shape[0] == M and np.array_equal(to_f32_np(y)[:, : want.shape[1]], want), f"axis {axis}"
+        del starts
+
+
+GCASES = [("balanced", 4, 1024, 512, 512), ("ragged", 8, 3000, 384, 1024), ("zeros", 8, 2048, 256, 512),
+          ("zipf", 32, 8192, 1024, 768), ("ragged", 3, 77, 96, 640), ("zipf", 16, 4096, 2048, 512)]
+
+
+@pytest.mark.parametrize("kind,G_,M,N,K", GCASES)
+@pytest.mark.parametrize("fa,fb", [(torch.float8_e4m3fn, torch.float8_e4m3fn), (torch.float8_e5m2, torch.float8_e4m3fn)])
+def test_grouped_mx_forward_product(kind, G_, M, N, K, fa, fb):
+    lens = group_lens(kind, G_, M, 43)
+    gl, offs = _offs(lens)
+    x = bf16_randn((M, K), seed=44)
+    w = bf16_randn((G_, N, K), seed=45)
+    rq, rs, lr, orow = qimpl.grouped_quantize_mxfp8_impl(x.cuda(), fa, 1, 32, gl, offs)
+    wq, ws = qimpl.quantize_mxfp8_impl(w.cuda(), fb, 2, 32, scaling_recipe=ScalingRecipe(use_2d_block=True))
+    out = gimpl.grouped_gemm_fp8_impl(rq, wq, rs, ws, gl, orow, False, True, torch.bfloat16, G.MX_BLOCKWISE.value, None, 0,
+                                      False, offs)
+    torch.cuda.synchronize()
+    assert out.shape == (rq.shape[0], N)
+    o = Q.mx_grouped_quant(x.float().numpy(), lens, FMT[fa])
+    a_pad = Q.mx_dequant(o["row"], o["row_scale"], FMT[fa])[:, :K]
+    a_deq = np.concatenate([a_pad[o["row_offs"][g] : o["row_offs"][g] + lens[g]] for g in range(G_)], axis=0)
+    w_deq = np.stack([Q.mx_dequant(codes_np(wq[g]), codes_np(ws[g]), FMT[fb])[:, :K] for g in range(G_)])
+    ref = OG.grouped_gemm_dequantized(a_deq, w_deq, lens, trans_b=True)
+    _gate(ref, to_f32_np(out[:M]), f"{kind} G={G_} {M}x{N}x{K}")
+    assert not bool(out[M:].float().abs().max() > 0) if out.shape[0] > M else True
+    # the dense (unpadded) row layout with one set of offsets gives the same rows
+    dq, dsc = qimpl.quantize_mxfp8_impl(x.cuda(), fa, 1, 32)
+    out2 = gimpl.grouped_gemm_fp8_impl(dq, wq, dsc, ws, gl, offs, False, True, torch.bfloat16, G.MX_BLOCKWISE.value, None, 0)
+    assert torch.equal(out2[:M], out[:M])
+
+
+@pytest.mark.parametrize("kind,G_,M,N,K", GCASES)
+@pytest.mark.parametrize("trans_c", [False, True])
+def test_grouped_mx_variable_k_product(kind, G_, M, N, K, trans_c):
+    lens = group_lens(kind, G_, M, 46)
+    gl, offs = _offs(lens)
+    x = bf16_randn((M, K), seed=47)
+    dy = bf16_randn((M, N), seed=48)
+    xq, xs, lc, ocol = qimpl.grouped_quantize_mxfp8_impl(x.cuda(), torch.float8_e4m3fn, 0, 32, gl, offs)
+    gq, gs, _, _ = qimpl.grouped_quantize_mxfp8_impl(dy.cuda(), torch.float8_e5m2, 0, 32, gl, offs)
+    out = gimpl.grouped_gemm_fp8_variable_k_impl(gq, xq, gs, xs, lc, ocol, False, False, trans_c, torch.float32,
+                                                 G.MX_BLOCKWISE.value, None, 0)
+    torch.cuda.synchronize()
+    assert out.shape == ((G_, K, N) if trans_c else (G_, N, K))
+    ox = Q.mx_grouped_quant(x.float().numpy(), lens, "e4m3")
+    og = Q.mx_grouped_quant(dy.float().numpy(), lens, "e5m2")
+    xd = Q.mx_dequant(ox["col"], ox["col_scale"], "e4m3")  # [K, Mc]
+    gd = Q.mx_dequant(og["col"], og["col_scale"], "e5m2")  # [N, Mc]
+    co = ox["col_offs"]
+    ref = np.stack([gd[:, co[g] : co[g + 1]].astype(np.float64) @ xd[:, co[g] : co[g + 1]].astype(np.float64).T
+                    for g in range(G_)]).astype(np.float32)
+    if trans_c:
+        ref = np.ascontiguousarray(ref.transpose(0, 2, 1))
+    _gate(ref, to_f32_np(out), f"variable-K {kind} G={G_}")
+    for g in range(G_):
+        if lens[g] == 0:
+            assert not bool(out[g].abs().max() > 0)
+    # beta = 1 epilogue
+    acc = torch.ones_like(out)
+    gimpl.grouped_gemm_fp8_variable_k_accum_impl(gq, xq, gs, xs, lc, ocol, False, False, trans_c, torch.float32,
+                                                 G.MX_BLOCKWISE.value, None, 0, acc)
+    assert torch.allclose(acc, out + 1, rtol=0, atol=1e-3 * float(out.abs().max()) + 1e-6)
