@@ -1,10 +1,15 @@
 """``grouped_gemm_fp8``: MoE grouped linear layer in FP8 with autograd
 (reference: primus_turbo/pytorch/ops/grouped_gemm_fp8.py:99-265,853-960).
 
-BLOCKWISE (128) is the granularity implemented here: one fused pass over the bf16 activation
-yields the row quantization (forward / dgrad operand) and the segment-padded column
-quantization (wgrad operand); the weight is quantized in 128 x 128 tiles that serve forward
-and backward unchanged.
+BLOCKWISE (128): one fused pass over the bf16 activation yields the row quantization (forward /
+dgrad operand) and the segment-padded column quantization (wgrad operand); the weight is
+quantized in 128 x 128 tiles that serve forward and backward unchanged.
+
+MX_BLOCKWISE (MXFP8, reference :604-840): activations and gradients go through the grouped MX
+quantizer (rows padded to 32 per group, transposed columns to 128), weights through the dense MX
+quantizer with 32 x 32 blocks in both directions; forward and dgrad are row-group NT products
+whose output is packed by the tight offsets, wgrad is a variable-K NT product over the padded
+column-direction operands. NT only (``trans_b=True``).
 """
 
 from __future__ import annotations
@@ -31,8 +36,10 @@ from primus_turbo.pytorch.kernels.grouped_gemm.grouped_gemm_fp8_impl import (
 )
 from primus_turbo.pytorch.kernels.grouped_gemm.grouped_gemm_utils import group_offs_from_lens
 from primus_turbo.pytorch.kernels.quantization.quantization_impl import (
+    grouped_quantize_mxfp8_impl,
     quant_fp8_blockwise_for_weight_impl,
     quant_fp8_blockwise_segment_m_row_col_impl,
+    quantize_mxfp8_impl,
 )
 from primus_turbo.pytorch.ops.utils import (
     _ensure_contiguous_grad_out,
@@ -118,6 +125,62 @@ class FP8GroupedGemmBlockFunc(torch.autograd.Function):
         return grad_a, grad_b, None, None, None, None, None, None, None, None, None
 
 
+class FP8GroupedGemmMXFunc(torch.autograd.Function):
+    """MX_BLOCKWISE (MXFP8) grouped GEMM autograd."""
+
+    @staticmethod
+    def forward(ctx, a, b, a_t, b_t, group_lens, group_offs, trans_b, out_dtype, config, num_cu,
+                fuse_bgrad_accum_pattern=None):
+        fuse_bgrad_accum, main_grad = _setup_fused_grad_accum(b, fuse_bgrad_accum_pattern)
+        assert config.granularity == ScalingGranularity.MX_BLOCKWISE
+        if isinstance(a, QuantizedTensor) or isinstance(b, QuantizedTensor):
+            raise NotImplementedError("FP8GroupedGemmMXFunc does not take pre-quantized operands in this build")
+        assert a.ndim == 2 and b.ndim == 3
+        assert trans_b, "MXFP8 grouped GEMM only supports trans_b=True (NT layout)."
+        assert group_lens.size(0) == b.size(0), "group_lens size must match b size(0)."
+        fdt = _get_fp8_dtype(config.format, True)
+        bs = config.block_size
+        total_m = int(a.size(0))
+        need_bwd = any(ctx.needs_input_grad[:2])
+        w_recipe = ScalingRecipe(use_2d_block=True)
+        if need_bwd:
+            a_row, a_row_s, a_col, a_col_s, _, offs_row, _, _ = grouped_quantize_mxfp8_impl(
+                a.contiguous(), fdt, None, bs, group_lens, group_offs, with_trans=True)
+            b_row, b_row_s, b_col, b_col_s = quantize_mxfp8_impl(
+                b.contiguous(), fdt, None, bs, with_trans=True, scaling_recipe=w_recipe, scaling_recipe_for_trans=w_recipe)
+        else:
+            a_row, a_row_s, _, offs_row = grouped_quantize_mxfp8_impl(a.contiguous(), fdt, 1, bs, group_lens, group_offs)
+            b_row, b_row_s = quantize_mxfp8_impl(b.contiguous(), fdt, 2, bs, scaling_recipe=w_recipe)
+            a_col = a_col_s = b_col = b_col_s = None
+        # the padded row layout is read through offs_row, the result is packed by group_offs
+        # into an output over-allocated to the padded rows
+        out = grouped_gemm_fp8_impl(a_row, b_row, a_row_s, b_row_s, group_lens, offs_row, False, True, out_dtype,
+                                    config.granularity.value, num_cu, _NATIVE, False, group_offs)[:total_m]
+        if need_bwd:
+            ctx.save_for_backward(a_col, a_col_s, b_col, b_col_s, group_lens, group_offs)
+        ctx.meta = (config, out_dtype, num_cu, total_m, fuse_bgrad_accum, main_grad)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        grad_out = _ensure_contiguous_grad_out(grad_out)
+        a_col, a_col_s, b_col, b_col_s, group_lens, group_offs = ctx.saved_tensors
+        config, out_dtype, num_cu, total_m, fuse_bgrad_accum, main_grad = ctx.meta
+        gdt = _get_fp8_dtype(config.format, False)
+        gran = config.granularity.value
+        g_row, g_row_s, g_col, g_col_s, _, offs_row, lens_col, offs_col = grouped_quantize_mxfp8_impl(
+            grad_out, gdt, None, config.block_size, group_lens, group_offs, with_trans=True)
+        # dgrad: grad_a = grad_out @ b, as an NT product with the transposed weight quantization [G, K, N]
+        grad_a = grouped_gemm_fp8_impl(g_row, b_col, g_row_s, b_col_s, group_lens, offs_row, False, True, out_dtype,
+                                       gran, num_cu, _NATIVE, False, group_offs)[:total_m]
+        # wgrad: grad_b[g] = grad_out_g^T @ a_g over the 128-padded segments -> [G, N, K]
+        grad_b = _grouped_gemm_fp8_variable_k_impl_wrapper(
+            g_col, a_col, g_col_s, a_col_s, lens_col, offs_col, False, False, False, out_dtype, gran, num_cu, _NATIVE,
+            inplace_add_to_out=fuse_bgrad_accum, out=main_grad,
+        )
+        return grad_a, grad_b, None, None, None, None, None, None, None, None, None
+
+
 def grouped_gemm_fp8(
     a: Union[torch.Tensor, QuantizedTensor, QuantizedTensorPair],
     b: Union[torch.Tensor, QuantizedTensor, QuantizedTensorPair],
@@ -145,6 +208,10 @@ def grouped_gemm_fp8(
     if config.granularity == ScalingGranularity.BLOCKWISE:
         return FP8GroupedGemmBlockFunc.apply(a_data, b_data, a_data_t, b_data_t, group_lens, group_offs, trans_b,
                                              out_dtype, config, num_cu, fuse_bgrad_accum_pattern)
+    if config.granularity == ScalingGranularity.MX_BLOCKWISE:
+        return FP8GroupedGemmMXFunc.apply(a_data, b_data, a_data_t, b_data_t, group_lens, group_offs, trans_b,
+                                          out_dtype, config, num_cu, fuse_bgrad_accum_pattern)
     raise NotImplementedError(
-        f"grouped_gemm_fp8: granularity {config.granularity} is not implemented (BLOCKWISE with block_size=128 is)"
+        f"grouped_gemm_fp8: granularity {config.granularity} is not implemented "
+        "(BLOCKWISE with block_size=128 and MX_BLOCKWISE are)"
     )

@@ -186,32 +186,46 @@ def dequantize_fp4(
     raise _unknown(granularity)
 
 
-# --- grouped MX quantizers: not part of this build's hot path ---------------------------
+# --- grouped MX quantizers (MoE experts): per-group padded MXFP8 layouts ---------------------
 def _grouped_mx_not_built(name):
     raise NotImplementedError(
-        f"{name}: the grouped MX quantizers (per-group padded MXFP8/MXFP4 layouts) are not built; "
-        "the grouped path of this library is the FP8 128-blockwise one (grouped_gemm_fp8 with BLOCKWISE)."
+        f"{name}: the grouped MXFP4 quantizers (per-group padded layouts) are not built; the grouped MX path "
+        "of this library is MXFP8 (grouped_quantize_fp8 / grouped_gemm_fp8 with MX_BLOCKWISE)."
     )
 
 
 def grouped_quantize_fp8(x, out_dtype, granularity, group_lens, group_offs, *, block_size=None, axis=None,
                          scaling_recipe=None):
+    """Quantize the packed rows of G groups (MX_BLOCKWISE): ``axis`` 1 (or -1) -> rows, every group
+    padded to 32 rows; ``axis`` 0 -> the transposed column direction, padded to 128.
+    Returns ``(x_fp8, scale_inv, group_lens_padded, group_offs_padded)``."""
     if granularity == _G.MX_BLOCKWISE:
-        _grouped_mx_not_built("grouped_quantize_fp8")
+        _need_mx_block(block_size, MXFP8_BLOCK_SIZE, "MXFP8")
+        assert axis is not None, "axis must be specified for grouped MXFP8 quantization"
+        return _impl.grouped_quantize_mxfp8_impl(x, out_dtype, axis % x.dim(), block_size, group_lens, group_offs,
+                                                 False, scaling_recipe)
     raise _unknown(granularity)
 
 
 def grouped_quantize_fp8_with_trans(x, out_dtype, granularity, group_lens, group_offs, *, block_size=None,
                                     scaling_recipe=None, scaling_recipe_for_trans=None):
+    """Both directions from one read of ``x``: ``(x_fp8_row, scale_row, x_fp8_col, scale_col,
+    lens_padded_row, offs_padded_row, lens_padded_col, offs_padded_col)``."""
     if granularity == _G.MX_BLOCKWISE:
-        _grouped_mx_not_built("grouped_quantize_fp8_with_trans")
+        _need_mx_block(block_size, MXFP8_BLOCK_SIZE, "MXFP8")
+        return _impl.grouped_quantize_mxfp8_impl(x, out_dtype, None, block_size, group_lens, group_offs, True,
+                                                 scaling_recipe, scaling_recipe_for_trans)
     raise _unknown(granularity)
 
 
 def grouped_dequantize_fp8(x, out_dtype, granularity, group_offs, group_offs_padded, *, block_size=None, axis=None,
                            scale_inv=None, scaling_recipe=None, total_M=None):
+    """Inverse of ``grouped_quantize_fp8``: the packed ``[total_M, N_pad]`` rows."""
     if granularity == _G.MX_BLOCKWISE:
-        _grouped_mx_not_built("grouped_dequantize_fp8")
+        _need_mx_block(block_size, MXFP8_BLOCK_SIZE, "MXFP8")
+        assert axis is not None and scale_inv is not None
+        return _impl.grouped_dequantize_mxfp8_impl(x, out_dtype, axis % 2, block_size, scale_inv, group_offs,
+                                                   group_offs_padded, total_M)
     raise _unknown(granularity)
 
 

@@ -139,3 +139,51 @@ def test_grouped_mx_variable_k_product(kind, G_, M, N, K, trans_c):
     gimpl.grouped_gemm_fp8_variable_k_accum_impl(gq, xq, gs, xs, lc, ocol, False, False, trans_c, torch.float32,
                                                  G.MX_BLOCKWISE.value, None, 0, acc)
     assert torch.allclose(acc, out + 1, rtol=0, atol=1e-3 * float(out.abs().max()) + 1e-6)
+
+
+@pytest.mark.parametrize("fmt,gate", [("E4M3", 25), ("E5M2", 20), ("HYBRID", 20)])
+@pytest.mark.parametrize("kind,G_,M,N,K", [("zipf", 8, 4096, 1024, 512), ("ragged", 4, 1000, 512, 1024)])
+def test_grouped_gemm_fp8_mx_autograd(fmt, gate, kind, G_, M, N, K):
+    """The MX_BLOCKWISE op end to end (grouped quantizers, forward, dgrad, wgrad) against the
+    unquantized grouped matmul; empty experts get a zero weight gradient; a forward-only call
+    gives the same output."""
+    lens = group_lens(kind, G_, M, 49)
+    gl, _ = _offs(lens)
+    a = bf16_randn((M, K), seed=50).cuda().requires_grad_(True)
+    b = bf16_randn((G_, N, K), seed=51).cuda().requires_grad_(True)
+    cfg = Float8QuantConfig(format=getattr(Format, fmt), granularity=G.MX_BLOCKWISE, block_size=32, scale_dtype=ScaleDtype.E8M0)
+    out = turbo.ops.grouped_gemm_fp8(a, b, gl, trans_b=True, config=cfg)
+    assert out.shape == (M, N) and out.dtype == torch.bfloat16
+    dy = bf16_randn((M, N), seed=52).cuda()
+    out.backward(dy)
+    torch.cuda.synchronize()
+    af, bf_, dyf = to_f32_np(a), to_f32_np(b), to_f32_np(dy)
+    ref_out = OG.grouped_gemm_dequantized(af, bf_, lens, trans_b=True)
+    ref_da = OG.grouped_gemm_dequantized(dyf, bf_, lens, trans_b=False)
+    ref_db = OG.grouped_gemm_variable_k_dequantized(af, dyf, lens).transpose(0, 2, 1)  # [G, N, K]
+    assert OG.snr_db(ref_out, to_f32_np(out)) > gate
+    assert OG.snr_db(ref_da, to_f32_np(a.grad)) > gate
+    assert OG.snr_db(ref_db, to_f32_np(b.grad)) > gate
+    for g in range(G_):
+        if lens[g] == 0:
+            assert torch.count_nonzero(b.grad[g]).item() == 0
+    with torch.no_grad():
+        out2 = turbo.ops.grouped_gemm_fp8(a, b, gl, trans_b=True, config=cfg)
+    assert torch.equal(out2, out)
+
+
+def test_grouped_quantize_fp8_ops_surface():
+    """``grouped_quantize_fp8`` / ``..._with_trans`` / ``grouped_dequantize_fp8`` of the op layer."""
+    lens = group_lens("ragged", 4, 600, 53)
+    gl, offs = _offs(lens)
+    x = bf16_randn((600, 256), seed=54).cuda()
+    q, s, lp, op = turbo.ops.grouped_quantize_fp8(x, turbo.float8_e4m3, G.MX_BLOCKWISE, gl, offs, block_size=32, axis=-1)
+    y = turbo.ops.grouped_dequantize_fp8(q, torch.float32, G.MX_BLOCKWISE, offs, op, block_size=32, axis=1, scale_inv=s,
+                                         total_M=600)
+    assert y.shape == (600, 256)
+    assert OG.snr_db(to_f32_np(x), to_f32_np(y)) > 25
+    out = turbo.ops.grouped_quantize_fp8_with_trans(x, turbo.float8_e4m3, G.MX_BLOCKWISE, gl, offs, block_size=32)
+    assert len(out) == 8 and torch.equal(out[0][: int(op[-1])], q[: int(op[-1])]) and torch.equal(out[5], op)
+    yc = turbo.ops.grouped_dequantize_fp8(out[2], torch.float32, G.MX_BLOCKWISE, offs, out[7], block_size=32, axis=0,
+                                          scale_inv=out[3], total_M=600)
+    assert OG.snr_db(to_f32_np(x), to_f32_np(yc)[:, :256]) > 25
