@@ -425,6 +425,104 @@ class GroupedGemmFp8(_GemmBase):
         )
 
 
+class GroupedGemmMxfp8(_GemmBase):
+    """The MoE configuration (32 experts, 32768 routed tokens, Zipf(1.2) counts with empty experts)
+    through the grouped MXFP8 path: grouped MX quantizers (rows padded to 32 per expert, transposed
+    columns to 128), forward + dgrad row-group GEMMs and the variable-K wgrad GEMM."""
+
+    dominant_name = "gemm_fp8_nt_kernel<256x256 tile, row groups, E8M0 block scales in the MFMA> (forward)"
+    dtype = "fp8_e4m3 with E8M0 block scales (fp32 accumulate)"
+
+    def __init__(self, dev, N=4096, K=7168, groups=32, tokens=32768):
+        import primus_turbo.pytorch as turbo
+        from primus_turbo.pytorch.core.low_precision import Float8QuantConfig, Format, ScaleDtype, ScalingGranularity, ScalingRecipe
+        from primus_turbo.pytorch.kernels.grouped_gemm import grouped_gemm_fp8_impl as gg
+        from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+        self.turbo, self.G, self.gg, self.qi = turbo, ScalingGranularity, gg, qi
+        self.M, self.N, self.K, self.groups = tokens, N, K, groups
+        self.name = (f"moe_grouped_gemm_mxfp8_{groups}experts_{tokens}tokens_zipf1.2_k{K}_n{N} "
+                     "(forward + dgrad + wgrad, quantizers included)")
+        self.cfg = Float8QuantConfig(format=Format.E4M3, granularity=ScalingGranularity.MX_BLOCKWISE, block_size=32,
+                                     scale_dtype=ScaleDtype.E8M0)
+        self.lens = _zipf_group_lens(groups, tokens, 7)
+        self.gl = torch.from_numpy(self.lens).to(dev)
+        self.offs = torch.ops.primus_turbo_cpp_extension.grouped_gemm_compute_offs(self.gl)
+        self.x_cpu = _randn_bf16((tokens, K), 7, 1.0)
+        self.w_cpu = _randn_bf16((groups, N, K), 8, 1.0)
+        self.x = self.x_cpu.to(dev).requires_grad_(True)
+        self.w = self.w_cpu.to(dev).requires_grad_(True)
+        self.dy = _randn_bf16((tokens, N), 9, 1.0).to(dev)
+        self.qr, self.sr, _, self.offs_row = qi.grouped_quantize_mxfp8_impl(self.x.detach(), torch.float8_e4m3fn, 1, 32,
+                                                                            self.gl, self.offs)
+        self.wq, self.ws = qi.quantize_mxfp8_impl(self.w.detach(), torch.float8_e4m3fn, 2, 32,
+                                                  scaling_recipe=ScalingRecipe(use_2d_block=True))
+
+    def step_work(self):
+        return 3 * 2.0 * self.M * self.N * self.K
+
+    def step(self):
+        self.x.grad = None
+        self.w.grad = None
+        y = self.turbo.ops.grouped_gemm_fp8(self.x, self.w, self.gl, self.offs, trans_b=True, config=self.cfg)
+        y.backward(self.dy)
+        return y
+
+    def dominant(self):
+        return self.gg.grouped_gemm_fp8_impl(self.qr, self.wq, self.sr, self.ws, self.gl, self.offs_row, False, True,
+                                             torch.bfloat16, self.G.MX_BLOCKWISE.value, None, 0, False, self.offs)
+
+    def check(self):
+        """Forward rows of the first and of the last non-empty expert (up to 64 each) against the
+        oracle's de-quantized matmul; their codes and E8M0 bytes bit-exact."""
+        import numpy as np
+
+        from oracle import gemm as OG
+        from oracle import quantize as Q
+
+        def u8(t):
+            return t.contiguous().view(torch.uint8).cpu().numpy()
+
+        out = self.dominant().float().cpu().numpy()
+        offs = np.concatenate([[0], np.cumsum(self.lens)])
+        orow = self.offs_row.cpu().numpy()
+        live = [g for g in range(self.groups) if self.lens[g] > 0]
+        same, rel, cos = True, 0.0, 1.0
+        for g in (live[0], live[-1]):
+            n = int(min(64, self.lens[g]))
+            r0, p0 = int(offs[g]), int(orow[g])
+            aq, asc = Q.mx_quant_rowwise(self.x_cpu.float().numpy()[r0 : r0 + n], "e4m3")
+            same = same and np.array_equal(u8(self.qr)[p0 : p0 + n], aq) and np.array_equal(u8(self.sr)[p0 : p0 + n], asc)
+            w_deq = Q.mx_dequant(u8(self.wq[g]), u8(self.ws[g]), "e4m3")
+            ref = OG.gemm_dequantized(Q.mx_dequant(aq, asc, "e4m3"), w_deq, trans_b=True)
+            ref_t = torch.from_numpy(np.ascontiguousarray(ref, dtype=np.float32)).to(torch.bfloat16).float().numpy()
+            rel = max(rel, OG.max_rel_err(ref_t, out[r0 : r0 + n]))
+            cos = min(cos, OG.cosine(out[r0 : r0 + n], ref_t))
+        ok = bool(same and rel <= 1e-2 and cos >= 0.9999)
+        return ok, f"codes and E8M0 bytes bit-exact: {same}; rows of two experts vs oracle: max_rel_err={rel:.2e}, cosine={cos:.6f}"
+
+    def cpu_baseline(self):
+        """The numpy oracle (MX quantize, de-quantize) plus an fp32 matmul for 256 tokens of the
+        largest expert against 2048 of its output features."""
+        import numpy as np
+
+        from oracle import quantize as Q
+
+        g = int(np.argmax(self.lens))
+        r0 = int(np.concatenate([[0], np.cumsum(self.lens)])[g])
+        a = self.x_cpu[r0 : r0 + 256].float().numpy()
+        b = self.w_cpu[g, :2048].float().numpy()
+        t0 = time.perf_counter()
+        aq, asc = Q.mx_quant_rowwise(a, "e4m3")
+        bq, bsc = Q.mx_quant_rowwise(b, "e4m3", use_2d_block=True)
+        y = Q.mx_dequant(aq, asc, "e4m3") @ Q.mx_dequant(bq, bsc, "e4m3").T
+        dt = time.perf_counter() - t0
+        del y
+        return dict(value=round(2.0 * 256 * 2048 * self.K / dt / 1e12, 5), unit="TFLOP/s", cores=torch.get_num_threads(),
+                    kind="port", sample=f"256 tokens of the largest expert against 2048 output features (MX quantize both, "
+                    f"dequantize, fp32 matmul), {dt:.1f} s, {os.cpu_count()} logical CPUs visible")
+
+
 def _keyed(key, make):
     def build(dev):
         wl = make(dev)
@@ -445,6 +543,8 @@ def register(workloads):
     workloads["gemm_mxfp8_n28672"] = lambda dev: GemmMx(dev, False, 8192, 28672, 8192)
     workloads["grouped_gemm_fp8"] = lambda dev: GroupedGemmFp8(dev, 4096, 7168)
     workloads["grouped_gemm_fp8_down"] = lambda dev: GroupedGemmFp8(dev, 7168, 2048)
+    workloads["grouped_gemm_mxfp8"] = lambda dev: GroupedGemmMxfp8(dev, 4096, 7168)
+    workloads["grouped_gemm_mxfp8_down"] = lambda dev: GroupedGemmMxfp8(dev, 7168, 2048)
     for key in list(workloads):
         if key in TRAFFIC_MIB:
             workloads[key] = _keyed(key, workloads[key])
