@@ -240,3 +240,35 @@ def test_fp4_packing_order():
     p = Q._pack_fp4(codes)
     assert p.tolist() == [[0x10, 0x32, 0x54, 0x76, 0x98, 0xBA, 0xDC, 0xFE]]  # even element in the low nibble
     assert np.array_equal(Q.unpack_fp4(p), codes)
+
+
+@pytest.mark.parametrize("lens", [[100, 0, 37, 163], [128, 128], [1], [0, 5, 0, 250, 31]])
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e2m1"])
+def test_mx_grouped_layout(lens, fmt):
+    """Grouped MX quantizer: group starts on multiples of 32 (rows) / 128 (transposed columns),
+    every group's slice equals the dense quantizer of that group's rows, pads are zero codes with
+    scale byte 0, and the round trip through the de-quantizer matches the dense round trip."""
+    lens = np.array(lens, dtype=np.int64)
+    M, N = int(lens.sum()), 160
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((M, N)) * np.exp(rng.standard_normal((M, 1)))).astype(np.float32)
+    o = Q.mx_grouped_quant(x, lens, fmt)
+    cpb = 2 if fmt == "e2m1" else 1
+    assert np.all(o["row_offs"] % 32 == 0) and np.all(o["col_offs"] % 128 == 0)
+    assert np.array_equal(o["row_lens"], (lens + 31) // 32 * 32) and np.array_equal(o["col_lens"], (lens + 127) // 128 * 128)
+    assert o["row"].shape == (o["row_offs"][-1], 256 // cpb) and o["col"].shape == (N, o["col_offs"][-1] // cpb)
+    starts = np.concatenate([[0], np.cumsum(lens)])
+    for g, n in enumerate(lens):
+        r0, c0, c1 = o["row_offs"][g], o["col_offs"][g], o["col_offs"][g + 1]
+        seg = x[starts[g] : starts[g] + n]
+        if n:
+            q, s = Q.mx_quant_rowwise(seg, fmt)
+            assert np.array_equal(o["row"][r0 : r0 + n], q) and np.array_equal(o["row_scale"][r0 : r0 + n], s)
+            deq = Q.mx_dequant(o["col"][:, c0 // cpb : c1 // cpb], o["col_scale"][:, c0 // 32 : c1 // 32], fmt)
+            qc, sc = Q.mx_quant_colwise(seg, fmt)
+            assert np.array_equal(deq[:, :n], Q.mx_dequant(qc, sc, fmt)[:, :n])
+            assert not deq[:, n:].any()
+        pad = slice(r0 + n, o["row_offs"][g + 1])
+        assert not o["row"][pad].any() and not o["row_scale"][pad].any()
+        # scale bytes of blocks that lie entirely in the column padding are zero
+        assert not o["col_scale"][:, (c0 + n + 31) // 32 : c1 // 32].any()
