@@ -306,6 +306,44 @@ PT_API int pt_grouped_gemm_fp8_variable_k(const void *lhs, int lhs_dtype, const 
                                           int accumulate, void *workspace, size_t workspace_bytes,
                                           int tile_cfg, void *stream);
 
+/* Grouped GEMM with vector scales (TENSORWISE / ROWWISE granularities) -----------------
+ *
+ * pt_grouped_gemm_fp8_vec replaces primus_turbo::grouped_gemm_fp8_impl for TENSORWISE and
+ * ROWWISE (kernels/grouped_gemm/grouped_gemm_fp8_impl.py:888-930; callers
+ * ops/grouped_gemm_fp8.py:265-603), forward and dgrad:
+ *   out[offs[g] : offs[g+1], n] = (A[offs[g] : offs[g+1]] . op(B[g]))[., n]
+ *                                 * a_scale[m * sa_stride] * b_scale[g * sb_gstride + n * sb_stride]
+ *   out[offs[G] : out_rows] = 0
+ * A [M, K] fp8; trans_b != 0: B [G, N, K], else [G, K, N]. Strides in floats: 0 = one scalar
+ * (TENSORWISE), 1 = one per row / column (ROWWISE). The workspace
+ * (pt_grouped_gemm_fp8_vec_workspace_bytes) holds the K-contiguous copy of B when trans_b == 0
+ * and zero-padded copies when K % 128 != 0 or K < 512.
+ *
+ * pt_grouped_gemm_fp8_vec_variable_k replaces primus_turbo::grouped_gemm_fp8_variable_k_impl for
+ * the same granularities (grouped_gemm_fp8_impl.py:933-1022), wgrad over tightly packed groups:
+ *   C[g][i, j] (+)= (L[offs[g] : offs[g+1]]^T . R[offs[g] : offs[g+1]])[i, j]
+ *                   * lhs_scale[i * sl_stride] * rhs_scale[j * sr_stride]
+ * L [M, Ml], R [M, Nr] fp8, C [G, Ml, Nr] (trans_c: [G, Nr, Ml]). The workspace holds the padded
+ * group offsets and both operands copied K-contiguous with every group padded to a multiple of
+ * 128 rows of zeros. */
+PT_API size_t pt_grouped_gemm_fp8_vec_workspace_bytes(int64_t G, int64_t M, int64_t N, int64_t K,
+                                                      int trans_b);
+PT_API int pt_grouped_gemm_fp8_vec(const void *a, int a_dtype, const float *a_scale, int64_t sa_stride,
+                                   const void *b, int b_dtype, const float *b_scale, int64_t sb_stride,
+                                   int64_t sb_gstride, void *c, int c_dtype, const int64_t *group_offs,
+                                   int64_t G, int64_t M, int64_t out_rows, int64_t N, int64_t K,
+                                   int trans_b, void *workspace, size_t workspace_bytes, int tile_cfg,
+                                   void *stream);
+PT_API size_t pt_grouped_gemm_fp8_vec_variable_k_workspace_bytes(int64_t G, int64_t M, int64_t Ml,
+                                                                 int64_t Nr);
+PT_API int pt_grouped_gemm_fp8_vec_variable_k(const void *lhs, int lhs_dtype, const float *lhs_scale,
+                                              int64_t sl_stride, const void *rhs, int rhs_dtype,
+                                              const float *rhs_scale, int64_t sr_stride, void *c,
+                                              int c_dtype, const int64_t *group_offs, int64_t G,
+                                              int64_t M, int64_t Ml, int64_t Nr, int trans_c,
+                                              int accumulate, void *workspace, size_t workspace_bytes,
+                                              int tile_cfg, void *stream);
+
 /* Grouped MXFP8 path (MoE experts with E8M0 block scales) ------------------------------
  *
  * pt_grouped_quantize_mx replaces the dispatcher ops grouped_quantize_mxfp8 /

@@ -108,6 +108,18 @@ _SIGNATURES = {
         [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_i64, c_i64, c_i64, c_i64,
          c_int, c_int, c_void_p, c_size_t, c_int, c_void_p],
     ),
+    "pt_grouped_gemm_fp8_vec_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_i64, c_int]),
+    "pt_grouped_gemm_fp8_vec": (
+        c_int,
+        [c_void_p, c_int, c_void_p, c_i64, c_void_p, c_int, c_void_p, c_i64, c_i64, c_void_p, c_int, c_void_p, c_i64, c_i64,
+         c_i64, c_i64, c_i64, c_int, c_void_p, c_size_t, c_int, c_void_p],
+    ),
+    "pt_grouped_gemm_fp8_vec_variable_k_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_i64]),
+    "pt_grouped_gemm_fp8_vec_variable_k": (
+        c_int,
+        [c_void_p, c_int, c_void_p, c_i64, c_void_p, c_int, c_void_p, c_i64, c_void_p, c_int, c_void_p, c_i64, c_i64, c_i64,
+         c_i64, c_int, c_int, c_void_p, c_size_t, c_int, c_void_p],
+    ),
     "pt_grouped_quantize_mx": (
         c_int,
         [c_void_p, c_int, c_i64, c_i64, c_int, c_void_p, c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_void_p, c_void_p,

@@ -5,8 +5,8 @@ on top of ``pt_grouped_gemm_fp8`` and ``pt_grouped_gemm_fp8_variable_k``.
 
 One backend exists here, so ``default_backend``, ``num_cu`` and ``maybe_pre_sync`` are accepted
 and ignored (the kernel is persistent over all CUs and never needs the group sizes on the
-host). BLOCKWISE (fp32 scales per 128 block) and MX_BLOCKWISE (E8M0 bytes per 32 elements,
-MXFP8) are the granularities these kernels implement.
+host). TENSORWISE / ROWWISE (vector scales applied in the epilogue), BLOCKWISE (fp32 scales per
+128 block) and MX_BLOCKWISE (E8M0 bytes per 32 elements, MXFP8) are implemented.
 """
 
 from __future__ import annotations
@@ -32,8 +32,80 @@ def _check(cond, msg):
 def _require_blockwise(granularity: int):
     if ScalingGranularity(granularity) != ScalingGranularity.BLOCKWISE:
         raise NotImplementedError(
-            f"grouped FP8 GEMM: only BLOCKWISE and MX_BLOCKWISE scaling are implemented, got {ScalingGranularity(granularity)}"
+            f"grouped FP8 GEMM: unknown granularity {ScalingGranularity(granularity)}"
         )
+
+
+def _is_vec(granularity: int) -> bool:
+    return ScalingGranularity(granularity) in (ScalingGranularity.TENSORWISE, ScalingGranularity.ROWWISE)
+
+
+def _vec_stride(scale: torch.Tensor, n: int, what: str) -> int:
+    """Stride (in floats) of a TENSORWISE (one element) or ROWWISE (``n`` elements) scale."""
+    _check(scale.dtype == torch.float32, f"{what} must be float32")
+    if scale.numel() == 1:
+        return 0
+    _check(scale.numel() == n, f"{what} must hold 1 or {n} elements, got {scale.numel()}")
+    return 1
+
+
+def _grouped_vec(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, out_dtype):
+    """TENSORWISE / ROWWISE row groups: ``out[rows of g] = (a[rows of g] @ op(b[g])) * sa[m] * sb[g, n]``."""
+    _check(not trans_a, "Only trans_a=False is supported.")
+    N.require_cuda(a, b, a_scales, b_scales, group_offs)
+    _check(a.dim() == 2 and b.dim() == 3, "a must be 2-D and b 3-D")
+    _check(a.dtype in _FP8 and b.dtype in _FP8, "operands must be float8_e4m3fn / float8_e5m2")
+    _check(out_dtype in (torch.float16, torch.bfloat16, torch.float32), "out_dtype must be float16, bfloat16 or float32")
+    a, b = a.contiguous(), b.contiguous()
+    a_scales, b_scales = a_scales.contiguous(), b_scales.contiguous()
+    G = b.shape[0]
+    M, K = a.shape
+    Nn, Kb = (b.shape[1], b.shape[2]) if trans_b else (b.shape[2], b.shape[1])
+    _check(K == Kb, f"reduction dims differ: {K} vs {Kb}")
+    _check(group_offs.dtype == torch.int64 and group_offs.numel() == G + 1, "group_offs must be int64 [G + 1]")
+    sa = _vec_stride(a_scales, M, "a_scales")
+    sb = 0 if b_scales.numel() == 1 else 1
+    _check(b_scales.dtype == torch.float32 and b_scales.numel() in (1, G * Nn), f"b_scales must hold 1 or G * N = {G * Nn} elements")
+    out = torch.empty((M, Nn), dtype=out_dtype, device=a.device)
+    lib = N.lib()
+    ws_bytes = lib.pt_grouped_gemm_fp8_vec_workspace_bytes(G, M, Nn, K, int(trans_b))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
+    N.check(
+        lib.pt_grouped_gemm_fp8_vec(
+            N.ptr(a), N.dtype_code(a.dtype), N.ptr(a_scales), sa, N.ptr(b), N.dtype_code(b.dtype), N.ptr(b_scales), sb,
+            Nn if sb else 0, N.ptr(out), N.dtype_code(out.dtype), N.ptr(group_offs.contiguous()), G, M, M, Nn, K,
+            int(trans_b), N.ptr(ws), ws_bytes, MX_TILE_CFG, N.stream_of(a),
+        )
+    )
+    return out
+
+
+def _variable_k_vec(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, accumulate):
+    """TENSORWISE / ROWWISE variable K: ``out[g] = (a[rows of g]^T @ b[rows of g]) * sa[i] * sb[j]``
+    over tightly packed groups (scales per column of ``a`` / ``b``, or scalars)."""
+    _check(trans_a and not trans_b, "variable-K grouped GEMM computes a^T @ b (trans_a=True, trans_b=False)")
+    N.require_cuda(a, b, a_scales, b_scales, group_offs, out)
+    _check(a.dim() == 2 and b.dim() == 2 and a.shape[0] == b.shape[0], "a and b must be 2-D with the same row count")
+    _check(a.dtype in _FP8 and b.dtype in _FP8, "operands must be float8_e4m3fn / float8_e5m2")
+    a, b = a.contiguous(), b.contiguous()
+    a_scales, b_scales = a_scales.contiguous(), b_scales.contiguous()
+    M, Ml = a.shape
+    Nr = b.shape[1]
+    G = group_offs.numel() - 1
+    sl, sr = _vec_stride(a_scales, Ml, "a_scales"), _vec_stride(b_scales, Nr, "b_scales")
+    want = (G, Nr, Ml) if trans_c else (G, Ml, Nr)
+    _check(tuple(out.shape) == want and out.is_contiguous(), f"out must be a contiguous {want} tensor")
+    lib = N.lib()
+    ws_bytes = lib.pt_grouped_gemm_fp8_vec_variable_k_workspace_bytes(G, M, Ml, Nr)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=a.device)
+    N.check(
+        lib.pt_grouped_gemm_fp8_vec_variable_k(
+            N.ptr(a), N.dtype_code(a.dtype), N.ptr(a_scales), sl, N.ptr(b), N.dtype_code(b.dtype), N.ptr(b_scales), sr,
+            N.ptr(out), N.dtype_code(out.dtype), N.ptr(group_offs.contiguous()), G, M, Ml, Nr, int(trans_c),
+            int(accumulate), N.ptr(ws), ws_bytes, MX_TILE_CFG, N.stream_of(a),
+        )
+    )
+    return out
 
 
 def _is_mx(granularity: int) -> bool:
@@ -124,6 +196,9 @@ def grouped_gemm_fp8_impl(
     or ``[G, K, N]`` fp8 with 128 x 128 tile scales."""
     if _is_mx(granularity):
         return _grouped_mx(a, b, a_scales, b_scales, group_offs, group_offs_out, trans_a, trans_b, out_dtype)
+    if _is_vec(granularity):
+        _check(group_offs_out is None, "group_offs_out belongs to the MX grouped path")
+        return _grouped_vec(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, out_dtype)
     _require_blockwise(granularity)
     _check(not trans_a, "Only trans_a=False is supported.")
     _check(group_offs_out is None, "group_offs_out belongs to the MX grouped path")
@@ -219,6 +294,10 @@ def grouped_gemm_fp8_variable_k_impl(
         shape = (G, b.shape[0], a.shape[0]) if trans_c else (G, a.shape[0], b.shape[0])
         out = torch.empty(shape, dtype=out_dtype, device=a.device)
         return _variable_k_mx(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, False)
+    if _is_vec(granularity):
+        shape = (G, b.shape[1], a.shape[1]) if trans_c else (G, a.shape[1], b.shape[1])
+        out = torch.empty(shape, dtype=out_dtype, device=a.device)
+        return _variable_k_vec(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, False)
     _require_blockwise(granularity)
     shape = (G, b.shape[1], a.shape[1]) if trans_c else (G, a.shape[1], b.shape[1])
     out = torch.empty(shape, dtype=out_dtype, device=a.device)
@@ -258,6 +337,9 @@ def grouped_gemm_fp8_variable_k_accum_impl(
     """Same product, added into ``out`` in the GEMM epilogue (beta = 1)."""
     if _is_mx(granularity):
         _variable_k_mx(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, True)
+        return
+    if _is_vec(granularity):
+        _variable_k_vec(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, True)
         return
     _require_blockwise(granularity)
     _variable_k(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, True)

@@ -1,6 +1,10 @@
 """``grouped_gemm_fp8``: MoE grouped linear layer in FP8 with autograd
 (reference: primus_turbo/pytorch/ops/grouped_gemm_fp8.py:99-265,853-960).
 
+TENSORWISE / ROWWISE (reference :265-603): the packed rows of all groups are quantized as one
+tensor (one scale, or one per token row / weight row); the vector scales are applied in the GEMM
+epilogue.
+
 BLOCKWISE (128): one fused pass over the bf16 activation yields the row quantization (forward /
 dgrad operand) and the segment-padded column quantization (wgrad operand); the weight is
 quantized in 128 x 128 tiles that serve forward and backward unchanged.
@@ -125,6 +129,96 @@ class FP8GroupedGemmBlockFunc(torch.autograd.Function):
         return grad_a, grad_b, None, None, None, None, None, None, None, None, None
 
 
+def _quantize_plain(x, config, fwd: bool, axis: int) -> QuantizedTensor:
+    """TENSORWISE / ROWWISE quantization treats the packed rows of all groups as one tensor
+    (reference: core/quantized_tensor.py:309-325)."""
+    if isinstance(x, QuantizedTensor):
+        check_quantized_tensor(x, config, axis=None if config.granularity == ScalingGranularity.TENSORWISE else axis)
+        return x
+    return QuantizedTensor.quantize(x.contiguous(), _get_fp8_dtype(config.format, fwd), config.granularity, axis=axis,
+                                    block_size=config.block_size)
+
+
+class FP8GroupedGemmRowFunc(torch.autograd.Function):
+    """ROWWISE grouped GEMM autograd (reference :265-447): activations scaled per token row, weights
+    per output row of every expert; the operands of the backward GEMMs are re-quantized along
+    their other axis from the de-quantized forward operands."""
+
+    @staticmethod
+    def forward(ctx, a, b, a_t, b_t, group_lens, group_offs, trans_b, out_dtype, config, num_cu,
+                fuse_bgrad_accum_pattern=None):
+        fuse_bgrad_accum, main_grad = _setup_fused_grad_accum(b, fuse_bgrad_accum_pattern)
+        assert config.granularity == ScalingGranularity.ROWWISE
+        b_row_axis, b_col_axis = (-1, -2) if trans_b else (-2, -1)
+        qa = _quantize_plain(a, config, True, -1)
+        qb = _quantize_plain(b, config, True, b_row_axis)
+        gran = config.granularity.value
+        out = grouped_gemm_fp8_impl(qa.qdata, qb.qdata, qa.scale_inv, qb.scale_inv, group_lens, group_offs, False, trans_b,
+                                    out_dtype, gran, num_cu, _NATIVE)
+        if any(ctx.needs_input_grad[:2]):
+            def other_axis(q, given, axis):
+                if given is not None:
+                    assert isinstance(given, QuantizedTensor)
+                    return given
+                return QuantizedTensor.quantize(q.dequantize(), q.real_dtype, config.granularity, axis=axis,
+                                                block_size=config.block_size)
+
+            qa_t, qb_t = other_axis(qa, a_t, -2), other_axis(qb, b_t, b_col_axis)
+            ctx.save_for_backward(qa_t.qdata, qb_t.qdata, qa_t.scale_inv, qb_t.scale_inv, group_lens, group_offs)
+        ctx.meta = (trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        grad_out = _ensure_contiguous_grad_out(grad_out)
+        a_col, b_col, a_col_s, b_col_s, group_lens, group_offs = ctx.saved_tensors
+        trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad = ctx.meta
+        gran = config.granularity.value
+        g_row = _quantize_plain(grad_out, config, False, -1)
+        grad_a = grouped_gemm_fp8_impl(g_row.qdata, b_col, g_row.scale_inv, b_col_s, group_lens, group_offs, False,
+                                       not trans_b, out_dtype, gran, num_cu, _NATIVE)
+        g_col = _quantize_plain(grad_out, config, False, -2)
+        grad_b = _grouped_gemm_fp8_variable_k_impl_wrapper(
+            a_col, g_col.qdata, a_col_s, g_col.scale_inv, group_lens, group_offs, True, False, trans_b, out_dtype, gran,
+            num_cu, _NATIVE, inplace_add_to_out=fuse_bgrad_accum, out=main_grad,
+        )
+        return grad_a, grad_b, None, None, None, None, None, None, None, None, None
+
+
+class FP8GroupedGemmTensorFunc(torch.autograd.Function):
+    """TENSORWISE grouped GEMM autograd (reference :450-603): one scale per tensor; backward reuses
+    the forward's quantized operands."""
+
+    @staticmethod
+    def forward(ctx, a, b, a_t, b_t, group_lens, group_offs, trans_b, out_dtype, config, num_cu,
+                fuse_bgrad_accum_pattern=None):
+        fuse_bgrad_accum, main_grad = _setup_fused_grad_accum(b, fuse_bgrad_accum_pattern)
+        assert config.granularity == ScalingGranularity.TENSORWISE
+        qa = _quantize_plain(a, config, True, -1)
+        qb = _quantize_plain(b, config, True, -1)
+        out = grouped_gemm_fp8_impl(qa.qdata, qb.qdata, qa.scale_inv, qb.scale_inv, group_lens, group_offs, False, trans_b,
+                                    out_dtype, config.granularity.value, num_cu, _NATIVE)
+        if any(ctx.needs_input_grad[:2]):
+            ctx.save_for_backward(qa.qdata, qb.qdata, qa.scale_inv, qb.scale_inv, group_lens, group_offs)
+        ctx.meta = (trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        grad_out = _ensure_contiguous_grad_out(grad_out)
+        a_q, b_q, a_s, b_s, group_lens, group_offs = ctx.saved_tensors
+        trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad = ctx.meta
+        gran = config.granularity.value
+        g = _quantize_plain(grad_out, config, False, -1)
+        grad_a = grouped_gemm_fp8_impl(g.qdata, b_q, g.scale_inv, b_s, group_lens, group_offs, False, not trans_b,
+                                       out_dtype, gran, num_cu, _NATIVE)
+        grad_b = _grouped_gemm_fp8_variable_k_impl_wrapper(
+            a_q, g.qdata, a_s, g.scale_inv, group_lens, group_offs, True, False, trans_b, out_dtype, gran, num_cu, _NATIVE,
+            inplace_add_to_out=fuse_bgrad_accum, out=main_grad,
+        )
+        return grad_a, grad_b, None, None, None, None, None, None, None, None, None
+
+
 class FP8GroupedGemmMXFunc(torch.autograd.Function):
     """MX_BLOCKWISE (MXFP8) grouped GEMM autograd."""
 
@@ -208,10 +302,15 @@ def grouped_gemm_fp8(
     if config.granularity == ScalingGranularity.BLOCKWISE:
         return FP8GroupedGemmBlockFunc.apply(a_data, b_data, a_data_t, b_data_t, group_lens, group_offs, trans_b,
                                              out_dtype, config, num_cu, fuse_bgrad_accum_pattern)
+    if config.granularity == ScalingGranularity.ROWWISE:
+        return FP8GroupedGemmRowFunc.apply(a_data, b_data, a_data_t, b_data_t, group_lens, group_offs, trans_b,
+                                           out_dtype, config, num_cu, fuse_bgrad_accum_pattern)
+    if config.granularity == ScalingGranularity.TENSORWISE:
+        return FP8GroupedGemmTensorFunc.apply(a_data, b_data, a_data_t, b_data_t, group_lens, group_offs, trans_b,
+                                              out_dtype, config, num_cu, fuse_bgrad_accum_pattern)
     if config.granularity == ScalingGranularity.MX_BLOCKWISE:
         return FP8GroupedGemmMXFunc.apply(a_data, b_data, a_data_t, b_data_t, group_lens, group_offs, trans_b,
                                           out_dtype, config, num_cu, fuse_bgrad_accum_pattern)
     raise NotImplementedError(
-        f"grouped_gemm_fp8: granularity {config.granularity} is not implemented "
-        "(BLOCKWISE with block_size=128 and MX_BLOCKWISE are)"
+        f"grouped_gemm_fp8: unknown granularity {config.granularity}"
     )
