@@ -22,13 +22,13 @@ FP8_PEAK_TFLOPS = 5000.0
 # summarised under profiles/. (fetched, written) in MiB.
 TRAFFIC_MIB = {
     "gemm_fp8_rowwise": (779.1, 151.6),
-    "gemm_fp8_blockwise": (493.5, 224.0),
-    "gemm_fp8_blockwise_k7168": (1434.1, 128.0),
-    "gemm_fp8_blockwise_8192": (1482.7, 128.0),
+    "gemm_fp8_blockwise": (567.5, 224.0),
+    "gemm_fp8_blockwise_k7168": (1155.2, 128.0),
+    "gemm_fp8_blockwise_8192": (1326.5, 128.0),
     "gemm_mxfp4": (3332.6, 754.7),
     "gemm_mxfp8": (6488.6, 700.2),
-    "grouped_gemm_fp8": (8922.6, 256.1),  # forward launches only
-    "grouped_gemm_fp8_down": (4180.1, 448.2),
+    "grouped_gemm_fp8": (5372.6, 256.1),  # forward launches only
+    "grouped_gemm_fp8_down": (2439.0, 448.2),
 }
 
 
