@@ -15,6 +15,7 @@ import time
 import torch
 
 FP8_PEAK_TFLOPS = 5000.0
+FP4_PEAK_TFLOPS = 10100.0
 
 # HBM-side bytes per launch of each workload's dominant kernel: rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a plain copy of
@@ -238,7 +239,7 @@ class GemmMx(_GemmBase):
         kind = "mxfp4_e2m1" if fp4 else "mxfp8_e4m3"
         self.name = f"{kind}_gemm_{M}x{N}x{K}_bf16_out (quantize A 1x32, quantize B 32x32, multiply)"
         self.dtype = ("fp4_e2m1" if fp4 else "fp8_e4m3") + " with E8M0 block scales (fp32 accumulate)"
-        self.peak = 10100.0 if fp4 else FP8_PEAK_TFLOPS
+        self.peak = FP4_PEAK_TFLOPS if fp4 else FP8_PEAK_TFLOPS
         self.dominant_name = "gemm_fp8_nt_kernel<256x256 tile, E8M0 block scales in the MFMA>"
         self.fmt = "e2m1" if fp4 else "e4m3"
         if fp4:
@@ -457,6 +458,7 @@ class GroupedGemmMxfp8(_GemmBase):
                                                                             self.gl, self.offs)
         self.wq, self.ws = qi.quantize_mxfp8_impl(self.w.detach(), torch.float8_e4m3fn, 2, 32,
                                                   scaling_recipe=ScalingRecipe(use_2d_block=True))
+        self.fmt = "e4m3"
 
     def step_work(self):
         return 3 * 2.0 * self.M * self.N * self.K
@@ -491,10 +493,10 @@ class GroupedGemmMxfp8(_GemmBase):
         for g in (live[0], live[-1]):
             n = int(min(64, self.lens[g]))
             r0, p0 = int(offs[g]), int(orow[g])
-            aq, asc = Q.mx_quant_rowwise(self.x_cpu.float().numpy()[r0 : r0 + n], "e4m3")
+            aq, asc = Q.mx_quant_rowwise(self.x_cpu.float().numpy()[r0 : r0 + n], self.fmt)
             same = same and np.array_equal(u8(self.qr)[p0 : p0 + n], aq) and np.array_equal(u8(self.sr)[p0 : p0 + n], asc)
-            w_deq = Q.mx_dequant(u8(self.wq[g]), u8(self.ws[g]), "e4m3")
-            ref = OG.gemm_dequantized(Q.mx_dequant(aq, asc, "e4m3"), w_deq, trans_b=True)
+            w_deq = Q.mx_dequant(u8(self.wq[g]), u8(self.ws[g]), self.fmt)
+            ref = OG.gemm_dequantized(Q.mx_dequant(aq, asc, self.fmt), w_deq, trans_b=True)
             ref_t = torch.from_numpy(np.ascontiguousarray(ref, dtype=np.float32)).to(torch.bfloat16).float().numpy()
             rel = max(rel, OG.max_rel_err(ref_t, out[r0 : r0 + n]))
             cos = min(cos, OG.cosine(out[r0 : r0 + n], ref_t))
@@ -513,14 +515,59 @@ class GroupedGemmMxfp8(_GemmBase):
         a = self.x_cpu[r0 : r0 + 256].float().numpy()
         b = self.w_cpu[g, :2048].float().numpy()
         t0 = time.perf_counter()
-        aq, asc = Q.mx_quant_rowwise(a, "e4m3")
-        bq, bsc = Q.mx_quant_rowwise(b, "e4m3", use_2d_block=True)
-        y = Q.mx_dequant(aq, asc, "e4m3") @ Q.mx_dequant(bq, bsc, "e4m3").T
+        aq, asc = Q.mx_quant_rowwise(a, self.fmt)
+        bq, bsc = Q.mx_quant_rowwise(b, self.fmt, use_2d_block=True)
+        y = Q.mx_dequant(aq, asc, self.fmt) @ Q.mx_dequant(bq, bsc, self.fmt).T
         dt = time.perf_counter() - t0
         del y
         return dict(value=round(2.0 * 256 * 2048 * self.K / dt / 1e12, 5), unit="TFLOP/s", cores=torch.get_num_threads(),
                     kind="port", sample=f"256 tokens of the largest expert against 2048 output features (MX quantize both, "
                     f"dequantize, fp32 matmul), {dt:.1f} s, {os.cpu_count()} logical CPUs visible")
+
+
+class GroupedGemmMxfp4(GroupedGemmMxfp8):
+    """The same MoE configuration through the grouped MXFP4 path: rows quantized in place,
+    transposed columns padded to 256 tokens per expert, packed E2M1 operands."""
+
+    dominant_name = "gemm_fp8_nt_kernel<256x256 tile, row groups, MXFP4 operands, E8M0 block scales in the MFMA> (forward)"
+    dtype = "fp4_e2m1 with E8M0 block scales (fp32 accumulate)"
+    peak = FP4_PEAK_TFLOPS
+
+    def __init__(self, dev, N=4096, K=7168, groups=32, tokens=32768):
+        import primus_turbo.pytorch as turbo
+        from primus_turbo.pytorch.core.low_precision import Float4QuantConfig, ScalingGranularity, ScalingRecipe, float4_e2m1fn_x2
+        from primus_turbo.pytorch.kernels.grouped_gemm import grouped_gemm_fp4_impl as gg
+        from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+        self.turbo, self.G, self.gg, self.qi = turbo, ScalingGranularity, gg, qi
+        self.M, self.N, self.K, self.groups = tokens, N, K, groups
+        self.name = (f"moe_grouped_gemm_mxfp4_{groups}experts_{tokens}tokens_zipf1.2_k{K}_n{N} "
+                     "(forward + dgrad + wgrad, quantizers included)")
+        self.cfg = Float4QuantConfig()
+        self.lens = _zipf_group_lens(groups, tokens, 7)
+        self.gl = torch.from_numpy(self.lens).to(dev)
+        self.offs = torch.ops.primus_turbo_cpp_extension.grouped_gemm_compute_offs(self.gl)
+        self.x_cpu = _randn_bf16((tokens, K), 7, 1.0)
+        self.w_cpu = _randn_bf16((groups, N, K), 8, 1.0)
+        self.x = self.x_cpu.to(dev).requires_grad_(True)
+        self.w = self.w_cpu.to(dev).requires_grad_(True)
+        self.dy = _randn_bf16((tokens, N), 9, 1.0).to(dev)
+        self.qr, self.sr, _, self.offs_row = qi.grouped_quantize_mxfp4_impl(self.x.detach(), float4_e2m1fn_x2, 1, 32,
+                                                                            self.gl, self.offs)
+        self.wq, self.ws = qi.quantize_mxfp4_impl(self.w.detach(), float4_e2m1fn_x2, 2, 32,
+                                                  scaling_recipe=ScalingRecipe(use_2d_block=True))
+        self.fmt = "e2m1"
+
+    def step(self):
+        self.x.grad = None
+        self.w.grad = None
+        y = self.turbo.ops.grouped_gemm_fp4(self.x, self.w, self.gl, self.offs, trans_b=True, config=self.cfg)
+        y.backward(self.dy)
+        return y
+
+    def dominant(self):
+        return self.gg.grouped_gemm_fp4_impl(self.qr, self.wq, self.sr, self.ws, self.gl, self.offs_row, False, True,
+                                             torch.bfloat16, self.G.MX_BLOCKWISE.value, None, 0, False, self.offs)
 
 
 def _keyed(key, make):
@@ -545,6 +592,8 @@ def register(workloads):
     workloads["grouped_gemm_fp8_down"] = lambda dev: GroupedGemmFp8(dev, 7168, 2048)
     workloads["grouped_gemm_mxfp8"] = lambda dev: GroupedGemmMxfp8(dev, 4096, 7168)
     workloads["grouped_gemm_mxfp8_down"] = lambda dev: GroupedGemmMxfp8(dev, 7168, 2048)
+    workloads["grouped_gemm_mxfp4"] = lambda dev: GroupedGemmMxfp4(dev, 4096, 7168)
+    workloads["grouped_gemm_mxfp4_down"] = lambda dev: GroupedGemmMxfp4(dev, 7168, 2048)
     for key in list(workloads):
         if key in TRAFFIC_MIB:
             workloads[key] = _keyed(key, workloads[key])

@@ -359,33 +359,43 @@ PT_API int pt_grouped_gemm_fp8_vec_variable_k(const void *lhs, int lhs_dtype, co
  *   128 rows with zero data, scale byte 0); col_ld is a multiple of 128 >= col_offs_padded[G];
  *   columns from col_offs_padded[G] on are not written.
  * Either pair may be NULL. The padded offsets come from pt_compute_group_offs (align 32 / 128).
+ * With q_dtype e2m1x2 it is the grouped MXFP4 quantizer (grouped_quantize_mxfp4[_dual],
+ * quantization.cpp:1209-1378; default dispatch flydsl/quantization/mxfp4_grouped_quant.py:320-349):
+ * two codes per byte, rows kept tight (row_offs_padded NULL) and column groups padded to 256.
  *
  * pt_grouped_gemm_mx replaces primus_turbo::grouped_gemm_fp8_impl for MX_BLOCKWISE
  * (kernels/grouped_gemm/grouped_gemm_fp8_impl.py:888-930 with group_offs_out; caller
- * ops/grouped_gemm_fp8.py:726-741,786-801), forward and dgrad:
+ * ops/grouped_gemm_fp8.py:726-741,786-801) and primus_turbo::grouped_gemm_fp4_impl
+ * (kernels/grouped_gemm/grouped_gemm_fp4_impl.py; caller ops/grouped_gemm_fp4.py:226-240,
+ * 279-293), forward and dgrad:
  *   out[oo[g] : oo[g] + len_g, :] = A[o[g] : o[g] + len_g, :] . B[g]^T,   out[oo[G] : out_rows] = 0
- * A [a_rows, K] MXFP8 codes with scale bytes [a_rows, sa_ld], B [G, N, K] with [G, N, sb_ld];
- * o = group_offs (rows of A, e.g. the padded row layout above), oo = group_offs_out (rows of the
- * output, packed tight; NULL = the same as o); len_g = oo[g + 1] - oo[g] when oo is given.
- * K is a multiple of 128 and at least 512.
+ * A [a_rows, lda bytes] MXFP8 (or, both operands, packed MXFP4) codes with scale bytes
+ * [a_rows, sa_ld], B [G, N, ldb bytes] with [G, N, sb_ld]; o = group_offs (rows of A, e.g. the
+ * padded row layout above), oo = group_offs_out (rows of the output, packed tight; NULL = the
+ * same as o); len_g = oo[g + 1] - oo[g] when oo is given. K counts elements (a multiple of 32);
+ * lda == ldb is a multiple of 128 bytes, at least 512, and the bytes of a row behind its K
+ * codes are zero.
  *
  * pt_grouped_gemm_mx_variable_k replaces primus_turbo::grouped_gemm_fp8_variable_k_impl for
- * MX_BLOCKWISE (grouped_gemm_fp8_impl.py:933-974; caller ops/grouped_gemm_fp8.py:809-825), wgrad:
+ * MX_BLOCKWISE (grouped_gemm_fp8_impl.py:933-974; caller ops/grouped_gemm_fp8.py:809-825) and
+ * primus_turbo::grouped_gemm_fp4_variable_k[_accum]_impl (caller ops/grouped_gemm_fp4.py:56-98,
+ * 296-312), wgrad:
  *   C[g] (+)= L[:, p[g] : p[g+1]] . R[:, p[g] : p[g+1]]^T      C is [G, Ml, Nr]
- * L [Ml, ld] and R [Nr, ld] are transposed column-direction outputs of pt_grouped_quantize_mx
- * with scale bytes [rows, ld / 32]; p = the 128-padded group offsets. An empty group yields
- * C[g] = 0 (or leaves it unchanged when accumulating). No workspace: both operands are read in
- * place. */
+ * L [Ml, ld] and R [Nr, ld] (ld in elements) are transposed column-direction outputs of
+ * pt_grouped_quantize_mx with scale bytes [rows, ld / 32]; p = the group offsets in elements,
+ * padded to whole 128-byte slabs (128 elements, MXFP4: 256). An empty group yields C[g] = 0 (or
+ * leaves it unchanged when accumulating). No workspace: both operands are read in place. */
 PT_API int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype,
                                   const int64_t *group_offs, const int64_t *row_offs_padded,
                                   const int64_t *col_offs_padded, int64_t G, void *row_q,
                                   void *row_scale, void *col_q, void *col_scale, int64_t col_ld,
                                   void *stream);
-PT_API int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, int64_t sa_ld,
-                              const void *b, int b_dtype, const void *b_scale, int64_t sb_ld, void *c,
-                              int c_dtype, const int64_t *group_offs, const int64_t *group_offs_out,
-                              int64_t G, int64_t a_rows, int64_t out_rows, int64_t N, int64_t K,
-                              int tile_cfg, void *stream);
+PT_API int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, int64_t lda,
+                              int64_t sa_ld, const void *b, int b_dtype, const void *b_scale,
+                              int64_t ldb, int64_t sb_ld, void *c, int c_dtype,
+                              const int64_t *group_offs, const int64_t *group_offs_out, int64_t G,
+                              int64_t a_rows, int64_t out_rows, int64_t N, int64_t K, int tile_cfg,
+                              void *stream);
 PT_API int pt_grouped_gemm_mx_variable_k(const void *lhs, int lhs_dtype, const void *lhs_scale,
                                          const void *rhs, int rhs_dtype, const void *rhs_scale, void *c,
                                          int c_dtype, const int64_t *group_offs, int64_t G, int64_t Ml,

@@ -344,7 +344,9 @@ def mx_grouped_quant(x: np.ndarray, group_lens: np.ndarray, fmt, row_align: int 
     /root/reference/primus_turbo/pytorch/kernels/quantization/quantization_impl.py:572-700:
     every group is virtually zero-padded along M, to ``row_align`` rows for the row direction
     and to ``col_align`` rows for the column direction; per-block numerics are those of the
-    dense MX quantizer). Composition of ``mx_quant_rowwise`` / ``mx_quant_colwise`` per group
+    dense MX quantizer; the grouped MXFP4 quantizer, quantization_impl.py:657-811 with the layout
+    of /root/reference/primus_turbo/flydsl/quantization/mxfp4_grouped_quant.py:320-349, is
+    ``row_align=1, col_align=256``). Composition of ``mx_quant_rowwise`` / ``mx_quant_colwise`` per group
     (pinned there); the padded placement is pinned by the round trip through ``mx_dequant``
     against the dense quantizer of each group.
 

@@ -63,8 +63,9 @@ struct GemmArgs {
     // Grouped problems (MoE experts); group_offs is a device array of G + 1 int64 prefix sums.
     //   GROUP_ROWS: rows [offs[g], offs[g+1]) of A and C belong to group g, which multiplies
     //               with B + g * b_gstride (scales sB + g * sb_gstride); M is the row count of A.
-    //   GROUP_K   : group g reduces over K columns [offs[g], offs[g+1]) of A and B (multiples
-    //               of 128) into C + g * c_gstride; scales start at K block offs[g] / 128.
+    //   GROUP_K   : group g reduces over K elements [offs[g], offs[g+1]) of A and B (whole
+    //               128-byte slabs: multiples of 128, MXFP4 256) into C + g * c_gstride; scales
+    //               start at the slab offs[g] / 128 (MXFP4: / 256).
     int            gmode;
     int            G;
     const int64_t *group_offs;
@@ -375,7 +376,7 @@ struct TileCtx {
 
 // GROUP_ROWS: prefix[g] = number of tiles of the groups before g (in LDS), `g` is a search
 // hint that only moves forward as a workgroup walks its tiles.
-template <int BM, int BN, int GMODE>
+template <int BM, int BN, int GMODE, bool F4 = false>
 __device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile, const int *prefix, int &g) {
     TileCtx t;
     int     tm, tn;
@@ -415,7 +416,8 @@ __device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile, const 
         const int per = a.tiles_m * a.tiles_n;
         g             = tile / per;
         tile_coords_local(tile - g * per, a.tiles_m, a.tiles_n, tm, tn);
-        const int64_t lo = a.group_offs[g], hi = a.group_offs[g + 1];
+        // K ranges are given in elements; two E2M1 codes share a byte
+        const int64_t lo = a.group_offs[g] >> (F4 ? 1 : 0), hi = a.group_offs[g + 1] >> (F4 ? 1 : 0);
         t.m0    = static_cast<int64_t>(tm) * BM;
         t.m_end = a.M;
         t.Ag    = a.A + t.m0 * a.lda + lo;
@@ -529,7 +531,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     if (tile >= total || (XPIPE && KT_ALL <= 2))
         return;
     int     g_cur = 0, g_nxt = 0;
-    TileCtx cur_t = make_tile<BM, BN, GMODE>(a, tile, prefix, g_cur);
+    TileCtx cur_t = make_tile<BM, BN, GMODE, FA == 4>(a, tile, prefix, g_cur);
     g_nxt         = g_cur;
 
     // ---- loader: two slabs ahead of the MFMAs ----
@@ -751,7 +753,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         const int next_tile = tile + gridDim.x;
         nxt_t               = cur_t;
         if (next_tile < total)
-            nxt_t = make_tile<BM, BN, GMODE>(a, next_tile, prefix, g_nxt);
+            nxt_t = make_tile<BM, BN, GMODE, FA == 4>(a, next_tile, prefix, g_nxt);
         const int KT = XPIPE ? KT_ALL : cur_t.KT;
         if constexpr (!XPIPE) {
             if (KT > 0)

@@ -1,14 +1,17 @@
-// MoE grouped MXFP8 GEMM on gfx950 (E8M0 scale per 32 elements of K, applied by the matrix core):
+// MoE grouped MXFP8 / MXFP4 GEMM on gfx950 (E8M0 scale per 32 elements of K, applied by the
+// matrix core):
 //   * row groups (forward / dgrad): out[rows of g] = A[rows of g] . B[g]^T, A [rows, K] and B
 //     [G, N, K] both K-contiguous; the rows of A may sit in a per-group padded layout while the
 //     output is packed tight (two offset arrays);
 //   * variable K (wgrad): C[g] = L[:, K range of g] . R[:, K range of g]^T with both operands
 //     K-contiguous over the segment-padded token axis (the transposed column-direction output of
-//     the grouped MX quantizer), K ranges on multiples of 128.
+//     the grouped MX quantizer), K ranges on whole 128-byte slabs (multiples of 128 elements,
+//     MXFP4 256).
 // Semantics of Primus-Turbo's grouped MXFP8 path (primus_turbo/pytorch/ops/grouped_gemm_fp8.py:
 // 604-840: forward and dgrad are one NT product per group over the padded rows with
 // group_offs_out packing the result, wgrad is a variable-K NT product over the 128-padded
-// column-direction operands).
+// column-direction operands) and of its grouped MXFP4 path (ops/grouped_gemm_fp4.py:101-309:
+// the same three products over tight rows and 256-padded column-direction operands).
 #include "gemm_fp8_kernel.h"
 
 namespace pt {
@@ -26,6 +29,8 @@ template <int GMODE, int FA, int FB> static int launch_mxg_tiles(const GemmArgs 
 }
 
 template <int GMODE> static int launch_mxg(const GemmArgs &a, int fa, int fb, int tile_cfg, hipStream_t stream) {
+    if (fa == 4)
+        return launch_mxg_tiles<GMODE, 4, 4>(a, tile_cfg, stream);
     if (fa == 0 && fb == 0)
         return launch_mxg_tiles<GMODE, 0, 0>(a, tile_cfg, stream);
     if (fa == 0 && fb == 1)
@@ -60,15 +65,20 @@ using namespace pt;
 
 extern "C" {
 
-int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, int64_t sa_ld, const void *b, int b_dtype,
-                       const void *b_scale, int64_t sb_ld, void *c, int c_dtype, const int64_t *group_offs,
-                       const int64_t *group_offs_out, int64_t G, int64_t a_rows, int64_t out_rows, int64_t N, int64_t K,
-                       int tile_cfg, void *stream) {
-    PT_REQUIRE(is_fp8_dtype(a_dtype) && is_fp8_dtype(b_dtype), "operands must be e4m3 or e5m2");
+int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, int64_t lda, int64_t sa_ld, const void *b,
+                       int b_dtype, const void *b_scale, int64_t ldb, int64_t sb_ld, void *c, int c_dtype,
+                       const int64_t *group_offs, const int64_t *group_offs_out, int64_t G, int64_t a_rows,
+                       int64_t out_rows, int64_t N, int64_t K, int tile_cfg, void *stream) {
+    const bool fp4 = a_dtype == PT_DTYPE_E2M1X2;
+    PT_REQUIRE(fp4 ? b_dtype == PT_DTYPE_E2M1X2 : (is_fp8_dtype(a_dtype) && is_fp8_dtype(b_dtype)),
+               "operands must both be fp8 (e4m3 / e5m2) or both e2m1x2");
     PT_REQUIRE(is_hp_dtype(c_dtype), "output must be bf16, fp16 or fp32");
     PT_REQUIRE(G >= 0 && a_rows >= 0 && out_rows >= 0 && N >= 0, "bad dimensions");
-    PT_REQUIRE(K >= GEMM_MIN_SLABS * KSTEP && K % KSTEP == 0, "K must be a multiple of 128 and at least 512");
-    PT_REQUIRE(K < (1LL << 24), "K must be below 2^24");
+    PT_REQUIRE(K > 0 && K % 32 == 0, "K must be a positive multiple of 32");
+    const int64_t kbytes = fp4 ? K / 2 : K;
+    PT_REQUIRE(lda == ldb && lda >= kbytes && lda % KSTEP == 0 && lda >= GEMM_MIN_SLABS * KSTEP,
+               "row pitches must be equal multiples of 128 bytes, at least 512, that hold K");
+    PT_REQUIRE(lda < (1LL << 24), "K must be below 2^24");
     PT_REQUIRE(tile_cfg >= 0 && tile_cfg <= 3, "tile_cfg must be 0..3");
     PT_REQUIRE(sa_ld >= K / 32 && sb_ld >= K / 32 && sa_ld % 4 == 0 && sb_ld % 4 == 0,
                "scale rows must hold K / 32 bytes and be 4-byte multiples");
@@ -88,9 +98,9 @@ int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, int64_t 
         g.sB             = static_cast<const float *>(b_scale); // E8M0 bytes, [G, N, sb_ld]
         g.M              = a_rows;
         g.N              = N;
-        g.K              = K;
-        g.lda            = K;
-        g.ldb            = K;
+        g.K              = lda; // bytes; what lies between K and the pitch is zero
+        g.lda            = lda;
+        g.ldb            = ldb;
         g.sa_m           = sa_ld;
         g.sb_n           = sb_ld;
         g.kb_valid       = static_cast<int>(K / 32);
@@ -98,9 +108,9 @@ int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, int64_t 
         g.G              = static_cast<int>(G);
         g.group_offs     = group_offs;
         g.group_offs_out = group_offs_out;
-        g.b_gstride      = N * K;
+        g.b_gstride      = N * ldb;
         g.sb_gstride     = N * sb_ld / 4; // the kernel steps a 4-byte pointer
-        const int rc = launch_mxg<GROUP_ROWS>(g, a_dtype == PT_DTYPE_E5M2, b_dtype == PT_DTYPE_E5M2, tile_cfg, st);
+        const int rc = launch_mxg<GROUP_ROWS>(g, fp4 ? 4 : a_dtype == PT_DTYPE_E5M2, b_dtype == PT_DTYPE_E5M2, tile_cfg, st);
         if (rc != PT_OK)
             return rc;
     }
@@ -114,9 +124,12 @@ int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, int64_t 
 int pt_grouped_gemm_mx_variable_k(const void *lhs, int lhs_dtype, const void *lhs_scale, const void *rhs, int rhs_dtype,
                                   const void *rhs_scale, void *c, int c_dtype, const int64_t *group_offs, int64_t G,
                                   int64_t Ml, int64_t Nr, int64_t ld, int accumulate, int tile_cfg, void *stream) {
-    PT_REQUIRE(is_fp8_dtype(lhs_dtype) && is_fp8_dtype(rhs_dtype), "operands must be e4m3 or e5m2");
+    const bool fp4 = lhs_dtype == PT_DTYPE_E2M1X2;
+    PT_REQUIRE(fp4 ? rhs_dtype == PT_DTYPE_E2M1X2 : (is_fp8_dtype(lhs_dtype) && is_fp8_dtype(rhs_dtype)),
+               "operands must both be fp8 (e4m3 / e5m2) or both e2m1x2");
     PT_REQUIRE(is_hp_dtype(c_dtype), "output must be bf16, fp16 or fp32");
-    PT_REQUIRE(G >= 0 && Ml >= 0 && Nr >= 0 && ld >= 0 && ld % 128 == 0, "bad dimensions (ld must be a multiple of 128)");
+    PT_REQUIRE(G >= 0 && Ml >= 0 && Nr >= 0 && ld >= 0 && ld % (fp4 ? 256 : 128) == 0,
+               "bad dimensions (ld must be a multiple of 128 elements, e2m1x2: 256)");
     PT_REQUIRE(ld < (1LL << 24), "at most 2^24 padded rows");
     PT_REQUIRE(tile_cfg >= 0 && tile_cfg <= 3, "tile_cfg must be 0..3");
     if (G == 0 || Ml == 0 || Nr == 0)
@@ -132,19 +145,19 @@ int pt_grouped_gemm_mx_variable_k(const void *lhs, int lhs_dtype, const void *lh
     g.M          = Ml;
     g.N          = Nr;
     g.K          = 0; // per group
-    g.lda        = ld;
-    g.ldb        = ld;
+    g.lda        = fp4 ? ld / 2 : ld;
+    g.ldb        = g.lda;
     g.sa_m       = ld / 32;
     g.sb_n       = ld / 32;
-    g.sa_k       = 1; // a slab's four scale bytes: one step of the kernel's 4-byte scale pointer
-    g.sb_k       = 1;
+    g.sa_k       = fp4 ? 2 : 1; // a slab's four (e2m1x2: eight) scale bytes, in steps of the kernel's 4-byte scale pointer
+    g.sb_k       = g.sa_k;
     g.kb_valid   = static_cast<int>(ld / 32);
     g.out_dtype  = c_dtype;
     g.accumulate = accumulate;
     g.G          = static_cast<int>(G);
     g.group_offs = group_offs;
     g.c_gstride  = Ml * Nr;
-    return launch_mxg<GROUP_K>(g, lhs_dtype == PT_DTYPE_E5M2, rhs_dtype == PT_DTYPE_E5M2, tile_cfg,
+    return launch_mxg<GROUP_K>(g, fp4 ? 4 : lhs_dtype == PT_DTYPE_E5M2, rhs_dtype == PT_DTYPE_E5M2, tile_cfg,
                                static_cast<hipStream_t>(stream));
 }
 

@@ -127,8 +127,8 @@ _SIGNATURES = {
     ),
     "pt_grouped_gemm_mx": (
         c_int,
-        [c_void_p, c_int, c_void_p, c_i64, c_void_p, c_int, c_void_p, c_i64, c_void_p, c_int, c_void_p, c_void_p, c_i64,
-         c_i64, c_i64, c_i64, c_i64, c_int, c_void_p],
+        [c_void_p, c_int, c_void_p, c_i64, c_i64, c_void_p, c_int, c_void_p, c_i64, c_i64, c_void_p, c_int, c_void_p,
+         c_void_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_int, c_void_p],
     ),
     "pt_grouped_gemm_mx_variable_k": (
         c_int,

@@ -116,56 +116,83 @@ def _u8(t: torch.Tensor) -> torch.Tensor:
     return t.contiguous().view(torch.uint8)
 
 
+_FP4X2 = getattr(torch, "float4_e2m1fn_x2", None)
+
+
+def _mx_pitch(t: torch.Tensor, kbytes: int) -> torch.Tensor:
+    """Rows of ``t`` (uint8, last dim = ``kbytes`` K bytes) at the pitch the kernel reads: whole
+    128-byte slabs, at least four, zeros behind the data. No copy when it already is."""
+    need = max(512, -(-kbytes // 128) * 128)
+    return t if t.shape[-1] == need else torch.nn.functional.pad(t, (0, need - t.shape[-1]))
+
+
 def _grouped_mx(a, b, a_scales, b_scales, group_offs, group_offs_out, trans_a, trans_b, out_dtype):
-    """MXFP8 row groups: ``out[oo[g] : oo[g+1]] = a[o[g] : o[g] + len_g] @ b[g]^T`` with ``a`` in
+    """MX row groups: ``out[oo[g] : oo[g+1]] = a[o[g] : o[g] + len_g] @ b[g]^T`` with ``a`` in
     the (possibly per-group padded) row layout of the grouped quantizer and the output packed
-    by ``group_offs_out`` (over-allocated to the rows of ``a``; the tail is zero)."""
-    _check(not trans_a and trans_b, "MXFP8 grouped GEMM only supports trans_a=False, trans_b=True (NT layout).")
+    by ``group_offs_out`` (over-allocated to the rows of ``a``; the tail is zero). Operands are
+    both MXFP8 or both packed MXFP4."""
+    _check(not trans_a and trans_b, "MX grouped GEMM only supports trans_a=False, trans_b=True (NT layout).")
     N.require_cuda(a, b, a_scales, b_scales, group_offs)
     _check(a.dim() == 2 and b.dim() == 3, "a must be 2-D and b 3-D")
-    _check(a.dtype in _FP8 and b.dtype in _FP8, "operands must be float8_e4m3fn / float8_e5m2")
+    fp4 = _FP4X2 is not None and a.dtype == _FP4X2
+    if fp4:
+        _check(b.dtype == _FP4X2, "operands must both be float4_e2m1fn_x2")
+    else:
+        _check(a.dtype in _FP8 and b.dtype in _FP8, "operands must be float8_e4m3fn / float8_e5m2")
     _check(out_dtype in (torch.float16, torch.bfloat16, torch.float32), "out_dtype must be float16, bfloat16 or float32")
-    G, Nn, K = b.shape
+    G, Nn, kb = b.shape  # kb: K bytes of a row
     rows = a.shape[0]
-    _check(a.shape[1] == K, f"reduction dims differ: {a.shape[1]} vs {K}")
-    _check(K % 128 == 0 and K >= 512, "grouped MXFP8 GEMM needs K to be a multiple of 128 and at least 512")
+    _check(a.shape[1] == kb, f"reduction dims differ: {a.shape[1]} vs {kb}")
+    K = kb * 2 if fp4 else kb
+    _check(K % 32 == 0, "MX grouped GEMM needs K to be a multiple of 32")
+    if not fp4:
+        _check(K % 128 == 0 and K >= 512, "grouped MXFP8 GEMM needs K to be a multiple of 128 and at least 512")
     _check(group_offs.dtype == torch.int64 and group_offs.numel() == G + 1, "group_offs must be int64 [G + 1]")
     a_s, b_s = _u8(a_scales), _u8(b_scales)
     _check(a_s.dim() == 2 and a_s.shape[0] == rows and a_s.shape[1] >= K // 32, "a_scales must be [rows, K/32]")
     _check(b_s.dim() == 3 and tuple(b_s.shape[:2]) == (G, Nn) and b_s.shape[2] >= K // 32, "b_scales must be [G, N, K/32]")
-    a, b = a.contiguous(), b.contiguous()
+    _check(a_s.shape[1] % 4 == 0 and b_s.shape[2] % 4 == 0, "scale rows must be multiples of 4 bytes")
+    da, db = N.dtype_code(a.dtype), N.dtype_code(b.dtype)
+    a, b = _mx_pitch(_u8(a), kb), _mx_pitch(_u8(b), kb)
     out = torch.empty((rows, Nn), dtype=out_dtype, device=a.device)
     oo = None if group_offs_out is None else group_offs_out.contiguous()
     N.check(
         N.lib().pt_grouped_gemm_mx(
-            N.ptr(a), N.dtype_code(a.dtype), N.ptr(a_s), a_s.shape[1], N.ptr(b), N.dtype_code(b.dtype), N.ptr(b_s),
-            b_s.shape[2], N.ptr(out), N.dtype_code(out.dtype), N.ptr(group_offs.contiguous()), N.ptr(oo), G, rows, rows,
-            Nn, K, MX_TILE_CFG, N.stream_of(a),
+            N.ptr(a), da, N.ptr(a_s), a.shape[1], a_s.shape[1], N.ptr(b), db, N.ptr(b_s), b.shape[2], b_s.shape[2], N.ptr(out),
+            N.dtype_code(out.dtype), N.ptr(group_offs.contiguous()), N.ptr(oo), G, rows, rows, Nn, K, MX_TILE_CFG,
+            N.stream_of(a),
         )
     )
     return out
 
 
 def _variable_k_mx(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, accumulate):
-    """MXFP8 variable K: ``out[g] = a[:, p[g]:p[g+1]] @ b[:, p[g]:p[g+1]]^T`` over the transposed
-    column-direction outputs of the grouped quantizer (both K-contiguous already)."""
-    _check(not trans_a and not trans_b, "MXFP8 variable-K grouped GEMM takes both operands transposed already")
+    """MX variable K: ``out[g] = a[:, p[g]:p[g+1]] @ b[:, p[g]:p[g+1]]^T`` over the transposed
+    column-direction outputs of the grouped quantizer (both K-contiguous already); ``p`` counts
+    elements (multiples of 128, MXFP4 256)."""
+    _check(not trans_a and not trans_b, "MX variable-K grouped GEMM takes both operands transposed already")
     N.require_cuda(a, b, a_scales, b_scales, group_offs, out)
     _check(a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[1], "a and b must be 2-D with the same padded length")
-    _check(a.dtype in _FP8 and b.dtype in _FP8, "operands must be float8_e4m3fn / float8_e5m2")
+    fp4 = _FP4X2 is not None and a.dtype == _FP4X2
+    if fp4:
+        _check(b.dtype == _FP4X2, "operands must both be float4_e2m1fn_x2")
+    else:
+        _check(a.dtype in _FP8 and b.dtype in _FP8, "operands must be float8_e4m3fn / float8_e5m2")
     if trans_c:
         a, b, a_scales, b_scales = b, a, b_scales, a_scales
-    Ml, ld = a.shape
+    Ml = a.shape[0]
+    ld = a.shape[1] * (2 if fp4 else 1)
     Nr = b.shape[0]
     G = group_offs.numel() - 1
-    _check(ld % 128 == 0, "the padded length must be a multiple of 128")
+    _check(ld % (256 if fp4 else 128) == 0, "the padded length must be a multiple of 128 (MXFP4: 256)")
     a_s, b_s = _u8(a_scales), _u8(b_scales)
     _check(tuple(a_s.shape) == (Ml, ld // 32) and tuple(b_s.shape) == (Nr, ld // 32), "scales must be [rows, padded length / 32]")
     _check(tuple(out.shape) == (G, Ml, Nr) and out.is_contiguous(), f"out must be a contiguous {(G, Ml, Nr)} tensor")
-    a, b = a.contiguous(), b.contiguous()
+    da, db = N.dtype_code(a.dtype), N.dtype_code(b.dtype)
+    a, b = _u8(a), _u8(b)
     N.check(
         N.lib().pt_grouped_gemm_mx_variable_k(
-            N.ptr(a), N.dtype_code(a.dtype), N.ptr(a_s), N.ptr(b), N.dtype_code(b.dtype), N.ptr(b_s), N.ptr(out),
+            N.ptr(a), da, N.ptr(a_s), N.ptr(b), db, N.ptr(b_s), N.ptr(out),
             N.dtype_code(out.dtype), N.ptr(group_offs.contiguous()), G, Ml, Nr, ld, int(accumulate), MX_TILE_CFG,
             N.stream_of(a),
         )

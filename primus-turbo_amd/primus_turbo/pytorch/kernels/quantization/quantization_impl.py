@@ -711,7 +711,13 @@ MXFP8_GROUP_M_PADDING_ALIGN_SIZE = 32
 MXFP8_K_DIM_PADDING_ALIGN_SIZE = 128
 
 
+MXFP4_GROUP_K_DIM_PADDING_ALIGN_SIZE = 256
+
+
 def _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, want_row: bool, want_col: bool):
+    """MXFP8: rows of every group padded to 32, transposed columns to 128. MXFP4: rows stay
+    where they are in ``x`` (their "padded" lens / offs are the originals), transposed columns
+    padded to 256 per group."""
     N.require_cuda(x, group_lens, group_offs)
     if x.dtype not in (torch.bfloat16, torch.float16):
         raise RuntimeError("Input must be BFloat16 or Half")
@@ -720,29 +726,34 @@ def _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, want_row: bool, w
     _check(group_lens.dim() == 1 and group_offs.dim() == 1 and group_offs.numel() == group_lens.numel() + 1,
            "group_offs.size(0) must equal group_lens.size(0) + 1")
     _check(group_lens.numel() >= 1, "must have at least one group")
-    _check(out_dtype in (torch.float8_e4m3fn, torch.float8_e5m2), "Output must be Float8_e4m3fn or Float8_e5m2")
+    fp4 = _FP4X2 is not None and out_dtype == _FP4X2
+    _check(fp4 or out_dtype in (torch.float8_e4m3fn, torch.float8_e5m2),
+           "Output must be Float8_e4m3fn, Float8_e5m2 or Float4_e2m1fn_x2")
     M, Nn = x.shape
     _check(Nn % 32 == 0, f"N must be divisible by 32, got N={Nn}")
     G = group_lens.numel()
-    ra, ca = MXFP8_GROUP_M_PADDING_ALIGN_SIZE, MXFP8_K_DIM_PADDING_ALIGN_SIZE
-    m_pad_row = -(-(M + G * ra) // ra) * ra
+    ra = MXFP8_GROUP_M_PADDING_ALIGN_SIZE
+    ca = MXFP4_GROUP_K_DIM_PADDING_ALIGN_SIZE if fp4 else MXFP8_K_DIM_PADDING_ALIGN_SIZE
+    pack = 2 if fp4 else 1
+    m_pad_row = M if fp4 else -(-(M + G * ra) // ra) * ra
     m_pad_col = -(-(M + G * ca) // ca) * ca
     n_pad = -(-Nn // _MX_PAD) * _MX_PAD
     dev = x.device
-    lens_row, offs_row = _group_offs(group_lens, ra, True)
+    group_offs = group_offs.contiguous()
+    lens_row, offs_row = (group_lens, group_offs) if fp4 else _group_offs(group_lens, ra, True)
     lens_col, offs_col = _group_offs(group_lens, ca, True)
     row_q = row_s = col_q = col_s = None
     if want_row:
-        row_q = torch.empty((m_pad_row, n_pad), dtype=torch.uint8, device=dev)
+        row_q = torch.empty((m_pad_row, n_pad // pack), dtype=torch.uint8, device=dev)
         row_s = torch.empty((m_pad_row, n_pad // 32), dtype=torch.uint8, device=dev)
     if want_col:
-        col_q = torch.empty((Nn, m_pad_col), dtype=torch.uint8, device=dev)
+        col_q = torch.empty((Nn, m_pad_col // pack), dtype=torch.uint8, device=dev)
         col_s = torch.empty((Nn, m_pad_col // 32), dtype=torch.uint8, device=dev)
     N.check(
         N.lib().pt_grouped_quantize_mx(
-            N.ptr(x), N.dtype_code(x.dtype), M, Nn, N.dtype_code(out_dtype), N.ptr(group_offs.contiguous()),
-            N.ptr(offs_row), N.ptr(offs_col), G, N.ptr(row_q), N.ptr(row_s), N.ptr(col_q), N.ptr(col_s), m_pad_col,
-            N.stream_of(x),
+            N.ptr(x), N.dtype_code(x.dtype), M, Nn, N.dtype_code(out_dtype), N.ptr(group_offs),
+            None if fp4 else N.ptr(offs_row), N.ptr(offs_col), G, N.ptr(row_q), N.ptr(row_s), N.ptr(col_q), N.ptr(col_s),
+            m_pad_col, N.stream_of(x),
         )
     )
     view = lambda t, dt: None if t is None else t.view(dt)  # noqa: E731
@@ -787,3 +798,28 @@ def grouped_dequantize_mxfp8_impl(x, out_dtype, axis, block_size, scale_inv, gro
     g = torch.searchsorted(group_offs[1:].contiguous(), rows, right=True)
     src = rows + (group_offs_padded[:-1] - group_offs[:-1])[g]
     return full.index_select(0, src)
+
+
+def grouped_quantize_mxfp4_impl(x, out_dtype, axis, block_size, group_lens, group_offs, with_trans=False,
+                                scaling_recipe=None, scaling_recipe_for_trans=None):
+    """MXFP4 quantization of the packed rows of G groups (reference: quantization_impl.py:657-811,
+    layout of its default dispatch flydsl/quantization/mxfp4_grouped_quant.py:320-349).
+
+    ``with_trans`` -> ``(row_q [M, N_pad/2], row_scale [M, N_pad/32], col_q [N, M_pad_col/2], col_scale
+    [N, M_pad_col/32], group_lens, group_offs, lens_padded_col, offs_padded_col)``: the row
+    direction keeps the rows where they are (row i = input row i), the transposed column
+    direction pads every group to a multiple of 256 rows of zero data; ``M_pad_col`` = ``total_M +
+    256 G`` rounded up to 256. Otherwise ``(q, scale, lens_padded, offs_padded)`` of the direction
+    ``axis`` asks for (1 = rows, 0 = transposed columns). Round-to-nearest-even only: stochastic
+    rounding, the random Hadamard transform, 2-D blocks and shuffled layouts raise."""
+    assert block_size == 32, "The block size must be 32 for MXFP4 quantization"
+    assert _FP4X2 is not None and out_dtype == _FP4X2, "The out_dtype must be float4_e2m1fn_x2 for MXFP4 quantization"
+    for r in (scaling_recipe, scaling_recipe_for_trans):
+        if r is not None and (r.use_2d_block or r.use_sr or r.use_rht or r.shuffle_scale or r.shuffle_out):
+            raise NotImplementedError(
+                "grouped MXFP4 quantization: 2-D blocks, stochastic rounding, RHT and shuffled layouts are not implemented")
+    if with_trans:
+        return _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, True, True)
+    assert axis in (0, 1), "The axis must be 0 (colwise) or 1 (rowwise) when with_trans is False."
+    rq, rs, cq, cs, lr, orow, lc, ocol = _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, axis == 1, axis == 0)
+    return (rq, rs, lr, orow) if axis == 1 else (cq, cs, lc, ocol)

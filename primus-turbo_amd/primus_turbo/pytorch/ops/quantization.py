@@ -29,6 +29,7 @@ __all__ = [
     "grouped_quantize_fp8_with_trans",
     "grouped_dequantize_fp8",
     "grouped_quantize_fp4",
+    "grouped_quantize_fp4_with_trans",
     "grouped_dequantize_fp4",
 ]
 
@@ -186,14 +187,7 @@ def dequantize_fp4(
     raise _unknown(granularity)
 
 
-# --- grouped MX quantizers (MoE experts): per-group padded MXFP8 layouts ---------------------
-def _grouped_mx_not_built(name):
-    raise NotImplementedError(
-        f"{name}: the grouped MXFP4 quantizers (per-group padded layouts) are not built; the grouped MX path "
-        "of this library is MXFP8 (grouped_quantize_fp8 / grouped_gemm_fp8 with MX_BLOCKWISE)."
-    )
-
-
+# --- grouped MX quantizers (MoE experts): per-group padded layouts ------------------------------
 def grouped_quantize_fp8(x, out_dtype, granularity, group_lens, group_offs, *, block_size=None, axis=None,
                          scaling_recipe=None):
     """Quantize the packed rows of G groups (MX_BLOCKWISE): ``axis`` 1 (or -1) -> rows, every group
@@ -231,13 +225,37 @@ def grouped_dequantize_fp8(x, out_dtype, granularity, group_offs, group_offs_pad
 
 def grouped_quantize_fp4(x, out_dtype, granularity, group_lens, group_offs, *, block_size=None, axis=None,
                          scaling_recipe=None):
+    """MXFP4 quantization of the packed rows ``[total_m, N]`` of G groups in one direction
+    (reference: ops/quantization.py:340-385): ``axis`` 1 -> rows, in place (row i = input row i, the
+    returned padded lens / offs are the originals); ``axis`` 0 -> the transposed column direction
+    ``[N, M_pad_col/2]`` with every group padded to 256 rows (the variable-K wgrad operand).
+    Returns ``(data, scale_inv, group_lens_padded, group_offs_padded)``."""
     if granularity == _G.MX_BLOCKWISE:
-        _grouped_mx_not_built("grouped_quantize_fp4")
+        _need_mx_block(block_size, MXFP4_BLOCK_SIZE, "MXFP4")
+        assert x.ndim == 2, "grouped MXFP4 quantize expects a 2D packed-M tensor"
+        assert axis in (0, 1), "axis must be 0 (colwise) or 1 (rowwise) for grouped MXFP4"
+        return _impl.grouped_quantize_mxfp4_impl(x, out_dtype, axis, block_size, group_lens, group_offs, False,
+                                                 scaling_recipe)
+    raise _unknown(granularity)
+
+
+def grouped_quantize_fp4_with_trans(x, out_dtype, granularity, group_lens, group_offs, *, block_size=None,
+                                    scaling_recipe=None, scaling_recipe_for_trans=None):
+    """Both directions from one read of ``x`` (reference: ops/quantization.py:388-443):
+    ``(row_q [total_m, N_pad/2], row_scale [total_m, N_pad/32], col_q [N, M_pad_col/2], col_scale
+    [N, M_pad_col/32], group_lens, group_offs, lens_padded_col, offs_padded_col)``."""
+    if granularity == _G.MX_BLOCKWISE:
+        _need_mx_block(block_size, MXFP4_BLOCK_SIZE, "MXFP4")
+        assert x.ndim == 2, "grouped MXFP4 quantize expects a 2D packed-M tensor"
+        return _impl.grouped_quantize_mxfp4_impl(x, out_dtype, None, block_size, group_lens, group_offs, True,
+                                                 scaling_recipe, scaling_recipe_for_trans)
     raise _unknown(granularity)
 
 
 def grouped_dequantize_fp4(x, out_dtype, granularity, *, block_size=None, axis=None, scale_inv=None,
                            scaling_recipe=None):
+    """Row-direction grouped MXFP4 data are plain rows: the dense de-quantizer
+    (reference: ops/quantization.py:519-537)."""
     if granularity == _G.MX_BLOCKWISE:
         _need_mx_block(block_size, MXFP4_BLOCK_SIZE, "MXFP4")
         return _impl.dequantize_mxfp4_impl(x, out_dtype, axis, block_size, scale_inv)

@@ -243,19 +243,22 @@ def test_fp4_packing_order():
 
 
 @pytest.mark.parametrize("lens", [[100, 0, 37, 163], [128, 128], [1], [0, 5, 0, 250, 31]])
-@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e2m1"])
-def test_mx_grouped_layout(lens, fmt):
-    """Grouped MX quantizer: group starts on multiples of 32 (rows) / 128 (transposed columns),
-    every group's slice equals the dense quantizer of that group's rows, pads are zero codes with
-    scale byte 0, and the round trip through the de-quantizer matches the dense round trip."""
+@pytest.mark.parametrize("fmt,ra,ca", [("e4m3", 32, 128), ("e5m2", 32, 128), ("e2m1", 32, 128), ("e2m1", 1, 256)])
+def test_mx_grouped_layout(lens, fmt, ra, ca):
+    """Grouped MX quantizer: group starts on multiples of 32 (rows) / 128 (transposed columns) --
+    grouped MXFP4: rows in place, columns on multiples of 256 --, every group's slice equals the
+    dense quantizer of that group's rows, pads are zero codes with scale byte 0, and the round
+    trip through the de-quantizer matches the dense round trip."""
     lens = np.array(lens, dtype=np.int64)
     M, N = int(lens.sum()), 160
     rng = np.random.default_rng(5)
     x = (rng.standard_normal((M, N)) * np.exp(rng.standard_normal((M, 1)))).astype(np.float32)
-    o = Q.mx_grouped_quant(x, lens, fmt)
+    o = Q.mx_grouped_quant(x, lens, fmt, row_align=ra, col_align=ca)
     cpb = 2 if fmt == "e2m1" else 1
-    assert np.all(o["row_offs"] % 32 == 0) and np.all(o["col_offs"] % 128 == 0)
-    assert np.array_equal(o["row_lens"], (lens + 31) // 32 * 32) and np.array_equal(o["col_lens"], (lens + 127) // 128 * 128)
+    assert np.all(o["row_offs"] % ra == 0) and np.all(o["col_offs"] % ca == 0)
+    assert np.array_equal(o["row_lens"], (lens + ra - 1) // ra * ra) and np.array_equal(o["col_lens"], (lens + ca - 1) // ca * ca)
+    if ra == 1:
+        assert np.array_equal(o["row_offs"], np.concatenate([[0], np.cumsum(lens)]))
     assert o["row"].shape == (o["row_offs"][-1], 256 // cpb) and o["col"].shape == (N, o["col_offs"][-1] // cpb)
     starts = np.concatenate([[0], np.cumsum(lens)])
     for g, n in enumerate(lens):
