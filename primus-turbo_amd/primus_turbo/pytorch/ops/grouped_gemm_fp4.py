@@ -84,8 +84,6 @@ class FP4GroupedGemmMXFunc(torch.autograd.Function):
             raise NotImplementedError("Float4QuantConfig.use_preshuffle is not implemented")
         if config.use_gradient_sr:
             raise NotImplementedError("Float4QuantConfig.use_gradient_sr (stochastic rounding) is not implemented")
-        if isinstance(a, QuantizedTensor):
-            raise NotImplementedError("FP4GroupedGemmMXFunc does not take a pre-quantized activation in this build")
         supported, reason = check_mxfp4_support()
         assert supported, reason
         N, K = int(b.shape[-2]), int(b.shape[-1])
@@ -97,7 +95,19 @@ class FP4GroupedGemmMXFunc(torch.autograd.Function):
         need_bwd = any(ctx.needs_input_grad[:2])
         w_recipe = ScalingRecipe(use_2d_block=True)
 
-        if need_bwd:
+        a_recipe = ScalingRecipe()
+        if isinstance(a, QuantizedTensor):
+            # a grouped (packed rows) quantization made by the caller
+            check_quantized_tensor(a, config, axis=-1, scaling_recipe=a_recipe)
+            a_row, a_row_s, offs_row = a.qdata, a.scale_inv, a.group_offs
+            a_col = a_col_s = None
+            if need_bwd:
+                if a_t is None:
+                    a_t = QuantizedTensor.quantize(a.dequantize(), a.real_dtype, gran, axis=-2, block_size=bs,
+                                                   scaling_recipe=a_recipe, group_lens=group_lens)
+                assert isinstance(a_t, QuantizedTensor)
+                a_col, a_col_s = a_t.qdata, a_t.scale_inv
+        elif need_bwd:
             a_row, a_row_s, a_col, a_col_s, _, offs_row, _, _ = grouped_quantize_fp4_with_trans(
                 a.contiguous(), float4_e2m1fn_x2, gran, group_lens, group_offs, block_size=bs)
         else:
@@ -162,9 +172,10 @@ def grouped_gemm_fp4(
 ) -> torch.Tensor:
     """Grouped GEMM with MXFP4 quantization: ``out[rows of group g] = a[rows of group g] @ b[g]^T``.
 
-    ``a``: ``[sum(group_lens), K]`` (fp16 / bf16); ``b``: ``[G, N, K]`` (``trans_b`` must be True), or
-    a pre-quantized 32 x 32-block ``QuantizedTensor`` / ``QuantizedTensorPair`` (``data_t`` = the
-    transposed quantization that dgrad reads); ``group_lens``: int64 ``[G]`` on the device
+    ``a``: ``[sum(group_lens), K]`` (fp16 / bf16), or a grouped ``QuantizedTensor`` / pair (``data_t`` =
+    the column-direction quantization that wgrad reads); ``b``: ``[G, N, K]`` (``trans_b`` must be
+    True), or a pre-quantized 32 x 32-block ``QuantizedTensor`` / ``QuantizedTensorPair`` (``data_t`` =
+    the transposed quantization that dgrad reads); ``group_lens``: int64 ``[G]`` on the device
     (groups may be empty); N and K multiples of 32. ``fuse_bgrad_accum_pattern="megatron"``
     accumulates the weight gradient into ``b.main_grad`` (any of fp32 / bf16 / fp16)."""
     if config is None:

@@ -227,25 +227,45 @@ class FP8GroupedGemmMXFunc(torch.autograd.Function):
                 fuse_bgrad_accum_pattern=None):
         fuse_bgrad_accum, main_grad = _setup_fused_grad_accum(b, fuse_bgrad_accum_pattern)
         assert config.granularity == ScalingGranularity.MX_BLOCKWISE
-        if isinstance(a, QuantizedTensor) or isinstance(b, QuantizedTensor):
-            raise NotImplementedError("FP8GroupedGemmMXFunc does not take pre-quantized operands in this build")
         assert a.ndim == 2 and b.ndim == 3
         assert trans_b, "MXFP8 grouped GEMM only supports trans_b=True (NT layout)."
         assert group_lens.size(0) == b.size(0), "group_lens size must match b size(0)."
         fdt = _get_fp8_dtype(config.format, True)
         bs = config.block_size
+        gran = config.granularity
         total_m = int(a.size(0))
         need_bwd = any(ctx.needs_input_grad[:2])
-        w_recipe = ScalingRecipe(use_2d_block=True)
-        if need_bwd:
+        a_recipe, w_recipe = ScalingRecipe(), ScalingRecipe(use_2d_block=True)
+        a_col = a_col_s = b_col = b_col_s = None
+        if isinstance(a, QuantizedTensor):
+            # a grouped (packed rows, per-group padded) quantization made by the caller
+            check_quantized_tensor(a, config, axis=-1, scaling_recipe=a_recipe)
+            a_row, a_row_s, offs_row = a.qdata, a.scale_inv, a.group_offs
+            if need_bwd:
+                if a_t is None:
+                    a_t = QuantizedTensor.quantize(a.dequantize(), a.real_dtype, gran, axis=-2, block_size=bs,
+                                                   scaling_recipe=a_recipe, group_lens=group_lens)
+                assert isinstance(a_t, QuantizedTensor)
+                a_col, a_col_s = a_t.qdata, a_t.scale_inv
+        elif need_bwd:
             a_row, a_row_s, a_col, a_col_s, _, offs_row, _, _ = grouped_quantize_mxfp8_impl(
                 a.contiguous(), fdt, None, bs, group_lens, group_offs, with_trans=True)
+        else:
+            a_row, a_row_s, _, offs_row = grouped_quantize_mxfp8_impl(a.contiguous(), fdt, 1, bs, group_lens, group_offs)
+        if isinstance(b, QuantizedTensor):
+            check_quantized_tensor(b, config, axis=-1, scaling_recipe=w_recipe)
+            b_row, b_row_s = b.qdata, b.scale_inv
+            if need_bwd:
+                if b_t is None:
+                    b_t = QuantizedTensor.quantize(b.dequantize(), b.real_dtype, gran, axis=-2, block_size=bs,
+                                                   scaling_recipe=w_recipe)
+                assert isinstance(b_t, QuantizedTensor)
+                b_col, b_col_s = b_t.qdata, b_t.scale_inv
+        elif need_bwd:
             b_row, b_row_s, b_col, b_col_s = quantize_mxfp8_impl(
                 b.contiguous(), fdt, None, bs, with_trans=True, scaling_recipe=w_recipe, scaling_recipe_for_trans=w_recipe)
         else:
-            a_row, a_row_s, _, offs_row = grouped_quantize_mxfp8_impl(a.contiguous(), fdt, 1, bs, group_lens, group_offs)
             b_row, b_row_s = quantize_mxfp8_impl(b.contiguous(), fdt, 2, bs, scaling_recipe=w_recipe)
-            a_col = a_col_s = b_col = b_col_s = None
         # the padded row layout is read through offs_row, the result is packed by group_offs
         # into an output over-allocated to the padded rows
         out = grouped_gemm_fp8_impl(a_row, b_row, a_row_s, b_row_s, group_lens, offs_row, False, True, out_dtype,
