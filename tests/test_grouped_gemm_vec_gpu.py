@@ -112,3 +112,37 @@ def test_grouped_gemm_fp8_vec_autograd(gran, fmt, gate, trans_b):
     for g in range(G_):
         if lens[g] == 0:
             assert torch.count_nonzero(b.grad[g]).item() == 0
+
+
+@pytest.mark.parametrize("gran", ["TENSORWISE", "ROWWISE", "BLOCKWISE", "MX_BLOCKWISE"])
+@pytest.mark.parametrize("main_dtype", [torch.float32, torch.bfloat16])
+def test_grouped_gemm_fp8_fused_grad_accum(gran, main_dtype):
+    """``fuse_bgrad_accum_pattern="megatron"`` for every grouped FP8 granularity: the wgrad GEMM adds
+    into ``b.main_grad`` (beta = 1 epilogue), flags the weight, and autograd receives a placeholder;
+    ``main_grad`` ends as previous + the gradient of the unfused call
+    (reference: primus_turbo/pytorch/ops/utils.py:37-89 and its callers in ops/grouped_gemm_fp8.py)."""
+    from primus_turbo.pytorch.core.low_precision import ScaleDtype
+
+    g = getattr(G, gran)
+    kw = {"BLOCKWISE": dict(block_size=128), "MX_BLOCKWISE": dict(block_size=32, scale_dtype=ScaleDtype.E8M0)}.get(gran, {})
+    cfg = Float8QuantConfig(format=Format.E4M3, granularity=g, **kw)
+    lens = group_lens("ragged", 4, 1024, 91)
+    gl, _ = _offs(lens)
+    a = bf16_randn((1024, 512), seed=92).cuda().requires_grad_(True)
+    b = bf16_randn((4, 768, 512), seed=93).cuda().requires_grad_(True)
+    dy = bf16_randn((1024, 768), seed=94).cuda()
+    turbo.ops.grouped_gemm_fp8(a, b, gl, trans_b=True, config=cfg).backward(dy)
+    plain, plain_da = b.grad.clone(), a.grad.clone()
+    a.grad = b.grad = None
+    b.main_grad = torch.full((4, 768, 512), 0.25, dtype=main_dtype, device="cuda")
+    b.grad_added_to_main_grad = False
+    turbo.ops.grouped_gemm_fp8(a, b, gl, trans_b=True, config=cfg, fuse_bgrad_accum_pattern="megatron").backward(dy)
+    torch.cuda.synchronize()
+    assert b.grad_added_to_main_grad and torch.equal(a.grad, plain_da)
+    want = plain.float() + 0.25
+    # fp32 accumulators differ from the unfused bf16 result by its rounding; bf16 ones round once more
+    tol = (2.0 ** -7 if main_dtype == torch.bfloat16 else 2.0 ** -8) * float(want.abs().max())
+    assert torch.allclose(b.main_grad.float(), want, rtol=0, atol=tol)
+    with pytest.raises(AssertionError):
+        c = bf16_randn((4, 768, 512), seed=95).cuda().requires_grad_(True)  # no main_grad set up
+        turbo.ops.grouped_gemm_fp8(a, c, gl, trans_b=True, config=cfg, fuse_bgrad_accum_pattern="megatron")
