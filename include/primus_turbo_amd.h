@@ -136,6 +136,14 @@ PT_API int pt_quantize_fp8_blockwise(const void *x, int x_dtype, int64_t M, int6
 PT_API int pt_quantize_fp8_blockwise_weight(const void *w, int w_dtype, int64_t B, int64_t M,
                                             int64_t N, void *q, int q_dtype, float *scale_inv,
                                             void *stream);
+/* The same, and from the same read of w also q_t [B, N, ldt]: the codes transposed per batch
+ * slice (q_t[b, n, m] = q[b, m, n]; M % 16 == 0, ldt >= M a multiple of 16; columns at and
+ * beyond M are not written). It is the operand the dgrad product of a linear layer reads (the
+ * reference hands the untransposed codes to backends that read either layout:
+ * ops/gemm_fp8.py:477-560, ops/grouped_gemm_fp8.py:190-262); the tile scales serve both. */
+PT_API int pt_quantize_fp8_blockwise_weight_dual(const void *w, int w_dtype, int64_t B, int64_t M,
+                                                 int64_t N, void *q, void *q_t, int64_t ldt,
+                                                 int q_dtype, float *scale_inv, void *stream);
 
 /* Prefix sums of group lengths, each rounded up to `align` first:
  *   padded_lens[i] = round_up(group_lens[i], align)   (optional output, may be NULL)
@@ -161,6 +169,14 @@ PT_API int pt_quantize_fp8_blockwise_segment_m_row_col(
     const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype, const int64_t *group_offs,
     const int64_t *padded_group_offs, int64_t num_groups, void *q_row, float *scale_inv_row,
     void *q_col_padded, float *scale_inv_col_padded, void *stream);
+/* The same with the column codes (also, or only: q_col_padded may be NULL) emitted transposed,
+ * q_col_t [N, ldt] with q_col_t[n, r] = q_col_padded[r, n]: the K-contiguous operand of the
+ * variable-K wgrad product. ldt >= M + G*128 rounded up to 128, a multiple of 16; columns at
+ * and beyond padded_group_offs[G] are not written. Scales as above. */
+PT_API int pt_quantize_fp8_blockwise_segment_m_row_col_t(
+    const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype, const int64_t *group_offs,
+    const int64_t *padded_group_offs, int64_t num_groups, void *q_row, float *scale_inv_row,
+    void *q_col_padded, void *q_col_t, int64_t ldt, float *scale_inv_col_padded, void *stream);
 
 /* De-quantize with one fp32 scale per (block_m x block_n) block of a [B, M, N] tensor:
  *   y[b, m, n] = T(float(q[b, m, n]) * scale_inv[b, m / block_m, n / block_n]).
@@ -290,6 +306,9 @@ PT_API int pt_gemm_mx(const void *a, const void *a_scale, const void *b, const v
  * rounded up to a multiple of 128, pad rows zero) with scales [Mp / 128, cols]; p = padded
  * group offsets (device int64 [G + 1], multiples of 128). An empty group yields C[g] = 0
  * (or leaves it unchanged when accumulating). The workspace holds both transposed operands.
+ * operands_kmajor != 0: LHS and RHS arrive transposed already, [Ml, Mp] and [Nr, Mp] (the
+ * q_col_t output of pt_quantize_fp8_blockwise_segment_m_row_col_t, scales unchanged); no
+ * workspace is used.
  */
 PT_API size_t pt_grouped_gemm_fp8_workspace_bytes(int64_t G, int64_t M, int64_t N, int64_t K,
                                                   int trans_b);
@@ -303,8 +322,8 @@ PT_API int pt_grouped_gemm_fp8_variable_k(const void *lhs, int lhs_dtype, const 
                                           const void *rhs, int rhs_dtype, const float *rhs_scale,
                                           void *c, int c_dtype, const int64_t *group_offs, int64_t G,
                                           int64_t Mp, int64_t Ml, int64_t Nr, int trans_c,
-                                          int accumulate, void *workspace, size_t workspace_bytes,
-                                          int tile_cfg, void *stream);
+                                          int accumulate, int operands_kmajor, void *workspace,
+                                          size_t workspace_bytes, int tile_cfg, void *stream);
 
 /* Grouped GEMM with vector scales (TENSORWISE / ROWWISE granularities) -----------------
  *

@@ -167,8 +167,8 @@ size_t pt_grouped_gemm_fp8_variable_k_workspace_bytes(int64_t Mp, int64_t Ml, in
 int pt_grouped_gemm_fp8_variable_k(const void *lhs, int lhs_dtype, const float *lhs_scale, const void *rhs,
                                    int rhs_dtype, const float *rhs_scale, void *c, int c_dtype,
                                    const int64_t *group_offs, int64_t G, int64_t Mp, int64_t Ml, int64_t Nr,
-                                   int trans_c, int accumulate, void *workspace, size_t workspace_bytes,
-                                   int tile_cfg, void *stream) {
+                                   int trans_c, int accumulate, int operands_kmajor, void *workspace,
+                                   size_t workspace_bytes, int tile_cfg, void *stream) {
     PT_REQUIRE(is_fp8_dtype(lhs_dtype) && is_fp8_dtype(rhs_dtype), "operands must be e4m3 or e5m2");
     PT_REQUIRE(is_hp_dtype(c_dtype), "output must be bf16, fp16 or fp32");
     PT_REQUIRE(G >= 0 && Mp >= 0 && Ml >= 0 && Nr >= 0, "bad dimensions");
@@ -179,16 +179,25 @@ int pt_grouped_gemm_fp8_variable_k(const void *lhs, int lhs_dtype, const float *
         return PT_OK;
     PT_REQUIRE(lhs && rhs && lhs_scale && rhs_scale && c && group_offs, "NULL pointer");
     PT_REQUIRE(aligned_to(lhs, 16) && aligned_to(rhs, 16) && aligned_to(c, 16), "operands must be 16-byte aligned");
-    const size_t need = pt_grouped_gemm_fp8_variable_k_workspace_bytes(Mp, Ml, Nr);
-    if (workspace == nullptr || workspace_bytes < need || !aligned_to(workspace, 16))
-        return fail(PT_ERR_WORKSPACE, "pt_grouped_gemm_fp8_variable_k: workspace missing, too small or misaligned");
-
-    // both operands become K-contiguous: [Mp, cols] -> [cols, ld] with the rows as K
-    const int64_t ld  = round_up(Mp, 128);
-    uint8_t      *lt  = static_cast<uint8_t *>(workspace);
-    uint8_t      *rt  = lt + round_up(Ml * ld, 256);
-    launch_transpose(static_cast<const uint8_t *>(lhs), lt, 1, Mp, Ml, ld, st);
-    launch_transpose(static_cast<const uint8_t *>(rhs), rt, 1, Mp, Nr, ld, st);
+    const int64_t  ld = round_up(Mp, 128);
+    const uint8_t *lt, *rt;
+    if (operands_kmajor) {
+        // the operands arrive with the rows as their contiguous axis already: [cols, Mp]
+        PT_REQUIRE(Mp % 128 == 0, "K-major operands need a padded row count that is a multiple of 128");
+        lt = static_cast<const uint8_t *>(lhs);
+        rt = static_cast<const uint8_t *>(rhs);
+    } else {
+        const size_t need = pt_grouped_gemm_fp8_variable_k_workspace_bytes(Mp, Ml, Nr);
+        if (workspace == nullptr || workspace_bytes < need || !aligned_to(workspace, 16))
+            return fail(PT_ERR_WORKSPACE, "pt_grouped_gemm_fp8_variable_k: workspace missing, too small or misaligned");
+        // both operands become K-contiguous: [Mp, cols] -> [cols, ld] with the rows as K
+        uint8_t *wl = static_cast<uint8_t *>(workspace);
+        uint8_t *wr = wl + round_up(Ml * ld, 256);
+        launch_transpose(static_cast<const uint8_t *>(lhs), wl, 1, Mp, Ml, ld, st);
+        launch_transpose(static_cast<const uint8_t *>(rhs), wr, 1, Mp, Nr, ld, st);
+        lt = wl;
+        rt = wr;
+    }
 
     // C[g] = lhs_g^T rhs_g ([Ml, Nr]); trans_c asks for its transpose: swap the operand roles
     GemmArgs g{};

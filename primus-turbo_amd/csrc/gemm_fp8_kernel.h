@@ -28,6 +28,7 @@
 #pragma once
 #include "pt_common.h"
 
+#include <atomic>
 #include <type_traits>
 
 // Timing probes for kernel development: a test translation unit may define this macro to
@@ -930,12 +931,17 @@ static int launch_gemm_cfg(const GemmArgs &args_in, hipStream_t stream) {
                              reinterpret_cast<uintptr_t>(a.sA) % 4 != 0 || reinterpret_cast<uintptr_t>(a.sB) % 4 != 0))
         return fail(PT_ERR_INVALID_ARGUMENT, "gemm_mx: scale rows must be 4-byte aligned");
     auto kern            = gemm_fp8_nt_kernel<TM, TN, MODE, SB_VEC, FA, FB, GMODE>;
-    static bool attr_set = false;
-    if (!attr_set) {
+    // the attribute belongs to the (kernel, device) pair: one bit per device, set once
+    static std::atomic<unsigned long long> attr_set{0};
+    int                                    dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+        return fail(PT_ERR_LAUNCH, "gemm_fp8: no current device (or a device index beyond 63)");
+    const unsigned long long dev_bit = 1ULL << dev;
+    if (!(attr_set.load(std::memory_order_acquire) & dev_bit)) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, LDS_MAX) != hipSuccess)
             return fail(PT_ERR_LAUNCH, "gemm_fp8: cannot raise the dynamic LDS limit");
-        attr_set = true;
+        attr_set.fetch_or(dev_bit, std::memory_order_release);
     }
     const int lds = STAGES + (GMODE == GROUP_ROWS ? (a.G + 2) * 4 : 0);
     // persistent grid: as many workgroups as fit on the machine at once (LDS-limited)

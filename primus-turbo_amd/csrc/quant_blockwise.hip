@@ -38,6 +38,10 @@ struct BlockQuantArgs {
     const int64_t *padded_offs; // [G+1] offsets with every group rounded up to 128 rows
     int            num_groups;
     float          qmax;
+    // optional transposed copy of the tile codes (MODE_TILE: [B, N, ldt]) or of the column
+    // codes (MODE_COL: [N, ldt]): the operand a GEMM reads when it reduces over the rows of x
+    uint8_t *q_t;
+    int64_t  ldt;
 };
 
 // Eight consecutive elements of a tile row as they come from memory (16-bit inputs stay packed:
@@ -114,11 +118,60 @@ __device__ __forceinline__ void store8(uint8_t *p, u32x2 v, bool vec, int64_t gn
     }
 }
 
+// Row of the tile that round r of thread row slot `rslot` handles: a thread owns two runs of four
+// consecutive rows, so that it can transpose its 4 x 4 byte blocks in registers.
+__device__ __forceinline__ int tile_row_of(int rslot, int r) {
+    return 4 * rslot + (r & 3) + 64 * (r >> 2);
+}
+
+constexpr int BQ_TP = 33; // words per row of the transposed LDS tile
+
+// Codes of four consecutive tile rows x eight columns (one u32x2 per row) -> eight words "four
+// rows of one column" in the transposed tile t[column][BQ_TP], word index = row / 4.
+__device__ __forceinline__ void stage_transposed(uint32_t *t, const u32x2 (&c)[4], int cseg, int rowgroup) {
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+        const uint32_t a0 = w ? c[0].y : c[0].x, a1 = w ? c[1].y : c[1].x, a2 = w ? c[2].y : c[2].x,
+                       a3 = w ? c[3].y : c[3].x;
+        const uint32_t t0 = __builtin_amdgcn_perm(a1, a0, 0x05010400u);
+        const uint32_t t1 = __builtin_amdgcn_perm(a1, a0, 0x07030602u);
+        const uint32_t t2 = __builtin_amdgcn_perm(a3, a2, 0x05010400u);
+        const uint32_t t3 = __builtin_amdgcn_perm(a3, a2, 0x07030602u);
+        const int      col = cseg * 8 + w * 4;
+        t[(col + 0) * BQ_TP + rowgroup] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+        t[(col + 1) * BQ_TP + rowgroup] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+        t[(col + 2) * BQ_TP + rowgroup] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+        t[(col + 3) * BQ_TP + rowgroup] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+    }
+}
+
+// The staged tile leaves as rows of the transposed output: out[(c0 + c) * ldt + m0 + 0..127] for
+// the columns c0 + c < cols; 16-byte chunks beyond `rows` (a multiple of 16) are not written.
+__device__ __forceinline__ void flush_transposed(const uint32_t *t, uint8_t *out, int64_t ldt, int64_t c0, int64_t cols,
+                                                 int64_t m0, int64_t rows, int tid) {
+    const int j = tid & 7;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int     c  = (tid >> 3) + 32 * p;
+        const int64_t gm = m0 + j * 16;
+        if (c0 + c < cols && gm < rows) {
+            u32x4 v;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                v[k] = t[c * BQ_TP + j * 4 + k];
+            *reinterpret_cast<u32x4 *>(out + (c0 + c) * ldt + gm) = v;
+        }
+    }
+}
+
 // MODE: bitmask of MODE_ROW / MODE_COL / MODE_TILE.  GROUPED: tiles live in the
 // segment-padded row space and map back to input rows through the group offsets.
 // VEC8: N % 8 == 0 and all pointers 16-byte aligned (128-bit loads, 64-bit stores).
-template <typename T, bool E5M2, int MODE, bool GROUPED, bool VEC8>
+// TRANS: also emit the transposed copy described at BlockQuantArgs::q_t.
+template <typename T, bool E5M2, int MODE, bool GROUPED, bool VEC8, bool TRANS = false>
 __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArgs a) {
+    static_assert(!TRANS || ((MODE & MODE_TILE) != 0) != ((MODE & MODE_COL) != 0), "one transposed output");
+    __shared__ uint32_t s_tr[TRANS ? BQ * BQ_TP : 1];
     const int     tid   = threadIdx.x;
     const int     cseg  = tid & 15; // which 8-column segment of the tile row
     const int     rslot = tid >> 4; // row within a round
@@ -151,7 +204,7 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
     Held8<T> held[BQ_ROUNDS];
 #pragma unroll
     for (int r = 0; r < BQ_ROUNDS; ++r) {
-        const int64_t in_m  = in_m0 + rslot + 16 * r;
+        const int64_t in_m  = in_m0 + tile_row_of(rslot, r);
         const bool    valid = in_m < in_end;
         if (valid && full)
             held[r].load(x + in_m * N + gn);
@@ -167,7 +220,7 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
 
 #pragma unroll
     for (int r = 0; r < BQ_ROUNDS; ++r) {
-        const int     lm    = rslot + 16 * r;
+        const int     lm    = tile_row_of(rslot, r);
         const int64_t in_m  = in_m0 + lm;
         const bool    valid = in_m < in_end;
         float         vals[BQ_PACK];
@@ -202,14 +255,24 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
         if (tid == 0)
             a.s_row[(batch * gridDim.y + tm) * gridDim.x + tn] = 1.0f / scale;
         const float s[8] = {scale, scale, scale, scale, scale, scale, scale, scale};
+        [[maybe_unused]] u32x2 code4[4];
 #pragma unroll
         for (int r = 0; r < BQ_ROUNDS; ++r) {
-            const int64_t in_m = in_m0 + rslot + 16 * r;
-            if (in_m < in_end) {
-                float vals[BQ_PACK];
-                held[r].get(vals);
-                store8(a.q_row + batch * M * N + in_m * N + gn, quant8<E5M2>(vals, s, qmax), full, gn, N);
+            const int64_t in_m = in_m0 + tile_row_of(rslot, r);
+            float         vals[BQ_PACK];
+            held[r].get(vals);
+            const u32x2 code = quant8<E5M2>(vals, s, qmax); // rows beyond the matrix hold zeros: code 0
+            if (in_m < in_end)
+                store8(a.q_row + batch * M * N + in_m * N + gn, code, full, gn, N);
+            if constexpr (TRANS) {
+                code4[r & 3] = code;
+                if ((r & 3) == 3)
+                    stage_transposed(s_tr, code4, cseg, rslot + 16 * (r >> 2));
             }
+        }
+        if constexpr (TRANS) {
+            __syncthreads();
+            flush_transposed(s_tr, a.q_t + batch * N * a.ldt, a.ldt, tn * BQ, N, tm * BQ, M, tid);
         }
     }
 
@@ -236,14 +299,24 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
 #pragma unroll
         for (int i = 0; i < BQ_PACK; ++i)
             s[i] = s_cscale[cseg * BQ_PACK + i];
+        [[maybe_unused]] u32x2 code4[4];
 #pragma unroll
         for (int r = 0; r < BQ_ROUNDS; ++r) {
-            const int64_t out_m = tm * BQ + rslot + 16 * r;
-            if (out_m < M_out) { // grouped: pad rows carry zeros -> code 0
-                float vals[BQ_PACK];
-                held[r].get(vals);
-                store8(a.q_col + out_m * N + gn, quant8<E5M2>(vals, s, qmax), full, gn, N);
+            const int64_t out_m = tm * BQ + tile_row_of(rslot, r);
+            float         vals[BQ_PACK];
+            held[r].get(vals);
+            const u32x2 code = quant8<E5M2>(vals, s, qmax); // grouped: pad rows carry zeros -> code 0
+            if (a.q_col != nullptr && out_m < M_out)
+                store8(a.q_col + out_m * N + gn, code, full, gn, N);
+            if constexpr (TRANS) {
+                code4[r & 3] = code;
+                if ((r & 3) == 3)
+                    stage_transposed(s_tr, code4, cseg, rslot + 16 * (r >> 2));
             }
+        }
+        if constexpr (TRANS) {
+            __syncthreads();
+            flush_transposed(s_tr, a.q_t, a.ldt, tn * BQ, N, tm * BQ, a.ldt, tid);
         }
     }
 }
@@ -255,6 +328,15 @@ static int launch_block128(const BlockQuantArgs &a, int64_t tiles_m, int64_t til
         return PT_OK;
     dim3 g(static_cast<unsigned>(tiles_n), static_cast<unsigned>(tiles_m),
            static_cast<unsigned>(batch));
+    if constexpr (MODE == MODE_TILE || (GROUPED && MODE == (MODE_ROW | MODE_COL))) {
+        if (a.q_t != nullptr) {
+            if (vec)
+                quant_block128_kernel<T, E5M2, MODE, GROUPED, true, true><<<g, 256, 0, stream>>>(a);
+            else
+                quant_block128_kernel<T, E5M2, MODE, GROUPED, false, true><<<g, 256, 0, stream>>>(a);
+            return check_launch("quant_block128_kernel");
+        }
+    }
     if (vec)
         quant_block128_kernel<T, E5M2, MODE, GROUPED, true><<<g, 256, 0, stream>>>(a);
     else
@@ -426,20 +508,25 @@ int pt_quantize_fp8_blockwise(const void *x, int x_dtype, int64_t M, int64_t N, 
 #undef CALL
 }
 
-int pt_quantize_fp8_blockwise_weight(const void *w, int w_dtype, int64_t B, int64_t M, int64_t N,
-                                     void *q, int q_dtype, float *scale_inv, void *stream) {
+static int quantize_weight_tiles(const void *w, int w_dtype, int64_t B, int64_t M, int64_t N, void *q, void *q_t,
+                                 int64_t ldt, int q_dtype, float *scale_inv, void *stream) {
     PT_REQUIRE(is_hp_dtype(w_dtype), "input must be bf16, fp16 or fp32");
     PT_REQUIRE(is_fp8_dtype(q_dtype), "output must be e4m3 or e5m2");
     PT_REQUIRE(B >= 0 && M >= 0 && N >= 0, "dimensions must be non-negative");
     if (B * M * N == 0)
         return PT_OK;
     PT_REQUIRE(w && q && scale_inv, "NULL tensor pointer");
+    if (q_t != nullptr)
+        PT_REQUIRE(M % 16 == 0 && ldt >= M && ldt % 16 == 0 && aligned_to(q_t, 16),
+                   "the transposed output needs M % 16 == 0 and a 16-byte aligned pitch >= M");
     const int64_t tm = cdiv(M, BQ), tn = cdiv(N, BQ);
     PT_REQUIRE(tm < 65536 && B < 65536, "too many tiles / batches");
     BlockQuantArgs a{};
     a.x = w;
     a.q_row = static_cast<uint8_t *>(q);
     a.s_row = scale_inv;
+    a.q_t = static_cast<uint8_t *>(q_t);
+    a.ldt = ldt;
     a.M = M;
     a.N = N;
     a.qmax = fp8_max_of(q_dtype);
@@ -448,6 +535,17 @@ int pt_quantize_fp8_blockwise_weight(const void *w, int w_dtype, int64_t B, int6
 #define CALL(T, E5) return launch_block128<T, E5, MODE_TILE, false>(a, tm, tn, B, vec, st)
     PT_DISPATCH_T_E5(w_dtype, q_dtype, CALL);
 #undef CALL
+}
+
+int pt_quantize_fp8_blockwise_weight(const void *w, int w_dtype, int64_t B, int64_t M, int64_t N,
+                                     void *q, int q_dtype, float *scale_inv, void *stream) {
+    return quantize_weight_tiles(w, w_dtype, B, M, N, q, nullptr, 0, q_dtype, scale_inv, stream);
+}
+
+int pt_quantize_fp8_blockwise_weight_dual(const void *w, int w_dtype, int64_t B, int64_t M, int64_t N, void *q,
+                                          void *q_t, int64_t ldt, int q_dtype, float *scale_inv, void *stream) {
+    PT_REQUIRE(q_t != nullptr || B * M * N == 0, "q_t must not be NULL");
+    return quantize_weight_tiles(w, w_dtype, B, M, N, q, q_t, ldt, q_dtype, scale_inv, stream);
 }
 
 int pt_compute_group_offs(const int64_t *group_lens, int64_t num_groups, int64_t align,
@@ -461,29 +559,31 @@ int pt_compute_group_offs(const int64_t *group_lens, int64_t num_groups, int64_t
     return check_launch("group_offs_kernel");
 }
 
-int pt_quantize_fp8_blockwise_segment_m_row_col(const void *x, int x_dtype, int64_t M, int64_t N,
-                                                int q_dtype, const int64_t *group_offs,
-                                                const int64_t *padded_group_offs,
-                                                int64_t num_groups, void *q_row,
-                                                float *scale_inv_row, void *q_col_padded,
-                                                float *scale_inv_col_padded, void *stream) {
+static int quantize_segment_m(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype, const int64_t *group_offs,
+                              const int64_t *padded_group_offs, int64_t num_groups, void *q_row, float *scale_inv_row,
+                              void *q_col_padded, void *q_col_t, int64_t ldt, float *scale_inv_col_padded,
+                              void *stream) {
     PT_REQUIRE(is_hp_dtype(x_dtype), "input must be bf16, fp16 or fp32");
     PT_REQUIRE(is_fp8_dtype(q_dtype), "output must be e4m3 or e5m2");
     PT_REQUIRE(M >= 0 && N >= 0 && num_groups >= 1, "bad dimensions");
     PT_REQUIRE(group_offs && padded_group_offs, "group offsets must not be NULL");
-    PT_REQUIRE(q_row && scale_inv_row && q_col_padded && scale_inv_col_padded,
-               "NULL output pointer");
+    PT_REQUIRE(q_row && scale_inv_row && (q_col_padded || q_col_t) && scale_inv_col_padded, "NULL output pointer");
     if (N == 0)
         return PT_OK;
     PT_REQUIRE(x != nullptr || M == 0, "x must not be NULL");
     const int64_t tm = cdiv(M + num_groups * BQ, BQ), tn = cdiv(N, BQ);
     PT_REQUIRE(tm < 65536, "too many row tiles");
+    if (q_col_t != nullptr)
+        PT_REQUIRE(ldt >= tm * BQ && ldt % 16 == 0 && aligned_to(q_col_t, 16),
+                   "the transposed column output needs a 16-byte aligned pitch that holds every padded group");
     BlockQuantArgs a{};
     a.x = x;
     a.q_row = static_cast<uint8_t *>(q_row);
     a.s_row = scale_inv_row;
     a.q_col = static_cast<uint8_t *>(q_col_padded);
     a.s_col = scale_inv_col_padded;
+    a.q_t = static_cast<uint8_t *>(q_col_t);
+    a.ldt = ldt;
     a.M = M;
     a.N = N;
     a.rs_m = 1; // row scales are stored transposed: [N / 128, M]
@@ -497,6 +597,27 @@ int pt_quantize_fp8_blockwise_segment_m_row_col(const void *x, int x_dtype, int6
 #define CALL(T, E5) return launch_block128<T, E5, MODE_ROW | MODE_COL, true>(a, tm, tn, 1, vec, st)
     PT_DISPATCH_T_E5(x_dtype, q_dtype, CALL);
 #undef CALL
+}
+
+int pt_quantize_fp8_blockwise_segment_m_row_col(const void *x, int x_dtype, int64_t M, int64_t N,
+                                                int q_dtype, const int64_t *group_offs,
+                                                const int64_t *padded_group_offs,
+                                                int64_t num_groups, void *q_row,
+                                                float *scale_inv_row, void *q_col_padded,
+                                                float *scale_inv_col_padded, void *stream) {
+    PT_REQUIRE(q_col_padded != nullptr, "NULL output pointer");
+    return quantize_segment_m(x, x_dtype, M, N, q_dtype, group_offs, padded_group_offs, num_groups, q_row, scale_inv_row,
+                              q_col_padded, nullptr, 0, scale_inv_col_padded, stream);
+}
+
+int pt_quantize_fp8_blockwise_segment_m_row_col_t(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype,
+                                                  const int64_t *group_offs, const int64_t *padded_group_offs,
+                                                  int64_t num_groups, void *q_row, float *scale_inv_row,
+                                                  void *q_col_padded, void *q_col_t, int64_t ldt,
+                                                  float *scale_inv_col_padded, void *stream) {
+    PT_REQUIRE(q_col_t != nullptr, "q_col_t must not be NULL");
+    return quantize_segment_m(x, x_dtype, M, N, q_dtype, group_offs, padded_group_offs, num_groups, q_row, scale_inv_row,
+                              q_col_padded, q_col_t, ldt, scale_inv_col_padded, stream);
 }
 
 int pt_dequantize_fp8_block(const void *q, int q_dtype, int64_t B, int64_t M, int64_t N,

@@ -72,6 +72,15 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_int, c_i64, c_i64, c_i64, c_void_p, c_int, c_void_p, c_void_p],
     ),
+    "pt_quantize_fp8_blockwise_weight_dual": (
+        c_int,
+        [c_void_p, c_int, c_i64, c_i64, c_i64, c_void_p, c_void_p, c_i64, c_int, c_void_p, c_void_p],
+    ),
+    "pt_quantize_fp8_blockwise_segment_m_row_col_t": (
+        c_int,
+        [c_void_p, c_int, c_i64, c_i64, c_int, c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_void_p, c_void_p, c_i64,
+         c_void_p, c_void_p],
+    ),
     "pt_compute_group_offs": (c_int, [c_void_p, c_i64, c_i64, c_void_p, c_void_p, c_void_p]),
     "pt_quantize_fp8_blockwise_segment_m_row_col": (
         c_int,
@@ -106,7 +115,7 @@ _SIGNATURES = {
     "pt_grouped_gemm_fp8_variable_k": (
         c_int,
         [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_i64, c_i64, c_i64, c_i64,
-         c_int, c_int, c_void_p, c_size_t, c_int, c_void_p],
+         c_int, c_int, c_int, c_void_p, c_size_t, c_int, c_void_p],
     ),
     "pt_grouped_gemm_fp8_vec_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_i64, c_int]),
     "pt_grouped_gemm_fp8_vec": (
@@ -188,7 +197,13 @@ def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 
 def stream_of(t: torch.Tensor) -> int:
-    """Raw hipStream_t of torch's current stream on ``t``'s device."""
+    """Raw hipStream_t of torch's current stream on ``t``'s device. Kernels are launched on the
+    current device, so that has to be the tensor's."""
+    if t.device.index != torch.cuda.current_device():
+        raise RuntimeError(
+            f"primus_turbo: tensor on {t.device} but the current device is cuda:{torch.cuda.current_device()}; "
+            "wrap the call in torch.cuda.device(tensor.device)"
+        )
     return torch.cuda.current_stream(t.device).cuda_stream
 
 

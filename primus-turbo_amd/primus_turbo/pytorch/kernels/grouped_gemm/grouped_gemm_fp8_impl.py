@@ -270,28 +270,37 @@ def _grouped_gemm_fp8_impl_fake(a, b, a_scales, b_scales, group_lens, group_offs
 
 
 def _variable_k(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, accumulate):
-    _check(trans_a and not trans_b, "variable-K grouped GEMM computes a^T @ b (trans_a=True, trans_b=False)")
+    """``trans_a=True, trans_b=False``: ``a [Mp, Ml]``, ``b [Mp, Nr]`` (the reference's layout; both get
+    transposed into a workspace). ``trans_a=False, trans_b=True``: ``a [Ml, Mp]``, ``b [Nr, Mp]`` with
+    the padded rows contiguous already (``Mp % 128 == 0``): read in place."""
+    kmajor = (not trans_a) and trans_b
+    _check(kmajor or (trans_a and not trans_b),
+           "variable-K grouped GEMM computes a^T @ b (trans_a=True, trans_b=False) or, with both operands "
+           "transposed already, a @ b^T (trans_a=False, trans_b=True)")
     N.require_cuda(a, b, a_scales, b_scales, group_offs, out)
-    _check(a.dim() == 2 and b.dim() == 2 and a.shape[0] == b.shape[0], "a and b must be 2-D with the same row count")
+    r = 1 if kmajor else 0  # the axis of the (padded) rows
+    _check(a.dim() == 2 and b.dim() == 2 and a.shape[r] == b.shape[r], "a and b must be 2-D with the same row count")
     _check(a.dtype in _FP8 and b.dtype in _FP8, "operands must be float8_e4m3fn / float8_e5m2")
     a, b = a.contiguous(), b.contiguous()
     a_scales, b_scales = a_scales.contiguous(), b_scales.contiguous()
-    Mp, Ml = a.shape
-    Nr = b.shape[1]
+    Mp, Ml, Nr = a.shape[r], a.shape[1 - r], b.shape[1 - r]
     G = group_offs.numel() - 1
-    _check(tuple(a_scales.shape) == ((Mp + 127) // 128, Ml) or a_scales.shape[1] == Ml, "a_scales must be [rows/128, a.shape[1]]")
-    _check(b_scales.shape[1] == Nr, "b_scales must be [rows/128, b.shape[1]]")
+    _check(not kmajor or Mp % 128 == 0, "K-major operands need a padded row count that is a multiple of 128")
+    _check(a_scales.dim() == 2 and a_scales.shape[1] == Ml, "a_scales must be [rows/128, Ml]")
+    _check(b_scales.dim() == 2 and b_scales.shape[1] == Nr, "b_scales must be [rows/128, Nr]")
     want = (G, Nr, Ml) if trans_c else (G, Ml, Nr)
     _check(tuple(out.shape) == want and out.is_contiguous(), f"out must be a contiguous {want} tensor")
     lib = N.lib()
-    ws_bytes = lib.pt_grouped_gemm_fp8_variable_k_workspace_bytes(Mp, Ml, Nr)
-    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=a.device)
+    ws, ws_bytes = None, 0
+    if not kmajor:
+        ws_bytes = lib.pt_grouped_gemm_fp8_variable_k_workspace_bytes(Mp, Ml, Nr)
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=a.device)
     N.check(
         lib.pt_grouped_gemm_fp8_variable_k(
             N.ptr(a), N.dtype_code(a.dtype), N.ptr(a_scales),
             N.ptr(b), N.dtype_code(b.dtype), N.ptr(b_scales),
             N.ptr(out), N.dtype_code(out.dtype), N.ptr(group_offs), G, Mp, Ml, Nr, int(trans_c), int(accumulate),
-            N.ptr(ws), ws_bytes, TILE_CFG, N.stream_of(a),
+            int(kmajor), N.ptr(ws), ws_bytes, TILE_CFG, N.stream_of(a),
         )
     )
     return out
@@ -326,7 +335,8 @@ def grouped_gemm_fp8_variable_k_impl(
         out = torch.empty(shape, dtype=out_dtype, device=a.device)
         return _variable_k_vec(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, False)
     _require_blockwise(granularity)
-    shape = (G, b.shape[1], a.shape[1]) if trans_c else (G, a.shape[1], b.shape[1])
+    f = 0 if ((not trans_a) and trans_b) else 1  # the free axis: 0 when the operands come K-major
+    shape = (G, b.shape[f], a.shape[f]) if trans_c else (G, a.shape[f], b.shape[f])
     out = torch.empty(shape, dtype=out_dtype, device=a.device)
     return _variable_k(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans_c, out, False)
 
@@ -336,10 +346,8 @@ def _grouped_gemm_fp8_variable_k_impl_fake(a, b, a_scales, b_scales, group_lens,
                                            trans_c, out_dtype, granularity, num_cu, default_backend,
                                            maybe_pre_sync=False):
     G = group_offs.numel() - 1
-    if _is_mx(granularity):
-        shape = (G, b.shape[0], a.shape[0]) if trans_c else (G, a.shape[0], b.shape[0])
-    else:
-        shape = (G, b.shape[1], a.shape[1]) if trans_c else (G, a.shape[1], b.shape[1])
+    f = 0 if (_is_mx(granularity) or ((not trans_a) and trans_b and not _is_vec(granularity))) else 1
+    shape = (G, b.shape[f], a.shape[f]) if trans_c else (G, a.shape[f], b.shape[f])
     return torch.empty(shape, dtype=out_dtype, device=a.device)
 
 

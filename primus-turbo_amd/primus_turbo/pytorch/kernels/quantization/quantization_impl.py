@@ -390,6 +390,43 @@ def _quant_fp8_blockwise_for_weight_impl_fake(w, dtype, block_size=128):
     return q, s
 
 
+@torch.library.custom_op("primus_turbo::quant_fp8_blockwise_for_weight_dual_impl", mutates_args=())
+def quant_fp8_blockwise_for_weight_dual_impl(
+    w: torch.Tensor, dtype: torch.dtype, block_size: int = 128
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """:func:`quant_fp8_blockwise_for_weight_impl` plus, from the same read of ``w``, the codes
+    transposed in their last two dimensions -> ``(w_fp8 [.., M, N], w_fp8_t [.., N, M], scale_inv)``.
+    The transposed copy is the K-contiguous operand of the product that reduces over M (dgrad of a
+    linear layer); it goes with ``scale_inv`` transposed in its last two dimensions. ``M % 16 == 0``.
+    (No counterpart in the reference, whose GEMM backends read either layout.)"""
+    N.require_cuda(w)
+    _check(w.dtype in _HP_DTYPES, "input must be bfloat16, float16 or float32")
+    _check_fp8_out(dtype)
+    _check(w.dim() in (2, 3), "weight quant requires 2D or 3D input")
+    _need_block_128(block_size)
+    w = w.contiguous()
+    B, M, Nn, sshape = _weight_shapes(w, block_size)
+    _check(M % 16 == 0, "the transposed copy needs a row count that is a multiple of 16")
+    q = torch.empty_like(w, dtype=dtype)
+    q_t = torch.empty(w.shape[:-2] + (Nn, M), dtype=dtype, device=w.device)
+    sc = torch.empty(sshape, dtype=torch.float32, device=w.device)
+    N.check(
+        N.lib().pt_quantize_fp8_blockwise_weight_dual(
+            N.ptr(w), N.dtype_code(w.dtype), B, M, Nn, N.ptr(q), N.ptr(q_t), M, N.dtype_code(dtype), N.ptr(sc),
+            N.stream_of(w),
+        )
+    )
+    return q, q_t, sc
+
+
+@quant_fp8_blockwise_for_weight_dual_impl.register_fake
+def _quant_fp8_blockwise_for_weight_dual_impl_fake(w, dtype, block_size=128):
+    _, M, Nn, sshape = _weight_shapes(w, block_size)
+    return (torch.empty(w.shape, dtype=dtype, device=w.device),
+            torch.empty(w.shape[:-2] + (Nn, M), dtype=dtype, device=w.device),
+            torch.empty(sshape, dtype=torch.float32, device=w.device))
+
+
 def _dequant_block(q: torch.Tensor, scale_inv: torch.Tensor, out_dtype, B, M, Nn, bm, bn):
     N.require_cuda(q, scale_inv)
     _check(q.dtype in _FP8_DTYPES, "input must be float8_e4m3fn or float8_e5m2")
@@ -558,6 +595,58 @@ def quant_fp8_blockwise_segment_m_row_col_impl(
 def _quant_fp8_blockwise_segment_m_row_col_impl_fake(x, dtype, block_size, group_lens, group_offs, gemm_other_dim=None):
     r = _quantize_fp8_blockwise_segment_m_row_col_meta(x, dtype, block_size, group_lens, group_offs)
     return r[0], r[1], r[2], r[3], r[4], r[5]
+
+
+def _segment_t_pitch(M: int, G: int, block_size: int) -> int:
+    return ceil_div(M + G * block_size, block_size) * block_size
+
+
+@torch.library.custom_op("primus_turbo::quant_fp8_blockwise_segment_m_row_col_t_impl", mutates_args=())
+def quant_fp8_blockwise_segment_m_row_col_t_impl(
+    x: torch.Tensor, dtype: torch.dtype, block_size: int, group_lens: torch.Tensor, group_offs: torch.Tensor
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """:func:`quant_fp8_blockwise_segment_m_row_col_impl` with the segment-padded column codes
+    emitted transposed: ``x_fp8_col_t [N, Mp]`` (``Mp`` = ``M + G * b`` rounded up to ``b``), the
+    K-contiguous operand of the variable-K wgrad product; everything else (row codes, both scale
+    tensors, padded lens / offs) as there. (No counterpart in the reference, whose GEMM backends
+    read the untransposed layout.)"""
+    N.require_cuda(x, group_lens, group_offs)
+    _check(x.dtype in _HP_DTYPES, "input must be bfloat16, float16 or float32")
+    _check_fp8_out(dtype)
+    _check(x.dim() == 2 and x.is_contiguous(), "input must be 2D and contiguous")
+    _need_block_128(block_size)
+    for t in (group_lens, group_offs):
+        _check(t.dtype == torch.int64 and t.is_contiguous(), "group_lens / group_offs must be contiguous int64")
+    G = group_lens.numel()
+    _check(group_offs.numel() == G + 1, "group_offs must have one more element than group_lens")
+    M, Nn = x.shape
+    _, rs_shape, cs_shape = _segment_shapes(M, Nn, G, block_size)
+    ldt = _segment_t_pitch(M, G, block_size)
+    dev = x.device
+    padded_lens, padded_offs = _group_offs(group_lens, block_size, True)
+    q_row = torch.empty((M, Nn), dtype=dtype, device=dev)
+    q_col_t = torch.empty((Nn, ldt), dtype=dtype, device=dev)
+    s_row = torch.empty(rs_shape, dtype=torch.float32, device=dev)
+    s_col = torch.empty(cs_shape, dtype=torch.float32, device=dev)
+    N.check(
+        N.lib().pt_quantize_fp8_blockwise_segment_m_row_col_t(
+            N.ptr(x), N.dtype_code(x.dtype), M, Nn, N.dtype_code(dtype), N.ptr(group_offs), N.ptr(padded_offs), G,
+            N.ptr(q_row), N.ptr(s_row), None, N.ptr(q_col_t), ldt, N.ptr(s_col), N.stream_of(x),
+        )
+    )
+    return q_row, q_col_t, s_row, s_col, padded_lens, padded_offs
+
+
+@quant_fp8_blockwise_segment_m_row_col_t_impl.register_fake
+def _quant_fp8_blockwise_segment_m_row_col_t_impl_fake(x, dtype, block_size, group_lens, group_offs):
+    M, Nn = x.shape
+    G = group_lens.numel()
+    _, rs_shape, cs_shape = _segment_shapes(M, Nn, G, block_size)
+    dev = x.device
+    return (torch.empty((M, Nn), dtype=dtype, device=dev),
+            torch.empty((Nn, _segment_t_pitch(M, G, block_size)), dtype=dtype, device=dev),
+            torch.empty(rs_shape, dtype=torch.float32, device=dev), torch.empty(cs_shape, dtype=torch.float32, device=dev),
+            torch.empty(G, dtype=torch.int64, device=dev), torch.empty(G + 1, dtype=torch.int64, device=dev))
 
 
 # ---------------------------------------------------------------------------------------

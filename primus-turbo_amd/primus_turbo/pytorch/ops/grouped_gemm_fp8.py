@@ -41,8 +41,10 @@ from primus_turbo.pytorch.kernels.grouped_gemm.grouped_gemm_fp8_impl import (
 from primus_turbo.pytorch.kernels.grouped_gemm.grouped_gemm_utils import group_offs_from_lens
 from primus_turbo.pytorch.kernels.quantization.quantization_impl import (
     grouped_quantize_mxfp8_impl,
+    quant_fp8_blockwise_for_weight_dual_impl,
     quant_fp8_blockwise_for_weight_impl,
     quant_fp8_blockwise_segment_m_row_col_impl,
+    quant_fp8_blockwise_segment_m_row_col_t_impl,
     quantize_mxfp8_impl,
 )
 from primus_turbo.pytorch.ops.utils import (
@@ -89,41 +91,63 @@ class FP8GroupedGemmBlockFunc(torch.autograd.Function):
         a_dtype = _get_fp8_dtype(config.format, True)
         b_dtype = _get_fp8_dtype(config.format, True)
 
-        gemm_n = b.size(-2) if trans_b else b.size(-1)
-        a_fp8_row, a_fp8_col, a_scale_row, a_scale_col, _, _ = quant_fp8_blockwise_segment_m_row_col_impl(
-            a.contiguous(), a_dtype, config.block_size, group_lens, group_offs, gemm_other_dim=gemm_n
-        )
+        need_bwd = any(ctx.needs_input_grad[:2])
+        bs = config.block_size
+        # Backward reduces over the tokens (wgrad) and over the other weight axis (dgrad): the
+        # quantizers emit those operands K-contiguous from the same read, so that no GEMM has to
+        # transpose anything. (A caller-quantized weight has no such copy: the GEMM transposes it.)
+        if need_bwd:
+            a_fp8_row, a_fp8_col_t, a_scale_row, a_scale_col, _, _ = quant_fp8_blockwise_segment_m_row_col_t_impl(
+                a.contiguous(), a_dtype, bs, group_lens, group_offs)
+        else:
+            a_fp8_row, _, a_scale_row, _, _, _ = quant_fp8_blockwise_segment_m_row_col_impl(
+                a.contiguous(), a_dtype, bs, group_lens, group_offs)
+            a_fp8_col_t = a_scale_col = None
         b_recipe = ScalingRecipe(use_2d_block=True)
+        b_fp8_t = None
         if isinstance(b, QuantizedTensor):
             check_quantized_tensor(b, config, scaling_recipe=b_recipe)
             b_fp8, b_scale = b.qdata, b.scale_inv
+        elif (need_bwd or not trans_b) and b.size(-2) % 16 == 0:
+            b_fp8, b_fp8_t, b_scale = quant_fp8_blockwise_for_weight_dual_impl(b, b_dtype, block_size=bs)
         else:
-            b_fp8, b_scale = quant_fp8_blockwise_for_weight_impl(b, b_dtype, block_size=config.block_size)
+            b_fp8, b_scale = quant_fp8_blockwise_for_weight_impl(b, b_dtype, block_size=bs)
 
-        out = grouped_gemm_fp8_impl(a_fp8_row, b_fp8, a_scale_row, b_scale, group_lens, group_offs, False, trans_b,
-                                    out_dtype, config.granularity.value, num_cu, _NATIVE)
-        ctx.save_for_backward(a_fp8_col, a_scale_col, b_fp8, b_scale, group_lens, group_offs)
-        ctx.meta = (trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad)
+        # fwd reduces over b's last axis when trans_b, else over its middle axis
+        fwd_b, dgrad_b = (b_fp8, b_fp8_t) if trans_b else (b_fp8_t, b_fp8)
+        b_scale_t = b_scale.transpose(-2, -1).contiguous() if b_fp8_t is not None else None
+        fwd_s, dgrad_s = (b_scale, b_scale_t) if trans_b else (b_scale_t, b_scale)
+        if fwd_b is not None:
+            out = grouped_gemm_fp8_impl(a_fp8_row, fwd_b, a_scale_row, fwd_s, group_lens, group_offs, False, True,
+                                        out_dtype, config.granularity.value, num_cu, _NATIVE)
+        else:
+            out = grouped_gemm_fp8_impl(a_fp8_row, b_fp8, a_scale_row, b_scale, group_lens, group_offs, False, trans_b,
+                                        out_dtype, config.granularity.value, num_cu, _NATIVE)
+        if need_bwd:
+            if dgrad_b is not None:
+                ctx.save_for_backward(a_fp8_col_t, a_scale_col, dgrad_b, dgrad_s, group_lens, group_offs)
+            else:
+                ctx.save_for_backward(a_fp8_col_t, a_scale_col, b_fp8, b_scale, group_lens, group_offs)
+        ctx.meta = (trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad, dgrad_b is not None)
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
         grad_out = _ensure_contiguous_grad_out(grad_out)
-        a_fp8_col, a_scale_col, b_fp8, b_scale, group_lens, group_offs = ctx.saved_tensors
-        trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad = ctx.meta
+        a_fp8_col_t, a_scale_col, b_fp8, b_scale, group_lens, group_offs = ctx.saved_tensors
+        trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad, b_ready = ctx.meta
         g_dtype = _get_fp8_dtype(config.format, False)
         gran = config.granularity.value
 
-        gemm_k = b_fp8.size(-1) if trans_b else b_fp8.size(-2)
-        g_row, g_col, g_scale_row, g_scale_col, var_k_lens, var_k_offs = quant_fp8_blockwise_segment_m_row_col_impl(
-            grad_out, g_dtype, config.block_size, group_lens, group_offs, gemm_other_dim=gemm_k
-        )
-        # grad_a = grad_out @ b^T
-        grad_a = grouped_gemm_fp8_impl(g_row, b_fp8, g_scale_row, b_scale, group_lens, group_offs, False, not trans_b,
-                                       out_dtype, gran, num_cu, _NATIVE)
-        # grad_b[g] = a_g^T @ grad_out_g
+        g_row, g_col_t, g_scale_row, g_scale_col, var_k_lens, var_k_offs = quant_fp8_blockwise_segment_m_row_col_t_impl(
+            grad_out, g_dtype, config.block_size, group_lens, group_offs)
+        # grad_a = grad_out @ b^T: the saved weight copy is contiguous along the reduction already,
+        # or (caller-quantized weight) the forward operand read the other way round
+        grad_a = grouped_gemm_fp8_impl(g_row, b_fp8, g_scale_row, b_scale, group_lens, group_offs, False,
+                                       True if b_ready else not trans_b, out_dtype, gran, num_cu, _NATIVE)
+        # grad_b[g] = a_g^T @ grad_out_g over the padded token ranges, both operands K-major
         grad_b = _grouped_gemm_fp8_variable_k_impl_wrapper(
-            a_fp8_col, g_col, a_scale_col, g_scale_col, var_k_lens, var_k_offs, True, False, trans_b, out_dtype, gran,
+            a_fp8_col_t, g_col_t, a_scale_col, g_scale_col, var_k_lens, var_k_offs, False, True, trans_b, out_dtype, gran,
             num_cu, _NATIVE, inplace_add_to_out=fuse_bgrad_accum, out=main_grad,
         )
         return grad_a, grad_b, None, None, None, None, None, None, None, None, None

@@ -168,3 +168,34 @@ def test_grouped_gemm_fp8_autograd(trans_b):
     for g in range(G_):
         if lens[g] == 0:
             assert torch.count_nonzero(b.grad[g]).item() == 0
+
+
+@pytest.mark.parametrize("kind,G_,M,N,K", CASES[:5])
+@pytest.mark.parametrize("trans_c", [True, False])
+def test_grouped_variable_k_kmajor_operands(kind, G_, M, N, K, trans_c):
+    """The variable-K product over operands that arrive transposed (``trans_a=False, trans_b=True``:
+    the transposed column output of the grouped quantizer) is bit-identical to the product that
+    transposes the untransposed ones itself, also with the beta = 1 epilogue."""
+    lens = group_lens(kind, G_, M, 39)
+    gl, offs = _offs(lens)
+    x = bf16_randn((M, K), seed=40).cuda()
+    dy = bf16_randn((M, N), seed=41).cuda()
+    seg, seg_t = qimpl.quant_fp8_blockwise_segment_m_row_col_impl, qimpl.quant_fp8_blockwise_segment_m_row_col_t_impl
+    _, xc, _, xs, plens, poffs = seg(x, torch.float8_e4m3fn, 128, gl, offs, N)
+    _, gc, _, gs, _, _ = seg(dy, torch.float8_e5m2, 128, gl, offs, K)
+    _, xct, _, xs2, _, _ = seg_t(x, torch.float8_e4m3fn, 128, gl, offs)
+    _, gct, _, gs2, _, _ = seg_t(dy, torch.float8_e5m2, 128, gl, offs)
+    args = (plens, poffs)
+    ref = gimpl.grouped_gemm_fp8_variable_k_impl(xc, gc, xs, gs, *args, True, False, trans_c, torch.bfloat16,
+                                                 G.BLOCKWISE.value, None, 0)
+    out = gimpl.grouped_gemm_fp8_variable_k_impl(xct, gct, xs2, gs2, *args, False, True, trans_c, torch.bfloat16,
+                                                 G.BLOCKWISE.value, None, 0)
+    torch.cuda.synchronize()
+    assert out.shape == ref.shape and torch.equal(out, ref)
+    acc = torch.full(ref.shape, 0.5, dtype=torch.float32, device="cuda")
+    acc_ref = acc.clone()
+    gimpl.grouped_gemm_fp8_variable_k_accum_impl(xct, gct, xs2, gs2, *args, False, True, trans_c, torch.float32,
+                                                 G.BLOCKWISE.value, None, 0, acc)
+    gimpl.grouped_gemm_fp8_variable_k_accum_impl(xc, gc, xs, gs, *args, True, False, trans_c, torch.float32,
+                                                 G.BLOCKWISE.value, None, 0, acc_ref)
+    assert torch.equal(acc, acc_ref)

@@ -128,3 +128,44 @@ def test_grouped_segment_row_col(kind, G_, M, N):
     # row scales are the plain 1x128 scales transposed
     _, s_plain = turbo.ops.quantize_fp8(x.cuda(), torch.float8_e4m3fn, G.BLOCKWISE, block_size=128, axis=1)
     assert torch.equal(sr, s_plain.t().contiguous())
+
+
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+@pytest.mark.parametrize("shape", [(7168, 2048), (4, 512, 384), (2, 144, 260), (112, 100), (3, 16, 8), (8, 4096, 1024)])
+def test_blockwise_weight_dual_transposed_copy(shape, dtype):
+    """The dual weight quantizer: codes and scales identical to the plain one, and the second output
+    is exactly the transpose of the codes (per batch slice)."""
+    from primus_turbo.pytorch.kernels.quantization.quantization_impl import quant_fp8_blockwise_for_weight_dual_impl as dual
+
+    x = bf16_randn(shape, seed=26).cuda()
+    q, s = turbo.ops.quantize_fp8(x, dtype, G.BLOCKWISE, block_size=128, scaling_recipe=ScalingRecipe(use_2d_block=True))
+    q2, qt, s2 = dual(x, dtype, 128)
+    torch.cuda.synchronize()
+    assert torch.equal(q2.view(torch.uint8), q.view(torch.uint8)) and torch.equal(s2, s)
+    assert qt.shape == x.shape[:-2] + (x.shape[-1], x.shape[-2])
+    assert torch.equal(qt.view(torch.uint8), q.view(torch.uint8).transpose(-2, -1).contiguous())
+    with pytest.raises(RuntimeError, match="multiple of 16"):
+        dual(bf16_randn((100, 128), seed=1).cuda(), dtype, 128)
+
+
+@pytest.mark.parametrize("kind,G_,M,N", [("balanced", 4, 1024, 512), ("ragged", 8, 3000, 384), ("zeros", 8, 16384, 256),
+                                         ("ragged", 3, 77, 104), ("zipf", 32, 8192, 7168)])
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+def test_grouped_segment_row_col_transposed(kind, G_, M, N, dtype):
+    """The grouped quantizer with the column codes emitted transposed: everything equals the plain
+    variant, the transposed codes are its column output transposed (up to the last padded group)."""
+    from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+    lens = group_lens(kind, G_, M, 27)
+    x = bf16_randn((M, N), seed=28, outlier_frac=0.001).cuda()
+    gl = torch.from_numpy(lens).cuda()
+    offs = torch.ops.primus_turbo_cpp_extension.grouped_gemm_compute_offs(gl)
+    qr, qc, sr, sc, plens, poffs = qi.quant_fp8_blockwise_segment_m_row_col_impl(x, dtype, 128, gl, offs, N)
+    qr2, qct, sr2, sc2, plens2, poffs2 = qi.quant_fp8_blockwise_segment_m_row_col_t_impl(x, dtype, 128, gl, offs)
+    torch.cuda.synchronize()
+    w = int(poffs[-1])
+    assert torch.equal(qr2.view(torch.uint8), qr.view(torch.uint8)) and torch.equal(sr2, sr)
+    assert torch.equal(plens2, plens) and torch.equal(poffs2, poffs)
+    assert torch.equal(sc2[: w // 128], sc[: w // 128])
+    assert qct.shape == (N, -(-(M + 128 * G_) // 128) * 128)
+    assert torch.equal(qct.view(torch.uint8)[:, :w], qc.view(torch.uint8)[:w].t().contiguous())
