@@ -488,7 +488,8 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     static_assert(MODE != SCALE_BLOCK || SB_VEC || TN * 16 <= 128, "one B scale per wavefront and slab");
     [[maybe_unused]] uint32_t unit_scale = 0x7f7f7f7fu; // E8M0 1.0 for all four K blocks
     // GROUP_K tiles have their own K extent (possibly none at all): they run the pipeline per
-    // tile instead of across tile boundaries
+    // tile instead of across tile boundaries; only the request for a tile's first two slabs is
+    // moved ahead of the previous tile's epilogue
     constexpr bool XPIPE = GMODE != GROUP_K;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
@@ -568,6 +569,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     const uint8_t *ld_ga, *ld_gb; // slab the loader points at
     uint32_t       ld_na, ld_nb;  // bytes from there to the end of the tile's rows
     int            ld_kt;
+    int            ld_KT = 0;     // slabs of the loader's tile (tiles with their own K extent)
     // scales of the loader's slab for the tile's first row / column, and the end of the scale
     // arrays (reads beyond return zero; they only ever meet rows that are never stored)
     [[maybe_unused]] const uint8_t *ld_sa = nullptr, *ld_sb = nullptr, *ld_sa_end = nullptr, *ld_sb_end = nullptr;
@@ -595,6 +597,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         ld_na = t.rows_a * static_cast<uint32_t>(a.lda);
         ld_nb = t.rows_b * static_cast<uint32_t>(a.ldb);
         ld_kt = 0;
+        ld_KT = t.KT;
         scales_to(t);
     };
     // bytes a scale copy may read: none for a slab of zero padding beyond the K blocks the
@@ -650,7 +653,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                 ld_sb_end         = wrap ? as_bytes(nxt_t.sB) + sb_extent : ld_sb_end;
             }
         } else {
-            const int adv = ld_kt + 1 < cur_t.KT ? KSTEP : 0;
+            const int adv = ld_kt + 1 < ld_KT ? KSTEP : 0;
             ld_kt += adv / KSTEP;
             ld_ga += adv;
             ld_gb += adv;
@@ -720,14 +723,21 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     const uint32_t a_part = wm * (TM * 16) * KSTEP;
     const uint32_t b_part = A_BYTES + wn * (TN * 16) * KSTEP;
 
-    // pipeline start at tile t: two slabs requested, the fragments of slab 0 on their way
-    auto start_pipeline = [&](const TileCtx &t) {
+    // pipeline start at tile t, in two steps: the first two slabs are requested (stages 0 and 1,
+    // which nobody may still be reading) ...
+    auto request_first_slabs = [&](const TileCtx &t) {
         loader_to(t);
         static_for<0, 2>([&](auto st) {
             static_for<0, NB>([&](auto c) { issue_part_b(c, st); });
             static_for<0, LA>([&](auto c) { issue_copy(c, st); });
             advance_loader();
         });
+    };
+    // ... and, once slab 0 has landed, its fragments go into registers. The wait leaves NL
+    // operations in flight: whatever else was issued after the two slabs (output stores of the
+    // previous tile), the copies of slab 0 are older than the NL copies of slab 1 and copies
+    // complete in order, so none of them can be among the NL youngest.
+    auto take_first_slab = [&]() {
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
         __builtin_amdgcn_s_barrier();
         buf = 0;
@@ -741,8 +751,13 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     };
     PT_GEMM_TRACE_DECL;
     PT_GEMM_TRACE_POINT(0);
-    if constexpr (XPIPE)
-        start_pipeline(cur_t);
+    if constexpr (XPIPE) {
+        request_first_slabs(cur_t);
+        take_first_slab();
+    } else {
+        if (cur_t.KT > 0)
+            request_first_slabs(cur_t);
+    }
 
     while (true) {
 #pragma unroll
@@ -758,7 +773,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         const int KT = XPIPE ? KT_ALL : cur_t.KT;
         if constexpr (!XPIPE) {
             if (KT > 0)
-                start_pipeline(cur_t);
+                take_first_slab(); // requested before the loop or before the previous tile's epilogue
         }
 
         // one K slab per iteration; the body must stay a single basic block (no branches), or
@@ -887,6 +902,9 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             // done reading the stages, before the next tile's first copies go into them
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_s_barrier();
+            // the next tile's first slabs travel while this tile's result is written out
+            if (next_tile < total && nxt_t.KT > 0)
+                request_first_slabs(nxt_t);
         }
 
         // the epilogue reads the accumulators with hand-written instructions the compiler's
