@@ -128,6 +128,15 @@ PT_API int pt_dequantize_fp8_rowwise(const void *q, int q_dtype, int64_t B, int6
 PT_API int pt_quantize_fp8_blockwise(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype,
                                      void *q_row, float *scale_inv_row, void *q_col,
                                      float *scale_inv_col, void *stream);
+/* The dual form with the column codes (also, or only: q_col may be NULL) emitted transposed,
+ * q_col_t [N, ldt] with q_col_t[n, m] = q_col[m, n] and zeros in columns [M, ldt), ldt = M
+ * rounded up to 128: the K-contiguous operand of the wgrad product of a linear layer (the
+ * reference hands the untransposed codes to backends that read either layout,
+ * ops/gemm_fp8.py:477-560). q_row / scale_inv_row are required. */
+PT_API int pt_quantize_fp8_blockwise_t(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype,
+                                       void *q_row, float *scale_inv_row, void *q_col,
+                                       void *q_col_t, int64_t ldt, float *scale_inv_col,
+                                       void *stream);
 
 /* Replaces torch.ops.primus_turbo_cpp_extension.quantize_fp8_blockwise_for_weight
  * (bindings_pytorch.cpp:52-93, csrc/pytorch/quantization/quantization.cpp:1443-1480,

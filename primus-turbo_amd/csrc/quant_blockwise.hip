@@ -328,7 +328,7 @@ static int launch_block128(const BlockQuantArgs &a, int64_t tiles_m, int64_t til
         return PT_OK;
     dim3 g(static_cast<unsigned>(tiles_n), static_cast<unsigned>(tiles_m),
            static_cast<unsigned>(batch));
-    if constexpr (MODE == MODE_TILE || (GROUPED && MODE == (MODE_ROW | MODE_COL))) {
+    if constexpr (MODE == MODE_TILE || MODE == (MODE_ROW | MODE_COL)) {
         if (a.q_t != nullptr) {
             if (vec)
                 quant_block128_kernel<T, E5M2, MODE, GROUPED, true, true><<<g, 256, 0, stream>>>(a);
@@ -468,13 +468,13 @@ using namespace pt;
 
 extern "C" {
 
-int pt_quantize_fp8_blockwise(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype,
-                              void *q_row, float *scale_inv_row, void *q_col, float *scale_inv_col,
-                              void *stream) {
+static int quantize_blocks(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype, void *q_row,
+                           float *scale_inv_row, void *q_col, void *q_col_t, int64_t ldt, float *scale_inv_col,
+                           void *stream) {
     PT_REQUIRE(is_hp_dtype(x_dtype), "input must be bf16, fp16 or fp32");
     PT_REQUIRE(is_fp8_dtype(q_dtype), "output must be e4m3 or e5m2");
     PT_REQUIRE(M >= 0 && N >= 0, "dimensions must be non-negative");
-    const bool row = q_row != nullptr, col = q_col != nullptr;
+    const bool row = q_row != nullptr, col = q_col != nullptr || q_col_t != nullptr;
     PT_REQUIRE(row || col, "at least one of q_row / q_col must be given");
     PT_REQUIRE(!row || scale_inv_row, "scale_inv_row must accompany q_row");
     PT_REQUIRE(!col || scale_inv_col, "scale_inv_col must accompany q_col");
@@ -483,12 +483,17 @@ int pt_quantize_fp8_blockwise(const void *x, int x_dtype, int64_t M, int64_t N, 
     PT_REQUIRE(x != nullptr, "x must not be NULL");
     const int64_t tm = cdiv(M, BQ), tn = cdiv(N, BQ);
     PT_REQUIRE(tm < 65536, "too many row tiles");
+    if (q_col_t != nullptr)
+        PT_REQUIRE(row && ldt == tm * BQ && aligned_to(q_col_t, 16),
+                   "the transposed column output comes with the row output, at a 16-byte aligned pitch of M rounded up to 128");
     BlockQuantArgs a{};
     a.x = x;
     a.q_row = static_cast<uint8_t *>(q_row);
     a.s_row = scale_inv_row;
     a.q_col = static_cast<uint8_t *>(q_col);
     a.s_col = scale_inv_col;
+    a.q_t = static_cast<uint8_t *>(q_col_t);
+    a.ldt = ldt;
     a.M = M;
     a.N = N;
     a.rs_m = tn;
@@ -506,6 +511,19 @@ int pt_quantize_fp8_blockwise(const void *x, int x_dtype, int64_t M, int64_t N, 
     } while (0)
     PT_DISPATCH_T_E5(x_dtype, q_dtype, CALL);
 #undef CALL
+}
+
+int pt_quantize_fp8_blockwise(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype,
+                              void *q_row, float *scale_inv_row, void *q_col, float *scale_inv_col,
+                              void *stream) {
+    return quantize_blocks(x, x_dtype, M, N, q_dtype, q_row, scale_inv_row, q_col, nullptr, 0, scale_inv_col, stream);
+}
+
+int pt_quantize_fp8_blockwise_t(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype, void *q_row,
+                                float *scale_inv_row, void *q_col, void *q_col_t, int64_t ldt, float *scale_inv_col,
+                                void *stream) {
+    PT_REQUIRE(q_col_t != nullptr || M * N == 0, "q_col_t must not be NULL");
+    return quantize_blocks(x, x_dtype, M, N, q_dtype, q_row, scale_inv_row, q_col, q_col_t, ldt, scale_inv_col, stream);
 }
 
 static int quantize_weight_tiles(const void *w, int w_dtype, int64_t B, int64_t M, int64_t N, void *q, void *q_t,

@@ -47,6 +47,11 @@ def _scale_desc(granularity, a_scale_inv, b_scale_inv, trans_a, trans_b, M, Nn, 
     if granularity == ScalingGranularity.BLOCKWISE:
         kb = (K + 127) // 128
         if not trans_a and trans_b:  # NT: A [M,K] 1x128 scales [M,kb]; B [N,K] tile scales [N/128,kb]
+            std = tuple(a_scale_inv.shape) == (M, kb) and tuple(b_scale_inv.shape) == ((Nn + 127) // 128, kb)
+            if not std and tuple(a_scale_inv.shape) == (kb, M) and tuple(b_scale_inv.shape) == (kb, Nn):
+                # both operands are transposed 128 x 1 column quantizations (K-contiguous data,
+                # scales still [K/128, rows]): the wgrad product without a transposition pass
+                return 1, 1, M, 1, Nn, 1, 1
             _check(tuple(a_scale_inv.shape) == (M, kb), "blockwise NT: a_scale_inv must be [M, K/128]")
             _check(tuple(b_scale_inv.shape) == ((Nn + 127) // 128, kb), "blockwise NT: b_scale_inv must be [N/128, K/128]")
             return 1, kb, 1, kb, 1, 1, 128

@@ -328,6 +328,47 @@ def _quant_fp8_blockwise_dual_impl_fake(x, dtype, block_size=128):
     )
 
 
+@torch.library.custom_op("primus_turbo::quant_fp8_blockwise_dual_t_impl", mutates_args=())
+def quant_fp8_blockwise_dual_t_impl(
+    x: torch.Tensor, dtype: torch.dtype, block_size: int = 128
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """:func:`quant_fp8_blockwise_dual_impl` with the column codes emitted transposed and zero-padded:
+    ``(x_fp8_row, scales_row [M, N/b], x_fp8_col_t [N, M_pad], scales_col [M/b, N])``, ``M_pad`` = ``M``
+    rounded up to ``b`` -- the K-contiguous operand of the product that reduces over the rows of ``x``
+    (wgrad). (No counterpart in the reference, whose GEMM backends read the untransposed layout.)"""
+    N.require_cuda(x)
+    _check(x.dtype in _HP_DTYPES, "input must be bfloat16, float16 or float32")
+    _check_fp8_out(dtype)
+    _check(x.dim() == 2 and x.is_contiguous(), "Input must be 2D and contiguous")
+    _need_block_128(block_size)
+    M, Nn = x.shape
+    Mp = ceil_div(M, block_size) * block_size
+    dev = x.device
+    q_row = torch.empty((M, Nn), dtype=dtype, device=dev)
+    s_row = torch.empty((M, ceil_div(Nn, block_size)), dtype=torch.float32, device=dev)
+    q_col_t = torch.empty((Nn, Mp), dtype=dtype, device=dev)
+    s_col = torch.empty((ceil_div(M, block_size), Nn), dtype=torch.float32, device=dev)
+    N.check(
+        N.lib().pt_quantize_fp8_blockwise_t(
+            N.ptr(x), N.dtype_code(x.dtype), M, Nn, N.dtype_code(dtype), N.ptr(q_row), N.ptr(s_row), None,
+            N.ptr(q_col_t), Mp, N.ptr(s_col), N.stream_of(x),
+        )
+    )
+    return q_row, s_row, q_col_t, s_col
+
+
+@quant_fp8_blockwise_dual_t_impl.register_fake
+def _quant_fp8_blockwise_dual_t_impl_fake(x, dtype, block_size=128):
+    M, Nn = x.shape
+    dev = x.device
+    return (
+        torch.empty((M, Nn), dtype=dtype, device=dev),
+        torch.empty((M, ceil_div(Nn, block_size)), dtype=torch.float32, device=dev),
+        torch.empty((Nn, ceil_div(M, block_size) * block_size), dtype=dtype, device=dev),
+        torch.empty((ceil_div(M, block_size), Nn), dtype=torch.float32, device=dev),
+    )
+
+
 # quantize_fp8_blockwise_for_weight(Tensor input, ScalarType dest_dtype, int block_size) -> Tensor[]
 _ext.define("quantize_fp8_blockwise_for_weight(Tensor input, ScalarType dest_dtype, int block_size) -> Tensor[]")
 

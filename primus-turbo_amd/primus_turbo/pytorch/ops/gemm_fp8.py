@@ -33,6 +33,10 @@ from primus_turbo.pytorch.core.quantized_tensor import (
     check_quantized_tensor,
 )
 from primus_turbo.pytorch.kernels.gemm.gemm_fp8_impl import gemm_fp8_accum_impl, gemm_fp8_impl
+from primus_turbo.pytorch.kernels.quantization.quantization_impl import (
+    quant_fp8_blockwise_dual_t_impl,
+    quant_fp8_blockwise_for_weight_dual_impl,
+)
 from primus_turbo.pytorch.ops.quantization import quantize_fp8, quantize_fp8_with_trans
 from primus_turbo.pytorch.ops.utils import _get_dummy_wgrad, _get_fp8_dtype, _setup_fused_grad_accum
 
@@ -143,44 +147,72 @@ class FP8GemmRowFunction(torch.autograd.Function):
 
 
 class FP8GemmBlockFunction(torch.autograd.Function):
+    """BLOCKWISE (128): activations and gradients in 1 x 128 blocks along the reduction of each
+    product, the weight in 128 x 128 tiles that serve forward and backward. When a gradient is
+    wanted the quantizers also emit, from the same read, the operands of the backward products with
+    their reduction axis contiguous (the transposed 128 x 1 column codes of ``a`` and ``grad_out``,
+    the transposed weight codes), so that every product is an NT product read in place."""
+
     @staticmethod
     def forward(ctx, a, b, a_t, b_t, trans_a, trans_b, out_dtype, config):
         assert trans_a == False, "trans_a has to be False"  # noqa: E712
         fdt = _get_fp8_dtype(config.format, True)
         gran, bs = config.granularity, config.block_size
+        need_bwd = any(ctx.needs_input_grad[:2])
+        a_col = a_col_s = None
+        a_kmajor = False
         if isinstance(a, QuantizedTensor):
             check_quantized_tensor(a, config, axis=-1)
             a_row, a_row_s = a.qdata, a.scale_inv
-            if a_t is None:
-                a_t = QuantizedTensor.quantize(a.dequantize(), fdt, gran, axis=-2, block_size=bs)
-            a_col, a_col_s = a_t.qdata, a_t.scale_inv
-        elif any(ctx.needs_input_grad[:2]):
-            a_row, a_row_s, a_col, a_col_s = quantize_fp8_with_trans(a, fdt, gran, block_size=bs)
+            if need_bwd:
+                if a_t is None:
+                    a_t = QuantizedTensor.quantize(a.dequantize(), fdt, gran, axis=-2, block_size=bs)
+                a_col, a_col_s = a_t.qdata, a_t.scale_inv
+        elif need_bwd:
+            a_row, a_row_s, a_col, a_col_s = quant_fp8_blockwise_dual_t_impl(a.contiguous(), fdt, bs)
+            a_kmajor = True
         else:
             # the column-direction copy of `a` only feeds wgrad: skip it when nothing asks for a gradient
             a_row, a_row_s = quantize_fp8(a, fdt, gran, axis=-1, block_size=bs)
-            a_col, a_col_s = a_row, a_row_s
         w_recipe = ScalingRecipe(use_2d_block=True)  # weight tiles serve forward and backward unchanged
+        b_q_t = None
         if isinstance(b, QuantizedTensor):
             check_quantized_tensor(b, config, scaling_recipe=w_recipe)
             b_q, b_s = b.qdata, b.scale_inv
+        elif (need_bwd or not trans_b) and b.dim() == 2 and b.size(0) % 16 == 0:
+            b_q, b_q_t, b_s = quant_fp8_blockwise_for_weight_dual_impl(b, fdt, bs)
         else:
             b_q, b_s = quantize_fp8(b, fdt, gran, block_size=bs, scaling_recipe=w_recipe)
-        out = _gemm(a_row, a_row_s, trans_a, b_q, b_s, trans_b, out_dtype, False, gran)
-        ctx.save_for_backward(a_col, a_col_s, b_q, b_s)
-        ctx.meta = (trans_a, trans_b, out_dtype, config)
+        b_s_t = b_s.t().contiguous() if b_q_t is not None else None
+        # forward reduces over b's last axis when trans_b, dgrad over the other one
+        fwd_b, fwd_s, dgrad_b, dgrad_s = (b_q, b_s, b_q_t, b_s_t) if trans_b else (b_q_t, b_s_t, b_q, b_s)
+        if fwd_b is not None:
+            out = _gemm(a_row, a_row_s, False, fwd_b, fwd_s, True, out_dtype, False, gran)
+        else:
+            out = _gemm(a_row, a_row_s, False, b_q, b_s, trans_b, out_dtype, False, gran)
+        if need_bwd:
+            b_ready = dgrad_b is not None
+            ctx.save_for_backward(a_col, a_col_s, dgrad_b if b_ready else b_q, dgrad_s if b_ready else b_s)
+            ctx.meta = (trans_a, trans_b, out_dtype, config, a_kmajor, b_ready)
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
-        trans_a, trans_b, out_dtype, config = ctx.meta
+        trans_a, trans_b, out_dtype, config, a_kmajor, b_ready = ctx.meta
         a_col, a_col_s, b_q, b_s = ctx.saved_tensors
         gran = config.granularity
-        g_row, g_row_s, g_col, g_col_s = quantize_fp8_with_trans(
-            grad_out.contiguous(), _get_fp8_dtype(config.format, False), gran, block_size=config.block_size
-        )
-        grad_a = _gemm(g_row, g_row_s, False, b_q, b_s, not trans_b, out_dtype, False, gran)
-        grad_b = _gemm(a_col, a_col_s, not trans_a, g_col, g_col_s, False, out_dtype, trans_b, gran)
+        gdt = _get_fp8_dtype(config.format, False)
+        g = grad_out.contiguous()
+        if a_kmajor:
+            g_row, g_row_s, g_col_t, g_col_s = quant_fp8_blockwise_dual_t_impl(g, gdt, config.block_size)
+        else:
+            g_row, g_row_s, g_col, g_col_s = quantize_fp8_with_trans(g, gdt, gran, block_size=config.block_size)
+        grad_a = _gemm(g_row, g_row_s, False, b_q, b_s, True if b_ready else not trans_b, out_dtype, False, gran)
+        if a_kmajor:
+            # [K, M_pad] x [N, M_pad]^T: both read in place; trans_c gives the [N, K] weight layout
+            grad_b = _gemm(a_col, a_col_s, False, g_col_t, g_col_s, True, out_dtype, trans_b, gran)
+        else:
+            grad_b = _gemm(a_col, a_col_s, not trans_a, g_col, g_col_s, False, out_dtype, trans_b, gran)
         return grad_a, grad_b, None, None, None, None, None, None
 
 

@@ -169,3 +169,22 @@ def test_grouped_segment_row_col_transposed(kind, G_, M, N, dtype):
     assert torch.equal(sc2[: w // 128], sc[: w // 128])
     assert qct.shape == (N, -(-(M + 128 * G_) // 128) * 128)
     assert torch.equal(qct.view(torch.uint8)[:, :w], qc.view(torch.uint8)[:w].t().contiguous())
+
+
+@pytest.mark.parametrize("shape", [(256, 384), (130, 257), (1000, 512), (16384, 2048), (77, 96)])
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+def test_blockwise_dual_transposed_column_output(shape, dtype):
+    """Dual quantizer with the column codes emitted transposed: rows / scales identical to the plain
+    dual quantizer, transposed codes = its column codes transposed, zero beyond M."""
+    from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+    M, N = shape
+    x = bf16_randn(shape, seed=29, outlier_frac=0.001).cuda()
+    qr, sr, qc, sc = qi.quant_fp8_blockwise_dual_impl(x, dtype, 128)
+    qr2, sr2, qct, sc2 = qi.quant_fp8_blockwise_dual_t_impl(x, dtype, 128)
+    torch.cuda.synchronize()
+    Mp = -(-M // 128) * 128
+    assert torch.equal(qr2.view(torch.uint8), qr.view(torch.uint8)) and torch.equal(sr2, sr) and torch.equal(sc2, sc)
+    assert qct.shape == (N, Mp)
+    assert torch.equal(qct.view(torch.uint8)[:, :M], qc.view(torch.uint8).t().contiguous())
+    assert not bool(qct.view(torch.uint8)[:, M:].any())
