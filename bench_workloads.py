@@ -22,14 +22,19 @@ FP4_PEAK_TFLOPS = 10100.0
 # 256 MiB launched in the same run (`bench.py --calib-copy`; factors 2.000 and 1.000); the runs are
 # summarised under profiles/. (fetched, written) in MiB.
 TRAFFIC_MIB = {
-    "gemm_fp8_rowwise": (779.1, 151.6),
-    "gemm_fp8_blockwise": (567.5, 224.0),
-    "gemm_fp8_blockwise_k7168": (1155.2, 128.0),
-    "gemm_fp8_blockwise_8192": (1326.5, 128.0),
-    "gemm_mxfp4": (3332.6, 754.7),
-    "gemm_mxfp8": (6488.6, 700.2),
-    "grouped_gemm_fp8": (5372.6, 256.1),  # forward launches only
-    "grouped_gemm_fp8_down": (2439.0, 448.2),
+    "gemm_fp8_rowwise": (779.3, 151.9),
+    "gemm_fp8_blockwise": (568.7, 224.0),
+    "gemm_fp8_blockwise_k7168": (1159.9, 128.1),
+    "gemm_fp8_blockwise_8192": (1327.5, 129.1),
+    "gemm_mxfp4": (3341.2, 761.7),
+    "gemm_mxfp8": (6414.0, 682.4),
+    # grouped workloads: forward launches only (the same kernel symbol also runs dgrad)
+    "grouped_gemm_fp8": (5333.5, 256.1),
+    "grouped_gemm_fp8_down": (2424.1, 448.2),
+    "grouped_gemm_mxfp8": (5495.4, 256.1),
+    "grouped_gemm_mxfp8_down": (2601.7, 448.2),
+    "grouped_gemm_mxfp4": (2767.3, 256.1),
+    "grouped_gemm_mxfp4_down": (1279.2, 448.2),
 }
 
 
