@@ -1,0 +1,92 @@
+"""The hot path under HIP graph capture (``torch.cuda.graph``): quantize -> GEMM steps, grouped
+forward + backward, are captured once and replayed with new contents in the static input buffers;
+every replay must equal the eager result bit for bit, with eager work and synchronizations between
+the replays (the reference captures its grouped MXFP4 GEMM the same way,
+tests/pytorch/ops/test_grouped_gemm_fp4.py:409-470). One eager call before the capture does the
+one-time set-up (kernel attributes, lazy library loading) outside the graph."""
+
+import pytest
+import torch
+
+from helpers import bf16_randn, group_lens
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _turbo(native_lib):
+    global turbo, G, F8, F4, Format, ScaleDtype
+    import primus_turbo.pytorch as turbo
+    from primus_turbo.pytorch.core.low_precision import Float4QuantConfig as F4
+    from primus_turbo.pytorch.core.low_precision import Float8QuantConfig as F8
+    from primus_turbo.pytorch.core.low_precision import Format, ScaleDtype
+    from primus_turbo.pytorch.core.low_precision import ScalingGranularity as G
+
+
+def _replay_check(fn, make_inputs, n_static, replays=3):
+    """``fn(*static) -> tuple of tensors``; ``make_inputs(seed) -> tuple`` of fresh CPU-made inputs."""
+    static = [t.cuda() for t in make_inputs(0)]
+    assert len(static) == n_static
+    fn(*static)  # one-time set-up outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn(*static)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = fn(*static)
+    for seed in range(1, replays + 1):
+        fresh = [t.cuda() for t in make_inputs(seed)]
+        for s, f in zip(static, fresh):
+            s.copy_(f)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        want = fn(*fresh)  # eager work between the replays
+        torch.cuda.synchronize()
+        for g, w in zip(got, want):
+            assert torch.equal(g.view(torch.uint8) if g.element_size() == 1 else g,
+                               w.view(torch.uint8) if w.element_size() == 1 else w), f"replay {seed} differs from eager"
+
+
+def test_graph_tensorwise_quantize_dequantize():
+    def fn(x):
+        q, s = turbo.ops.quantize_fp8(x, turbo.float8_e4m3, G.TENSORWISE)
+        return q, s, turbo.ops.dequantize_fp8(q, torch.bfloat16, G.TENSORWISE, scale_inv=s)
+
+    _replay_check(fn, lambda seed: (bf16_randn((1024, 1024), seed=100 + seed, outlier_frac=0.001) * (1 + seed),), 1)
+
+
+@pytest.mark.parametrize("gran", ["ROWWISE", "BLOCKWISE", "MX_BLOCKWISE"])
+def test_graph_gemm_fp8_forward(gran):
+    kw = {"BLOCKWISE": dict(block_size=128), "MX_BLOCKWISE": dict(block_size=32, scale_dtype=ScaleDtype.E8M0)}.get(gran, {})
+    cfg = F8(format=Format.E4M3, granularity=getattr(G, gran), **kw)
+
+    def fn(a, b):
+        return (turbo.ops.gemm_fp8(a, b, trans_b=True, config=cfg),)
+
+    _replay_check(fn, lambda seed: (bf16_randn((512, 1024), seed=110 + seed), bf16_randn((768, 1024), seed=120 + seed)), 2)
+
+
+@pytest.mark.parametrize("kind", ["blockwise", "mxfp8", "mxfp4"])
+def test_graph_grouped_gemm_forward_backward(kind):
+    lens = group_lens("ragged", 4, 1024, 130)
+    gl = torch.from_numpy(lens).cuda()
+    if kind == "mxfp4":
+        cfg, op = F4(), turbo.ops.grouped_gemm_fp4
+    else:
+        kw = dict(block_size=128) if kind == "blockwise" else dict(block_size=32, scale_dtype=ScaleDtype.E8M0)
+        cfg = F8(format=Format.E4M3, granularity=G.BLOCKWISE if kind == "blockwise" else G.MX_BLOCKWISE, **kw)
+        op = turbo.ops.grouped_gemm_fp8
+
+    def fn(a, b, dy):
+        a = a.detach().requires_grad_(True)
+        b = b.detach().requires_grad_(True)
+        y = op(a, b, gl, trans_b=True, config=cfg)
+        da, db = torch.autograd.grad(y, (a, b), dy)
+        return y, da, db
+
+    _replay_check(fn, lambda seed: (bf16_randn((1024, 1024), seed=140 + seed), bf16_randn((4, 512, 1024), seed=150 + seed),
+                                    bf16_randn((1024, 512), seed=160 + seed)), 3)
