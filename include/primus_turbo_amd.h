@@ -213,8 +213,12 @@ PT_API int pt_dequantize_fp8_block(const void *q, int q_dtype, int64_t B, int64_
  * Row direction (blocks of 32 along N): row_q [B, M, Npad] codes (FP4: Npad / 2 bytes per
  * row), row_scale [B, M, Npad / 32]; Npad = N rounded up to 128, the padding is zero data
  * with scale byte 0. Column direction (blocks of 32 along M), emitted transposed:
- * col_q [B, N, Mpad], col_scale [B, N, Mpad / 32]. Either pair may be NULL. row_2d / col_2d
- * != 0 share one exponent per 32 x 32 tile (weights).
+ * col_q [B, N, Mpad], col_scale [B, N, Mpad / 32]. Either pair may be NULL. row_flags /
+ * col_flags: bit 0 shares one exponent per 32 x 32 tile (weights); bit 1 (MXFP4 only, not with
+ * bit 0) quantizes the Hadamard-transformed values: every 16 consecutive elements along the
+ * direction (of the zero-padded tensor) are replaced by (H4 (x) H4) / 4 times themselves, in fp32
+ * with the operation order of flydsl/quantization/mxfp4_quant_kernel.py:92-118 -- the recipe's
+ * "RHT" of the two wgrad operands, which cancels in their product.
  *
  * pt_dequantize_mx replaces dequantize_mxfp8 / dequantize_mxfp4 (quantization.cpp:285-359,
  * 436-508; kernels dequantization_mxfp8.cu:29-113, dequantization_mxfp4.cu:28-160):
@@ -222,8 +226,8 @@ PT_API int pt_dequantize_fp8_block(const void *q, int q_dtype, int64_t B, int64_
  * over q [rows, cols] (cols % 32 == 0; FP4 packed), written as y [rows, cols] or, for
  * column-direction data, transposed back as y [cols, rows]. */
 PT_API int pt_quantize_mx(const void *x, int x_dtype, int64_t B, int64_t M, int64_t N, int q_dtype,
-                          void *row_q, void *row_scale, int row_2d, void *col_q, void *col_scale,
-                          int col_2d, void *stream);
+                          void *row_q, void *row_scale, int row_flags, void *col_q, void *col_scale,
+                          int col_flags, void *stream);
 PT_API int pt_dequantize_mx(const void *q, int q_dtype, const void *scale, int64_t rows,
                             int64_t cols, void *y, int y_dtype, int transpose, void *stream);
 
@@ -389,7 +393,8 @@ PT_API int pt_grouped_gemm_fp8_vec_variable_k(const void *lhs, int lhs_dtype, co
  * Either pair may be NULL. The padded offsets come from pt_compute_group_offs (align 32 / 128).
  * With q_dtype e2m1x2 it is the grouped MXFP4 quantizer (grouped_quantize_mxfp4[_dual],
  * quantization.cpp:1209-1378; default dispatch flydsl/quantization/mxfp4_grouped_quant.py:320-349):
- * two codes per byte, rows kept tight (row_offs_padded NULL) and column groups padded to 256.
+ * two codes per byte, rows kept tight (row_offs_padded NULL) and column groups padded to 256;
+ * row_flags / col_flags as for pt_quantize_mx (bit 1 only: grouped data have no 2-D blocks).
  *
  * pt_grouped_gemm_mx replaces primus_turbo::grouped_gemm_fp8_impl for MX_BLOCKWISE
  * (kernels/grouped_gemm/grouped_gemm_fp8_impl.py:888-930 with group_offs_out; caller
@@ -416,8 +421,8 @@ PT_API int pt_grouped_gemm_fp8_vec_variable_k(const void *lhs, int lhs_dtype, co
 PT_API int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype,
                                   const int64_t *group_offs, const int64_t *row_offs_padded,
                                   const int64_t *col_offs_padded, int64_t G, void *row_q,
-                                  void *row_scale, void *col_q, void *col_scale, int64_t col_ld,
-                                  void *stream);
+                                  void *row_scale, int row_flags, void *col_q, void *col_scale,
+                                  int col_flags, int64_t col_ld, void *stream);
 PT_API int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, int64_t lda,
                               int64_t sa_ld, const void *b, int b_dtype, const void *b_scale,
                               int64_t ldb, int64_t sb_ld, void *c, int c_dtype,

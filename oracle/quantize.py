@@ -31,8 +31,10 @@ What each function follows, and what pins it (tests/test_oracle_*.py):
   The HIP sources of the reference MX quantizers are absent from the snapshot, so
   bit-identity with them is PARITY UNPINNED; what is pinned is the published rule:
   brute force over every bf16 amax, the saturation invariant, 2-D blocks constant
-  over 32x32 tiles, round trips through the de-quantizer. Random Hadamard transform
-  and stochastic rounding recipes are not restated (unpinned, not implemented).
+  over 32x32 tiles, round trips through the de-quantizer. ``hadamard16`` restates the
+  recipe's fixed 16-point Hadamard transform (``use_rht``; pinned against scipy's
+  Sylvester matrix and by its involution, rounding order PARITY UNPINNED as above).
+  Stochastic rounding is not restated (random by design, not implemented).
 * ``mx_grouped_quant`` — per-group composition of the two above in the padded layouts of
   /root/reference/csrc/pytorch/quantization/quantization.cpp:971-1100 (rows of a group padded
   to 32 / 128 with zero data); pinned by the group-by-group round trip against the dense
@@ -300,14 +302,40 @@ def unpack_fp4(packed: np.ndarray) -> np.ndarray:
     return out
 
 
-def mx_quant_rowwise(x: np.ndarray, fmt, use_2d_block: bool = False, pad: int = 128):
+def hadamard16(v: np.ndarray) -> np.ndarray:
+    """The fixed 16-point Hadamard transform of the MXFP4 recipe along the last axis (length a
+    multiple of 16, transformed in groups of 16), in fp32 with the operation order of
+    /root/reference/primus_turbo/flydsl/quantization/mxfp4_quant_kernel.py:92-118: an H4 butterfly
+    inside each run of four elements, an H4 butterfly across the four runs, times 0.25 -- i.e.
+    (H4 (x) H4) / 4, the orthonormal Sylvester matrix of order 16. There are no random signs:
+    the transform is its own inverse and cancels between two operands that both carry it.
+    Pinned against scipy's Sylvester matrix on inputs where fp32 is exact, and by the involution.
+    Bit-identity of the rounding order with the reference's HIP kernel is PARITY UNPINNED (its
+    source is absent); the FlyDSL text states that the two agree."""
+    v = np.asarray(v, dtype=F32)
+    g = v.reshape(v.shape[:-1] + (v.shape[-1] // 16, 4, 4))  # [.., group, block, local]
+
+    def h4(v0, v1, v2, v3):
+        a0, a1, a2, a3 = (v0 + v1).astype(F32), (v0 - v1).astype(F32), (v2 + v3).astype(F32), (v2 - v3).astype(F32)
+        return (a0 + a2).astype(F32), (a1 + a3).astype(F32), (a0 - a2).astype(F32), (a1 - a3).astype(F32)
+
+    with np.errstate(over="ignore", invalid="ignore"):
+        o = np.stack(h4(g[..., 0], g[..., 1], g[..., 2], g[..., 3]), axis=-1)       # within each block
+        r = np.stack(h4(o[..., 0, :], o[..., 1, :], o[..., 2, :], o[..., 3, :]), axis=-2)  # across the blocks
+        r = (r * F32(0.25)).astype(F32)
+    return r.reshape(v.shape)
+
+
+def mx_quant_rowwise(x: np.ndarray, fmt, use_2d_block: bool = False, pad: int = 128, use_rht: bool = False):
     """MX quantization along the last axis of a 2-D ``x [M, K]``.
 
     -> (codes [M, K_pad] (FP4: packed [M, K_pad/2]), e8m0 bytes [M, K_pad/32]) with
     K_pad = K rounded up to ``pad``; the K padding is zero data (scale byte 0 for a
     fully padded block). With ``use_2d_block`` one exponent is shared by each 32x32
     tile (rows beyond M count as zeros) and replicated into the scale slot of each of
-    its rows.
+    its rows. ``use_rht`` (MXFP4 recipe): every 16 consecutive elements (of the zero-padded
+    row) go through ``hadamard16`` first; abs-max, scale and codes are those of the
+    transformed values (mxfp4_quant_kernel.py:176-199).
     """
     fmt = _fmt(fmt)
     x = np.asarray(x, dtype=F32)
@@ -315,6 +343,9 @@ def mx_quant_rowwise(x: np.ndarray, fmt, use_2d_block: bool = False, pad: int = 
     Kp = _cdiv(K, pad) * pad
     xp = np.zeros((M, Kp), dtype=F32)
     xp[:, :K] = x
+    if use_rht:
+        assert not use_2d_block, "the recipe never combines 2-D blocks with the Hadamard transform"
+        xp = hadamard16(xp)
     blk = xp.reshape(M, Kp // 32, 32)
     if use_2d_block:
         Mp = _cdiv(M, 32) * 32
@@ -331,14 +362,15 @@ def mx_quant_rowwise(x: np.ndarray, fmt, use_2d_block: bool = False, pad: int = 
     return codes, byte.reshape(M, Kp // 32)
 
 
-def mx_quant_colwise(x: np.ndarray, fmt, use_2d_block: bool = False, pad: int = 128):
+def mx_quant_colwise(x: np.ndarray, fmt, use_2d_block: bool = False, pad: int = 128, use_rht: bool = False):
     """MX quantization along axis 0 of ``x [M, K]``, emitted transposed:
     codes [K, M_pad] (FP4 packed [K, M_pad/2]) and bytes [K, M_pad/32]."""
     x = np.asarray(x, dtype=F32)
-    return mx_quant_rowwise(np.ascontiguousarray(x.T), fmt, use_2d_block, pad)
+    return mx_quant_rowwise(np.ascontiguousarray(x.T), fmt, use_2d_block, pad, use_rht)
 
 
-def mx_grouped_quant(x: np.ndarray, group_lens: np.ndarray, fmt, row_align: int = 32, col_align: int = 128):
+def mx_grouped_quant(x: np.ndarray, group_lens: np.ndarray, fmt, row_align: int = 32, col_align: int = 128,
+                     row_rht: bool = False, col_rht: bool = False):
     """Grouped MX quantizer of a packed-M activation ``x [M, N]`` (layout rules of
     /root/reference/csrc/pytorch/quantization/quantization.cpp:971-1100 and
     /root/reference/primus_turbo/pytorch/kernels/quantization/quantization_impl.py:572-700:
@@ -375,10 +407,10 @@ def mx_grouped_quant(x: np.ndarray, group_lens: np.ndarray, fmt, row_align: int 
         if n == 0:
             continue
         seg = x[offs[g] : offs[g] + n]
-        q, sc = mx_quant_rowwise(seg, fmt)
+        q, sc = mx_quant_rowwise(seg, fmt, use_rht=row_rht)
         row[ro[g] : ro[g] + n] = q
         row_scale[ro[g] : ro[g] + n] = sc
-        q, sc = mx_quant_colwise(seg, fmt, pad=col_align)
+        q, sc = mx_quant_colwise(seg, fmt, pad=col_align, use_rht=col_rht)
         col[:, co[g] // cpb : co[g + 1] // cpb] = q
         col_scale[:, co[g] // 32 : co[g + 1] // 32] = sc
     return dict(row=row, row_scale=row_scale, col=col, col_scale=col_scale, row_lens=rl, row_offs=ro, col_lens=cl,

@@ -94,15 +94,43 @@ struct MxArgs {
     int            G;
 };
 
+// The MXFP4 recipe's fixed 16-point Hadamard transform of v[base .. base + 16), in place:
+// (H4 (x) H4) / 4 with the operation order of Primus-Turbo's
+// primus_turbo/flydsl/quantization/mxfp4_quant_kernel.py:92-118 (an H4 butterfly inside each run
+// of four, one across the four runs, then * 0.25). Additions only and one exact scaling: there is
+// nothing here for the compiler to contract.
+__device__ __forceinline__ void h4(float &v0, float &v1, float &v2, float &v3) {
+    const float a0 = v0 + v1, a1 = v0 - v1, a2 = v2 + v3, a3 = v2 - v3;
+    v0 = a0 + a2;
+    v1 = a1 + a3;
+    v2 = a0 - a2;
+    v3 = a1 - a3;
+}
+__device__ __forceinline__ void hadamard16(float (&v)[32], int base) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+        h4(v[base + 4 * b], v[base + 4 * b + 1], v[base + 4 * b + 2], v[base + 4 * b + 3]);
+#pragma unroll
+    for (int l = 0; l < 4; ++l) {
+        h4(v[base + l], v[base + 4 + l], v[base + 8 + l], v[base + 12 + l]);
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+            v[base + 4 * b + l] *= 0.25f;
+    }
+}
+
 // fabsf(x) with NaN mapped to 0 (fmaxf-style abs-max ignores NaN)
 __device__ __forceinline__ float abs_or_zero(float x) {
     const float a = fabsf(x);
     return a == a ? a : 0.f;
 }
 
-template <typename T, int FMT, bool ROW, bool COL, bool ROW2D, bool COL2D>
+// RHT: bit 0 / bit 1 = the row / column direction quantizes the Hadamard-transformed values
+// (16 consecutive elements along the direction; never together with 2-D blocks).
+template <typename T, int FMT, bool ROW, bool COL, bool ROW2D, bool COL2D, int RHT = 0>
 __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
     constexpr bool ANY2D = (ROW && ROW2D) || (COL && COL2D);
+    static_assert(RHT == 0 || !ANY2D, "the Hadamard transform is not combined with 2-D blocks");
     __shared__ __attribute__((aligned(16))) uint16_t tile[MX_TILE * MX_PITCH];
     __shared__ float                                 amax_rc[ANY2D ? MX_TILE * 4 : 1]; // [row][32-col block]
     __shared__ __attribute__((aligned(4))) uint8_t   sbytes[MX_TILE * 4]; // E8M0 bytes of the tile, [row or column][block]
@@ -177,6 +205,14 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
                     am = fmaxf(am, fmaxf(abs_or_zero(lo), abs_or_zero(hi)));
                 }
             }
+            if constexpr ((RHT & 1) != 0) {
+                hadamard16(rv[p], 0);
+                hadamard16(rv[p], 16);
+                am = 0.f;
+#pragma unroll
+                for (int k = 0; k < 32; ++k)
+                    am = fmaxf(am, abs_or_zero(rv[p][k]));
+            }
             ram[p] = am;
             if constexpr (ANY2D)
                 amax_rc[r * 4 + c] = am;
@@ -240,6 +276,14 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
                 v[i] = elem(tile[(rb * 32 + i) * MX_PITCH + c]);
                 am   = fmaxf(am, abs_or_zero(v[i]));
             }
+            if constexpr ((RHT & 2) != 0) {
+                hadamard16(v, 0);
+                hadamard16(v, 16);
+                am = 0.f;
+#pragma unroll
+                for (int i = 0; i < 32; ++i)
+                    am = fmaxf(am, abs_or_zero(v[i]));
+            }
             if constexpr (COL2D) {
                 am = 0.f;
 #pragma unroll 8
@@ -299,6 +343,23 @@ static void launch_mx_dir(const MxArgs &a, bool row2d, bool col2d, dim3 grid, hi
         launch_mx_2d<T, FMT, true, false>(a, row2d, false, grid, st);
     else
         launch_mx_2d<T, FMT, false, true>(a, false, col2d, grid, st);
+}
+
+// MXFP4 with the Hadamard transform in one or both directions (1-D blocks only)
+template <typename T> static void launch_mx_rht(const MxArgs &a, bool row_rht, bool col_rht, dim3 grid, hipStream_t st) {
+    const bool row = a.row_q != nullptr, col = a.col_q != nullptr;
+    if (row && col) {
+        if (row_rht && col_rht)
+            mx_quant_kernel<T, MX_E2M1, true, true, false, false, 3><<<grid, 256, 0, st>>>(a);
+        else if (col_rht)
+            mx_quant_kernel<T, MX_E2M1, true, true, false, false, 2><<<grid, 256, 0, st>>>(a);
+        else
+            mx_quant_kernel<T, MX_E2M1, true, true, false, false, 1><<<grid, 256, 0, st>>>(a);
+    } else if (row) {
+        mx_quant_kernel<T, MX_E2M1, true, false, false, false, 1><<<grid, 256, 0, st>>>(a);
+    } else {
+        mx_quant_kernel<T, MX_E2M1, false, true, false, false, 2><<<grid, 256, 0, st>>>(a);
+    }
 }
 
 template <typename T> static void launch_mx_fmt(const MxArgs &a, int fmt, bool row2d, bool col2d, dim3 grid, hipStream_t st) {
@@ -452,8 +513,17 @@ using namespace pt;
 
 extern "C" {
 
+// direction flags: bit 0 = 2-D (32 x 32) blocks, bit 1 = Hadamard transform (MXFP4, 1-D blocks)
+static int check_mx_flags(int fmt, int row_flags, int col_flags) {
+    PT_REQUIRE((row_flags & ~3) == 0 && (col_flags & ~3) == 0, "unknown direction flags");
+    const bool rht = ((row_flags | col_flags) & 2) != 0;
+    PT_REQUIRE(!rht || fmt == MX_E2M1, "the Hadamard transform belongs to the MXFP4 recipe");
+    PT_REQUIRE(!rht || ((row_flags | col_flags) & 1) == 0, "the Hadamard transform is not combined with 2-D blocks");
+    return PT_OK;
+}
+
 int pt_quantize_mx(const void *x, int x_dtype, int64_t B, int64_t M, int64_t N, int q_dtype, void *row_q,
-                   void *row_scale, int row_2d, void *col_q, void *col_scale, int col_2d, void *stream) {
+                   void *row_scale, int row_flags, void *col_q, void *col_scale, int col_flags, void *stream) {
     PT_REQUIRE(x_dtype == PT_DTYPE_BF16 || x_dtype == PT_DTYPE_F16, "input must be bf16 or fp16");
     const int fmt = mx_fmt_of(q_dtype);
     PT_REQUIRE(fmt >= 0, "q_dtype must be e4m3, e5m2 or e2m1x2");
@@ -461,6 +531,9 @@ int pt_quantize_mx(const void *x, int x_dtype, int64_t B, int64_t M, int64_t N, 
     PT_REQUIRE((row_q != nullptr) == (row_scale != nullptr) && (col_q != nullptr) == (col_scale != nullptr),
                "codes and scales come in pairs");
     PT_REQUIRE(row_q || col_q, "nothing to produce");
+    if (const int rc = check_mx_flags(fmt, row_q ? row_flags : 0, col_q ? col_flags : 0))
+        return rc;
+    const bool rht = (((row_q ? row_flags : 0) | (col_q ? col_flags : 0)) & 2) != 0;
     if (B == 0 || M == 0 || N == 0)
         return PT_OK;
     PT_REQUIRE(x, "NULL input");
@@ -482,16 +555,23 @@ int pt_quantize_mx(const void *x, int x_dtype, int64_t B, int64_t M, int64_t N, 
     PT_REQUIRE(a.Mpad / 128 < 65536 && B < 65536, "grid dimension out of range");
     dim3 grid(static_cast<unsigned>(a.Npad / 128), static_cast<unsigned>(a.Mpad / 128), static_cast<unsigned>(B));
     auto st = static_cast<hipStream_t>(stream);
-    if (x_dtype == PT_DTYPE_BF16)
-        launch_mx_fmt<bf16_t>(a, fmt, row_2d != 0, col_2d != 0, grid, st);
-    else
-        launch_mx_fmt<f16_t>(a, fmt, row_2d != 0, col_2d != 0, grid, st);
+    if (rht) {
+        if (x_dtype == PT_DTYPE_BF16)
+            launch_mx_rht<bf16_t>(a, (row_flags & 2) != 0, (col_flags & 2) != 0, grid, st);
+        else
+            launch_mx_rht<f16_t>(a, (row_flags & 2) != 0, (col_flags & 2) != 0, grid, st);
+    } else if (x_dtype == PT_DTYPE_BF16) {
+        launch_mx_fmt<bf16_t>(a, fmt, (row_flags & 1) != 0, (col_flags & 1) != 0, grid, st);
+    } else {
+        launch_mx_fmt<f16_t>(a, fmt, (row_flags & 1) != 0, (col_flags & 1) != 0, grid, st);
+    }
     return check_launch("mx_quant_kernel");
 }
 
 int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype, const int64_t *group_offs,
                            const int64_t *row_offs_padded, const int64_t *col_offs_padded, int64_t G, void *row_q,
-                           void *row_scale, void *col_q, void *col_scale, int64_t col_ld, void *stream) {
+                           void *row_scale, int row_flags, void *col_q, void *col_scale, int col_flags, int64_t col_ld,
+                           void *stream) {
     PT_REQUIRE(x_dtype == PT_DTYPE_BF16 || x_dtype == PT_DTYPE_F16, "input must be bf16 or fp16");
     const int fmt = mx_fmt_of(q_dtype);
     PT_REQUIRE(fmt >= 0, "q_dtype must be e4m3, e5m2 or e2m1x2");
@@ -499,6 +579,10 @@ int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t N, int
     PT_REQUIRE((row_q != nullptr) == (row_scale != nullptr) && (col_q != nullptr) == (col_scale != nullptr),
                "codes and scales come in pairs");
     PT_REQUIRE(row_q || col_q, "nothing to produce");
+    if (const int rc = check_mx_flags(fmt, row_q ? row_flags : 0, col_q ? col_flags : 0))
+        return rc;
+    PT_REQUIRE(((row_flags | col_flags) & 1) == 0, "grouped MX quantization has no 2-D blocks");
+    const bool rht = (((row_q ? row_flags : 0) | (col_q ? col_flags : 0)) & 2) != 0;
     PT_REQUIRE(col_ld % 128 == 0 && col_ld >= M, "col_ld must be a multiple of 128 that holds every padded group");
     if (M == 0 || N == 0)
         return PT_OK;
@@ -523,10 +607,16 @@ int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t N, int
     PT_REQUIRE(col_ld / 128 < 65536, "grid dimension out of range");
     dim3 grid(static_cast<unsigned>(a.Npad / 128), static_cast<unsigned>(col_ld / 128), 1);
     auto st = static_cast<hipStream_t>(stream);
-    if (x_dtype == PT_DTYPE_BF16)
+    if (rht) {
+        if (x_dtype == PT_DTYPE_BF16)
+            launch_mx_rht<bf16_t>(a, (row_flags & 2) != 0, (col_flags & 2) != 0, grid, st);
+        else
+            launch_mx_rht<f16_t>(a, (row_flags & 2) != 0, (col_flags & 2) != 0, grid, st);
+    } else if (x_dtype == PT_DTYPE_BF16) {
         launch_mx_fmt<bf16_t>(a, fmt, false, false, grid, st);
-    else
+    } else {
         launch_mx_fmt<f16_t>(a, fmt, false, false, grid, st);
+    }
     return check_launch("mx_quant_kernel");
 }
 

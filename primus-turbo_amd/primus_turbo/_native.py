@@ -135,8 +135,8 @@ _SIGNATURES = {
     ),
     "pt_grouped_quantize_mx": (
         c_int,
-        [c_void_p, c_int, c_i64, c_i64, c_int, c_void_p, c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_void_p, c_void_p,
-         c_i64, c_void_p],
+        [c_void_p, c_int, c_i64, c_i64, c_int, c_void_p, c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_int, c_void_p,
+         c_void_p, c_int, c_i64, c_void_p],
     ),
     "pt_grouped_gemm_mx": (
         c_int,

@@ -92,7 +92,7 @@ class ScalingRecipe(NamedTuple):
 
     use_2d_block  one scale per square tile (128x128 FP8 blockwise, 32x32 MX) instead of 1-D blocks
     use_sr        stochastic rounding (MXFP4 only)
-    use_rht       random Hadamard transform before quantization (MXFP4 only)
+    use_rht       the recipe's fixed 16-point Hadamard transform before quantization (MXFP4 only)
     shuffle_scale / shuffle_out  pre-shuffled memory layouts (MXFP4 only)
     """
 

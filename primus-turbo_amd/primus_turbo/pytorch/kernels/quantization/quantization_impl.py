@@ -706,12 +706,21 @@ def _mx_recipes(with_trans, scaling_recipe, scaling_recipe_for_trans, what):
     r = ScalingRecipe() if scaling_recipe is None else scaling_recipe
     rt = (ScalingRecipe() if scaling_recipe_for_trans is None else scaling_recipe_for_trans) if with_trans else r
     for rec in (r, rt):
-        if rec.use_sr or rec.use_rht or rec.shuffle_scale or rec.shuffle_out:
+        if rec.use_sr or rec.shuffle_scale or rec.shuffle_out:
             raise NotImplementedError(
-                f"{what}: stochastic rounding, RHT and shuffled layouts are not implemented "
+                f"{what}: stochastic rounding and shuffled layouts are not implemented "
                 "(round-to-nearest-even, plain layouts are)"
             )
+        if rec.use_rht and what != "MXFP4":
+            raise NotImplementedError(f"{what}: the Hadamard transform belongs to the MXFP4 recipe")
+        if rec.use_rht and rec.use_2d_block:
+            raise NotImplementedError(f"{what}: the Hadamard transform is not combined with 2-D blocks")
     return r, rt
+
+
+def _mx_flags(recipe) -> int:
+    """Direction flags of the native quantizer: bit 0 = 2-D blocks, bit 1 = Hadamard transform."""
+    return (1 if recipe.use_2d_block else 0) | (2 if recipe.use_rht else 0)
 
 
 def _mx_check_axis(x, axis, with_trans):
@@ -727,8 +736,9 @@ def _mx_check_axis(x, axis, with_trans):
         assert x.ndim in (2, 3), f"The input tensor must be 2D or 3D but got {x.ndim}D."
 
 
-def _mx_quantize(x: torch.Tensor, out_dtype: torch.dtype, want_row: bool, want_col: bool, row_2d: bool, col_2d: bool):
-    """-> (row_q, row_scale, col_q, col_scale); the pair of an unwanted direction is None."""
+def _mx_quantize(x: torch.Tensor, out_dtype: torch.dtype, want_row: bool, want_col: bool, row_flags: int, col_flags: int):
+    """-> (row_q, row_scale, col_q, col_scale); the pair of an unwanted direction is None.
+    ``row_flags`` / ``col_flags``: see ``_mx_flags``."""
     N.require_cuda(x)
     if x.dtype not in (torch.bfloat16, torch.float16):
         raise RuntimeError("Input must be BFloat16 or Half")
@@ -756,7 +766,7 @@ def _mx_quantize(x: torch.Tensor, out_dtype: torch.dtype, want_row: bool, want_c
     N.check(
         N.lib().pt_quantize_mx(
             N.ptr(x), N.dtype_code(x.dtype), B, M, Nn, N.dtype_code(out_dtype),
-            N.ptr(row_q), N.ptr(row_s), int(row_2d), N.ptr(col_q), N.ptr(col_s), int(col_2d), N.stream_of(x),
+            N.ptr(row_q), N.ptr(row_s), int(row_flags), N.ptr(col_q), N.ptr(col_s), int(col_flags), N.stream_of(x),
         )
     )
     view = lambda t, dt: None if t is None else t.view(dt)  # noqa: E731
@@ -768,9 +778,9 @@ def _quantize_mx_impl(x, out_dtype, axis, block_size, with_trans, scaling_recipe
     r, rt = _mx_recipes(with_trans, scaling_recipe, scaling_recipe_for_trans, what)
     _mx_check_axis(x, axis, with_trans)
     if with_trans:
-        return _mx_quantize(x, out_dtype, True, True, r.use_2d_block, rt.use_2d_block)
+        return _mx_quantize(x, out_dtype, True, True, _mx_flags(r), _mx_flags(rt))
     rowwise = axis == x.ndim - 1
-    rq, rs, cq, cs = _mx_quantize(x, out_dtype, rowwise, not rowwise, r.use_2d_block, r.use_2d_block)
+    rq, rs, cq, cs = _mx_quantize(x, out_dtype, rowwise, not rowwise, _mx_flags(r), _mx_flags(r))
     return (rq, rs) if rowwise else (cq, cs)
 
 
@@ -786,7 +796,8 @@ def quantize_mxfp8_impl(x, out_dtype, axis, block_size, with_trans=False, scalin
 def quantize_mxfp4_impl(x, out_dtype, axis, block_size, with_trans=False, scaling_recipe=None,
                         scaling_recipe_for_trans=None):
     """MXFP4 (E2M1, two codes per byte, even element in the low nibble); shapes as MXFP8 with
-    the code tensors half as wide."""
+    the code tensors half as wide. ``use_rht`` in a recipe quantizes the values after the recipe's
+    fixed 16-point Hadamard transform along that direction (1-D blocks only)."""
     assert x.is_contiguous(), "The x tensor must be contiguous."
     return _quantize_mx_impl(x, out_dtype, axis, block_size, with_trans, scaling_recipe, scaling_recipe_for_trans, "MXFP4")
 
@@ -844,7 +855,8 @@ MXFP8_K_DIM_PADDING_ALIGN_SIZE = 128
 MXFP4_GROUP_K_DIM_PADDING_ALIGN_SIZE = 256
 
 
-def _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, want_row: bool, want_col: bool):
+def _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, want_row: bool, want_col: bool, row_flags: int = 0,
+                         col_flags: int = 0):
     """MXFP8: rows of every group padded to 32, transposed columns to 128. MXFP4: rows stay
     where they are in ``x`` (their "padded" lens / offs are the originals), transposed columns
     padded to 256 per group."""
@@ -882,8 +894,8 @@ def _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, want_row: bool, w
     N.check(
         N.lib().pt_grouped_quantize_mx(
             N.ptr(x), N.dtype_code(x.dtype), M, Nn, N.dtype_code(out_dtype), N.ptr(group_offs),
-            None if fp4 else N.ptr(offs_row), N.ptr(offs_col), G, N.ptr(row_q), N.ptr(row_s), N.ptr(col_q), N.ptr(col_s),
-            m_pad_col, N.stream_of(x),
+            None if fp4 else N.ptr(offs_row), N.ptr(offs_col), G, N.ptr(row_q), N.ptr(row_s), int(row_flags), N.ptr(col_q),
+            N.ptr(col_s), int(col_flags), m_pad_col, N.stream_of(x),
         )
     )
     view = lambda t, dt: None if t is None else t.view(dt)  # noqa: E731
@@ -940,16 +952,21 @@ def grouped_quantize_mxfp4_impl(x, out_dtype, axis, block_size, group_lens, grou
     direction keeps the rows where they are (row i = input row i), the transposed column
     direction pads every group to a multiple of 256 rows of zero data; ``M_pad_col`` = ``total_M +
     256 G`` rounded up to 256. Otherwise ``(q, scale, lens_padded, offs_padded)`` of the direction
-    ``axis`` asks for (1 = rows, 0 = transposed columns). Round-to-nearest-even only: stochastic
-    rounding, the random Hadamard transform, 2-D blocks and shuffled layouts raise."""
+    ``axis`` asks for (1 = rows, 0 = transposed columns). ``use_rht`` in a recipe applies the fixed
+    16-point Hadamard transform along that direction (within each group's padded rows for the
+    column direction). Round-to-nearest-even only: stochastic rounding, 2-D blocks and shuffled
+    layouts raise."""
     assert block_size == 32, "The block size must be 32 for MXFP4 quantization"
     assert _FP4X2 is not None and out_dtype == _FP4X2, "The out_dtype must be float4_e2m1fn_x2 for MXFP4 quantization"
     for r in (scaling_recipe, scaling_recipe_for_trans):
-        if r is not None and (r.use_2d_block or r.use_sr or r.use_rht or r.shuffle_scale or r.shuffle_out):
+        if r is not None and (r.use_2d_block or r.use_sr or r.shuffle_scale or r.shuffle_out):
             raise NotImplementedError(
-                "grouped MXFP4 quantization: 2-D blocks, stochastic rounding, RHT and shuffled layouts are not implemented")
+                "grouped MXFP4 quantization: 2-D blocks, stochastic rounding and shuffled layouts are not implemented")
+    rf = 2 if (scaling_recipe is not None and scaling_recipe.use_rht) else 0
     if with_trans:
-        return _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, True, True)
+        cf = 2 if (scaling_recipe_for_trans is not None and scaling_recipe_for_trans.use_rht) else 0
+        return _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, True, True, rf, cf)
     assert axis in (0, 1), "The axis must be 0 (colwise) or 1 (rowwise) when with_trans is False."
-    rq, rs, cq, cs, lr, orow, lc, ocol = _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, axis == 1, axis == 0)
+    rq, rs, cq, cs, lr, orow, lc, ocol = _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, axis == 1, axis == 0,
+                                                              rf, rf)
     return (rq, rs, lr, orow) if axis == 1 else (cq, cs, lc, ocol)

@@ -3,9 +3,10 @@
 
 Forward, dgrad and wgrad are all NT products of MX-quantized operands: activations and
 gradients use 1 x 32 blocks, the weight 32 x 32 blocks; each tensor is quantized in both
-directions from one read. Differences from the reference's recipe, both of which only change
-how much quantization noise the backward products carry, not what they estimate: the random
-Hadamard transform on the wgrad operands and stochastic rounding of gradients are not
+directions from one read. As in the reference's recipe (its lines 108-160, 220-240) the two wgrad
+operands -- the column-direction quantizations of ``a`` and of ``grad_out`` -- carry the fixed
+16-point Hadamard transform along the token axis, which cancels in their product and spreads
+outliers over 16 values before they are quantized. Stochastic rounding of gradients is not
 implemented (``use_gradient_sr=True`` raises), and pre-shuffled layouts do not exist here
 (``use_preshuffle=True`` raises).
 """
@@ -68,22 +69,25 @@ class FP4GemmMXFunction(torch.autograd.Function):
 
         need_bwd = any(ctx.needs_input_grad[:2])
 
-        def both_ways(x, x_t, recipe):
+        def both_ways(x, x_t, recipe, recipe_t):
             if isinstance(x, QuantizedTensor):
                 check_quantized_tensor(x, config, scaling_recipe=recipe)
                 if x_t is None:
                     x_t = QuantizedTensor.quantize(x.dequantize(), x.real_dtype, gran, axis=-2, block_size=bs,
-                                                   scaling_recipe=recipe)
+                                                   scaling_recipe=recipe_t)
+                else:
+                    check_quantized_tensor(x_t, config, scaling_recipe=recipe_t)
                 return x.qdata, x.scale_inv, x_t.qdata, x_t.scale_inv
             if not need_bwd:
                 # the transposed copies only feed backward: skip them when nothing asks for a gradient
                 q, sc = quantize_mxfp4_impl(x, dt, x.dim() - 1, bs, scaling_recipe=recipe)
                 return q, sc, q, sc
             return quantize_fp4_with_trans(x, dt, gran, block_size=bs, scaling_recipe=recipe,
-                                           scaling_recipe_for_trans=recipe)
+                                           scaling_recipe_for_trans=recipe_t)
 
-        a_row, a_row_s, a_col, a_col_s = both_ways(a, a_t, ScalingRecipe())
-        b_row, b_row_s, b_col, b_col_s = both_ways(b, b_t, ScalingRecipe(use_2d_block=True))
+        w_recipe = ScalingRecipe(use_2d_block=True)
+        a_row, a_row_s, a_col, a_col_s = both_ways(a, a_t, ScalingRecipe(), ScalingRecipe(use_rht=True))
+        b_row, b_row_s, b_col, b_col_s = both_ways(b, b_t, w_recipe, w_recipe)
         out = gemm_fp4_impl(a_row, a_row_s, False, b_row, b_row_s, True, out_dtype, False, gran.value, _NATIVE)
         ctx.save_for_backward(a_col, a_col_s, b_col, b_col_s)
         ctx.meta = (out_dtype, config, fuse, main_grad)
@@ -98,7 +102,7 @@ class FP4GemmMXFunction(torch.autograd.Function):
         g = grad_out.reshape(grad_out.shape[0], -1).contiguous()
         g_row, g_row_s, g_col, g_col_s = quantize_fp4_with_trans(
             g, dt, gran, block_size=config.block_size, scaling_recipe=ScalingRecipe(),
-            scaling_recipe_for_trans=ScalingRecipe(),
+            scaling_recipe_for_trans=ScalingRecipe(use_rht=True),  # pairs with a_col in wgrad
         )
         # both directions are stored transposed, so dgrad and wgrad are NT products as well
         grad_a = gemm_fp4_impl(g_row, g_row_s, False, b_col, b_col_s, True, out_dtype, False, gran.value, _NATIVE)

@@ -7,9 +7,10 @@ autograd (reference: primus_turbo/pytorch/ops/grouped_gemm_fp4.py:101-400).
 
 Activations and gradients use 1 x 32 blocks and are quantized in both directions from one read
 (rows in place, transposed columns padded to 256 tokens per group); the weight uses 32 x 32
-blocks. As in ``gemm_fp4``, the recipe extras that only change how much quantization noise the
-backward products carry are not implemented: no random Hadamard transform on the wgrad operands,
-no stochastic rounding (``use_gradient_sr=True`` raises), no pre-shuffled layouts.
+blocks. As in the reference the two wgrad operands (the column-direction quantizations of ``a`` and
+``grad_out``) carry the recipe's fixed 16-point Hadamard transform along the token axis, which
+cancels in their product. Not implemented: stochastic rounding (``use_gradient_sr=True`` raises)
+and pre-shuffled layouts.
 """
 
 from __future__ import annotations
@@ -95,7 +96,7 @@ class FP4GroupedGemmMXFunc(torch.autograd.Function):
         need_bwd = any(ctx.needs_input_grad[:2])
         w_recipe = ScalingRecipe(use_2d_block=True)
 
-        a_recipe = ScalingRecipe()
+        a_recipe, a_t_recipe = ScalingRecipe(), ScalingRecipe(use_rht=True)
         if isinstance(a, QuantizedTensor):
             # a grouped (packed rows) quantization made by the caller
             check_quantized_tensor(a, config, axis=-1, scaling_recipe=a_recipe)
@@ -104,12 +105,14 @@ class FP4GroupedGemmMXFunc(torch.autograd.Function):
             if need_bwd:
                 if a_t is None:
                     a_t = QuantizedTensor.quantize(a.dequantize(), a.real_dtype, gran, axis=-2, block_size=bs,
-                                                   scaling_recipe=a_recipe, group_lens=group_lens)
+                                                   scaling_recipe=a_t_recipe, group_lens=group_lens)
                 assert isinstance(a_t, QuantizedTensor)
+                check_quantized_tensor(a_t, config, scaling_recipe=a_t_recipe)
                 a_col, a_col_s = a_t.qdata, a_t.scale_inv
         elif need_bwd:
             a_row, a_row_s, a_col, a_col_s, _, offs_row, _, _ = grouped_quantize_fp4_with_trans(
-                a.contiguous(), float4_e2m1fn_x2, gran, group_lens, group_offs, block_size=bs)
+                a.contiguous(), float4_e2m1fn_x2, gran, group_lens, group_offs, block_size=bs,
+                scaling_recipe=a_recipe, scaling_recipe_for_trans=a_t_recipe)
         else:
             a_row, a_row_s, _, offs_row = grouped_quantize_fp4(
                 a.contiguous(), float4_e2m1fn_x2, gran, group_lens, group_offs, block_size=bs, axis=1)
@@ -147,7 +150,8 @@ class FP4GroupedGemmMXFunc(torch.autograd.Function):
         config, out_dtype, num_cu, total_m, fuse_bgrad_accum, main_grad = ctx.meta
         gran = config.granularity
         g_row, g_row_s, g_col, g_col_s, _, offs_row, lens_col, offs_col = grouped_quantize_fp4_with_trans(
-            grad_out, float4_e2m1fn_x2, gran, group_lens, group_offs, block_size=config.block_size)
+            grad_out, float4_e2m1fn_x2, gran, group_lens, group_offs, block_size=config.block_size,
+            scaling_recipe=ScalingRecipe(), scaling_recipe_for_trans=ScalingRecipe(use_rht=True))
         # dgrad: grad_a = grad_out @ b as an NT product with the transposed weight quantization [G, K, N]
         grad_a = grouped_gemm_fp4_impl(g_row, b_col, g_row_s, b_col_s, group_lens, offs_row, False, True, out_dtype,
                                        gran.value, num_cu, _NATIVE, False, group_offs)[:total_m]

@@ -213,4 +213,43 @@ def test_grouped_quantize_fp4_ops_surface():
     assert int(oc[-1]) % 256 == 0 and bool((lc % 256 == 0).all())
     with pytest.raises(NotImplementedError):
         turbo.ops.grouped_quantize_fp4(x, FP4, G.MX_BLOCKWISE, gl, offs, block_size=32, axis=1,
-                                       scaling_recipe=ScalingRecipe(use_rht=True))
+                                       scaling_recipe=ScalingRecipe(use_sr=True))
+
+
+@pytest.mark.parametrize("kind,G_,M,N", [("ragged", 8, 1000, 384), ("zeros", 8, 640, 128), ("zipf", 32, 4096, 512),
+                                         ("ragged", 3, 77, 96)])
+def test_grouped_mxfp4_quantizer_hadamard_bit_exact(kind, G_, M, N):
+    """The recipe's Hadamard transform in the grouped quantizer (column direction = the wgrad
+    operand, also the row direction) bit for bit against the oracle."""
+    lens = group_lens(kind, G_, M, 82)
+    gl, offs = _offs(lens)
+    x = bf16_randn((M, N), seed=83, outlier_frac=0.002)
+    rq, rs, cq, cs, _, _, _, ocol = qimpl.grouped_quantize_mxfp4_impl(
+        x.cuda(), FP4, None, 32, gl, offs, with_trans=True, scaling_recipe=ScalingRecipe(),
+        scaling_recipe_for_trans=ScalingRecipe(use_rht=True))
+    o = Q.mx_grouped_quant(x.float().numpy(), lens, "e2m1", row_align=1, col_align=256, col_rht=True)
+    mc = int(o["col_offs"][-1])
+    assert np.array_equal(codes_np(rq), o["row"]) and np.array_equal(codes_np(rs), o["row_scale"])
+    assert np.array_equal(codes_np(cq)[:, : mc // 2], o["col"]) and np.array_equal(codes_np(cs)[:, : mc // 32], o["col_scale"])
+    q1, s1, _, _ = qimpl.grouped_quantize_mxfp4_impl(x.cuda(), FP4, 1, 32, gl, offs, scaling_recipe=ScalingRecipe(use_rht=True))
+    o1 = Q.mx_grouped_quant(x.float().numpy(), lens, "e2m1", row_align=1, col_align=256, row_rht=True)
+    assert np.array_equal(codes_np(q1), o1["row"]) and np.array_equal(codes_np(s1), o1["row_scale"])
+
+
+def test_grouped_mxfp4_hadamard_cancels_in_wgrad():
+    """Both wgrad operands carry the transform along the token axis: the variable-K product of the
+    transformed quantizations estimates the same dW as the plain ones, at least as well."""
+    lens = group_lens("ragged", 4, 2048, 84)
+    gl, offs = _offs(lens)
+    x = bf16_randn((2048, 512), seed=85, outlier_frac=0.01)
+    dy = bf16_randn((2048, 384), seed=86, outlier_frac=0.01)
+    ref = OG.grouped_gemm_variable_k_dequantized(x.float().numpy(), dy.float().numpy(), lens).transpose(0, 2, 1)
+    snr = {}
+    for rht in (False, True):
+        rec = ScalingRecipe(use_rht=rht)
+        xq, xs, lc, ocol = qimpl.grouped_quantize_mxfp4_impl(x.cuda(), FP4, 0, 32, gl, offs, scaling_recipe=rec)
+        gq, gs, _, _ = qimpl.grouped_quantize_mxfp4_impl(dy.cuda(), FP4, 0, 32, gl, offs, scaling_recipe=rec)
+        out = gimpl.grouped_gemm_fp4_variable_k_impl(gq, xq, gs, xs, lc, ocol, False, False, False, torch.float32,
+                                                     G.MX_BLOCKWISE.value, None, 0)
+        snr[rht] = OG.snr_db(ref, to_f32_np(out))
+    assert snr[True] > SNR_GATE and snr[True] > snr[False] - 1.0, snr

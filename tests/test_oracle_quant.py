@@ -275,3 +275,50 @@ def test_mx_grouped_layout(lens, fmt, ra, ca):
         assert not o["row"][pad].any() and not o["row_scale"][pad].any()
         # scale bytes of blocks that lie entirely in the column padding are zero
         assert not o["col_scale"][:, (c0 + n + 31) // 32 : c1 // 32].any()
+
+
+def test_hadamard16_is_the_orthonormal_sylvester_matrix():
+    """``hadamard16`` against scipy's Sylvester construction where fp32 arithmetic is exact (small
+    integers), its involution, norm preservation, and what the recipe relies on: the transform
+    cancels in a product of two operands that both carry it along the reduction axis."""
+    import scipy.linalg
+
+    H = scipy.linalg.hadamard(16).astype(np.float64)
+    rng = np.random.default_rng(11)
+    x = rng.integers(-64, 65, size=(7, 48)).astype(np.float32)
+    y = Q.hadamard16(x)
+    want = np.concatenate([x[:, 16 * i : 16 * i + 16].astype(np.float64) @ H.T / 4 for i in range(3)], axis=1)
+    assert np.array_equal(y.astype(np.float64), want)
+    assert np.array_equal(Q.hadamard16(y), x)
+    e = np.zeros((16, 16), np.float32)
+    np.fill_diagonal(e, 4.0)
+    assert np.array_equal(Q.hadamard16(e), H.astype(np.float32))  # rows of 4 I -> rows of H (symmetric)
+    g = rng.standard_normal((64, 5)).astype(np.float32)
+    a = rng.standard_normal((64, 3)).astype(np.float32)
+    gt, at = Q.hadamard16(g.T.copy()), Q.hadamard16(a.T.copy())
+    assert np.allclose(gt @ at.T, g.T @ a, rtol=1e-5, atol=1e-5)
+    assert np.allclose(np.linalg.norm(gt, axis=1), np.linalg.norm(g.T, axis=1), rtol=1e-6)
+
+
+@pytest.mark.parametrize("shape", [(64, 64), (40, 96), (33, 160)])
+def test_mxfp4_hadamard_quantizer(shape):
+    """With ``use_rht`` the quantizer is the plain MXFP4 quantizer of the transformed, zero-padded
+    tensor; an outlier is spread over its 16 neighbours (smaller block maximum, better SNR of the
+    de-quantized inverse transform on spiky data)."""
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal(shape).astype(np.float32)
+    x[rng.integers(0, shape[0], 6), rng.integers(0, shape[1], 6)] *= 40
+    x = F.bf16_bits_to_f32(F.f32_to_bf16_bits(x))
+    q, s = Q.mx_quant_rowwise(x, "e2m1", use_rht=True)
+    Kp = -(-shape[1] // 128) * 128
+    xp = np.zeros((shape[0], Kp), np.float32)
+    xp[:, : shape[1]] = x
+    q2, s2 = Q.mx_quant_rowwise(Q.hadamard16(xp), "e2m1")
+    assert np.array_equal(q, q2) and np.array_equal(s, s2)
+    qc, sc = Q.mx_quant_colwise(x, "e2m1", use_rht=True)
+    q3, s3 = Q.mx_quant_rowwise(np.ascontiguousarray(x.T), "e2m1", use_rht=True)
+    assert np.array_equal(qc, q3) and np.array_equal(sc, s3)
+    back = Q.hadamard16(Q.mx_dequant(q, s, "e2m1"))[:, : shape[1]]
+    plain = Q.mx_dequant(*Q.mx_quant_rowwise(x, "e2m1"), "e2m1")[:, : shape[1]]
+    err = lambda y: float(np.linalg.norm(y - x) / np.linalg.norm(x))  # noqa: E731
+    assert err(back) < 0.25 and err(plain) < 0.25

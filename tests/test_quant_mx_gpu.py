@@ -140,3 +140,40 @@ def test_mx_public_ops():
         q, s = turbo.ops.quantize_fp4(x, FP4, G.MX_BLOCKWISE, block_size=32, axis=1)
         oq, os_ = Q.mx_quant_rowwise(to_f32_np(x), "e2m1")
         assert np.array_equal(codes_np(q), oq) and np.array_equal(codes_np(s), os_)
+
+
+@pytest.mark.skipif(FP4 is None, reason="torch has no float4_e2m1fn_x2")
+@pytest.mark.parametrize("row_rht,col_rht", [(False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("M,N", [(128, 128), (200, 96), (33, 32), (1000, 2080), (4096, 1024)])
+def test_mxfp4_hadamard_recipe_matches_oracle(row_rht, col_rht, M, N):
+    """``use_rht``: codes and scale bytes of the Hadamard-transformed values, per direction (the recipe
+    uses it on the column direction of ``a`` and ``grad_out``; padding rows / columns take part as
+    zeros). Dual call, single-direction calls, fp16 input."""
+    x = bf16_randn((M, N), seed=55, outlier_frac=0.002)
+    r, rt = ScalingRecipe(use_rht=row_rht), ScalingRecipe(use_rht=col_rht)
+    rq, rs, cq, cs = qi.quantize_mxfp4_impl(x.cuda(), FP4, None, 32, with_trans=True, scaling_recipe=r,
+                                            scaling_recipe_for_trans=rt)
+    xf = to_f32_np(x)
+    oq, os_ = Q.mx_quant_rowwise(xf, "e2m1", use_rht=row_rht)
+    assert np.array_equal(codes_np(rs), os_) and np.array_equal(codes_np(rq), oq), "row direction"
+    oq, os_ = Q.mx_quant_colwise(xf, "e2m1", use_rht=col_rht)
+    assert np.array_equal(codes_np(cs), os_) and np.array_equal(codes_np(cq), oq), "column direction"
+    q0, s0 = qi.quantize_mxfp4_impl(x.cuda(), FP4, 0, 32, scaling_recipe=rt)
+    assert torch.equal(q0.view(torch.uint8), cq.view(torch.uint8)) and torch.equal(s0.view(torch.uint8), cs.view(torch.uint8))
+    q1, s1 = qi.quantize_mxfp4_impl(x.cuda(), FP4, 1, 32, scaling_recipe=r)
+    assert torch.equal(q1.view(torch.uint8), rq.view(torch.uint8)) and torch.equal(s1.view(torch.uint8), rs.view(torch.uint8))
+    xh = x.to(torch.float16)
+    hq, hs = qi.quantize_mxfp4_impl(xh.cuda(), FP4, 0, 32, scaling_recipe=ScalingRecipe(use_rht=True))
+    oq, os_ = Q.mx_quant_colwise(to_f32_np(xh), "e2m1", use_rht=True)
+    assert np.array_equal(codes_np(hs), os_) and np.array_equal(codes_np(hq), oq), "fp16 input"
+
+
+@pytest.mark.skipif(FP4 is None, reason="torch has no float4_e2m1fn_x2")
+def test_mx_hadamard_recipe_limits():
+    x = bf16_randn((128, 128), seed=56).cuda()
+    with pytest.raises(NotImplementedError):  # MXFP8 has no Hadamard recipe
+        qi.quantize_mxfp8_impl(x, torch.float8_e4m3fn, 1, 32, scaling_recipe=ScalingRecipe(use_rht=True))
+    with pytest.raises(NotImplementedError):  # never together with 2-D blocks
+        qi.quantize_mxfp4_impl(x, FP4, 1, 32, scaling_recipe=ScalingRecipe(use_rht=True, use_2d_block=True))
+    with pytest.raises(NotImplementedError):  # stochastic rounding stays out
+        qi.quantize_mxfp4_impl(x, FP4, 1, 32, scaling_recipe=ScalingRecipe(use_sr=True))

@@ -263,7 +263,9 @@ def test_grouped_gemm_prequantized_operands(case):
     y_ref = op(a1, w1, gl, trans_b=True, config=cfg)
     y_ref.backward(dy)
     qa = QT.quantize(a, dt, G.MX_BLOCKWISE, axis=-1, group_lens=gl, block_size=32, scaling_recipe=Recipe())
-    qa_t = QT.quantize(a, dt, G.MX_BLOCKWISE, axis=-2, group_lens=gl, block_size=32, scaling_recipe=Recipe())
+    # (the MXFP4 recipe puts the Hadamard transform on the wgrad operands)
+    qa_t = QT.quantize(a, dt, G.MX_BLOCKWISE, axis=-2, group_lens=gl, block_size=32,
+                       scaling_recipe=Recipe(use_rht=(case == "mxfp4")))
     qw, qw_t = create_quantized_weight(w, dt, cfg, need_weight_transpose_cache=True)
     with torch.no_grad():
         assert torch.equal(op(qa, qw, gl, trans_b=True, config=cfg), y_ref)
