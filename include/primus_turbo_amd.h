@@ -218,7 +218,10 @@ PT_API int pt_dequantize_fp8_block(const void *q, int q_dtype, int64_t B, int64_
  * bit 0) quantizes the Hadamard-transformed values: every 16 consecutive elements along the
  * direction (of the zero-padded tensor) are replaced by (H4 (x) H4) / 4 times themselves, in fp32
  * with the operation order of flydsl/quantization/mxfp4_quant_kernel.py:92-118 -- the recipe's
- * "RHT" of the two wgrad operands, which cancels in their product.
+ * "RHT" of the two wgrad operands, which cancels in their product. Bit 2 (MXFP4 only) rounds
+ * the codes stochastically (unbiased; scales unchanged) from sr_seed, which the caller changes
+ * from launch to launch (mxfp4_quant_kernel.py:48-75: random by design, not reproducible bit
+ * for bit against the reference).
  *
  * pt_dequantize_mx replaces dequantize_mxfp8 / dequantize_mxfp4 (quantization.cpp:285-359,
  * 436-508; kernels dequantization_mxfp8.cu:29-113, dequantization_mxfp4.cu:28-160):
@@ -227,7 +230,7 @@ PT_API int pt_dequantize_fp8_block(const void *q, int q_dtype, int64_t B, int64_
  * column-direction data, transposed back as y [cols, rows]. */
 PT_API int pt_quantize_mx(const void *x, int x_dtype, int64_t B, int64_t M, int64_t N, int q_dtype,
                           void *row_q, void *row_scale, int row_flags, void *col_q, void *col_scale,
-                          int col_flags, void *stream);
+                          int col_flags, uint32_t sr_seed, void *stream);
 PT_API int pt_dequantize_mx(const void *q, int q_dtype, const void *scale, int64_t rows,
                             int64_t cols, void *y, int y_dtype, int transpose, void *stream);
 
@@ -394,7 +397,8 @@ PT_API int pt_grouped_gemm_fp8_vec_variable_k(const void *lhs, int lhs_dtype, co
  * With q_dtype e2m1x2 it is the grouped MXFP4 quantizer (grouped_quantize_mxfp4[_dual],
  * quantization.cpp:1209-1378; default dispatch flydsl/quantization/mxfp4_grouped_quant.py:320-349):
  * two codes per byte, rows kept tight (row_offs_padded NULL) and column groups padded to 256;
- * row_flags / col_flags as for pt_quantize_mx (bit 1 only: grouped data have no 2-D blocks).
+ * row_flags / col_flags / sr_seed as for pt_quantize_mx (bits 1 and 2: grouped data have no 2-D
+ * blocks).
  *
  * pt_grouped_gemm_mx replaces primus_turbo::grouped_gemm_fp8_impl for MX_BLOCKWISE
  * (kernels/grouped_gemm/grouped_gemm_fp8_impl.py:888-930 with group_offs_out; caller
@@ -422,7 +426,7 @@ PT_API int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t
                                   const int64_t *group_offs, const int64_t *row_offs_padded,
                                   const int64_t *col_offs_padded, int64_t G, void *row_q,
                                   void *row_scale, int row_flags, void *col_q, void *col_scale,
-                                  int col_flags, int64_t col_ld, void *stream);
+                                  int col_flags, int64_t col_ld, uint32_t sr_seed, void *stream);
 PT_API int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, int64_t lda,
                               int64_t sa_ld, const void *b, int b_dtype, const void *b_scale,
                               int64_t ldb, int64_t sb_ld, void *c, int c_dtype,

@@ -34,7 +34,7 @@ What each function follows, and what pins it (tests/test_oracle_*.py):
   over 32x32 tiles, round trips through the de-quantizer. ``hadamard16`` restates the
   recipe's fixed 16-point Hadamard transform (``use_rht``; pinned against scipy's
   Sylvester matrix and by its involution, rounding order PARITY UNPINNED as above).
-  Stochastic rounding is not restated (random by design, not implemented).
+  Stochastic rounding is not restated (random by design: the tests check its properties).
 * ``mx_grouped_quant`` — per-group composition of the two above in the padded layouts of
   /root/reference/csrc/pytorch/quantization/quantization.cpp:971-1100 (rows of a group padded
   to 32 / 128 with zero data); pinned by the group-by-group round trip against the dense

@@ -73,6 +73,37 @@ template <int FMT> __device__ __forceinline__ void mx_encode32(const float (&v)[
     }
 }
 
+// Stochastic rounding (MXFP4 gradients): the hardware converter adds the seed's bits below the
+// kept mantissa before truncating, so a value lands on its upper neighbour with a probability
+// equal to its position between the two neighbours (unbiased; measured on uniform seeds). The
+// scale stays the deterministic one. Every pair of values gets its own seed; the converter's
+// destination bytes other than the selected one are not preserved, hence byte 0 and a mask.
+// (Primus-Turbo's recipe: flydsl/quantization/mxfp4_quant_kernel.py:48-75,120-150.)
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t sr_hash(uint32_t s) {
+    s = (s ^ 61u) ^ (s >> 16);
+    s *= 9u;
+    s ^= s >> 4;
+    s *= 0x27D4EB2Du;
+    s ^= s >> 15;
+    return s;
+}
+__device__ __forceinline__ void mx_encode32_fp4_sr(const float (&v)[32], float inv, uint32_t seed, uint32_t (&out)[8]) {
+    constexpr float Q = MxFmt<MX_E2M1>::QMAX;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        uint32_t w = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const f32x2_t pair = {scale_clamp(v[8 * d + 2 * k], inv, Q), scale_clamp(v[8 * d + 2 * k + 1], inv, Q)};
+            seed += 0x9E3779B9u;
+            const uint32_t b = __builtin_amdgcn_cvt_scalef32_sr_pk_fp4_f32(0u, pair, seed, 1.0f, 0) & 0xffu;
+            w |= b << (8 * k);
+        }
+        out[d] = w;
+    }
+}
+
 constexpr int MX_TILE  = 128;
 constexpr int MX_PITCH = MX_TILE + 8; // 16-bit elements per LDS row (272 B: 16-byte aligned rows)
 
@@ -92,6 +123,9 @@ struct MxArgs {
     const int64_t *row_offs_pad; // [G + 1] or NULL
     const int64_t *col_offs_pad; // [G + 1]
     int            G;
+    // MXFP4 stochastic rounding: bit 0 / bit 1 = row / column direction; one seed per launch
+    int      sr_mask;
+    uint32_t sr_seed;
 };
 
 // The MXFP4 recipe's fixed 16-point Hadamard transform of v[base .. base + 16), in place:
@@ -234,7 +268,13 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
             }
             const int e = mx_exponent<FMT>(am);
             uint32_t  code[8];
-            mx_encode32<FMT>(rv[p], mx_inv_scale(e), code);
+            if (FMT == MX_E2M1 && (a.sr_mask & 1)) {
+                // a seed per 32-element block: launch seed, tile and task mixed
+                const uint32_t id = (static_cast<uint32_t>(blockIdx.z) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+                mx_encode32_fp4_sr(rv[p], mx_inv_scale(e), sr_hash(a.sr_seed ^ (id * 512u + t)), code);
+            } else {
+                mx_encode32<FMT>(rv[p], mx_inv_scale(e), code);
+            }
             sbytes[r * 4 + c] = static_cast<uint8_t>(e + 127);
             if (r < row_cnt) {
                 const int64_t nb = (n0 >> 5) + c; // 32-column block index in the padded row
@@ -291,7 +331,12 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
                     am = fmaxf(am, amax_rc[(rb * 32 + i) * 4 + (c >> 5)]);
             }
             const int e = mx_exponent<FMT>(am);
-            mx_encode32<FMT>(v, mx_inv_scale(e), code[p]);
+            if (FMT == MX_E2M1 && (a.sr_mask & 2)) {
+                const uint32_t id = (static_cast<uint32_t>(blockIdx.z) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+                mx_encode32_fp4_sr(v, mx_inv_scale(e), sr_hash(a.sr_seed ^ 0x5BD1E995u ^ (id * 512u + t)), code[p]);
+            } else {
+                mx_encode32<FMT>(v, mx_inv_scale(e), code[p]);
+            }
             sbytes[c * 4 + rb] = static_cast<uint8_t>(e + 127);
         }
         __syncthreads(); // everybody is done with the input tile
@@ -513,17 +558,20 @@ using namespace pt;
 
 extern "C" {
 
-// direction flags: bit 0 = 2-D (32 x 32) blocks, bit 1 = Hadamard transform (MXFP4, 1-D blocks)
+// direction flags: bit 0 = 2-D (32 x 32) blocks, bit 1 = Hadamard transform (MXFP4, 1-D blocks),
+// bit 2 = stochastic rounding (MXFP4)
 static int check_mx_flags(int fmt, int row_flags, int col_flags) {
-    PT_REQUIRE((row_flags & ~3) == 0 && (col_flags & ~3) == 0, "unknown direction flags");
+    PT_REQUIRE((row_flags & ~7) == 0 && (col_flags & ~7) == 0, "unknown direction flags");
     const bool rht = ((row_flags | col_flags) & 2) != 0;
     PT_REQUIRE(!rht || fmt == MX_E2M1, "the Hadamard transform belongs to the MXFP4 recipe");
+    PT_REQUIRE(((row_flags | col_flags) & 4) == 0 || fmt == MX_E2M1, "stochastic rounding belongs to the MXFP4 recipe");
     PT_REQUIRE(!rht || ((row_flags | col_flags) & 1) == 0, "the Hadamard transform is not combined with 2-D blocks");
     return PT_OK;
 }
 
 int pt_quantize_mx(const void *x, int x_dtype, int64_t B, int64_t M, int64_t N, int q_dtype, void *row_q,
-                   void *row_scale, int row_flags, void *col_q, void *col_scale, int col_flags, void *stream) {
+                   void *row_scale, int row_flags, void *col_q, void *col_scale, int col_flags, uint32_t sr_seed,
+                   void *stream) {
     PT_REQUIRE(x_dtype == PT_DTYPE_BF16 || x_dtype == PT_DTYPE_F16, "input must be bf16 or fp16");
     const int fmt = mx_fmt_of(q_dtype);
     PT_REQUIRE(fmt >= 0, "q_dtype must be e4m3, e5m2 or e2m1x2");
@@ -552,6 +600,8 @@ int pt_quantize_mx(const void *x, int x_dtype, int64_t B, int64_t M, int64_t N, 
     a.col_s = static_cast<uint8_t *>(col_scale);
     a.group_offs = a.row_offs_pad = a.col_offs_pad = nullptr;
     a.G          = 0;
+    a.sr_mask    = ((row_q && (row_flags & 4)) ? 1 : 0) | ((col_q && (col_flags & 4)) ? 2 : 0);
+    a.sr_seed    = sr_seed;
     PT_REQUIRE(a.Mpad / 128 < 65536 && B < 65536, "grid dimension out of range");
     dim3 grid(static_cast<unsigned>(a.Npad / 128), static_cast<unsigned>(a.Mpad / 128), static_cast<unsigned>(B));
     auto st = static_cast<hipStream_t>(stream);
@@ -571,7 +621,7 @@ int pt_quantize_mx(const void *x, int x_dtype, int64_t B, int64_t M, int64_t N, 
 int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype, const int64_t *group_offs,
                            const int64_t *row_offs_padded, const int64_t *col_offs_padded, int64_t G, void *row_q,
                            void *row_scale, int row_flags, void *col_q, void *col_scale, int col_flags, int64_t col_ld,
-                           void *stream) {
+                           uint32_t sr_seed, void *stream) {
     PT_REQUIRE(x_dtype == PT_DTYPE_BF16 || x_dtype == PT_DTYPE_F16, "input must be bf16 or fp16");
     const int fmt = mx_fmt_of(q_dtype);
     PT_REQUIRE(fmt >= 0, "q_dtype must be e4m3, e5m2 or e2m1x2");
@@ -604,6 +654,8 @@ int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t N, int
     a.row_offs_pad = row_offs_padded;
     a.col_offs_pad = col_offs_padded;
     a.G            = static_cast<int>(G);
+    a.sr_mask      = ((row_q && (row_flags & 4)) ? 1 : 0) | ((col_q && (col_flags & 4)) ? 2 : 0);
+    a.sr_seed      = sr_seed;
     PT_REQUIRE(col_ld / 128 < 65536, "grid dimension out of range");
     dim3 grid(static_cast<unsigned>(a.Npad / 128), static_cast<unsigned>(col_ld / 128), 1);
     auto st = static_cast<hipStream_t>(stream);

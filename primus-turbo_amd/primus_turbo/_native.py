@@ -106,7 +106,8 @@ _SIGNATURES = {
     ),
     "pt_quantize_mx": (
         c_int,
-        [c_void_p, c_int, c_i64, c_i64, c_i64, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p],
+        [c_void_p, c_int, c_i64, c_i64, c_i64, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, ctypes.c_uint32,
+         c_void_p],
     ),
     "pt_dequantize_mx": (c_int, [c_void_p, c_int, c_void_p, c_i64, c_i64, c_void_p, c_int, c_int, c_void_p]),
     "pt_grouped_gemm_fp8_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_i64, c_int]),
@@ -136,7 +137,7 @@ _SIGNATURES = {
     "pt_grouped_quantize_mx": (
         c_int,
         [c_void_p, c_int, c_i64, c_i64, c_int, c_void_p, c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_int, c_void_p,
-         c_void_p, c_int, c_i64, c_void_p],
+         c_void_p, c_int, c_i64, ctypes.c_uint32, c_void_p],
     ),
     "pt_grouped_gemm_mx": (
         c_int,

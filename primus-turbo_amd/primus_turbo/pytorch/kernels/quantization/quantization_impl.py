@@ -706,21 +706,33 @@ def _mx_recipes(with_trans, scaling_recipe, scaling_recipe_for_trans, what):
     r = ScalingRecipe() if scaling_recipe is None else scaling_recipe
     rt = (ScalingRecipe() if scaling_recipe_for_trans is None else scaling_recipe_for_trans) if with_trans else r
     for rec in (r, rt):
-        if rec.use_sr or rec.shuffle_scale or rec.shuffle_out:
-            raise NotImplementedError(
-                f"{what}: stochastic rounding and shuffled layouts are not implemented "
-                "(round-to-nearest-even, plain layouts are)"
-            )
-        if rec.use_rht and what != "MXFP4":
-            raise NotImplementedError(f"{what}: the Hadamard transform belongs to the MXFP4 recipe")
+        if rec.shuffle_scale or rec.shuffle_out:
+            raise NotImplementedError(f"{what}: shuffled layouts are not implemented (plain layouts are)")
+        if (rec.use_rht or rec.use_sr) and what != "MXFP4":
+            raise NotImplementedError(f"{what}: the Hadamard transform and stochastic rounding belong to the MXFP4 recipe")
         if rec.use_rht and rec.use_2d_block:
             raise NotImplementedError(f"{what}: the Hadamard transform is not combined with 2-D blocks")
     return r, rt
 
 
 def _mx_flags(recipe) -> int:
-    """Direction flags of the native quantizer: bit 0 = 2-D blocks, bit 1 = Hadamard transform."""
-    return (1 if recipe.use_2d_block else 0) | (2 if recipe.use_rht else 0)
+    """Direction flags of the native quantizer: bit 0 = 2-D blocks, bit 1 = Hadamard transform,
+    bit 2 = stochastic rounding."""
+    if recipe is None:
+        return 0
+    return (1 if recipe.use_2d_block else 0) | (2 if recipe.use_rht else 0) | (4 if recipe.use_sr else 0)
+
+
+_sr_counter = [0]
+
+
+def _next_sr_seed(*flags: int) -> int:
+    """A fresh 32-bit seed per stochastic-rounding launch (a process-wide counter, as the
+    reference's quantizers keep one: reproducible for a fixed order of calls); 0 otherwise."""
+    if not any(f & 4 for f in flags):
+        return 0
+    _sr_counter[0] = (_sr_counter[0] + 1) & 0xFFFFFFFF
+    return (_sr_counter[0] * 0x9E3779B1) & 0xFFFFFFFF
 
 
 def _mx_check_axis(x, axis, with_trans):
@@ -766,7 +778,8 @@ def _mx_quantize(x: torch.Tensor, out_dtype: torch.dtype, want_row: bool, want_c
     N.check(
         N.lib().pt_quantize_mx(
             N.ptr(x), N.dtype_code(x.dtype), B, M, Nn, N.dtype_code(out_dtype),
-            N.ptr(row_q), N.ptr(row_s), int(row_flags), N.ptr(col_q), N.ptr(col_s), int(col_flags), N.stream_of(x),
+            N.ptr(row_q), N.ptr(row_s), int(row_flags), N.ptr(col_q), N.ptr(col_s), int(col_flags),
+            _next_sr_seed(row_flags if want_row else 0, col_flags if want_col else 0), N.stream_of(x),
         )
     )
     view = lambda t, dt: None if t is None else t.view(dt)  # noqa: E731
@@ -797,7 +810,8 @@ def quantize_mxfp4_impl(x, out_dtype, axis, block_size, with_trans=False, scalin
                         scaling_recipe_for_trans=None):
     """MXFP4 (E2M1, two codes per byte, even element in the low nibble); shapes as MXFP8 with
     the code tensors half as wide. ``use_rht`` in a recipe quantizes the values after the recipe's
-    fixed 16-point Hadamard transform along that direction (1-D blocks only)."""
+    fixed 16-point Hadamard transform along that direction (1-D blocks only); ``use_sr`` rounds the
+    codes stochastically (unbiased, a fresh seed per call; the scales stay deterministic)."""
     assert x.is_contiguous(), "The x tensor must be contiguous."
     return _quantize_mx_impl(x, out_dtype, axis, block_size, with_trans, scaling_recipe, scaling_recipe_for_trans, "MXFP4")
 
@@ -895,7 +909,8 @@ def _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, want_row: bool, w
         N.lib().pt_grouped_quantize_mx(
             N.ptr(x), N.dtype_code(x.dtype), M, Nn, N.dtype_code(out_dtype), N.ptr(group_offs),
             None if fp4 else N.ptr(offs_row), N.ptr(offs_col), G, N.ptr(row_q), N.ptr(row_s), int(row_flags), N.ptr(col_q),
-            N.ptr(col_s), int(col_flags), m_pad_col, N.stream_of(x),
+            N.ptr(col_s), int(col_flags), m_pad_col,
+            _next_sr_seed(row_flags if want_row else 0, col_flags if want_col else 0), N.stream_of(x),
         )
     )
     view = lambda t, dt: None if t is None else t.view(dt)  # noqa: E731
@@ -954,17 +969,16 @@ def grouped_quantize_mxfp4_impl(x, out_dtype, axis, block_size, group_lens, grou
     256 G`` rounded up to 256. Otherwise ``(q, scale, lens_padded, offs_padded)`` of the direction
     ``axis`` asks for (1 = rows, 0 = transposed columns). ``use_rht`` in a recipe applies the fixed
     16-point Hadamard transform along that direction (within each group's padded rows for the
-    column direction). Round-to-nearest-even only: stochastic rounding, 2-D blocks and shuffled
-    layouts raise."""
+    column direction), ``use_sr`` rounds the codes stochastically. 2-D blocks and shuffled layouts
+    raise."""
     assert block_size == 32, "The block size must be 32 for MXFP4 quantization"
     assert _FP4X2 is not None and out_dtype == _FP4X2, "The out_dtype must be float4_e2m1fn_x2 for MXFP4 quantization"
     for r in (scaling_recipe, scaling_recipe_for_trans):
-        if r is not None and (r.use_2d_block or r.use_sr or r.shuffle_scale or r.shuffle_out):
-            raise NotImplementedError(
-                "grouped MXFP4 quantization: 2-D blocks, stochastic rounding and shuffled layouts are not implemented")
-    rf = 2 if (scaling_recipe is not None and scaling_recipe.use_rht) else 0
+        if r is not None and (r.use_2d_block or r.shuffle_scale or r.shuffle_out):
+            raise NotImplementedError("grouped MXFP4 quantization: 2-D blocks and shuffled layouts are not implemented")
+    rf = _mx_flags(scaling_recipe)
     if with_trans:
-        cf = 2 if (scaling_recipe_for_trans is not None and scaling_recipe_for_trans.use_rht) else 0
+        cf = _mx_flags(scaling_recipe_for_trans)
         return _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, True, True, rf, cf)
     assert axis in (0, 1), "The axis must be 0 (colwise) or 1 (rowwise) when with_trans is False."
     rq, rs, cq, cs, lr, orow, lc, ocol = _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, axis == 1, axis == 0,

@@ -6,9 +6,9 @@ gradients use 1 x 32 blocks, the weight 32 x 32 blocks; each tensor is quantized
 directions from one read. As in the reference's recipe (its lines 108-160, 220-240) the two wgrad
 operands -- the column-direction quantizations of ``a`` and of ``grad_out`` -- carry the fixed
 16-point Hadamard transform along the token axis, which cancels in their product and spreads
-outliers over 16 values before they are quantized. Stochastic rounding of gradients is not
-implemented (``use_gradient_sr=True`` raises), and pre-shuffled layouts do not exist here
-(``use_preshuffle=True`` raises).
+outliers over 16 values before they are quantized; ``use_gradient_sr`` rounds both quantizations of
+``grad_out`` stochastically. Pre-shuffled layouts do not exist here (``use_preshuffle=True``
+raises).
 """
 
 from __future__ import annotations
@@ -61,8 +61,6 @@ class FP4GemmMXFunction(torch.autograd.Function):
         assert ok, why
         if config.use_preshuffle:
             raise NotImplementedError("Float4QuantConfig.use_preshuffle is not implemented")
-        if config.use_gradient_sr:
-            raise NotImplementedError("Float4QuantConfig.use_gradient_sr (stochastic rounding) is not implemented")
         fuse, main_grad = _setup_fused_grad_accum(b, fuse_bgrad_accum_pattern)
         dt = FP4GemmMXFunction.get_fp4_dtype(config.format)
         gran, bs = config.granularity, config.block_size
@@ -101,8 +99,8 @@ class FP4GemmMXFunction(torch.autograd.Function):
         gran = config.granularity
         g = grad_out.reshape(grad_out.shape[0], -1).contiguous()
         g_row, g_row_s, g_col, g_col_s = quantize_fp4_with_trans(
-            g, dt, gran, block_size=config.block_size, scaling_recipe=ScalingRecipe(),
-            scaling_recipe_for_trans=ScalingRecipe(use_rht=True),  # pairs with a_col in wgrad
+            g, dt, gran, block_size=config.block_size, scaling_recipe=ScalingRecipe(use_sr=config.use_gradient_sr),
+            scaling_recipe_for_trans=ScalingRecipe(use_sr=config.use_gradient_sr, use_rht=True),  # pairs with a_col
         )
         # both directions are stored transposed, so dgrad and wgrad are NT products as well
         grad_a = gemm_fp4_impl(g_row, g_row_s, False, b_col, b_col_s, True, out_dtype, False, gran.value, _NATIVE)

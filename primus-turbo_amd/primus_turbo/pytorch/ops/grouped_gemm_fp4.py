@@ -9,8 +9,8 @@ Activations and gradients use 1 x 32 blocks and are quantized in both directions
 (rows in place, transposed columns padded to 256 tokens per group); the weight uses 32 x 32
 blocks. As in the reference the two wgrad operands (the column-direction quantizations of ``a`` and
 ``grad_out``) carry the recipe's fixed 16-point Hadamard transform along the token axis, which
-cancels in their product. Not implemented: stochastic rounding (``use_gradient_sr=True`` raises)
-and pre-shuffled layouts.
+cancels in their product; ``use_gradient_sr`` rounds both quantizations of ``grad_out``
+stochastically. Pre-shuffled layouts are not implemented.
 """
 
 from __future__ import annotations
@@ -83,8 +83,6 @@ class FP4GroupedGemmMXFunc(torch.autograd.Function):
         assert trans_b, "MXFP4 grouped GEMM only supports trans_b=True (NT layout)."
         if config.use_preshuffle:
             raise NotImplementedError("Float4QuantConfig.use_preshuffle is not implemented")
-        if config.use_gradient_sr:
-            raise NotImplementedError("Float4QuantConfig.use_gradient_sr (stochastic rounding) is not implemented")
         supported, reason = check_mxfp4_support()
         assert supported, reason
         N, K = int(b.shape[-2]), int(b.shape[-1])
@@ -151,7 +149,8 @@ class FP4GroupedGemmMXFunc(torch.autograd.Function):
         gran = config.granularity
         g_row, g_row_s, g_col, g_col_s, _, offs_row, lens_col, offs_col = grouped_quantize_fp4_with_trans(
             grad_out, float4_e2m1fn_x2, gran, group_lens, group_offs, block_size=config.block_size,
-            scaling_recipe=ScalingRecipe(), scaling_recipe_for_trans=ScalingRecipe(use_rht=True))
+            scaling_recipe=ScalingRecipe(use_sr=config.use_gradient_sr),
+            scaling_recipe_for_trans=ScalingRecipe(use_sr=config.use_gradient_sr, use_rht=True))
         # dgrad: grad_a = grad_out @ b as an NT product with the transposed weight quantization [G, K, N]
         grad_a = grouped_gemm_fp4_impl(g_row, b_col, g_row_s, b_col_s, group_lens, offs_row, False, True, out_dtype,
                                        gran.value, num_cu, _NATIVE, False, group_offs)[:total_m]

@@ -213,7 +213,7 @@ def test_grouped_quantize_fp4_ops_surface():
     assert int(oc[-1]) % 256 == 0 and bool((lc % 256 == 0).all())
     with pytest.raises(NotImplementedError):
         turbo.ops.grouped_quantize_fp4(x, FP4, G.MX_BLOCKWISE, gl, offs, block_size=32, axis=1,
-                                       scaling_recipe=ScalingRecipe(use_sr=True))
+                                       scaling_recipe=ScalingRecipe(use_2d_block=True))
 
 
 @pytest.mark.parametrize("kind,G_,M,N", [("ragged", 8, 1000, 384), ("zeros", 8, 640, 128), ("zipf", 32, 4096, 512),
@@ -253,3 +253,35 @@ def test_grouped_mxfp4_hadamard_cancels_in_wgrad():
                                                      G.MX_BLOCKWISE.value, None, 0)
         snr[rht] = OG.snr_db(ref, to_f32_np(out))
     assert snr[True] > SNR_GATE and snr[True] > snr[False] - 1.0, snr
+
+
+@pytest.mark.parametrize("grouped", [True, False])
+def test_fp4_gradient_stochastic_rounding(grouped):
+    """``Float4QuantConfig(use_gradient_sr=True)``: forward is unchanged, the gradients pass the same
+    SNR gate, and two backward passes differ (the gradient quantizers draw a fresh seed)."""
+    lens = group_lens("ragged", 4, 1024, 87)
+    gl, _ = _offs(lens)
+    a = bf16_randn((1024, 512), seed=88).cuda().requires_grad_(True)
+    b = (bf16_randn((4, 384, 512), seed=89) if grouped else bf16_randn((384, 512), seed=89)).cuda().requires_grad_(True)
+    dy = bf16_randn((1024, 384), seed=90).cuda()
+    cfg, cfg_sr = Float4QuantConfig(), Float4QuantConfig(use_gradient_sr=True)
+
+    def run(c):
+        a.grad = b.grad = None
+        y = turbo.ops.grouped_gemm_fp4(a, b, gl, config=c) if grouped else turbo.ops.gemm_fp4(a, b, trans_b=True, config=c)
+        y.backward(dy)
+        return y.detach().clone(), a.grad.clone(), b.grad.clone()
+
+    y0, da0, db0 = run(cfg)
+    y1, da1, db1 = run(cfg_sr)
+    y2, da2, db2 = run(cfg_sr)
+    assert torch.equal(y0, y1) and torch.equal(y1, y2)
+    assert not torch.equal(da1, da2) and not torch.equal(db1, db2)
+    af, bf_, dyf = to_f32_np(a), to_f32_np(b), to_f32_np(dy)
+    if grouped:
+        ref_da = OG.grouped_gemm_dequantized(dyf, bf_, lens, trans_b=False)
+        ref_db = OG.grouped_gemm_variable_k_dequantized(af, dyf, lens).transpose(0, 2, 1)
+    else:
+        ref_da, ref_db = dyf @ bf_, dyf.T @ af
+    for da, db in ((da1, db1), (da2, db2)):
+        assert OG.snr_db(ref_da, to_f32_np(da)) > SNR_GATE and OG.snr_db(ref_db, to_f32_np(db)) > SNR_GATE

@@ -175,5 +175,54 @@ def test_mx_hadamard_recipe_limits():
         qi.quantize_mxfp8_impl(x, torch.float8_e4m3fn, 1, 32, scaling_recipe=ScalingRecipe(use_rht=True))
     with pytest.raises(NotImplementedError):  # never together with 2-D blocks
         qi.quantize_mxfp4_impl(x, FP4, 1, 32, scaling_recipe=ScalingRecipe(use_rht=True, use_2d_block=True))
-    with pytest.raises(NotImplementedError):  # stochastic rounding stays out
-        qi.quantize_mxfp4_impl(x, FP4, 1, 32, scaling_recipe=ScalingRecipe(use_sr=True))
+    with pytest.raises(NotImplementedError):  # MXFP8 has no stochastic rounding either
+        qi.quantize_mxfp8_impl(x, torch.float8_e4m3fn, 1, 32, scaling_recipe=ScalingRecipe(use_sr=True))
+    with pytest.raises(NotImplementedError):  # shuffled layouts do not exist here
+        qi.quantize_mxfp4_impl(x, FP4, 1, 32, scaling_recipe=ScalingRecipe(shuffle_out=True))
+
+
+@pytest.mark.skipif(FP4 is None, reason="torch has no float4_e2m1fn_x2")
+@pytest.mark.parametrize("axis", [1, 0])
+@pytest.mark.parametrize("rht", [False, True])
+def test_mxfp4_stochastic_rounding(axis, rht):
+    """``use_sr``: the scale bytes are those of round-to-nearest; every code is one of the two E2M1
+    neighbours of the scaled value; two calls differ (fresh seed) yet the mean over many calls
+    converges to the unrounded value (unbiased) where round-to-nearest keeps its systematic error."""
+    M, N = 256, 128
+    x = bf16_randn((M, N), seed=57)
+    xf = to_f32_np(x)
+    plain = ScalingRecipe(use_rht=rht)
+    q0, s0 = qi.quantize_mxfp4_impl(x.cuda(), FP4, axis, 32, scaling_recipe=plain)
+    rec = ScalingRecipe(use_sr=True, use_rht=rht)
+    n_calls = 192
+    acc = None
+    codes = []
+    for _ in range(n_calls):
+        q, sc = qi.quantize_mxfp4_impl(x.cuda(), FP4, axis, 32, scaling_recipe=rec)
+        assert torch.equal(sc.view(torch.uint8), s0.view(torch.uint8)), "scales are deterministic"
+        d = Q.mx_dequant(codes_np(q), codes_np(sc), "e2m1").astype(np.float64)
+        acc = d if acc is None else acc + d
+        if len(codes) < 2:
+            codes.append(codes_np(q).copy())
+    assert not np.array_equal(codes[0], codes[1]), "a fresh seed per call"
+    # the exact values the codes approximate: the (transformed) tensor in the quantizer's layout
+    t = xf if axis == 1 else np.ascontiguousarray(xf.T)
+    pad = np.zeros((t.shape[0], -(-t.shape[1] // 128) * 128), np.float32)
+    pad[:, : t.shape[1]] = t
+    target = (Q.hadamard16(pad) if rht else pad).astype(np.float64)
+    scale = np.repeat(Q.e8m0_to_f32(codes_np(s0)).astype(np.float64), 32, axis=-1)
+    grid = np.array([0, .5, 1, 1.5, 2, 3, 4, 6], dtype=np.float64)
+    # each code is a neighbour of the clamped scaled value
+    one = Q.mx_dequant(codes[0], codes_np(s0), "e2m1").astype(np.float64) / scale
+    v = np.clip(target / scale, -6, 6)
+    lo = grid[np.searchsorted(grid, np.abs(v), side="right") - 1]
+    hi = grid[np.minimum(np.searchsorted(grid, np.abs(v), side="left"), 7)]
+    assert np.all((np.abs(one) == lo) | (np.abs(one) == hi))
+    # unbiased: the mean error shrinks like 1 / sqrt(n), far below round-to-nearest's
+    mean = acc / n_calls
+    inside = np.abs(target / scale) <= 6  # the saturated sliver of a block is clamped, not rounded
+    err_sr = np.abs(mean - target)[inside] / scale[inside]
+    rne = Q.mx_dequant(codes_np(q0), codes_np(s0), "e2m1").astype(np.float64)
+    err_rne = np.abs(rne - target)[inside] / scale[inside]
+    assert err_sr.mean() < 0.35 * err_rne.mean(), (err_sr.mean(), err_rne.mean())
+    assert err_sr.max() < 6 * 1.0 / np.sqrt(n_calls) + 1e-6  # within six standard errors of the largest step
