@@ -340,7 +340,60 @@ class QuantMx(_QuantBase):
         return self._cpu(fn, self.step_work() * rows / self.M, f"numpy oracle on the first {rows} rows")
 
 
+class SwigluWithProbs(_QuantBase):
+    """SwiGLU with router probabilities between the two grouped GEMMs of the MoE configuration:
+    32768 routed tokens, fc1 output 2 x 2048 -> 2048, forward + backward."""
+
+    name = "swiglu_with_probs_32768tokens_hidden2048_bf16 (forward + backward)"
+    dominant_name = "glu_fwd_kernel<bf16, SiLU> (one workgroup per token row, 16-byte accesses)"
+    dtype = "bf16 (fp32 arithmetic)"
+
+    def __init__(self, dev, tokens=32768, hidden=2048):
+        import primus_turbo.pytorch as turbo
+
+        self.turbo, self.T, self.H = turbo, tokens, hidden
+        self.x_cpu = _randn_bf16((tokens, 2 * hidden), 31, 1.0)
+        g = torch.Generator().manual_seed(32)
+        self.p_cpu = torch.rand(tokens, generator=g, dtype=torch.float32)
+        self.x = self.x_cpu.to(dev).requires_grad_(True)
+        self.p = self.p_cpu.to(dev).requires_grad_(True)
+        self.go = _randn_bf16((tokens, hidden), 33, 1.0).to(dev)
+
+    def dominant_work(self):  # 2 H read + H written per token, 2 bytes each, + the probability
+        return 6.0 * self.T * self.H + 4.0 * self.T
+
+    def step_work(self):  # backward: 3 H read, 2 H written
+        return 16.0 * self.T * self.H + 12.0 * self.T
+
+    def dominant(self):
+        with torch.no_grad():
+            return self.turbo.ops.swiglu_with_probs(self.x, self.p)
+
+    def step(self):
+        self.x.grad = None
+        self.p.grad = None
+        y = self.turbo.ops.swiglu_with_probs(self.x, self.p)
+        y.backward(self.go)
+        return y
+
+    def check(self):
+        from oracle import activation as A
+
+        y = self.dominant().float().cpu().numpy()[:256]
+        ref = A.glu_with_probs(self.x_cpu[:256].float().numpy(), self.p_cpu[:256].numpy(), "silu")
+        ok = bool(np.all(np.abs(y - ref) <= 1.01 * 2.0 ** -8 * np.abs(ref) + 1e-6 * np.abs(ref).max()))
+        return ok, "256 rows within one bf16 rounding of the float64 formula"
+
+    def cpu_baseline(self):
+        def fn():
+            a, b = self.x_cpu[:4096].float().chunk(2, dim=-1)
+            (torch.nn.functional.silu(a) * b * self.p_cpu[:4096, None]).to(torch.bfloat16)
+
+        return self._cpu(fn, self.dominant_work() * 4096 / self.T, "forward of the first 4096 tokens in PyTorch")
+
+
 def register(workloads):
+    workloads["swiglu_with_probs"] = SwigluWithProbs
     workloads["quant_rowwise"] = QuantRowwise
     workloads["quant_blockwise"] = lambda dev: QuantBlockwise(dev, False)
     workloads["quant_blockwise_dual"] = lambda dev: QuantBlockwise(dev, True)

@@ -439,6 +439,24 @@ PT_API int pt_grouped_gemm_mx_variable_k(const void *lhs, int lhs_dtype, const v
                                          int64_t Nr, int64_t ld, int accumulate, int tile_cfg,
                                          void *stream);
 
+/* Gated activation of an MoE expert MLP with the router probability folded in -------------
+ *
+ * Replaces swiglu_fwd_with_probs / swiglu_bwd_with_probs and geglu_fwd_with_probs /
+ * geglu_bwd_with_probs (primus_turbo/pytorch/kernels/activation/swiglu_impl.py:20-117,
+ * geglu_impl.py; Triton kernels primus_turbo/triton/activation/swiglu_kernel.py:11-248):
+ *   out[t, c]     = act(x[t, c]) * x[t, H + c] * probs[t]                      x [rows, 2 H]
+ *   grad_x[t, c]     = grad_out[t, c] * probs[t] * x[t, H + c] * act'(x[t, c])
+ *   grad_x[t, H + c] = grad_out[t, c] * probs[t] * act(x[t, c])
+ *   grad_probs[t]    = sum_c grad_out[t, c] * act(x[t, c]) * x[t, H + c]
+ * act: 0 = SiLU, 1 = exact (erf) GELU; x / out / grad in bf16 or fp16, probs and grad_probs fp32,
+ * arithmetic in fp32. row_mask (device int64 [rows], may be NULL): rows with 0 produce zeros. */
+PT_API int pt_glu_with_probs_fwd(const void *x, int x_dtype, const float *probs,
+                                 const int64_t *row_mask, void *out, int64_t rows, int64_t H, int act,
+                                 void *stream);
+PT_API int pt_glu_with_probs_bwd(const void *grad_out, const void *x, int x_dtype, const float *probs,
+                                 const int64_t *row_mask, void *grad_x, float *grad_probs,
+                                 int64_t rows, int64_t H, int act, void *stream);
+
 /* Byte-matrix transpose out[b, c, r] = in[b, r, c] (fp8 payloads; replaces the 2-D
  * transpose used for tensorwise `.t()` copies, csrc/kernels/transpose/). */
 PT_API int pt_transpose_u8(const void *in, void *out, int64_t batch, int64_t R, int64_t C,

@@ -97,6 +97,11 @@ _SIGNATURES = {
         [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_i64, c_i64, c_i64, c_int, c_int,
          c_int, c_i64, c_i64, c_i64, c_i64, c_int, c_int, c_int, c_void_p, c_size_t, c_int, c_void_p],
     ),
+    "pt_glu_with_probs_fwd": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_int, c_void_p]),
+    "pt_glu_with_probs_bwd": (
+        c_int,
+        [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_int, c_void_p],
+    ),
     "pt_transpose_u8": (c_int, [c_void_p, c_void_p, c_i64, c_i64, c_i64, c_void_p]),
     "pt_gemm_mx_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_i64, c_i64, c_int]),
     "pt_gemm_mx": (
