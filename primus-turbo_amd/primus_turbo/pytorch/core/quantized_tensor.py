@@ -51,6 +51,7 @@ def _is_fp4(dtype) -> bool:
     return float4_e2m1fn_x2 is not None and dtype == float4_e2m1fn_x2
 
 
+@torch.library.custom_op("primus_turbo::transpose_last_two", mutates_args=())
 def transpose_last_two(t: torch.Tensor) -> torch.Tensor:
     """Physical transpose of the last two dimensions of a contiguous 1-byte tensor (fp8 codes)."""
     assert t.element_size() == 1 and t.is_contiguous() and t.dim() in (2, 3)
@@ -59,6 +60,11 @@ def transpose_last_two(t: torch.Tensor) -> torch.Tensor:
     out = torch.empty(t.shape[:-2] + (C, R), dtype=t.dtype, device=t.device)
     N.check(N.lib().pt_transpose_u8(N.ptr(t), N.ptr(out), batch, R, C, N.stream_of(t)))
     return out
+
+
+@transpose_last_two.register_fake
+def _transpose_last_two_fake(t):
+    return torch.empty(tuple(t.shape[:-2]) + (t.shape[-1], t.shape[-2]), dtype=t.dtype, device=t.device)
 
 
 class QuantizedTensor(torch.Tensor):

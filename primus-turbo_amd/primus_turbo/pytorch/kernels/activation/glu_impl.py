@@ -30,6 +30,7 @@ def _common(x, probs, row_mask):
     return x.contiguous(), probs.contiguous().view(-1), row_mask
 
 
+@torch.library.custom_op("primus_turbo::glu_fwd_with_probs", mutates_args=())
 def glu_fwd_with_probs(x: torch.Tensor, probs: torch.Tensor, row_mask: Optional[torch.Tensor], act: int) -> torch.Tensor:
     """``out[t] = act(x[t, :H]) * x[t, H:] * probs[t]``; rows with ``row_mask == 0`` come out as zeros."""
     x, probs, row_mask = _common(x, probs, row_mask)
@@ -40,6 +41,12 @@ def glu_fwd_with_probs(x: torch.Tensor, probs: torch.Tensor, row_mask: Optional[
     return out
 
 
+@glu_fwd_with_probs.register_fake
+def _glu_fwd_with_probs_fake(x, probs, row_mask, act):
+    return torch.empty((x.shape[0], x.shape[1] // 2), dtype=x.dtype, device=x.device)
+
+
+@torch.library.custom_op("primus_turbo::glu_bwd_with_probs", mutates_args=())
 def glu_bwd_with_probs(grad_out: torch.Tensor, x: torch.Tensor, probs: torch.Tensor, row_mask: Optional[torch.Tensor],
                        act: int) -> Tuple[torch.Tensor, torch.Tensor]:
     """-> ``(grad_x [tokens, 2 H], grad_probs`` shaped like ``probs)``."""
@@ -53,6 +60,12 @@ def glu_bwd_with_probs(grad_out: torch.Tensor, x: torch.Tensor, probs: torch.Ten
     N.check(N.lib().pt_glu_with_probs_bwd(N.ptr(grad_out), N.ptr(x), N.dtype_code(x.dtype), N.ptr(probs), N.ptr(row_mask),
                                           N.ptr(grad_x), N.ptr(grad_probs), T, H, act, N.stream_of(x)))
     return grad_x, grad_probs.view(shape)
+
+
+@glu_bwd_with_probs.register_fake
+def _glu_bwd_with_probs_fake(grad_out, x, probs, row_mask, act):
+    return torch.empty(x.shape, dtype=x.dtype, device=x.device), torch.empty(probs.shape, dtype=torch.float32,
+                                                                              device=x.device)
 
 
 def swiglu_fwd_with_probs(x, probs, row_mask=None):

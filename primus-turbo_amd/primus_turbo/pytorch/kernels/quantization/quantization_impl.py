@@ -748,9 +748,33 @@ def _mx_check_axis(x, axis, with_trans):
         assert x.ndim in (2, 3), f"The input tensor must be 2D or 3D but got {x.ndim}D."
 
 
+def _mx_shapes(x, out_dtype, want_row, want_col):
+    fp4 = _FP4X2 is not None and out_dtype == _FP4X2
+    lead = tuple(x.shape[:-2])
+    M, Nn = x.shape[-2], x.shape[-1]
+    Mp, Np = -(-M // _MX_PAD) * _MX_PAD, -(-Nn // _MX_PAD) * _MX_PAD
+    pack = 2 if fp4 else 1
+    none = (0,)
+    return (lead + (M, Np // pack) if want_row else none, lead + (M, Np // 32) if want_row else none,
+            lead + (Nn, Mp // pack) if want_col else none, lead + (Nn, Mp // 32) if want_col else none)
+
+
 def _mx_quantize(x: torch.Tensor, out_dtype: torch.dtype, want_row: bool, want_col: bool, row_flags: int, col_flags: int):
     """-> (row_q, row_scale, col_q, col_scale); the pair of an unwanted direction is None.
     ``row_flags`` / ``col_flags``: see ``_mx_flags``."""
+    rq, rs, cq, cs = _quantize_mx_op(x, out_dtype, want_row, want_col, int(row_flags), int(col_flags))
+    if not want_row:
+        rq = rs = None
+    if not want_col:
+        cq = cs = None
+    return rq, rs, cq, cs
+
+
+@torch.library.custom_op("primus_turbo::quantize_mx", mutates_args=())
+def _quantize_mx_op(x: torch.Tensor, out_dtype: torch.dtype, want_row: bool, want_col: bool, row_flags: int,
+                    col_flags: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """The four outputs of ``_mx_quantize`` with an empty tensor for an unwanted direction (an
+    operator returns tensors, not ``None``)."""
     N.require_cuda(x)
     if x.dtype not in (torch.bfloat16, torch.float16):
         raise RuntimeError("Input must be BFloat16 or Half")
@@ -782,8 +806,16 @@ def _mx_quantize(x: torch.Tensor, out_dtype: torch.dtype, want_row: bool, want_c
             _next_sr_seed(row_flags if want_row else 0, col_flags if want_col else 0), N.stream_of(x),
         )
     )
-    view = lambda t, dt: None if t is None else t.view(dt)  # noqa: E731
+    empty = lambda: torch.empty(0, dtype=torch.uint8, device=dev)  # noqa: E731
+    view = lambda t, dt: (empty() if t is None else t).view(dt)  # noqa: E731
     return view(row_q, out_dtype), view(row_s, _E8M0), view(col_q, out_dtype), view(col_s, _E8M0)
+
+
+@_quantize_mx_op.register_fake
+def _quantize_mx_op_fake(x, out_dtype, want_row, want_col, row_flags, col_flags):
+    shapes = _mx_shapes(x, out_dtype, want_row, want_col)
+    mk = lambda shp, dt: torch.empty(shp, dtype=torch.uint8, device=x.device).view(dt)  # noqa: E731
+    return mk(shapes[0], out_dtype), mk(shapes[1], _E8M0), mk(shapes[2], out_dtype), mk(shapes[3], _E8M0)
 
 
 def _quantize_mx_impl(x, out_dtype, axis, block_size, with_trans, scaling_recipe, scaling_recipe_for_trans, what):
@@ -816,6 +848,26 @@ def quantize_mxfp4_impl(x, out_dtype, axis, block_size, with_trans=False, scalin
     return _quantize_mx_impl(x, out_dtype, axis, block_size, with_trans, scaling_recipe, scaling_recipe_for_trans, "MXFP4")
 
 
+@torch.library.custom_op("primus_turbo::dequantize_mx", mutates_args=())
+def _dequantize_mx_op(x: torch.Tensor, scale_inv: torch.Tensor, out_dtype: torch.dtype, rows: int, cols: int,
+                      rowwise: bool) -> torch.Tensor:
+    """``[rows, cols]`` codes with ``[rows, cols / 32]`` E8M0 scales -> ``[rows, cols]`` values, or
+    their transpose ``[cols, rows]`` when not ``rowwise``."""
+    out = torch.empty((rows, cols) if rowwise else (cols, rows), dtype=out_dtype, device=x.device)
+    N.check(
+        N.lib().pt_dequantize_mx(
+            N.ptr(x), N.dtype_code(x.dtype), N.ptr(scale_inv), rows, cols, N.ptr(out), N.dtype_code(out_dtype),
+            int(not rowwise), N.stream_of(x),
+        )
+    )
+    return out
+
+
+@_dequantize_mx_op.register_fake
+def _dequantize_mx_op_fake(x, scale_inv, out_dtype, rows, cols, rowwise):
+    return torch.empty((rows, cols) if rowwise else (cols, rows), dtype=out_dtype, device=x.device)
+
+
 def _dequantize_mx(x, out_dtype, axis, block_size, scale_inv, fp4):
     assert x.is_contiguous(), "The x tensor must be contiguous."
     assert x.dim() in (2, 3), "The x must be a 2D or 3D tensor."
@@ -833,13 +885,7 @@ def _dequantize_mx(x, out_dtype, axis, block_size, scale_inv, fp4):
     cols = x.shape[-1] * (2 if fp4 else 1)
     assert cols % block_size == 0, "The last dimension of the x tensor must be divisible by the block size."
     assert scale_inv.numel() == rows * (cols // 32), "scale_inv does not match x"
-    out = torch.empty((rows, cols) if rowwise else (cols, rows), dtype=out_dtype, device=x.device)
-    N.check(
-        N.lib().pt_dequantize_mx(
-            N.ptr(x), N.dtype_code(x.dtype), N.ptr(scale_inv), rows, cols, N.ptr(out), N.dtype_code(out_dtype),
-            int(not rowwise), N.stream_of(x),
-        )
-    )
+    out = _dequantize_mx_op(x, scale_inv, out_dtype, rows, cols, rowwise)
     if x.dim() == 3:
         if rowwise:
             return out.reshape(x.shape[0], x.shape[1], cols)
@@ -873,7 +919,36 @@ def _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, want_row: bool, w
                          col_flags: int = 0):
     """MXFP8: rows of every group padded to 32, transposed columns to 128. MXFP4: rows stay
     where they are in ``x`` (their "padded" lens / offs are the originals), transposed columns
-    padded to 256 per group."""
+    padded to 256 per group.
+    -> (row_q, row_scale, col_q, col_scale, lens_row, offs_row, lens_col, offs_col); the pair of an
+    unwanted direction is None."""
+    rq, rs, cq, cs, lr, orow, lc, ocol = _grouped_quantize_mx_op(x, out_dtype, group_lens, group_offs, want_row, want_col,
+                                                                 int(row_flags), int(col_flags))
+    if not want_row:
+        rq = rs = None
+    if not want_col:
+        cq = cs = None
+    if _FP4X2 is not None and out_dtype == _FP4X2:
+        lr, orow = group_lens, group_offs
+    return rq, rs, cq, cs, lr, orow, lc, ocol
+
+
+def _grouped_mx_dims(M, Nn, G, fp4):
+    ra = MXFP8_GROUP_M_PADDING_ALIGN_SIZE
+    ca = MXFP4_GROUP_K_DIM_PADDING_ALIGN_SIZE if fp4 else MXFP8_K_DIM_PADDING_ALIGN_SIZE
+    m_pad_row = M if fp4 else -(-(M + G * ra) // ra) * ra
+    m_pad_col = -(-(M + G * ca) // ca) * ca
+    n_pad = -(-Nn // _MX_PAD) * _MX_PAD
+    return ra, ca, m_pad_row, m_pad_col, n_pad
+
+
+@torch.library.custom_op("primus_turbo::grouped_quantize_mx", mutates_args=())
+def _grouped_quantize_mx_op(
+    x: torch.Tensor, out_dtype: torch.dtype, group_lens: torch.Tensor, group_offs: torch.Tensor, want_row: bool,
+    want_col: bool, row_flags: int, col_flags: int,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """The outputs of ``_grouped_mx_quantize`` with an empty tensor where that returns None, and
+    empty row lens / offs for MXFP4 (an operator may not hand its inputs back)."""
     N.require_cuda(x, group_lens, group_offs)
     if x.dtype not in (torch.bfloat16, torch.float16):
         raise RuntimeError("Input must be BFloat16 or Half")
@@ -888,12 +963,8 @@ def _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, want_row: bool, w
     M, Nn = x.shape
     _check(Nn % 32 == 0, f"N must be divisible by 32, got N={Nn}")
     G = group_lens.numel()
-    ra = MXFP8_GROUP_M_PADDING_ALIGN_SIZE
-    ca = MXFP4_GROUP_K_DIM_PADDING_ALIGN_SIZE if fp4 else MXFP8_K_DIM_PADDING_ALIGN_SIZE
     pack = 2 if fp4 else 1
-    m_pad_row = M if fp4 else -(-(M + G * ra) // ra) * ra
-    m_pad_col = -(-(M + G * ca) // ca) * ca
-    n_pad = -(-Nn // _MX_PAD) * _MX_PAD
+    ra, ca, m_pad_row, m_pad_col, n_pad = _grouped_mx_dims(M, Nn, G, fp4)
     dev = x.device
     group_offs = group_offs.contiguous()
     lens_row, offs_row = (group_lens, group_offs) if fp4 else _group_offs(group_lens, ra, True)
@@ -913,9 +984,28 @@ def _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, want_row: bool, w
             _next_sr_seed(row_flags if want_row else 0, col_flags if want_col else 0), N.stream_of(x),
         )
     )
-    view = lambda t, dt: None if t is None else t.view(dt)  # noqa: E731
+    empty = lambda dt=torch.uint8: torch.empty(0, dtype=dt, device=dev)  # noqa: E731
+    view = lambda t, dt: (empty() if t is None else t).view(dt)  # noqa: E731
+    if fp4:
+        lens_row, offs_row = empty(torch.int64), empty(torch.int64)
     return (view(row_q, out_dtype), view(row_s, _E8M0), view(col_q, out_dtype), view(col_s, _E8M0),
             lens_row, offs_row, lens_col, offs_col)
+
+
+@_grouped_quantize_mx_op.register_fake
+def _grouped_quantize_mx_op_fake(x, out_dtype, group_lens, group_offs, want_row, want_col, row_flags, col_flags):
+    fp4 = _FP4X2 is not None and out_dtype == _FP4X2
+    M, Nn = x.shape
+    G = group_lens.numel()
+    pack = 2 if fp4 else 1
+    _, _, m_pad_row, m_pad_col, n_pad = _grouped_mx_dims(M, Nn, G, fp4)
+    mk = lambda shp, dt: torch.empty(shp, dtype=torch.uint8, device=x.device).view(dt)  # noqa: E731
+    i64 = lambda n: torch.empty(n, dtype=torch.int64, device=x.device)  # noqa: E731
+    return (mk((m_pad_row, n_pad // pack) if want_row else (0,), out_dtype),
+            mk((m_pad_row, n_pad // 32) if want_row else (0,), _E8M0),
+            mk((Nn, m_pad_col // pack) if want_col else (0,), out_dtype),
+            mk((Nn, m_pad_col // 32) if want_col else (0,), _E8M0),
+            i64(0 if fp4 else G), i64(0 if fp4 else G + 1), i64(G), i64(G + 1))
 
 
 def grouped_quantize_mxfp8_impl(x, out_dtype, axis, block_size, group_lens, group_offs, with_trans=False,

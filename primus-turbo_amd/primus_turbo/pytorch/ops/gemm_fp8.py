@@ -31,13 +31,14 @@ from primus_turbo.pytorch.core.quantized_tensor import (
     QuantizedTensor,
     QuantizedTensorPair,
     check_quantized_tensor,
+    transpose_last_two,
 )
 from primus_turbo.pytorch.kernels.gemm.gemm_fp8_impl import gemm_fp8_accum_impl, gemm_fp8_impl
 from primus_turbo.pytorch.kernels.quantization.quantization_impl import (
     quant_fp8_blockwise_dual_t_impl,
     quant_fp8_blockwise_for_weight_dual_impl,
 )
-from primus_turbo.pytorch.ops.quantization import quantize_fp8, quantize_fp8_with_trans
+from primus_turbo.pytorch.ops.quantization import dequantize_fp8, quantize_fp8, quantize_fp8_with_trans
 from primus_turbo.pytorch.ops.utils import _get_dummy_wgrad, _get_fp8_dtype, _setup_fused_grad_accum
 
 __all__ = ["gemm_fp8"]
@@ -60,32 +61,35 @@ def _wgrad_gemm(a, a_s, trans_a, b, b_s, trans_b, out_dtype, trans_c, granularit
     return _get_dummy_wgrad(accumulate_into.shape, out_dtype)
 
 
-def _as_quantized(x, config, fwd: bool, axis, recipe=None) -> QuantizedTensor:
+def _quantized_parts(x, config, fwd: bool, axis):
+    """-> ``(codes, scale_inv, original dtype)`` of an operand: the fields of a ``QuantizedTensor``
+    that the caller quantized already, else a fresh quantization along ``axis``. Plain tensors, not
+    wrappers, so that ``torch.compile`` traces the functions below into one graph."""
     if isinstance(x, QuantizedTensor):
-        check_quantized_tensor(x, config, axis=axis, scaling_recipe=recipe)
-        return x
-    return QuantizedTensor.quantize(
-        x, _get_fp8_dtype(config.format, fwd), config.granularity, axis=axis, block_size=config.block_size,
-        scaling_recipe=recipe,
-    )
+        check_quantized_tensor(x, config, axis=axis)
+        return x.qdata, x.scale_inv, x.dtype
+    q, s = quantize_fp8(x.contiguous(), _get_fp8_dtype(config.format, fwd), config.granularity, axis=axis % x.ndim,
+                        block_size=config.block_size)
+    return q, s, x.dtype
 
 
 class FP8GemmTensorFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, a, b, a_t, b_t, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum_pattern=None):
         fuse, main_grad = _setup_fused_grad_accum(b, fuse_bgrad_accum_pattern)
-        qa = _as_quantized(a, config, True, -1)
-        qb = _as_quantized(b, config, True, -1)
-        out = _gemm(qa.qdata, qa.scale_inv, trans_a, qb.qdata, qb.scale_inv, trans_b, out_dtype, False, config.granularity)
+        qa, qa_s, _ = _quantized_parts(a, config, True, -1)
+        qb, qb_s, _ = _quantized_parts(b, config, True, -1)
+        out = _gemm(qa, qa_s, trans_a, qb, qb_s, trans_b, out_dtype, False, config.granularity)
         # NT forward: keep physically transposed fp8 copies so that both backward GEMMs
         # are NT as well (contiguous-K operands need no transposition pass inside the GEMM)
         nt_bwd = (not trans_a) and trans_b
         if nt_bwd:
-            qa_t = a_t if isinstance(a_t, QuantizedTensor) else qa.t()
-            qb_t = b_t if isinstance(b_t, QuantizedTensor) else qb.t()
-            ctx.save_for_backward(qa_t.qdata, qa_t.scale_inv, qb_t.qdata, qb_t.scale_inv)
+            # a tensorwise transpose moves the codes and shares the scalar scale
+            sa, sa_s = (a_t.qdata, a_t.scale_inv) if isinstance(a_t, QuantizedTensor) else (transpose_last_two(qa), qa_s)
+            sb, sb_s = (b_t.qdata, b_t.scale_inv) if isinstance(b_t, QuantizedTensor) else (transpose_last_two(qb), qb_s)
+            ctx.save_for_backward(sa, sa_s, sb, sb_s)
         else:
-            ctx.save_for_backward(qa.qdata, qa.scale_inv, qb.qdata, qb.scale_inv)
+            ctx.save_for_backward(qa, qa_s, qb, qb_s)
         ctx.meta = (trans_a, trans_b, out_dtype, config, nt_bwd, fuse, main_grad)
         return out
 
@@ -93,17 +97,16 @@ class FP8GemmTensorFunction(torch.autograd.Function):
     def backward(ctx, grad_out):
         trans_a, trans_b, out_dtype, config, nt_bwd, fuse, main_grad = ctx.meta
         sa, sa_s, sb, sb_s = ctx.saved_tensors
-        g = QuantizedTensor.quantize(grad_out.contiguous(), _get_fp8_dtype(config.format, False), config.granularity, axis=-1)
         gran = config.granularity
+        g, g_s = quantize_fp8(grad_out.contiguous(), _get_fp8_dtype(config.format, False), gran)
         acc = main_grad if fuse else None
         if nt_bwd:
             # saved: A^T [K, M], B^T [K, N]
-            grad_a = _gemm(g.qdata, g.scale_inv, False, sb, sb_s, True, out_dtype, False, gran)
-            g_t = g.t()
-            grad_b = _wgrad_gemm(sa, sa_s, False, g_t.qdata, g_t.scale_inv, True, out_dtype, trans_b, gran, acc)
+            grad_a = _gemm(g, g_s, False, sb, sb_s, True, out_dtype, False, gran)
+            grad_b = _wgrad_gemm(sa, sa_s, False, transpose_last_two(g), g_s, True, out_dtype, trans_b, gran, acc)
         else:
-            grad_a = _gemm(g.qdata, g.scale_inv, False, sb, sb_s, not trans_b, out_dtype, trans_a, gran)
-            grad_b = _wgrad_gemm(sa, sa_s, not trans_a, g.qdata, g.scale_inv, False, out_dtype, trans_b, gran, acc)
+            grad_a = _gemm(g, g_s, False, sb, sb_s, not trans_b, out_dtype, trans_a, gran)
+            grad_b = _wgrad_gemm(sa, sa_s, not trans_a, g, g_s, False, out_dtype, trans_b, gran, acc)
         return grad_a, grad_b, None, None, None, None, None, None, None
 
 
@@ -111,24 +114,27 @@ class FP8GemmRowFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, a, b, a_t, b_t, trans_a, trans_b, out_dtype, config):
         assert trans_a == False, "trans_a has to be False"  # noqa: E712
+        gran = config.granularity
         b_axis = -1 if trans_b else -2
-        qa = _as_quantized(a, config, True, -1)
-        qb = _as_quantized(b, config, True, b_axis)
+        qa, qa_s, a_hp = _quantized_parts(a, config, True, -1)
+        qb, qb_s, b_hp = _quantized_parts(b, config, True, b_axis)
 
-        def other_axis(q: QuantizedTensor, given, axis):
+        def other_axis(q, q_s, hp_dtype, from_axis, given, axis):
+            # the operand as backward reads it: what the forward codes stand for, quantized again
+            # along the other axis
             if given is not None:
                 assert isinstance(given, QuantizedTensor)
-                return given
-            return QuantizedTensor.quantize(q.dequantize(), q.real_dtype, config.granularity, axis=axis,
-                                            block_size=config.block_size)
+                return given.qdata, given.scale_inv
+            hp = dequantize_fp8(q, hp_dtype, gran, axis=from_axis % q.ndim, scale_inv=q_s, block_size=config.block_size)
+            return quantize_fp8(hp, q.dtype, gran, axis=axis % q.ndim, block_size=config.block_size)
 
-        out = _gemm(qa.qdata, qa.scale_inv, trans_a, qb.qdata, qb.scale_inv, trans_b, out_dtype, False, config.granularity)
+        out = _gemm(qa, qa_s, trans_a, qb, qb_s, trans_b, out_dtype, False, gran)
         # the operands quantized along their other axis only feed backward: skip them when no
         # input asks for a gradient (same outputs, two quantizer passes less)
         if any(ctx.needs_input_grad[:2]):
-            qa_t = other_axis(qa, a_t, -2)
-            qb_t = other_axis(qb, b_t, -2 if trans_b else -1)
-            ctx.save_for_backward(qa_t.qdata, qa_t.scale_inv, qb_t.qdata, qb_t.scale_inv)
+            a_c, a_cs = other_axis(qa, qa_s, a_hp, -1, a_t, -2)
+            b_c, b_cs = other_axis(qb, qb_s, b_hp, b_axis, b_t, -2 if trans_b else -1)
+            ctx.save_for_backward(a_c, a_cs, b_c, b_cs)
         ctx.meta = (trans_a, trans_b, out_dtype, config)
         return out
 
@@ -139,10 +145,10 @@ class FP8GemmRowFunction(torch.autograd.Function):
         grad_out = grad_out.contiguous()
         gdt = _get_fp8_dtype(config.format, False)
         gran = config.granularity
-        g_row = QuantizedTensor.quantize(grad_out, gdt, gran, axis=-1, block_size=config.block_size)
-        grad_a = _gemm(g_row.qdata, g_row.scale_inv, False, b_c, b_cs, not trans_b, out_dtype, trans_a, gran)
-        g_col = QuantizedTensor.quantize(grad_out, gdt, gran, axis=-2, block_size=config.block_size)
-        grad_b = _gemm(a_c, a_cs, not trans_a, g_col.qdata, g_col.scale_inv, False, out_dtype, trans_b, gran)
+        g_row, g_row_s = quantize_fp8(grad_out, gdt, gran, axis=1, block_size=config.block_size)
+        grad_a = _gemm(g_row, g_row_s, False, b_c, b_cs, not trans_b, out_dtype, trans_a, gran)
+        g_col, g_col_s = quantize_fp8(grad_out, gdt, gran, axis=0, block_size=config.block_size)
+        grad_b = _gemm(a_c, a_cs, not trans_a, g_col, g_col_s, False, out_dtype, trans_b, gran)
         return grad_a, grad_b, None, None, None, None, None, None
 
 

@@ -161,7 +161,6 @@ class FP4GroupedGemmMXFunc(torch.autograd.Function):
         return grad_a, grad_b, None, None, None, None, None, None, None, None, None
 
 
-@torch._dynamo.disable(recursive=True, reason="packed FP4 / E8M0 tensors inside an autograd.Function")
 def grouped_gemm_fp4(
     a: Union[torch.Tensor, QuantizedTensor, QuantizedTensorPair],
     b: Union[torch.Tensor, QuantizedTensor, QuantizedTensorPair],

@@ -47,6 +47,7 @@ from primus_turbo.pytorch.kernels.quantization.quantization_impl import (
     quant_fp8_blockwise_segment_m_row_col_t_impl,
     quantize_mxfp8_impl,
 )
+from primus_turbo.pytorch.ops.quantization import dequantize_fp8, quantize_fp8
 from primus_turbo.pytorch.ops.utils import (
     _ensure_contiguous_grad_out,
     _get_dummy_wgrad,
@@ -153,14 +154,16 @@ class FP8GroupedGemmBlockFunc(torch.autograd.Function):
         return grad_a, grad_b, None, None, None, None, None, None, None, None, None
 
 
-def _quantize_plain(x, config, fwd: bool, axis: int) -> QuantizedTensor:
-    """TENSORWISE / ROWWISE quantization treats the packed rows of all groups as one tensor
-    (reference: core/quantized_tensor.py:309-325)."""
+def _quantize_plain(x, config, fwd: bool, axis: int):
+    """-> ``(codes, scale_inv, original dtype)``. TENSORWISE / ROWWISE quantization treats the
+    packed rows of all groups as one tensor (reference: core/quantized_tensor.py:309-325). Plain
+    tensors rather than wrappers, so that ``torch.compile`` traces the functions below into one graph."""
     if isinstance(x, QuantizedTensor):
         check_quantized_tensor(x, config, axis=None if config.granularity == ScalingGranularity.TENSORWISE else axis)
-        return x
-    return QuantizedTensor.quantize(x.contiguous(), _get_fp8_dtype(config.format, fwd), config.granularity, axis=axis,
-                                    block_size=config.block_size)
+        return x.qdata, x.scale_inv, x.dtype
+    q, s = quantize_fp8(x.contiguous(), _get_fp8_dtype(config.format, fwd), config.granularity, axis=axis % x.ndim,
+                        block_size=config.block_size)
+    return q, s, x.dtype
 
 
 class FP8GroupedGemmRowFunc(torch.autograd.Function):
@@ -174,21 +177,23 @@ class FP8GroupedGemmRowFunc(torch.autograd.Function):
         fuse_bgrad_accum, main_grad = _setup_fused_grad_accum(b, fuse_bgrad_accum_pattern)
         assert config.granularity == ScalingGranularity.ROWWISE
         b_row_axis, b_col_axis = (-1, -2) if trans_b else (-2, -1)
-        qa = _quantize_plain(a, config, True, -1)
-        qb = _quantize_plain(b, config, True, b_row_axis)
+        qa, qa_s, a_hp = _quantize_plain(a, config, True, -1)
+        qb, qb_s, b_hp = _quantize_plain(b, config, True, b_row_axis)
         gran = config.granularity.value
-        out = grouped_gemm_fp8_impl(qa.qdata, qb.qdata, qa.scale_inv, qb.scale_inv, group_lens, group_offs, False, trans_b,
-                                    out_dtype, gran, num_cu, _NATIVE)
+        out = grouped_gemm_fp8_impl(qa, qb, qa_s, qb_s, group_lens, group_offs, False, trans_b, out_dtype, gran, num_cu,
+                                    _NATIVE)
         if any(ctx.needs_input_grad[:2]):
-            def other_axis(q, given, axis):
+            def other_axis(q, q_s, hp_dtype, from_axis, given, axis):
                 if given is not None:
                     assert isinstance(given, QuantizedTensor)
-                    return given
-                return QuantizedTensor.quantize(q.dequantize(), q.real_dtype, config.granularity, axis=axis,
-                                                block_size=config.block_size)
+                    return given.qdata, given.scale_inv
+                hp = dequantize_fp8(q, hp_dtype, config.granularity, axis=from_axis % q.ndim, scale_inv=q_s,
+                                    block_size=config.block_size)
+                return quantize_fp8(hp, q.dtype, config.granularity, axis=axis % q.ndim, block_size=config.block_size)
 
-            qa_t, qb_t = other_axis(qa, a_t, -2), other_axis(qb, b_t, b_col_axis)
-            ctx.save_for_backward(qa_t.qdata, qb_t.qdata, qa_t.scale_inv, qb_t.scale_inv, group_lens, group_offs)
+            a_col, a_col_s = other_axis(qa, qa_s, a_hp, -1, a_t, -2)
+            b_col, b_col_s = other_axis(qb, qb_s, b_hp, b_row_axis, b_t, b_col_axis)
+            ctx.save_for_backward(a_col, b_col, a_col_s, b_col_s, group_lens, group_offs)
         ctx.meta = (trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad)
         return out
 
@@ -198,12 +203,12 @@ class FP8GroupedGemmRowFunc(torch.autograd.Function):
         a_col, b_col, a_col_s, b_col_s, group_lens, group_offs = ctx.saved_tensors
         trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad = ctx.meta
         gran = config.granularity.value
-        g_row = _quantize_plain(grad_out, config, False, -1)
-        grad_a = grouped_gemm_fp8_impl(g_row.qdata, b_col, g_row.scale_inv, b_col_s, group_lens, group_offs, False,
-                                       not trans_b, out_dtype, gran, num_cu, _NATIVE)
-        g_col = _quantize_plain(grad_out, config, False, -2)
+        g_row, g_row_s, _ = _quantize_plain(grad_out, config, False, -1)
+        grad_a = grouped_gemm_fp8_impl(g_row, b_col, g_row_s, b_col_s, group_lens, group_offs, False, not trans_b,
+                                       out_dtype, gran, num_cu, _NATIVE)
+        g_col, g_col_s, _ = _quantize_plain(grad_out, config, False, -2)
         grad_b = _grouped_gemm_fp8_variable_k_impl_wrapper(
-            a_col, g_col.qdata, a_col_s, g_col.scale_inv, group_lens, group_offs, True, False, trans_b, out_dtype, gran,
+            a_col, g_col, a_col_s, g_col_s, group_lens, group_offs, True, False, trans_b, out_dtype, gran,
             num_cu, _NATIVE, inplace_add_to_out=fuse_bgrad_accum, out=main_grad,
         )
         return grad_a, grad_b, None, None, None, None, None, None, None, None, None
@@ -218,12 +223,12 @@ class FP8GroupedGemmTensorFunc(torch.autograd.Function):
                 fuse_bgrad_accum_pattern=None):
         fuse_bgrad_accum, main_grad = _setup_fused_grad_accum(b, fuse_bgrad_accum_pattern)
         assert config.granularity == ScalingGranularity.TENSORWISE
-        qa = _quantize_plain(a, config, True, -1)
-        qb = _quantize_plain(b, config, True, -1)
-        out = grouped_gemm_fp8_impl(qa.qdata, qb.qdata, qa.scale_inv, qb.scale_inv, group_lens, group_offs, False, trans_b,
-                                    out_dtype, config.granularity.value, num_cu, _NATIVE)
+        qa, qa_s, _ = _quantize_plain(a, config, True, -1)
+        qb, qb_s, _ = _quantize_plain(b, config, True, -1)
+        out = grouped_gemm_fp8_impl(qa, qb, qa_s, qb_s, group_lens, group_offs, False, trans_b, out_dtype,
+                                    config.granularity.value, num_cu, _NATIVE)
         if any(ctx.needs_input_grad[:2]):
-            ctx.save_for_backward(qa.qdata, qb.qdata, qa.scale_inv, qb.scale_inv, group_lens, group_offs)
+            ctx.save_for_backward(qa, qb, qa_s, qb_s, group_lens, group_offs)
         ctx.meta = (trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad)
         return out
 
@@ -233,11 +238,11 @@ class FP8GroupedGemmTensorFunc(torch.autograd.Function):
         a_q, b_q, a_s, b_s, group_lens, group_offs = ctx.saved_tensors
         trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad = ctx.meta
         gran = config.granularity.value
-        g = _quantize_plain(grad_out, config, False, -1)
-        grad_a = grouped_gemm_fp8_impl(g.qdata, b_q, g.scale_inv, b_s, group_lens, group_offs, False, not trans_b,
-                                       out_dtype, gran, num_cu, _NATIVE)
+        g, g_s, _ = _quantize_plain(grad_out, config, False, -1)
+        grad_a = grouped_gemm_fp8_impl(g, b_q, g_s, b_s, group_lens, group_offs, False, not trans_b, out_dtype, gran,
+                                       num_cu, _NATIVE)
         grad_b = _grouped_gemm_fp8_variable_k_impl_wrapper(
-            a_q, g.qdata, a_s, g.scale_inv, group_lens, group_offs, True, False, trans_b, out_dtype, gran, num_cu, _NATIVE,
+            a_q, g, a_s, g_s, group_lens, group_offs, True, False, trans_b, out_dtype, gran, num_cu, _NATIVE,
             inplace_add_to_out=fuse_bgrad_accum, out=main_grad,
         )
         return grad_a, grad_b, None, None, None, None, None, None, None, None, None
