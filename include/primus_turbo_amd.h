@@ -462,6 +462,23 @@ PT_API int pt_glu_with_probs_bwd(const void *grad_out, const void *x, int x_dtyp
 PT_API int pt_transpose_u8(const void *in, void *out, int64_t batch, int64_t R, int64_t C,
                            void *stream);
 
+/* Pre-shuffled MX operand layouts (the (16, 16) tile orders that the reference hands to AITER's
+ * a4w4 GEMM). Replaces shuffle_weight / shuffle_e8m0_scale (csrc/include/primus_turbo/shuffle.h:26-32,
+ * csrc/kernels/shuffle/shuffle.cu:32-160; index maps csrc/include/primus_turbo/device/shuffle.cuh:39-80)
+ * and the shuffle_out / shuffle_scale outputs of the MX quantizers
+ * (csrc/pytorch/quantization/quantization.cpp:553-603). `inverse` != 0 brings a shuffled tensor back
+ * to the plain row-major layout (no counterpart in the reference, whose GEMMs read the shuffled one).
+ *
+ * pt_shuffle_mx_codes: [rows, row_bytes] code bytes (FP4 pairs or FP8), rows % 16 == 0,
+ *   row_bytes % 32 == 0; every 16-row x 32-byte tile is stored as two contiguous 16 x 16-byte halves.
+ * pt_shuffle_e8m0_scale: `batch` matrices [M, N] of E8M0 bytes <-> [M_pad, N_pad] (M_pad % 32 == 0,
+ *   N_pad % 8 == 0, the reference pads M to 256 and N to 8), zero outside [M, N]; every 32 x 8 tile is
+ *   stored in the order (col % 4, row % 16, (col % 8) / 4, (row % 32) / 16). */
+PT_API int pt_shuffle_mx_codes(const void *in, void *out, int64_t rows, int64_t row_bytes, int inverse,
+                               void *stream);
+PT_API int pt_shuffle_e8m0_scale(const void *in, void *out, int64_t batch, int64_t M, int64_t N,
+                                 int64_t M_pad, int64_t N_pad, int inverse, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -700,14 +700,186 @@ _E8M0 = getattr(torch, "float8_e8m0fnu", torch.uint8)
 _FP4X2 = getattr(torch, "float4_e2m1fn_x2", None)
 
 
+# ---------------------------------------------------------------------------
+# Pre-shuffled MX layouts: shuffle_scale(Tensor scale, int[] layout) -> Tensor and
+# shuffle_weight(Tensor weight, int[] layout) -> Tensor of the reference
+# (csrc/pytorch/bindings_pytorch.cpp, csrc/pytorch/shuffle/shuffle.cpp:15-83), their inverses, and the
+# quantizers' shuffle_scale / shuffle_out outputs (csrc/pytorch/quantization/quantization.cpp:553-603).
+# ---------------------------------------------------------------------------
+_SHUFFLE_ROWS, _SHUFFLE_SCALE_M_ALIGN, _SHUFFLE_SCALE_N_ALIGN = 16, 256, 8
+
+
+def _check_layout(layout):
+    _check(len(layout) == 2, "layout must have exactly 2 elements")
+    _check(tuple(layout) == (16, 16), "Unsupported shuffle layout.")
+
+
+def _scale_pad(M: int, Nn: int) -> Tuple[int, int]:
+    a, b = _SHUFFLE_SCALE_M_ALIGN, _SHUFFLE_SCALE_N_ALIGN
+    return -(-M // a) * a, -(-Nn // b) * b
+
+
+def _shuffle_scale_launch(scale: torch.Tensor, batch: int, M: int, Nn: int) -> torch.Tensor:
+    """``batch`` stacked ``[M, Nn]`` E8M0 matrices -> ``[batch * M_pad, N_pad]`` shuffled."""
+    Mp, Np = _scale_pad(M, Nn)
+    out = torch.empty((batch * Mp, Np), dtype=torch.uint8, device=scale.device)
+    N.check(N.lib().pt_shuffle_e8m0_scale(N.ptr(scale), N.ptr(out), batch, M, Nn, Mp, Np, 0, N.stream_of(scale)))
+    return out.view(_E8M0)
+
+
+_ext.define("shuffle_scale(Tensor scale, int[] layout) -> Tensor")
+
+
+def _shuffle_scale(scale: torch.Tensor, layout: List[int]) -> torch.Tensor:
+    N.require_cuda(scale)
+    _check(scale.dtype == _E8M0, "Scale must be Float8_e8m0fnu.")
+    _check(scale.dim() == 2, "Scale must be 2D")
+    _check_layout(layout)
+    return _shuffle_scale_launch(scale.contiguous(), 1, scale.shape[0], scale.shape[1])
+
+
+def _shuffle_scale_meta(scale, layout):
+    Mp, Np = _scale_pad(scale.shape[0], scale.shape[1])
+    return torch.empty((Mp, Np), dtype=torch.uint8, device=scale.device).view(_E8M0)
+
+
+_ext.impl("shuffle_scale", _shuffle_scale, "CUDA")
+_ext.impl("shuffle_scale", _shuffle_scale, "CPU")  # raises: no CPU path
+_ext.impl("shuffle_scale", _shuffle_scale_meta, "Meta")
+
+_ext.define("unshuffle_scale(Tensor shuffled, int M, int N) -> Tensor")
+
+
+def _unshuffle_scale(shuffled: torch.Tensor, M: int, Nn: int) -> torch.Tensor:
+    """Inverse of ``shuffle_scale``: the plain ``[M, N]`` scales of a shuffled ``[M_pad, N_pad]`` tensor
+    (no counterpart in the reference, whose GEMM backends read the shuffled form)."""
+    N.require_cuda(shuffled)
+    _check(shuffled.dtype == _E8M0 and shuffled.dim() == 2, "shuffled scale must be a 2-D Float8_e8m0fnu tensor")
+    _check(tuple(shuffled.shape) == _scale_pad(M, Nn), f"shuffled scale of [{M}, {Nn}] must be {_scale_pad(M, Nn)}")
+    shuffled = shuffled.contiguous()
+    out = torch.empty((M, Nn), dtype=torch.uint8, device=shuffled.device)
+    N.check(N.lib().pt_shuffle_e8m0_scale(N.ptr(shuffled), N.ptr(out), 1, M, Nn, shuffled.shape[0], shuffled.shape[1], 1,
+                                          N.stream_of(shuffled)))
+    return out.view(_E8M0)
+
+
+_ext.impl("unshuffle_scale", _unshuffle_scale, "CUDA")
+_ext.impl("unshuffle_scale", _unshuffle_scale, "CPU")
+_ext.impl("unshuffle_scale", lambda s, M, Nn: torch.empty((M, Nn), dtype=torch.uint8, device=s.device).view(_E8M0), "Meta")
+
+
+def _shuffle_codes_launch(codes: torch.Tensor, inverse: bool) -> torch.Tensor:
+    rows, row_bytes = codes.numel() // codes.shape[-1], codes.shape[-1] * codes.element_size()
+    out = torch.empty_like(codes)
+    N.check(N.lib().pt_shuffle_mx_codes(N.ptr(codes), N.ptr(out), rows, row_bytes, int(inverse), N.stream_of(codes)))
+    return out
+
+
+def _check_weight(weight, layout):
+    N.require_cuda(weight)
+    _check(_FP4X2 is not None and weight.dtype == _FP4X2, "Weight must be Float4_e2m1fn_x2.")
+    _check(weight.dim() == 2, "Weight must be 2D")
+    _check(weight.is_contiguous(), "Weight must be contiguous")
+    M, Nn = weight.shape
+    _check(M % 16 == 0, f"M must be divisible by 16 for shuffled FP4. But got M={M}")
+    _check(Nn % 32 == 0, f"N must be divisible by 32 for shuffled FP4. But got N={Nn}")
+    _check_layout(layout)
+
+
+_ext.define("shuffle_weight(Tensor weight, int[] layout) -> Tensor")
+_ext.define("unshuffle_weight(Tensor shuffled, int[] layout) -> Tensor")
+
+
+def _shuffle_weight(weight: torch.Tensor, layout: List[int]) -> torch.Tensor:
+    _check_weight(weight, layout)
+    return _shuffle_codes_launch(weight, False)
+
+
+def _unshuffle_weight(shuffled: torch.Tensor, layout: List[int]) -> torch.Tensor:
+    """Inverse of ``shuffle_weight`` (no counterpart in the reference)."""
+    _check_weight(shuffled, layout)
+    return _shuffle_codes_launch(shuffled, True)
+
+
+for _name, _fn in (("shuffle_weight", _shuffle_weight), ("unshuffle_weight", _unshuffle_weight)):
+    _ext.impl(_name, _fn, "CUDA")
+    _ext.impl(_name, _fn, "CPU")
+    _ext.impl(_name, lambda w, layout: torch.empty_like(w), "Meta")
+
+
+def _apply_mx_shuffles(q, s, recipe, direction: str):
+    """The ``shuffle_out`` / ``shuffle_scale`` forms of one direction's outputs ``q [.., R, W]`` /
+    ``s [.., R, W / 32]``: a pass over the plain outputs of the quantizer. Batched scales are shuffled
+    per matrix, each padded on its own (quantization.cpp:563-603)."""
+    if q is None:
+        return q, s
+    if recipe.shuffle_out:
+        R = q.shape[-2]
+        what = "M" if direction == "rowwise" else "N"
+        _check(R % _SHUFFLE_ROWS == 0,
+               f"{what} must be divisible by {_SHUFFLE_ROWS} for shuffled {direction} output. But got {what}={R}")
+        q = torch.ops.primus_turbo_cpp_extension.shuffle_mx_codes(q)
+    if recipe.shuffle_scale:
+        s = torch.ops.primus_turbo_cpp_extension.shuffle_scale_batched(s)
+    return q, s
+
+
+_ext.define("shuffle_mx_codes(Tensor codes) -> Tensor")
+_ext.define("shuffle_scale_batched(Tensor scale) -> Tensor")
+
+
+def _shuffle_mx_codes(codes: torch.Tensor) -> torch.Tensor:
+    N.require_cuda(codes)
+    return _shuffle_codes_launch(codes.contiguous(), False)
+
+
+def _shuffle_scale_batched(scale: torch.Tensor) -> torch.Tensor:
+    N.require_cuda(scale)
+    batch = scale.shape[0] if scale.dim() == 3 else 1
+    out = _shuffle_scale_launch(scale.contiguous(), batch, scale.shape[-2], scale.shape[-1])
+    return out.view(batch, -1, out.shape[-1]) if scale.dim() == 3 else out
+
+
+def _shuffle_scale_batched_meta(scale):
+    Mp, Np = _scale_pad(scale.shape[-2], scale.shape[-1])
+    return torch.empty(tuple(scale.shape[:-2]) + (Mp, Np), dtype=torch.uint8, device=scale.device).view(_E8M0)
+
+
+_ext.impl("shuffle_mx_codes", _shuffle_mx_codes, "CUDA")
+_ext.impl("shuffle_mx_codes", lambda c: torch.empty_like(c), "Meta")
+_ext.impl("shuffle_scale_batched", _shuffle_scale_batched, "CUDA")
+_ext.impl("shuffle_scale_batched", _shuffle_scale_batched_meta, "Meta")
+
+
+def mx_plain_layout(q: torch.Tensor, scale: torch.Tensor, shuffled_out: bool, shuffled_scale: bool):
+    """``(codes, scales)`` of a 2-D MX operand in the plain row-major layout that the GEMM and
+    de-quantization kernels read, from outputs produced with ``shuffle_out`` / ``shuffle_scale``."""
+    if shuffled_out:
+        q = _shuffle_codes_op(q, True)
+    if shuffled_scale:
+        cols = q.shape[-1] * (2 if (_FP4X2 is not None and q.dtype == _FP4X2) else 1) // 32
+        scale = torch.ops.primus_turbo_cpp_extension.unshuffle_scale(scale, q.shape[-2], cols)
+    return q, scale
+
+
+@torch.library.custom_op("primus_turbo::shuffle_mx_codes_impl", mutates_args=())
+def _shuffle_codes_op(codes: torch.Tensor, inverse: bool) -> torch.Tensor:
+    N.require_cuda(codes)
+    _check(codes.dim() in (2, 3), "codes must be 2-D or 3-D")
+    return _shuffle_codes_launch(codes.contiguous(), inverse)
+
+
+@_shuffle_codes_op.register_fake
+def _shuffle_codes_op_fake(codes, inverse):
+    return torch.empty_like(codes)
+
+
 def _mx_recipes(with_trans, scaling_recipe, scaling_recipe_for_trans, what):
     from primus_turbo.pytorch.core.low_precision import ScalingRecipe
 
     r = ScalingRecipe() if scaling_recipe is None else scaling_recipe
     rt = (ScalingRecipe() if scaling_recipe_for_trans is None else scaling_recipe_for_trans) if with_trans else r
     for rec in (r, rt):
-        if rec.shuffle_scale or rec.shuffle_out:
-            raise NotImplementedError(f"{what}: shuffled layouts are not implemented (plain layouts are)")
         if (rec.use_rht or rec.use_sr) and what != "MXFP4":
             raise NotImplementedError(f"{what}: the Hadamard transform and stochastic rounding belong to the MXFP4 recipe")
         if rec.use_rht and rec.use_2d_block:
@@ -823,10 +995,11 @@ def _quantize_mx_impl(x, out_dtype, axis, block_size, with_trans, scaling_recipe
     r, rt = _mx_recipes(with_trans, scaling_recipe, scaling_recipe_for_trans, what)
     _mx_check_axis(x, axis, with_trans)
     if with_trans:
-        return _mx_quantize(x, out_dtype, True, True, _mx_flags(r), _mx_flags(rt))
+        rq, rs, cq, cs = _mx_quantize(x, out_dtype, True, True, _mx_flags(r), _mx_flags(rt))
+        return _apply_mx_shuffles(rq, rs, r, "rowwise") + _apply_mx_shuffles(cq, cs, rt, "colwise")
     rowwise = axis == x.ndim - 1
     rq, rs, cq, cs = _mx_quantize(x, out_dtype, rowwise, not rowwise, _mx_flags(r), _mx_flags(r))
-    return (rq, rs) if rowwise else (cq, cs)
+    return _apply_mx_shuffles(rq, rs, r, "rowwise") if rowwise else _apply_mx_shuffles(cq, cs, r, "colwise")
 
 
 def quantize_mxfp8_impl(x, out_dtype, axis, block_size, with_trans=False, scaling_recipe=None,

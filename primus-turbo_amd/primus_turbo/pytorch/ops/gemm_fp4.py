@@ -7,8 +7,10 @@ directions from one read. As in the reference's recipe (its lines 108-160, 220-2
 operands -- the column-direction quantizations of ``a`` and of ``grad_out`` -- carry the fixed
 16-point Hadamard transform along the token axis, which cancels in their product and spreads
 outliers over 16 values before they are quantized; ``use_gradient_sr`` rounds both quantizations of
-``grad_out`` stochastically. Pre-shuffled layouts do not exist here (``use_preshuffle=True``
-raises).
+``grad_out`` stochastically. ``use_preshuffle`` selects, in the reference, the shuffled operand
+layouts of AITER's kernel; the kernel here reads plain layouts, so the flag only decides which
+layout pre-quantized operands are expected in (they are brought back to the plain one on entry)
+and leaves the result unchanged.
 """
 
 from __future__ import annotations
@@ -30,7 +32,7 @@ from primus_turbo.pytorch.core.quantized_tensor import (
     check_quantized_tensor,
 )
 from primus_turbo.pytorch.kernels.gemm.gemm_fp4_impl import gemm_fp4_accum_impl, gemm_fp4_impl
-from primus_turbo.pytorch.kernels.quantization.quantization_impl import quantize_mxfp4_impl
+from primus_turbo.pytorch.kernels.quantization.quantization_impl import mx_plain_layout, quantize_mxfp4_impl
 from primus_turbo.pytorch.ops.quantization import quantize_fp4_with_trans
 from primus_turbo.pytorch.ops.utils import _get_dummy_wgrad, _setup_fused_grad_accum
 
@@ -59,8 +61,7 @@ class FP4GemmMXFunction(torch.autograd.Function):
     def forward(ctx, a, b, a_t, b_t, trans_a, trans_b, out_dtype, config, fuse_bgrad_accum_pattern=None):
         ok, why = check_mxfp4_support()
         assert ok, why
-        if config.use_preshuffle:
-            raise NotImplementedError("Float4QuantConfig.use_preshuffle is not implemented")
+        pre = config.use_preshuffle
         fuse, main_grad = _setup_fused_grad_accum(b, fuse_bgrad_accum_pattern)
         dt = FP4GemmMXFunction.get_fp4_dtype(config.format)
         gran, bs = config.granularity, config.block_size
@@ -68,6 +69,8 @@ class FP4GemmMXFunction(torch.autograd.Function):
         need_bwd = any(ctx.needs_input_grad[:2])
 
         def both_ways(x, x_t, recipe, recipe_t):
+            """Row- and column-direction quantizations in the plain layout. ``recipe`` / ``recipe_t`` are
+            what a pre-quantized operand must carry (the reference's recipes, shuffle flags included)."""
             if isinstance(x, QuantizedTensor):
                 check_quantized_tensor(x, config, scaling_recipe=recipe)
                 if x_t is None:
@@ -75,7 +78,11 @@ class FP4GemmMXFunction(torch.autograd.Function):
                                                    scaling_recipe=recipe_t)
                 else:
                     check_quantized_tensor(x_t, config, scaling_recipe=recipe_t)
-                return x.qdata, x.scale_inv, x_t.qdata, x_t.scale_inv
+                q, sc = mx_plain_layout(x.qdata, x.scale_inv, recipe.shuffle_out, recipe.shuffle_scale)
+                q_t, sc_t = mx_plain_layout(x_t.qdata, x_t.scale_inv, recipe_t.shuffle_out, recipe_t.shuffle_scale)
+                return q, sc, q_t, sc_t
+            recipe = recipe._replace(shuffle_out=False, shuffle_scale=False)
+            recipe_t = recipe_t._replace(shuffle_out=False, shuffle_scale=False)
             if not need_bwd:
                 # the transposed copies only feed backward: skip them when nothing asks for a gradient
                 q, sc = quantize_mxfp4_impl(x, dt, x.dim() - 1, bs, scaling_recipe=recipe)
@@ -83,8 +90,10 @@ class FP4GemmMXFunction(torch.autograd.Function):
             return quantize_fp4_with_trans(x, dt, gran, block_size=bs, scaling_recipe=recipe,
                                            scaling_recipe_for_trans=recipe_t)
 
-        w_recipe = ScalingRecipe(use_2d_block=True)
-        a_row, a_row_s, a_col, a_col_s = both_ways(a, a_t, ScalingRecipe(), ScalingRecipe(use_rht=True))
+        # reference lines 112-160: the second operand of each product is the one held pre-shuffled
+        w_recipe = ScalingRecipe(use_2d_block=True, shuffle_scale=pre, shuffle_out=pre)
+        a_row, a_row_s, a_col, a_col_s = both_ways(a, a_t, ScalingRecipe(shuffle_scale=pre),
+                                                   ScalingRecipe(use_rht=True, shuffle_scale=pre, shuffle_out=pre))
         b_row, b_row_s, b_col, b_col_s = both_ways(b, b_t, w_recipe, w_recipe)
         out = gemm_fp4_impl(a_row, a_row_s, False, b_row, b_row_s, True, out_dtype, False, gran.value, _NATIVE)
         ctx.save_for_backward(a_col, a_col_s, b_col, b_col_s)

@@ -10,7 +10,7 @@ Activations and gradients use 1 x 32 blocks and are quantized in both directions
 blocks. As in the reference the two wgrad operands (the column-direction quantizations of ``a`` and
 ``grad_out``) carry the recipe's fixed 16-point Hadamard transform along the token axis, which
 cancels in their product; ``use_gradient_sr`` rounds both quantizations of ``grad_out``
-stochastically. Pre-shuffled layouts are not implemented.
+stochastically. ``use_preshuffle`` must be off, as in the reference.
 """
 
 from __future__ import annotations
@@ -81,8 +81,8 @@ class FP4GroupedGemmMXFunc(torch.autograd.Function):
         assert a.ndim == 2 and b.ndim == 3
         assert out_dtype in (torch.float16, torch.bfloat16)
         assert trans_b, "MXFP4 grouped GEMM only supports trans_b=True (NT layout)."
-        if config.use_preshuffle:
-            raise NotImplementedError("Float4QuantConfig.use_preshuffle is not implemented")
+        # as the reference (its line 126): the grouped product has no pre-shuffled form
+        assert not config.use_preshuffle, "MXFP4 grouped GEMM does not use preshuffle."
         supported, reason = check_mxfp4_support()
         assert supported, reason
         N, K = int(b.shape[-2]), int(b.shape[-1])

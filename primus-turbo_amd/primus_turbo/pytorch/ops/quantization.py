@@ -123,6 +123,9 @@ def dequantize_fp8(
         return _impl.dequant_fp8_blockwise_impl(x, scale_inv, out_dtype, axis, block_size)
     if granularity == _G.MX_BLOCKWISE:
         _need_mx_block(block_size, MXFP8_BLOCK_SIZE, "MXFP8")
+        if scaling_recipe is not None and (scaling_recipe.shuffle_out or scaling_recipe.shuffle_scale):
+            assert x.dim() == 2, "shuffled layouts are de-quantized as 2-D tensors"
+            x, scale_inv = _impl.mx_plain_layout(x, scale_inv, scaling_recipe.shuffle_out, scaling_recipe.shuffle_scale)
         return _impl.dequantize_mxfp8_impl(x, out_dtype, axis, block_size, scale_inv)
     raise _unknown(granularity)
 
@@ -183,6 +186,9 @@ def dequantize_fp4(
 ) -> torch.Tensor:
     if granularity == _G.MX_BLOCKWISE:
         _need_mx_block(block_size, MXFP4_BLOCK_SIZE, "MXFP4")
+        if scaling_recipe is not None and (scaling_recipe.shuffle_out or scaling_recipe.shuffle_scale):
+            assert x.dim() == 2, "shuffled layouts are de-quantized as 2-D tensors"
+            x, scale_inv = _impl.mx_plain_layout(x, scale_inv, scaling_recipe.shuffle_out, scaling_recipe.shuffle_scale)
         return _impl.dequantize_mxfp4_impl(x, out_dtype, axis, block_size, scale_inv)
     raise _unknown(granularity)
 
@@ -258,5 +264,8 @@ def grouped_dequantize_fp4(x, out_dtype, granularity, *, block_size=None, axis=N
     (reference: ops/quantization.py:519-537)."""
     if granularity == _G.MX_BLOCKWISE:
         _need_mx_block(block_size, MXFP4_BLOCK_SIZE, "MXFP4")
+        if scaling_recipe is not None and (scaling_recipe.shuffle_out or scaling_recipe.shuffle_scale):
+            assert x.dim() == 2, "shuffled layouts are de-quantized as 2-D tensors"
+            x, scale_inv = _impl.mx_plain_layout(x, scale_inv, scaling_recipe.shuffle_out, scaling_recipe.shuffle_scale)
         return _impl.dequantize_mxfp4_impl(x, out_dtype, axis, block_size, scale_inv)
     raise _unknown(granularity)

@@ -177,8 +177,8 @@ def test_mx_hadamard_recipe_limits():
         qi.quantize_mxfp4_impl(x, FP4, 1, 32, scaling_recipe=ScalingRecipe(use_rht=True, use_2d_block=True))
     with pytest.raises(NotImplementedError):  # MXFP8 has no stochastic rounding either
         qi.quantize_mxfp8_impl(x, torch.float8_e4m3fn, 1, 32, scaling_recipe=ScalingRecipe(use_sr=True))
-    with pytest.raises(NotImplementedError):  # shuffled layouts do not exist here
-        qi.quantize_mxfp4_impl(x, FP4, 1, 32, scaling_recipe=ScalingRecipe(shuffle_out=True))
+    with pytest.raises(RuntimeError, match="divisible by 16"):  # shuffled codes come in bands of 16 rows
+        qi.quantize_mxfp4_impl(x[:120].contiguous(), FP4, 1, 32, scaling_recipe=ScalingRecipe(shuffle_out=True))
 
 
 @pytest.mark.skipif(FP4 is None, reason="torch has no float4_e2m1fn_x2")
