@@ -345,6 +345,7 @@ class SwigluWithProbs(_QuantBase):
     32768 routed tokens, fc1 output 2 x 2048 -> 2048, forward + backward."""
 
     name = "swiglu_with_probs_32768tokens_hidden2048_bf16 (forward + backward)"
+    metric = "gated activation GB/s (algorithmic bytes) & fraction of HBM peak"
     dominant_name = "glu_fwd_kernel<bf16, SiLU> (one workgroup per token row, 16-byte accesses)"
     dtype = "bf16 (fp32 arithmetic)"
 
