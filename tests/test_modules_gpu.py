@@ -132,3 +132,53 @@ def test_moe_expert_mlp_composition(kind):
     for name, g, w, slack in zip(("out", "dx", "dw1", "dw2"), got, want, (0, 3, 3, 0)):
         snr = OG.snr_db(w, g)
         assert snr > gate - slack, f"{kind} {name}: SNR {snr:.1f} dB"
+
+
+@pytest.mark.parametrize("kind", ["tensorwise", "rowwise", "blockwise", "mxfp8", "mxfp4"])
+@pytest.mark.parametrize("B,M,N,K", [(4, 256, 1024, 2048), (8, 512, 512, 1024)])
+@pytest.mark.parametrize("balance", [True, False])
+@pytest.mark.parametrize("compiled", [False, True])
+def test_grouped_linear(kind, B, M, N, K, balance, compiled):
+    """``GroupedLinear`` against one bf16 ``x_g @ W_g^T`` per group: the shapes of the reference's
+    tests/pytorch/modules/test_grouped_linear.py:19-60 (B groups of M tokens on average, balanced or
+    not, with and without ``torch.compile(fullgraph=True)``), at the SNR gates of the grouped GEMM
+    tests (25 dB FP8, 8 dB MXFP4) since the module multiplies in low precision."""
+    import numpy as np
+
+    from helpers import group_lens
+    from primus_turbo.pytorch.core.low_precision import Float4QuantConfig, ScaleDtype
+    from primus_turbo.pytorch.modules import GroupedLinear
+
+    if kind == "mxfp4":
+        cfg, gate = Float4QuantConfig(), 8.0
+    else:
+        kw = {"tensorwise": dict(granularity=G.TENSORWISE), "rowwise": dict(granularity=G.ROWWISE),
+              "blockwise": dict(granularity=G.BLOCKWISE, block_size=128),
+              "mxfp8": dict(granularity=G.MX_BLOCKWISE, block_size=32, scale_dtype=ScaleDtype.E8M0)}[kind]
+        cfg, gate = Float8QuantConfig(format=Format.E4M3, **kw), 25.0
+    torch.manual_seed(3)
+    torch._dynamo.reset()
+    lens = group_lens("balanced" if balance else "ragged", B, B * M, 5)
+    gl = torch.from_numpy(lens).cuda()
+    mod = GroupedLinear(B, K, N, "cuda", dtype=torch.bfloat16, config=cfg)
+    assert tuple(mod.weight.shape) == (B, N, K) and f"group_num={B}" in repr(mod)
+    fn = torch.compile(mod, fullgraph=True) if compiled else mod
+    x1 = torch.randn((B * M, K), device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    x2 = x1.detach().clone().requires_grad_()
+    w2 = mod.weight.detach().clone().requires_grad_()
+    out1 = fn(x1, gl)
+    offs = np.concatenate([[0], np.cumsum(lens)])
+    out2 = torch.cat([x2[offs[g]:offs[g + 1]] @ w2[g].t() for g in range(B)], dim=0)
+    assert out1.shape == out2.shape and out1.dtype == torch.bfloat16
+    go = torch.randn_like(out1)
+    out1.backward(go)
+    out2.backward(go)
+    for name, got, want in (("out", out1, out2), ("dx", x1.grad, x2.grad), ("dw", mod.weight.grad, w2.grad)):
+        assert _snr(want, got) > gate, f"{kind} {name}: SNR {_snr(want, got):.1f} dB"
+
+
+def test_grouped_linear_needs_a_config():
+    from primus_turbo.pytorch.modules import GroupedLinear
+
+    with pytest.raises(NotImplementedError, match="Float8QuantConfig"):
+        GroupedLinear(4, 128, 128, "cuda", dtype=torch.bfloat16)

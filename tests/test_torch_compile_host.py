@@ -96,3 +96,16 @@ def test_gated_activation_traces_fullgraph(turbo, kind):
     x, p = _meta(300, 512), _meta(300, 1, dtype=torch.float32)
     out = _trace(lambda x, p: fn(x, p, None), x, p)
     assert out.shape == (300, 256) and x.grad.shape == x.shape and p.grad.shape == p.shape
+
+
+@pytest.mark.parametrize("gran", GRANS + ["mxfp4"])
+def test_grouped_linear_traces_fullgraph(turbo, gran):
+    from primus_turbo.pytorch.core.low_precision import Float4QuantConfig
+    from primus_turbo.pytorch.modules import GroupedLinear
+
+    cfg = Float4QuantConfig() if gran == "mxfp4" else _cfg(gran)
+    mod = GroupedLinear(4, 512, 512, "meta", dtype=torch.bfloat16, config=cfg)
+    x = _meta(1024, 512)
+    lens = torch.empty(4, device="meta", dtype=torch.int64)
+    out = _trace(mod, x, lens)
+    assert out.shape == (1024, 512) and x.grad.shape == x.shape and mod.weight.grad.shape == (4, 512, 512)
