@@ -393,7 +393,75 @@ class SwigluWithProbs(_QuantBase):
         return self._cpu(fn, self.dominant_work() * 4096 / self.T, "forward of the first 4096 tokens in PyTorch")
 
 
+class MoePermute(_QuantBase):
+    """MoE permute + unpermute around the expert bank of the MoE configuration: 4096 tokens with
+    top-8 routing over 32 local experts (32768 routed rows), hidden 7168, bf16, rows padded per
+    expert to 128. Dominant kernel: the permute copy (reads every token once, writes its 8 rows)."""
+
+    name = "moe_permute_unpermute_4096tokens_top8_32experts_hidden7168_bf16 (pad 128)"
+    metric = "MoE permute GB/s (algorithmic bytes) & fraction of HBM peak"
+    dominant_name = "moe_permute_kernel (one workgroup per token row, 16-byte accesses, streaming stores)"
+    dtype = "bf16 (byte copy; fp32 sum in unpermute)"
+
+    def __init__(self, dev, tokens=4096, experts=32, topk=8, hidden=7168, pad=128):
+        import primus_turbo.pytorch as turbo
+
+        self.turbo, self.T, self.E, self.K, self.H, self.pad = turbo, tokens, experts, topk, hidden, pad
+        rng = np.random.default_rng(41)
+        self.topk_cpu = np.stack([rng.choice(experts, topk, replace=False) for _ in range(tokens)]).astype(np.int64)
+        self.x_cpu = _randn_bf16((tokens, hidden), 42, 1.0)
+        self.x = self.x_cpu.to(dev)
+        self.topk = torch.from_numpy(self.topk_cpu).to(dev)
+        self.ext = torch.ops.primus_turbo_cpp_extension
+        pre = self.ext.permute_preprocessing(self.topk, experts, topk, pad, -1, 0)
+        self.rmap, self.tpe, _, self.nd = pre
+        self.rows = int(self.tpe.sum().item())
+        self.out = torch.empty((self.rows, hidden), dtype=torch.bfloat16, device=dev)
+        self.back = torch.empty((tokens, hidden), dtype=torch.bfloat16, device=dev)
+
+    def dominant_work(self):  # every token read once, every permuted row (zero rows included) written once
+        return 2.0 * self.H * (self.T + self.rows)
+
+    def step_work(self):  # + the row map pass and the unpermute (reads the routed rows, writes the tokens)
+        return 2.0 * self.dominant_work() + 8.0 * self.T * self.K
+
+    def dominant(self):
+        self.ext.permute(self.x, self.out, None, None, None, None, self.rmap, self.nd, self.pad, self.E, self.H, 0,
+                         False, False, self.rows, 0)
+        return self.out
+
+    def step(self):
+        pre = self.ext.permute_preprocessing(self.topk, self.E, self.K, self.pad, self.rows, 0)
+        self.ext.permute(self.x, self.out, None, None, None, None, pre[0], pre[3], self.pad, self.E, self.H, 0, False,
+                         False, self.rows, 0)
+        self.ext.unpermute(self.out, self.back, None, None, pre[0], pre[3], self.E, self.H, False, 0)
+        return self.back
+
+    def check(self):
+        from oracle import moe_permute as P
+
+        rmap, tpe, _, _ = P.preprocess(self.topk_cpu, self.E, self.pad)
+        ok = np.array_equal(self.rmap.cpu().numpy(), rmap) and np.array_equal(self.tpe.cpu().numpy(), tpe)
+        want, _, _, written = P.permute(self.x_cpu.view(torch.int16).numpy(), rmap, self.E, self.rows, self.pad)
+        ok = ok and bool(written.all()) and np.array_equal(self.dominant().view(torch.int16).cpu().numpy(), want)
+        back = self.step()
+        ok = ok and torch.equal(back.cpu(), (self.x_cpu.float() * self.K).to(torch.bfloat16))
+        return bool(ok), "row map, tokens_per_expert and all permuted rows bit-exact vs oracle; unpermute = top-k x tokens"
+
+    def cpu_baseline(self):
+        from oracle import moe_permute as P
+
+        x = self.x_cpu.view(torch.int16).numpy()
+        rmap, _, _, _ = P.preprocess(self.topk_cpu, self.E, self.pad)
+
+        def fn():
+            P.permute(x, rmap, self.E, self.rows, self.pad)
+
+        return self._cpu(fn, self.dominant_work(), "numpy oracle permute of the full workload (row map precomputed)")
+
+
 def register(workloads):
+    workloads["moe_permute"] = MoePermute
     workloads["swiglu_with_probs"] = SwigluWithProbs
     workloads["quant_rowwise"] = QuantRowwise
     workloads["quant_blockwise"] = lambda dev: QuantBlockwise(dev, False)

@@ -479,6 +479,47 @@ PT_API int pt_shuffle_mx_codes(const void *in, void *out, int64_t rows, int64_t 
 PT_API int pt_shuffle_e8m0_scale(const void *in, void *out, int64_t batch, int64_t M, int64_t N,
                                  int64_t M_pad, int64_t N_pad, int inverse, void *stream);
 
+/* MoE token permute / unpermute (the step before and after the grouped GEMMs of an expert bank).
+ * Replaces permute_preprocessing_impl / permute_impl / unpermute_impl
+ * (csrc/include/primus_turbo/moe_permute.h, csrc/kernels/moe_permute/moe_permute.cu:84-330, :425-510,
+ * :553-745; schemas csrc/pytorch/bindings_pytorch.cpp:100-112).
+ *
+ * pt_moe_permute_preprocess: expert_map is bool [T, E] (map_kind 0) or topk_idx [T, num_topk] of
+ *   int32 / int64 (1 / 2; entries outside [0, E) are ignored). Writes row_id_map
+ *   [T + pad_multiple, 2 E + 1] (row of a token: [2E] = n routed experts, [0, n) = 1-based destination
+ *   rows in ascending expert order, [E, E + n) = expert id, or the top-k slot when
+ *   topk_aligned_probs; rows T + i: negative 1-based rows of the i-th zero pad row of every expert that
+ *   has one; other entries are left as they are), tokens_per_expert [E] (padded to pad_multiple,
+ *   clipped at num_permuted_tokens when that is > 0), overflow_flag (1 when rows were dropped for
+ *   that limit), num_dispatched_tokens (tokens routed to at least one local expert). E <= 240.
+ *   workspace: pt_moe_permute_workspace_bytes(T, E) bytes, contents irrelevant. Three launches, no host
+ *   synchronisation, no inter-block waiting.
+ * pt_moe_permute: copies token rows (hidden_bytes each, a multiple of 16) to their destination rows
+ *   and writes the zero pad rows; optional per-token scale factors (scale_bytes_per_token raw bytes)
+ *   and probs (prob_bytes 2 or 4; source row stride probs_stride elements, column from the map) ride
+ *   along. Rows of permuted_tokens that no map entry names are left untouched; map entries at or
+ *   beyond num_permuted_rows (the rows the permuted tensors hold) are skipped, also in pt_moe_unpermute.
+ * pt_moe_unpermute: tokens[t] = sum over the token's experts of permuted_tokens[row] (fp32
+ *   accumulation in map order, bf16 / fp16 storage; zeros for a token routed nowhere); optional probs
+ *   scattered back into zero-filled rows of probs_stride elements. */
+PT_API size_t pt_moe_permute_workspace_bytes(int64_t num_tokens, int64_t num_local_experts);
+PT_API int pt_moe_permute_preprocess(const void *expert_map, int map_kind, int64_t num_tokens,
+                                     int64_t num_local_experts, int64_t num_topk, int64_t pad_multiple,
+                                     int64_t num_permuted_tokens, int topk_aligned_probs, int *row_id_map,
+                                     int64_t *tokens_per_expert, int *overflow_flag,
+                                     int *num_dispatched_tokens, void *workspace, size_t workspace_bytes,
+                                     void *stream);
+PT_API int pt_moe_permute(const void *tokens, void *permuted_tokens, int64_t hidden_bytes,
+                          const void *scaling_factor, void *permuted_scaling_factor,
+                          int64_t scale_bytes_per_token, const void *probs, void *permuted_probs,
+                          int prob_bytes, int64_t probs_stride, const int *row_id_map, int64_t num_tokens,
+                          int64_t pad_multiple, int64_t num_local_experts, int64_t num_permuted_rows,
+                          void *stream);
+PT_API int pt_moe_unpermute(const void *permuted_tokens, void *tokens, int dtype, int64_t hidden,
+                            const void *permuted_probs, void *probs, int prob_bytes, int64_t probs_stride,
+                            const int *row_id_map, int64_t num_tokens, int64_t num_local_experts,
+                            int64_t num_permuted_rows, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

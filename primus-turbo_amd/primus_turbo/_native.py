@@ -103,6 +103,21 @@ _SIGNATURES = {
         [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_int, c_void_p],
     ),
     "pt_transpose_u8": (c_int, [c_void_p, c_void_p, c_i64, c_i64, c_i64, c_void_p]),
+    "pt_moe_permute_workspace_bytes": (c_size_t, [c_i64, c_i64]),
+    "pt_moe_permute_preprocess": (
+        c_int,
+        [c_void_p, c_int, c_i64, c_i64, c_i64, c_i64, c_i64, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_size_t, c_void_p],
+    ),
+    "pt_moe_permute": (
+        c_int,
+        [c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_int, c_i64, c_void_p, c_i64, c_i64,
+         c_i64, c_i64, c_void_p],
+    ),
+    "pt_moe_unpermute": (
+        c_int,
+        [c_void_p, c_void_p, c_int, c_i64, c_void_p, c_void_p, c_int, c_i64, c_void_p, c_i64, c_i64, c_i64, c_void_p],
+    ),
     "pt_shuffle_mx_codes": (c_int, [c_void_p, c_void_p, c_i64, c_i64, c_int, c_void_p]),
     "pt_shuffle_e8m0_scale": (c_int, [c_void_p, c_void_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_int, c_void_p]),
     "pt_gemm_mx_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_i64, c_i64, c_int]),
