@@ -243,17 +243,11 @@ def require_cuda(*tensors: torch.Tensor) -> None:
 
 
 # ---------------------------------------------------------------------------
-# Small persistent device workspaces (zero-filled once, left zeroed by the kernels).
-# One per (device, stream) so launches on different streams never share one.
+# Small zero-filled device workspace for one launch (the kernels leave it zeroed, but it is not
+# kept: a buffer that outlives the call would have to live outside the private memory pool of
+# whatever graph capture, or warm-up run for one, happens to be active -- torch.compile's CUDA-graph
+# trees insist that nothing allocated there stays alive -- and an op cannot tell. A fill kernel of
+# 256 bytes per call is the price; it is capturable and belongs to nobody afterwards).
 # ---------------------------------------------------------------------------
-_workspaces: dict = {}
-
-
 def zeroed_workspace(device: torch.device, nbytes: int, tag: str) -> torch.Tensor:
-    stream = torch.cuda.current_stream(device)
-    key = (tag, device.index if device.index is not None else torch.cuda.current_device(), stream.cuda_stream)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
-    return ws
+    return torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=device)

@@ -97,3 +97,23 @@ def test_gated_activation_compiled(kind):
     x = _rand(300, 512)
     p = torch.rand(300, 1, generator=torch.Generator().manual_seed(2)).cuda().requires_grad_(True)
     _same_as_eager(lambda x, p: fn(x, p, None), (x, p), True)
+
+
+@pytest.mark.parametrize("gran", GRANS)
+def test_float8_linear_max_autotune(gran):
+    """``mode="max-autotune"``, the setting of the reference's test: Inductor then runs the graph
+    through CUDA-graph trees (warm-up, capture, replays), so the ops must be capturable and must keep
+    nothing alive in the graph's memory pool. Fresh inputs on every call; each call equals eager."""
+    from primus_turbo.pytorch.modules import Float8Linear
+
+    torch._dynamo.reset()
+    torch.manual_seed(2)
+    lin = Float8Linear(512, 256, bias=True, config=_cfg(gran), device="cuda", dtype=torch.bfloat16)
+    compiled = torch.compile(lin, fullgraph=False, mode="max-autotune")
+    for it in range(4):
+        x = _rand(128, 512, seed=10 + it)
+        out_e, grads_e = _run(lin, (x,), list(lin.parameters()))
+        out_c, grads_c = _run(compiled, (x,), list(lin.parameters()))
+        assert torch.equal(out_e, out_c), f"call {it}: forward differs"
+        for e, c in zip(grads_e, grads_c):
+            assert torch.equal(e, c), f"call {it}: a gradient differs"
