@@ -182,3 +182,58 @@ def test_grouped_linear_needs_a_config():
 
     with pytest.raises(NotImplementedError, match="Float8QuantConfig"):
         GroupedLinear(4, 128, 128, "cuda", dtype=torch.bfloat16)
+
+
+@pytest.mark.parametrize("kind", ["rowwise", "blockwise", "mxfp8"])
+def test_moe_layer_permute_experts_unpermute(kind):
+    """A whole MoE expert layer on the path: ``moe_permute`` (top-k routing, groups padded to 32 rows)
+    -> grouped fc1 -> ``swiglu_with_probs`` -> grouped fc2 -> ``moe_unpermute``, forward and all
+    gradients, against the same layer computed token by token in fp32 from the bf16 values. The
+    permute's ``tokens_per_expert`` is the group-length tensor of the grouped GEMMs as it stands (no
+    host round trip). Gates as in the two-GEMM composition above (20 dB, 17 dB for gradients through
+    both products); the gradient of the router probabilities passes through one product: 20 dB."""
+    import primus_turbo.pytorch as turbo
+    from primus_turbo.pytorch.core.low_precision import ScaleDtype
+
+    T, E, K, H, F, pad = 512, 8, 2, 512, 768, 32
+    kw = {"blockwise": dict(granularity=G.BLOCKWISE, block_size=128), "rowwise": dict(granularity=G.ROWWISE),
+          "mxfp8": dict(granularity=G.MX_BLOCKWISE, block_size=32, scale_dtype=ScaleDtype.E8M0)}[kind]
+    cfg = Float8QuantConfig(format=Format.E4M3, **kw)
+    g = torch.Generator().manual_seed(77)
+    x0 = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    w1_0 = (torch.randn(E, 2 * F, H, generator=g) * H ** -0.5).to(torch.bfloat16)
+    w2_0 = (torch.randn(E, H, F, generator=g) * F ** -0.5).to(torch.bfloat16)
+    p0 = torch.rand(T, K, generator=g) + 0.25
+    topk = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)])
+    dy = torch.randn(T, H, generator=g).to(torch.bfloat16).cuda()
+
+    def leaves(dtype):
+        return [t.clone().to(dtype).cuda().requires_grad_(True) for t in (x0, w1_0, w2_0, p0)]
+
+    x, w1, w2, p = leaves(torch.bfloat16)
+    p = p0.clone().cuda().requires_grad_(True)
+    rows = T * K + E * pad  # an upper bound keeps the op free of a host read-back
+    px, rmap, tpe, overflow, nd, _, pp = turbo.ops.moe_permute(
+        x, topk.cuda(), num_local_experts=E, num_topk=K, pad_multiple=pad, num_permuted_tokens=rows, probs=p,
+        probs_layout="topk")
+    assert px.shape[0] == rows and int(overflow.item()) == 0
+    used = int(tpe.sum().item())
+    px, pp = px[:used], pp[:used]  # the rows the experts own; the tail of the bound is unused
+    h = turbo.ops.grouped_gemm_fp8(px, w1, tpe, trans_b=True, config=cfg)
+    a = turbo.ops.swiglu_with_probs(h, pp.unsqueeze(-1), None)
+    y = turbo.ops.grouped_gemm_fp8(a, w2, tpe, trans_b=True, config=cfg)
+    y = torch.cat([y, y.new_zeros(rows - used, H)])
+    out, _ = turbo.ops.moe_unpermute(y, rmap, nd, restore_shape=x.shape, num_local_experts=E, pad_multiple=pad)
+    out.backward(dy)
+
+    xr, w1r, w2r, pr = leaves(torch.float32)
+    ref = torch.zeros(T, H, device="cuda")
+    for k in range(K):
+        e = topk[:, k].cuda()
+        hk = torch.einsum("th,tfh->tf", xr, w1r[e])
+        ak = torch.nn.functional.silu(hk[:, :F]) * hk[:, F:] * pr[:, k:k + 1]
+        ref = ref + torch.einsum("tf,thf->th", ak, w2r[e])
+    ref.backward(dy.float())
+    for name, got, want, gate in (("out", out, ref, 20.0), ("dx", x.grad, xr.grad, 17.0), ("dw1", w1.grad, w1r.grad, 17.0),
+                                  ("dw2", w2.grad, w2r.grad, 20.0), ("dprobs", p.grad, pr.grad, 20.0)):
+        assert _snr(want, got) > gate, f"{kind} {name}: SNR {_snr(want, got):.1f} dB"
