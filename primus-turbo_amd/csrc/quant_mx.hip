@@ -306,16 +306,24 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
         uint32_t code[2][8];
         if constexpr (ROW)
             __syncthreads(); // the row pass's scale bytes have been read
+        // a thread owns two neighbouring columns of one 32-row block: one 32-bit LDS read per row
+        // serves both (task p: column c, numbered t = 128 rb + c as the seeds of stochastic rounding expect)
+        const int rb = tid >> 6, c0 = (tid & 63) * 2;
+        float     v2[2][32];
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const uint32_t w = *reinterpret_cast<const uint32_t *>(&tile[(rb * 32 + i) * MX_PITCH + c0]);
+            v2[0][i]         = elem(static_cast<uint16_t>(w & 0xffffu));
+            v2[1][i]         = elem(static_cast<uint16_t>(w >> 16));
+        }
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
-            const int t = tid + 256 * p, c = t & 127, rb = t >> 7;
-            float     v[32];
-            float     am = 0.f;
+            const int c = c0 + p, t = 128 * rb + c;
+            float (&v)[32] = v2[p];
+            float am = 0.f;
 #pragma unroll
-            for (int i = 0; i < 32; ++i) {
-                v[i] = elem(tile[(rb * 32 + i) * MX_PITCH + c]);
-                am   = fmaxf(am, abs_or_zero(v[i]));
-            }
+            for (int i = 0; i < 32; ++i)
+                am = fmaxf(am, abs_or_zero(v[i]));
             if constexpr ((RHT & 2) != 0) {
                 hadamard16(v, 0);
                 hadamard16(v, 16);
@@ -343,7 +351,7 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
         uint8_t *stage = reinterpret_cast<uint8_t *>(tile);
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
-            const int t = tid + 256 * p, c = t & 127, rb = t >> 7;
+            const int c = c0 + p;
             uint8_t  *d = stage + c * CPITCH + rb * CB;
             *reinterpret_cast<u32x4 *>(d) = u32x4{code[p][0], code[p][1], code[p][2], code[p][3]};
             if constexpr (FMT != MX_E2M1)
