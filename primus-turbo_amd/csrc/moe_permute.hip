@@ -147,6 +147,10 @@ __global__ __launch_bounds__(256) void moe_rowmap_kernel(const MapT *__restrict_
     int     *s_wcnt = reinterpret_cast<int *>(lds + TOK * E);
     const int64_t tok0 = blockIdx.x * static_cast<int64_t>(TOK);
     fill_flags(s_flag, map, tok0, T, E, K);
+    // first destination row of this block's tokens per expert, fetched once instead of per iteration
+    __shared__ int s_base[MAX_E];
+    for (int e = threadIdx.x; e < E; e += 256)
+        s_base[e] = counts_excl[blockIdx.x * static_cast<int64_t>(E + 1) + e] + pref[e];
     wave_counts(s_flag, s_wcnt, E);
     const int     t = threadIdx.x, w = t >> 6, lane = t & 63;
     const int64_t gt  = tok0 + t;
@@ -160,8 +164,7 @@ __global__ __launch_bounds__(256) void moe_rowmap_kernel(const MapT *__restrict_
         int before = __popcll(mask & ((1ull << lane) - 1ull));
         for (int w2 = 0; w2 < w; ++w2)
             before += s_wcnt[e * 4 + w2];
-        const int64_t dest = static_cast<int64_t>(counts_excl[blockIdx.x * static_cast<int64_t>(E + 1) + e]) + before + 1 +
-                             pref[e];
+        const int64_t dest = static_cast<int64_t>(s_base[e]) + before + 1;
         if (dest > npt)
             continue;
         int aux = e;
