@@ -120,7 +120,7 @@ class QuantTensorwise:
             lib = N.lib()
             out = torch.empty_like(self.x, dtype=torch.float8_e4m3fn)
             sinv = torch.empty((), dtype=torch.float32, device=self.x.device)
-            ws = N.zeroed_workspace(self.x.device, lib.pt_quantize_fp8_tensorwise_workspace_bytes(), "tw")
+            ws = N.zeroed_workspace(self.x.device, lib.pt_quantize_fp8_tensorwise_workspace_bytes())
             args = (N.ptr(self.x), N.dtype_code(self.x.dtype), self.x.numel(), N.ptr(out), N.dtype_code(out.dtype),
                     None, N.ptr(sinv), N.ptr(ws), ws.numel(), N.stream_of(self.x))
             self._dom = (lib.pt_quantize_fp8_tensorwise, args, out, sinv, ws)

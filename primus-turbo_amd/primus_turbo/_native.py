@@ -249,5 +249,5 @@ def require_cuda(*tensors: torch.Tensor) -> None:
 # trees insist that nothing allocated there stays alive -- and an op cannot tell. A fill kernel of
 # 256 bytes per call is the price; it is capturable and belongs to nobody afterwards).
 # ---------------------------------------------------------------------------
-def zeroed_workspace(device: torch.device, nbytes: int, tag: str) -> torch.Tensor:
+def zeroed_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     return torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=device)

@@ -68,7 +68,7 @@ def _quantize_fp8_tensorwise(input: torch.Tensor, dest_dtype: torch.dtype, scale
         _check(scale_opt.numel() == 1, "tensorwise scale must be scalar tensor")
         scale_in = scale_opt.to(torch.float32).contiguous()
     else:
-        ws = N.zeroed_workspace(input.device, lib.pt_quantize_fp8_tensorwise_workspace_bytes(), "tw")
+        ws = N.zeroed_workspace(input.device, lib.pt_quantize_fp8_tensorwise_workspace_bytes())
     N.check(
         lib.pt_quantize_fp8_tensorwise(
             N.ptr(input),
@@ -818,19 +818,13 @@ def _apply_mx_shuffles(q, s, recipe, direction: str):
         what = "M" if direction == "rowwise" else "N"
         _check(R % _SHUFFLE_ROWS == 0,
                f"{what} must be divisible by {_SHUFFLE_ROWS} for shuffled {direction} output. But got {what}={R}")
-        q = torch.ops.primus_turbo_cpp_extension.shuffle_mx_codes(q)
+        q = _shuffle_codes_op(q, False)
     if recipe.shuffle_scale:
         s = torch.ops.primus_turbo_cpp_extension.shuffle_scale_batched(s)
     return q, s
 
 
-_ext.define("shuffle_mx_codes(Tensor codes) -> Tensor")
 _ext.define("shuffle_scale_batched(Tensor scale) -> Tensor")
-
-
-def _shuffle_mx_codes(codes: torch.Tensor) -> torch.Tensor:
-    N.require_cuda(codes)
-    return _shuffle_codes_launch(codes.contiguous(), False)
 
 
 def _shuffle_scale_batched(scale: torch.Tensor) -> torch.Tensor:
@@ -845,8 +839,6 @@ def _shuffle_scale_batched_meta(scale):
     return torch.empty(tuple(scale.shape[:-2]) + (Mp, Np), dtype=torch.uint8, device=scale.device).view(_E8M0)
 
 
-_ext.impl("shuffle_mx_codes", _shuffle_mx_codes, "CUDA")
-_ext.impl("shuffle_mx_codes", lambda c: torch.empty_like(c), "Meta")
 _ext.impl("shuffle_scale_batched", _shuffle_scale_batched, "CUDA")
 _ext.impl("shuffle_scale_batched", _shuffle_scale_batched_meta, "Meta")
 
