@@ -193,3 +193,26 @@ def test_no_tokens_and_argument_checks():
         ext.permute_preprocessing(torch.zeros(4, 300, dtype=torch.bool, device="cuda"), 300, 2, 0, -1, 0)
     with pytest.raises(RuntimeError, match="bool or int or int64"):
         ext.permute_preprocessing(torch.zeros(4, E, dtype=torch.float32, device="cuda"), E, 2, 0, -1, 0)
+
+
+@pytest.mark.parametrize("layout", ["routing_map", "topk"])
+def test_half_precision_probs(layout):
+    """Probabilities are moved as raw 2-byte values too (bf16 routers)."""
+    T, E, K, H, pad = 333, 8, 2, 256, 4
+    flags = _routing(T, E, K, seed=51)
+    topk = _topk(flags, K, np.int64, 52)
+    emap = flags if layout == "routing_map" else topk
+    g = torch.Generator().manual_seed(53)
+    tokens = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    probs = torch.rand(T, E if layout == "routing_map" else K, generator=g).to(torch.bfloat16)
+    out, rmap_d, tpe_d, _, nd_d, _, out_p = turbo.ops.moe_permute(
+        tokens.cuda(), torch.from_numpy(emap).cuda(), num_local_experts=E, num_topk=K, pad_multiple=pad,
+        probs=probs.cuda(), probs_layout=layout)
+    rmap, tpe, _, _ = P.preprocess(emap, E, pad, topk_aligned_probs=layout == "topk")
+    _, _, want_p, _ = P.permute(_bits(tokens), rmap, E, int(tpe.sum()), pad, probs=_bits(probs))
+    assert out_p.dtype == torch.bfloat16 and np.array_equal(_bits(out_p), want_p)
+    stride = K if layout == "topk" else 0
+    _, back_p = turbo.ops.moe_unpermute(out, rmap_d, nd_d, restore_shape=tokens.shape, num_local_experts=E,
+                                        permuted_probs=out_p, probs_topk_stride=stride, pad_multiple=pad)
+    _, want_back = P.unpermute(np.zeros((int(tpe.sum()), 1), np.float32), rmap, E, T, want_p, stride if stride else E)
+    assert back_p.dtype == torch.bfloat16 and np.array_equal(_bits(back_p), want_back)
