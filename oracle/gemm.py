@@ -13,9 +13,10 @@ fp32 summation order and the final rounding to the output dtype:
 * grouped forward / variable-K
   (/root/reference/tests/pytorch/ref/gemm_ref.py:13-41)
 
-Pinned by: identity with a float64 block-by-block python evaluation on tiny shapes,
-transposition identities (NT vs NN vs TN of the same operands), and exact small-integer
-cases where fp32 accumulation is exact (tests/test_oracle_gemm.py).
+Pinned by (tests/test_oracle_gemm.py): float64 python-loop evaluation on tiny shapes in all
+four operand layouts, hand-computed values, exact small-integer cases where fp32 accumulation
+is exact, grouped cases with empty groups and rows past the last group, the adjoint identity
+between the grouped forward and the variable-K product, and hand values of the metrics.
 """
 
 from __future__ import annotations

@@ -309,9 +309,11 @@ def hadamard16(v: np.ndarray) -> np.ndarray:
     inside each run of four elements, an H4 butterfly across the four runs, times 0.25 -- i.e.
     (H4 (x) H4) / 4, the orthonormal Sylvester matrix of order 16. There are no random signs:
     the transform is its own inverse and cancels between two operands that both carry it.
-    Pinned against scipy's Sylvester matrix on inputs where fp32 is exact, and by the involution.
-    Bit-identity of the rounding order with the reference's HIP kernel is PARITY UNPINNED (its
-    source is absent); the FlyDSL text states that the two agree."""
+    Pinned against scipy's Sylvester matrix on inputs where fp32 is exact, by the involution, and
+    bit for bit against a one-operation-at-a-time evaluation of the FlyDSL text on data whose
+    rounding depends on the order (tests/test_oracle_gemm.py). Bit-identity of the rounding order
+    with the reference's HIP kernel is PARITY UNPINNED (its source is absent); the FlyDSL text
+    states that the two agree."""
     v = np.asarray(v, dtype=F32)
     g = v.reshape(v.shape[:-1] + (v.shape[-1] // 16, 4, 4))  # [.., group, block, local]
 
