@@ -75,15 +75,34 @@ PT_API int pt_device_cu_count(void);
  * scale_inv : device fp32[1] output.
  * workspace : device memory of at least pt_quantize_fp8_tensorwise_workspace_bytes()
  *             bytes, 16-byte aligned, ZERO-FILLED before its first use. The
- *             kernels keep an epoch counter and per-workgroup slots in it and
- *             maintain them from then on, so one buffer serves any number of
- *             successive calls on one stream without being cleared again; calls
- *             that may overlap (different streams) need separate buffers.
+ *             kernels keep a generation counter and generation-tagged per-workgroup
+ *             slots in it and maintain them from then on, so one buffer serves any
+ *             number of successive calls on one stream (HIP-graph replays included)
+ *             without being cleared again; calls that may overlap (different
+ *             streams) need separate buffers. Unused when scale_in is given.
+ *
+ * The exchange waits for every workgroup of the launch with a bounded number of
+ * probes. The launch is sized so that all its workgroups are resident (one per CU), so
+ * the bound is only reached when something outside the library takes CUs away (CU
+ * masking, a long kernel on another stream). Every wave still exits; the launch then
+ * writes NaN into scale_inv, so that everything de-quantized or multiplied from the
+ * result is NaN rather than plausible, and the _ex form raises *status.
  */
 PT_API size_t pt_quantize_fp8_tensorwise_workspace_bytes(void);
 PT_API int    pt_quantize_fp8_tensorwise(const void *x, int x_dtype, int64_t numel, void *q,
                                          int q_dtype, const float *scale_in, float *scale_inv,
                                          void *workspace, size_t workspace_bytes, void *stream);
+/* Same operation with the exchange's failure handling exposed.
+ * status         : optional device int32; every workgroup that gives up waiting stores 1
+ *                  (never cleared by the library; NULL = not reported).
+ * max_probes     : probe bound of the wait, 0 = the library's default (2^21).
+ * phantom_blocks : number of additional, never-published slots the launch waits for;
+ *                  0 in production. Tests pass 1 with a small max_probes to drive the
+ *                  wait to its bound from the host while every wave exits normally. */
+PT_API int pt_quantize_fp8_tensorwise_ex(const void *x, int x_dtype, int64_t numel, void *q,
+                                         int q_dtype, const float *scale_in, float *scale_inv,
+                                         void *workspace, size_t workspace_bytes, int32_t *status,
+                                         uint32_t max_probes, int64_t phantom_blocks, void *stream);
 
 /* Replaces torch.ops.primus_turbo_cpp_extension.dequantize_fp8_tensorwise
  * (csrc/pytorch/bindings_pytorch.cpp:38, quantization.cpp:211-230,

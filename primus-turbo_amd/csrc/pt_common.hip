@@ -51,7 +51,7 @@ const char *pt_last_error(void) {
 }
 
 int pt_abi_version(void) {
-    return 1;
+    return 2;
 }
 
 int pt_device_cu_count(void) {

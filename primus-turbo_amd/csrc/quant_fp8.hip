@@ -11,6 +11,8 @@
 // amax crosses the grid, so HBM sees x exactly once.
 #include "pt_common.h"
 
+#include <mutex>
+
 namespace pt {
 
 // ===========================================================================
@@ -21,53 +23,97 @@ constexpr int TW_VEC     = 16; // elements per thread per unit (16 fp8 bytes = o
 
 // Grid-wide abs-max exchange without read-modify-write atomics (same-address
 // device-scope atomics serialise at ~12 ns each on this part, far too slow for a
-// 256-workgroup launch). Workspace layout, in 32-bit words:
-//   [0]            epoch k, advanced by one per launch
-//   [1]            sticky time-out flag
-//   [64 + s*1024 + b]  slot of workgroup b in slot set s (s = 0, 1)
-// Launch k publishes into set k & 1: workgroup b stores its abs-max bit pattern
-// with bit 31 raised (abs-max >= 0, so bit 31 is free to mean "published"), then
-// thread t polls slot t until it is published and the block reduces what it read.
-// Workgroup 0 clears the other set for launch k + 1 (nobody reads it during launch
-// k, and launch k - 1, its last user, has finished) and advances the epoch once it
-// is past the exchange, i.e. after every workgroup has read the old epoch.
-constexpr int      WS_EPOCH = 0, WS_TIMEOUT = 1, WS_SLOTS = 64, WS_MAX_BLOCKS = 1024;
-constexpr int      WS_WORDS = WS_SLOTS + 2 * WS_MAX_BLOCKS;
+// 256-workgroup launch). Workspace layout, in 64-bit words (zero-filled before its
+// first use, maintained by the kernels from then on):
+//   [WS_GEN]       generation g: the tag of the last launch that completed its exchange
+//   [WS_GAVE_UP]   tag of the last launch in which a workgroup gave up waiting
+//   [WS_SLOTS + b] slot of workgroup b: (tag << 32) | abs-max bits
+// A launch takes tag = g + 1 (never 0). Thread 0 of every workgroup reads g BEFORE it
+// publishes (the published word depends on the value read, so the two cannot swap) and
+// hands the tag to its workgroup through LDS; wavefront 0 then polls the slots of all
+// workgroups until each carries the tag. Slots of earlier launches carry older tags and
+// need no clearing; workgroup 0 zeroes the slots this launch does not use, so a stale tag
+// can never be 2^32 launches old. Workgroup 0 stores g = tag once its own poll is over,
+// i.e. after every workgroup has read the old g. Successive launches that share a
+// workspace must be ordered (one stream, or a graph's dependencies).
+constexpr int WS_GEN = 0, WS_GAVE_UP = 1, WS_SLOTS = 8, WS_MAX_BLOCKS = 1024;
+constexpr int WS_WORDS = WS_SLOTS + WS_MAX_BLOCKS;
 // Probe bound of the poll (each probe sleeps ~64 cycles plus one memory round trip).
 // Every workgroup of the launch is resident (grid <= CU count, one workgroup per
 // CU), so the wait normally ends within microseconds; the bound only guarantees that
-// every wave exits even if residency is broken by something outside this library.
-// A timed-out launch raises WS_TIMEOUT (sticky) and its output is invalid.
+// every wave exits even if residency is broken by something outside this library (CU
+// masking, a long kernel of another stream holding the CUs). A workgroup that gives up
+// raises *status (when given) and WS_GAVE_UP; workgroup 0 then writes NaN into scale_inv,
+// so the failure travels with the data: everything de-quantized from it is NaN.
 constexpr uint32_t GRID_WAIT_MAX_PROBES = 1u << 21;
 
-__device__ __forceinline__ float grid_max_exchange(float block_amax, uint32_t *ws,
-                                                   uint32_t nblocks, float *s_red) {
-    const uint32_t k   = ws[WS_EPOCH];
-    uint32_t      *cur = ws + WS_SLOTS + (k & 1u) * WS_MAX_BLOCKS;
-    uint32_t      *nxt = ws + WS_SLOTS + ((k + 1u) & 1u) * WS_MAX_BLOCKS;
-    if (blockIdx.x == 0)
-        for (int t = threadIdx.x; t < WS_MAX_BLOCKS; t += blockDim.x)
-            nxt[t] = 0u;
-    if (threadIdx.x == 0)
-        __hip_atomic_store(&cur[blockIdx.x], __float_as_uint(block_amax) | 0x80000000u,
+struct GridWait {
+    uint64_t *ws;         // workspace words
+    int32_t  *status;     // optional device word, set to 1 by every workgroup that gives up
+    uint32_t  max_probes; // probe bound
+    uint32_t  wait_for;   // number of slots to wait for (the grid size; tests pass more)
+};
+
+// Returns the grid-wide abs-max. s_tag[1] != 0 afterwards when this workgroup's poll ended at
+// the probe bound (the value returned is then only a partial maximum) or, in workgroup 0,
+// when any workgroup of the launch is known to have given up.
+__device__ __forceinline__ float grid_max_exchange(float block_amax, const GridWait &gw,
+                                                   float *s_red, uint32_t *s_tag) {
+    uint64_t *slots = gw.ws + WS_SLOTS;
+    if (threadIdx.x == 0) {
+        const uint32_t g =
+            static_cast<uint32_t>(__hip_atomic_load(&gw.ws[WS_GEN], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        const uint32_t tag = (g + 1u == 0u) ? 1u : g + 1u;
+        s_tag[0]           = tag;
+        s_tag[1]           = 0u;
+        __hip_atomic_store(&slots[blockIdx.x],
+                           (static_cast<uint64_t>(tag) << 32) | __float_as_uint(block_amax),
                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    const uint32_t tag = s_tag[0];
+    if (blockIdx.x == 0)
+        for (uint32_t t = gw.wait_for + threadIdx.x; t < WS_MAX_BLOCKS; t += blockDim.x)
+            slots[t] = 0ull;
     float v = 0.f;
-    for (uint32_t t = threadIdx.x; t < nblocks; t += blockDim.x) {
-        uint32_t probes = 0, w;
-        while (((w = __hip_atomic_load(&cur[t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) &
-                0x80000000u) == 0u) {
-            __builtin_amdgcn_s_sleep(1);
-            if (++probes >= GRID_WAIT_MAX_PROBES) {
-                __hip_atomic_store(&ws[WS_TIMEOUT], 1u, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-                break;
+    if (threadIdx.x < 64) {
+        bool bad = false;
+        for (uint32_t t = threadIdx.x; t < gw.wait_for; t += 64) {
+            uint32_t probes = 0;
+            uint64_t w;
+            while (static_cast<uint32_t>((w = __hip_atomic_load(&slots[t], __ATOMIC_RELAXED,
+                                                                __HIP_MEMORY_SCOPE_AGENT)) >>
+                                         32) != tag) {
+                if (++probes >= gw.max_probes) {
+                    bad = true;
+                    w   = 0ull;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
             }
+            v = fmaxf(v, __uint_as_float(static_cast<uint32_t>(w) & 0x7fffffffu));
         }
-        v = fmaxf(v, __uint_as_float(w & 0x7fffffffu));
+        if (bad)
+            s_tag[1] = 1u; // same value from every lane that writes
     }
     v = block_max(v, s_red);
-    if (blockIdx.x == 0 && threadIdx.x == 0)
-        ws[WS_EPOCH] = k + 1u;
+    if (threadIdx.x == 0) {
+        if (s_tag[1] != 0u) {
+            __hip_atomic_store(&gw.ws[WS_GAVE_UP], static_cast<uint64_t>(tag), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+            if (gw.status != nullptr)
+                __hip_atomic_store(gw.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (blockIdx.x == 0) {
+            // a workgroup that started late (after one that gave up had left) can find every
+            // slot published although others quantized with a partial maximum: look at the flag
+            if (static_cast<uint32_t>(__hip_atomic_load(&gw.ws[WS_GAVE_UP], __ATOMIC_RELAXED,
+                                                        __HIP_MEMORY_SCOPE_AGENT)) == tag)
+                s_tag[1] = 1u;
+            __hip_atomic_store(&gw.ws[WS_GEN], static_cast<uint64_t>(tag), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
     return v;
 }
 
@@ -141,9 +187,10 @@ template <bool E5M2> __device__ __forceinline__ uint8_t quant1(float x, float sc
 template <typename T, bool E5M2, bool VEC16, bool DYNAMIC, int RET>
 __global__ __launch_bounds__(TW_THREADS) void quant_tensorwise_kernel(
     const T *__restrict__ x, uint8_t *__restrict__ q, const int64_t n,
-    const float *__restrict__ scale_in, float *__restrict__ scale_inv_out, uint32_t *ws,
+    const float *__restrict__ scale_in, float *__restrict__ scale_inv_out, const GridWait gw,
     const float qmax) {
-    __shared__ float s_red[TW_THREADS / 64];
+    __shared__ float    s_red[TW_THREADS / 64];
+    __shared__ uint32_t s_tag[2];
     const int64_t    stride = static_cast<int64_t>(gridDim.x) * TW_THREADS;
     const int64_t    tid0   = static_cast<int64_t>(blockIdx.x) * TW_THREADS + threadIdx.x;
 
@@ -172,7 +219,7 @@ __global__ __launch_bounds__(TW_THREADS) void quant_tensorwise_kernel(
             if (blockIdx.x == 0 && tail0 + threadIdx.x < n)
                 amax = fmaxf(amax, fabsf(HP<T>::to_f32(x[tail0 + threadIdx.x])));
             amax = block_max(amax, s_red);
-            amax = grid_max_exchange(amax, ws, gridDim.x, s_red);
+            amax = grid_max_exchange(amax, gw, s_red, s_tag);
         }
         float scale;
         if constexpr (DYNAMIC)
@@ -180,7 +227,7 @@ __global__ __launch_bounds__(TW_THREADS) void quant_tensorwise_kernel(
         else
             scale = scale_in[0];
         if (tid0 == 0)
-            scale_inv_out[0] = 1.0f / scale;
+            scale_inv_out[0] = (DYNAMIC && s_tag[1] != 0u) ? __builtin_nanf("") : 1.0f / scale;
 
         if constexpr (DYNAMIC) {
 #pragma unroll
@@ -204,7 +251,7 @@ __global__ __launch_bounds__(TW_THREADS) void quant_tensorwise_kernel(
             for (int64_t i = tid0; i < n; i += stride)
                 amax = fmaxf(amax, fabsf(HP<T>::to_f32(x[i])));
             amax = block_max(amax, s_red);
-            amax = grid_max_exchange(amax, ws, gridDim.x, s_red);
+            amax = grid_max_exchange(amax, gw, s_red, s_tag);
         }
         float scale;
         if constexpr (DYNAMIC)
@@ -212,7 +259,7 @@ __global__ __launch_bounds__(TW_THREADS) void quant_tensorwise_kernel(
         else
             scale = scale_in[0];
         if (tid0 == 0)
-            scale_inv_out[0] = 1.0f / scale;
+            scale_inv_out[0] = (DYNAMIC && s_tag[1] != 0u) ? __builtin_nanf("") : 1.0f / scale;
         for (int64_t i = tid0; i < n; i += stride)
             q[i] = quant1<E5M2>(HP<T>::to_f32(x[i]), scale, qmax);
     }
@@ -220,7 +267,8 @@ __global__ __launch_bounds__(TW_THREADS) void quant_tensorwise_kernel(
 
 template <typename T, bool E5M2>
 static int launch_quant_tensorwise(const void *x, int64_t n, void *q, const float *scale_in,
-                                   float *scale_inv, uint32_t *ws, hipStream_t stream) {
+                                   float *scale_inv, uint64_t *ws, int32_t *status,
+                                   uint32_t max_probes, int64_t phantom_blocks, hipStream_t stream) {
     constexpr int RET   = 4;
     const float   qmax  = E5M2 ? 57344.0f : 448.0f;
     const bool    vec   = aligned_to(x, 16) && aligned_to(q, 16);
@@ -233,16 +281,20 @@ static int launch_quant_tensorwise(const void *x, int64_t n, void *q, const floa
         grid = cus; // one workgroup per CU: all of them are resident at the grid exchange
     if (grid > WS_MAX_BLOCKS)
         grid = WS_MAX_BLOCKS;
-    const T *xp = static_cast<const T *>(x);
-    auto    *qp = static_cast<uint8_t *>(q);
-    dim3     g(static_cast<unsigned>(grid)), b(TW_THREADS);
+    if (grid + phantom_blocks > WS_MAX_BLOCKS)
+        return fail(PT_ERR_INVALID_ARGUMENT, "quant_tensorwise: phantom_blocks exceeds the slot count");
+    const T       *xp = static_cast<const T *>(x);
+    auto          *qp = static_cast<uint8_t *>(q);
+    dim3           g(static_cast<unsigned>(grid)), b(TW_THREADS);
+    const GridWait gw{ws, status, max_probes ? max_probes : GRID_WAIT_MAX_PROBES,
+                      static_cast<uint32_t>(grid + phantom_blocks)};
     if (scale_in == nullptr) {
         if (vec)
             quant_tensorwise_kernel<T, E5M2, true, true, RET>
-                <<<g, b, 0, stream>>>(xp, qp, n, nullptr, scale_inv, ws, qmax);
+                <<<g, b, 0, stream>>>(xp, qp, n, nullptr, scale_inv, gw, qmax);
         else
             quant_tensorwise_kernel<T, E5M2, false, true, 0>
-                <<<g, b, 0, stream>>>(xp, qp, n, nullptr, scale_inv, ws, qmax);
+                <<<g, b, 0, stream>>>(xp, qp, n, nullptr, scale_inv, gw, qmax);
     } else {
         // no grid exchange: oversubscribe the CUs for latency hiding
         const int64_t full = cdiv(units, TW_THREADS);
@@ -250,10 +302,10 @@ static int launch_quant_tensorwise(const void *x, int64_t n, void *q, const floa
         dim3          g2(static_cast<unsigned>(gg));
         if (vec)
             quant_tensorwise_kernel<T, E5M2, true, false, 0>
-                <<<g2, b, 0, stream>>>(xp, qp, n, scale_in, scale_inv, ws, qmax);
+                <<<g2, b, 0, stream>>>(xp, qp, n, scale_in, scale_inv, gw, qmax);
         else
             quant_tensorwise_kernel<T, E5M2, false, false, 0>
-                <<<g2, b, 0, stream>>>(xp, qp, n, scale_in, scale_inv, ws, qmax);
+                <<<g2, b, 0, stream>>>(xp, qp, n, scale_in, scale_inv, gw, qmax);
     }
     return check_launch("quant_tensorwise_kernel");
 }
@@ -687,29 +739,49 @@ using namespace pt;
 extern "C" {
 
 size_t pt_quantize_fp8_tensorwise_workspace_bytes(void) {
-    return WS_WORDS * sizeof(uint32_t);
+    return WS_WORDS * sizeof(uint64_t);
 }
 
-int pt_quantize_fp8_tensorwise(const void *x, int x_dtype, int64_t numel, void *q, int q_dtype,
-                               const float *scale_in, float *scale_inv, void *workspace,
-                               size_t workspace_bytes, void *stream) {
-    PT_REQUIRE(is_hp_dtype(x_dtype), "input must be bf16, fp16 or fp32");
-    PT_REQUIRE(is_fp8_dtype(q_dtype), "output must be e4m3 or e5m2");
-    PT_REQUIRE(numel >= 0, "numel must be non-negative");
-    PT_REQUIRE(scale_inv != nullptr, "scale_inv must not be NULL");
-    PT_REQUIRE(numel == 0 || (x != nullptr && q != nullptr), "x and q must not be NULL");
+static int quantize_fp8_tensorwise_common(const void *x, int x_dtype, int64_t numel, void *q,
+                                          int q_dtype, const float *scale_in, float *scale_inv,
+                                          uint64_t *ws, int32_t *status, uint32_t max_probes,
+                                          int64_t phantom_blocks, hipStream_t st) {
+#define CALL(T, E5)                                                                                \
+    return launch_quant_tensorwise<T, E5>(x, numel, q, scale_in, scale_inv, ws, status,            \
+                                          max_probes, phantom_blocks, st)
+    PT_DISPATCH_HP_FP8(x_dtype, q_dtype, CALL);
+#undef CALL
+}
+
+#define PT_TW_CHECK_ARGS()                                                                         \
+    PT_REQUIRE(is_hp_dtype(x_dtype), "input must be bf16, fp16 or fp32");                          \
+    PT_REQUIRE(is_fp8_dtype(q_dtype), "output must be e4m3 or e5m2");                              \
+    PT_REQUIRE(numel >= 0, "numel must be non-negative");                                          \
+    PT_REQUIRE(scale_inv != nullptr, "scale_inv must not be NULL");                                \
+    PT_REQUIRE(numel == 0 || (x != nullptr && q != nullptr), "x and q must not be NULL")
+
+int pt_quantize_fp8_tensorwise_ex(const void *x, int x_dtype, int64_t numel, void *q, int q_dtype,
+                                  const float *scale_in, float *scale_inv, void *workspace,
+                                  size_t workspace_bytes, int32_t *status, uint32_t max_probes,
+                                  int64_t phantom_blocks, void *stream) {
+    PT_TW_CHECK_ARGS();
+    PT_REQUIRE(phantom_blocks >= 0, "phantom_blocks must be non-negative");
     if (scale_in == nullptr) {
         if (workspace == nullptr || workspace_bytes < pt_quantize_fp8_tensorwise_workspace_bytes() ||
             !aligned_to(workspace, 16))
             return fail(PT_ERR_WORKSPACE,
                         "pt_quantize_fp8_tensorwise: workspace missing, too small or misaligned");
     }
-    auto *ws = static_cast<uint32_t *>(workspace);
-    auto  st = static_cast<hipStream_t>(stream);
-#define CALL(T, E5)                                                                                \
-    return launch_quant_tensorwise<T, E5>(x, numel, q, scale_in, scale_inv, ws, st)
-    PT_DISPATCH_HP_FP8(x_dtype, q_dtype, CALL);
-#undef CALL
+    return quantize_fp8_tensorwise_common(x, x_dtype, numel, q, q_dtype, scale_in, scale_inv,
+                                          static_cast<uint64_t *>(workspace), status, max_probes,
+                                          phantom_blocks, static_cast<hipStream_t>(stream));
+}
+
+int pt_quantize_fp8_tensorwise(const void *x, int x_dtype, int64_t numel, void *q, int q_dtype,
+                               const float *scale_in, float *scale_inv, void *workspace,
+                               size_t workspace_bytes, void *stream) {
+    return pt_quantize_fp8_tensorwise_ex(x, x_dtype, numel, q, q_dtype, scale_in, scale_inv,
+                                         workspace, workspace_bytes, nullptr, 0, 0, stream);
 }
 
 int pt_dequantize_fp8_tensorwise(const void *q, int q_dtype, int64_t numel, const float *scale_inv,

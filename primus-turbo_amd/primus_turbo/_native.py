@@ -37,6 +37,9 @@ if hasattr(torch, "float8_e8m0fnu"):
 _lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
 
+# status codes of include/primus_turbo_amd.h
+PT_OK, PT_ERR_INVALID_ARGUMENT, PT_ERR_UNSUPPORTED, PT_ERR_WORKSPACE, PT_ERR_LAUNCH = 0, -1, -2, -3, -4
+
 c_void_p, c_int, c_i64, c_size_t, c_float = (
     ctypes.c_void_p,
     ctypes.c_int,
@@ -54,6 +57,11 @@ _SIGNATURES = {
     "pt_quantize_fp8_tensorwise": (
         c_int,
         [c_void_p, c_int, c_i64, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
+    ),
+    "pt_quantize_fp8_tensorwise_ex": (
+        c_int,
+        [c_void_p, c_int, c_i64, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p, ctypes.c_uint32,
+         c_i64, c_void_p],
     ),
     "pt_dequantize_fp8_tensorwise": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p, c_int, c_void_p]),
     "pt_quantize_fp8_rowwise": (
@@ -243,11 +251,11 @@ def require_cuda(*tensors: torch.Tensor) -> None:
 
 
 # ---------------------------------------------------------------------------
-# Small zero-filled device workspace for one launch (the kernels leave it zeroed, but it is not
-# kept: a buffer that outlives the call would have to live outside the private memory pool of
-# whatever graph capture, or warm-up run for one, happens to be active -- torch.compile's CUDA-graph
-# trees insist that nothing allocated there stays alive -- and an op cannot tell. A fill kernel of
-# 256 bytes per call is the price; it is capturable and belongs to nobody afterwards).
+# Zero-filled device workspace for one launch. Not kept between calls: a buffer that outlives the
+# call would have to live outside the private memory pool of whatever graph capture, or warm-up
+# run for one, happens to be active -- torch.compile's CUDA-graph trees insist that nothing
+# allocated there stays alive -- and an op cannot tell. Only the fallback of the tensorwise
+# quantizer uses it (its normal path keeps the exchange words in the library's static scratch).
 # ---------------------------------------------------------------------------
 def zeroed_workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     return torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=device)

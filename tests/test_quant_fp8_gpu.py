@@ -154,3 +154,58 @@ def test_literal_python_reference_within_its_tolerance():
     d = turbo.ops.dequantize_fp8(q, torch.bfloat16, G.TENSORWISE, scale_inv=sinv).cpu()
     rd = R.dequantize_fp8_ref(rq, torch.bfloat16, rsinv)
     torch.testing.assert_close(d.float(), rd.float(), rtol=1e-1, atol=1e-1)
+
+
+def _tw_ex(lib, x, q, sinv, ws, status, max_probes, phantom):
+    from primus_turbo import _native as N
+
+    return lib.pt_quantize_fp8_tensorwise_ex(
+        N.ptr(x), N.dtype_code(x.dtype), x.numel(), N.ptr(q), N.dtype_code(q.dtype), None, N.ptr(sinv),
+        N.ptr(ws), ws.numel(), N.ptr(status), max_probes, phantom, N.stream_of(x))
+
+
+def test_tensorwise_lost_grid_exchange_is_visible():
+    """The bounded wait of the grid exchange is driven to its bound from the host: the launch
+    waits for one slot more than it has workgroups, with a bound of a few hundred probes, so every
+    wave exits normally. The failure has to show: NaN in scale_inv, the status word raised. The
+    same workspace then serves a normal launch (generation-tagged slots need no clearing), and a
+    launch with fewer workgroups after one with more."""
+    from primus_turbo import _native as N
+
+    lib = N.lib()
+    x = bf16_randn((1024, 1024), seed=5, outlier_frac=0.001).cuda()
+    oq, osinv = Q.fp8_tensorwise(to_f32_np(x), "e4m3")
+    q = torch.empty_like(x, dtype=torch.float8_e4m3fn)
+    sinv = torch.zeros((), dtype=torch.float32, device="cuda")
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    ws = torch.zeros(lib.pt_quantize_fp8_tensorwise_workspace_bytes(), dtype=torch.uint8, device="cuda")
+
+    N.check(_tw_ex(lib, x, q, sinv, ws, status, 200, 1))
+    torch.cuda.synchronize()
+    assert status.item() == 1, "a workgroup that gave up must raise the status word"
+    assert torch.isnan(sinv).item(), "a lost exchange must poison scale_inv"
+    y = turbo.ops.dequantize_fp8(q, torch.bfloat16, G.TENSORWISE, scale_inv=sinv)
+    assert torch.isnan(y).all().item()
+
+    # the same workspace, now a normal launch: bit-exact, status untouched
+    status.zero_()
+    N.check(_tw_ex(lib, x, q, sinv, ws, status, 0, 0))
+    torch.cuda.synchronize()
+    assert status.item() == 0
+    assert bits_np(sinv).item() == osinv.view(np.uint32).item()
+    assert np.array_equal(codes_np(q), oq)
+
+    # fewer workgroups than the launch before (stale slots of the larger grid stay behind)
+    xs = x[:3].contiguous()
+    qs = torch.empty_like(xs, dtype=torch.float8_e4m3fn)
+    for _ in range(3):
+        N.check(_tw_ex(lib, xs, qs, sinv, ws, status, 0, 0))
+    torch.cuda.synchronize()
+    oq, osinv = Q.fp8_tensorwise(to_f32_np(xs), "e4m3")
+    assert status.item() == 0 and bits_np(sinv).item() == osinv.view(np.uint32).item()
+    assert np.array_equal(codes_np(qs), oq)
+    # and more again
+    N.check(_tw_ex(lib, x, q, sinv, ws, status, 0, 0))
+    torch.cuda.synchronize()
+    oq, osinv = Q.fp8_tensorwise(to_f32_np(x), "e4m3")
+    assert status.item() == 0 and np.array_equal(codes_np(q), oq)
