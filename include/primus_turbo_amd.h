@@ -104,6 +104,29 @@ PT_API int pt_quantize_fp8_tensorwise_ex(const void *x, int x_dtype, int64_t num
                                          void *workspace, size_t workspace_bytes, int32_t *status,
                                          uint32_t max_probes, int64_t phantom_blocks, void *stream);
 
+/* pt_quantize_fp8_tensorwise without a workspace argument, for callers that cannot
+ * allocate device memory (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc). It has no counterpart in Primus-Turbo. The exchange words live
+ * in a static device array inside the library (66 KB per GPU, zero-initialised when the
+ * code object loads, held until the process ends); neither this entry point nor anything
+ * it calls allocates or frees memory. Same kernels and results as
+ * pt_quantize_fp8_tensorwise.
+ *
+ * Each stream that calls it on a device is given its own slot set, at most
+ * PT_TENSORWISE_STATIC_MAX_STREAMS per device; one more stream is rejected with
+ * PT_ERR_WORKSPACE, and numel above PT_TENSORWISE_STATIC_MAX_NUMEL with
+ * PT_ERR_INVALID_ARGUMENT. Calls on one stream are ordered and share that stream's slot
+ * set; the set keeps the last call's words (they are generation-tagged, so nothing has
+ * to be cleared). Work that overlaps on one GPU while using ONE slot set races: a graph
+ * captured on stream S and replayed on another stream while S is also calling, or the
+ * same graph replayed concurrently on two streams.
+ * status : as in pt_quantize_fp8_tensorwise_ex (optional). */
+#define PT_TENSORWISE_STATIC_MAX_STREAMS 8
+#define PT_TENSORWISE_STATIC_MAX_NUMEL (1LL << 37)
+PT_API int pt_quantize_fp8_tensorwise_static(const void *x, int x_dtype, int64_t numel, void *q,
+                                             int q_dtype, const float *scale_in, float *scale_inv,
+                                             int32_t *status, void *stream);
+
 /* Replaces torch.ops.primus_turbo_cpp_extension.dequantize_fp8_tensorwise
  * (csrc/pytorch/bindings_pytorch.cpp:38, quantization.cpp:211-230,
  * quantization_tensorwise.cu:113-154):  y[i] = T(float(q[i]) * scale_inv[0]). */

@@ -720,6 +720,58 @@ static int launch_dequant_rowwise(const void *q, int64_t B, int64_t M, int64_t N
 }
 
 // ---------------------------------------------------------------------------
+// Static scratch of pt_quantize_fp8_tensorwise_static: the exchange words live in the code
+// object's own zero-initialised device memory, so that entry point needs no workspace and
+// neither it nor its caller allocates anything. One slot set per stream that has used the
+// entry point on the device (calls on one stream are ordered, calls on different streams
+// must not share slots), PT_TENSORWISE_STATIC_MAX_STREAMS of them: 66 KB per GPU, held
+// until the process ends.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) uint64_t tw_scratch[PT_TENSORWISE_STATIC_MAX_STREAMS * WS_WORDS];
+
+// Device address of tw_scratch on the current device (the array's name is only a host-side
+// handle; every GPU holds its own copy at its own address) and the slot set of `stream`.
+static int static_scratch_for(hipStream_t stream, uint64_t **out) {
+    constexpr int MAX_DEV = 64;
+    struct PerDevice {
+        uint64_t   *base = nullptr;
+        int         used = 0;
+        hipStream_t streams[PT_TENSORWISE_STATIC_MAX_STREAMS];
+    };
+    static PerDevice  table[MAX_DEV];
+    static std::mutex mu;
+    int               dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEV)
+        return fail(PT_ERR_LAUNCH, "pt_quantize_fp8_tensorwise_static: no current device");
+    std::lock_guard<std::mutex> lock(mu);
+    PerDevice                  &pd = table[dev];
+    if (pd.base == nullptr) {
+        void            *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(tw_scratch));
+        if (e != hipSuccess || p == nullptr)
+            return fail(PT_ERR_LAUNCH, std::string("pt_quantize_fp8_tensorwise_static: "
+                                                   "hipGetSymbolAddress failed: ") +
+                                           hipGetErrorString(e));
+        pd.base = static_cast<uint64_t *>(p);
+    }
+    int idx = -1;
+    for (int i = 0; i < pd.used; ++i)
+        if (pd.streams[i] == stream)
+            idx = i;
+    if (idx < 0) {
+        if (pd.used == PT_TENSORWISE_STATIC_MAX_STREAMS)
+            return fail(PT_ERR_WORKSPACE,
+                        "pt_quantize_fp8_tensorwise_static: more distinct streams on this device "
+                        "than PT_TENSORWISE_STATIC_MAX_STREAMS; use pt_quantize_fp8_tensorwise "
+                        "with a workspace per stream");
+        idx             = pd.used++;
+        pd.streams[idx] = stream;
+    }
+    *out = pd.base + static_cast<size_t>(idx) * WS_WORDS;
+    return PT_OK;
+}
+
+// ---------------------------------------------------------------------------
 // dtype dispatch
 // ---------------------------------------------------------------------------
 #define PT_DISPATCH_HP_FP8(hp, fp8, CALL)                                                          \
@@ -782,6 +834,22 @@ int pt_quantize_fp8_tensorwise(const void *x, int x_dtype, int64_t numel, void *
                                size_t workspace_bytes, void *stream) {
     return pt_quantize_fp8_tensorwise_ex(x, x_dtype, numel, q, q_dtype, scale_in, scale_inv,
                                          workspace, workspace_bytes, nullptr, 0, 0, stream);
+}
+
+int pt_quantize_fp8_tensorwise_static(const void *x, int x_dtype, int64_t numel, void *q,
+                                      int q_dtype, const float *scale_in, float *scale_inv,
+                                      int32_t *status, void *stream) {
+    PT_TW_CHECK_ARGS();
+    PT_REQUIRE(numel <= PT_TENSORWISE_STATIC_MAX_NUMEL,
+               "numel exceeds PT_TENSORWISE_STATIC_MAX_NUMEL; use pt_quantize_fp8_tensorwise with a workspace");
+    uint64_t *ws = nullptr;
+    if (scale_in == nullptr) {
+        const int rc = static_scratch_for(static_cast<hipStream_t>(stream), &ws);
+        if (rc != PT_OK)
+            return rc;
+    }
+    return quantize_fp8_tensorwise_common(x, x_dtype, numel, q, q_dtype, scale_in, scale_inv, ws,
+                                          status, 0, 0, static_cast<hipStream_t>(stream));
 }
 
 int pt_dequantize_fp8_tensorwise(const void *q, int q_dtype, int64_t numel, const float *scale_inv,

@@ -63,6 +63,10 @@ _SIGNATURES = {
         [c_void_p, c_int, c_i64, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p, ctypes.c_uint32,
          c_i64, c_void_p],
     ),
+    "pt_quantize_fp8_tensorwise_static": (
+        c_int,
+        [c_void_p, c_int, c_i64, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
+    ),
     "pt_dequantize_fp8_tensorwise": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p, c_int, c_void_p]),
     "pt_quantize_fp8_rowwise": (
         c_int,

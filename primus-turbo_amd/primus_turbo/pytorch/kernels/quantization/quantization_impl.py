@@ -62,15 +62,28 @@ def _quantize_fp8_tensorwise(input: torch.Tensor, dest_dtype: torch.dtype, scale
     lib = N.lib()
     out = torch.empty_like(input, dtype=dest_dtype)
     scale_inv = torch.empty((), dtype=torch.float32, device=input.device)
-    ws = None
     scale_in = None
     if scale_opt is not None:
         _check(scale_opt.numel() == 1, "tensorwise scale must be scalar tensor")
         scale_in = scale_opt.to(torch.float32).contiguous()
-    else:
+    # The grid exchange of the fused kernel keeps its words in the library's static device
+    # scratch (one slot set per stream): no per-call allocation or fill. A lost exchange shows
+    # as NaN in scale_inv (see the header), so nothing is read back here.
+    status = lib.pt_quantize_fp8_tensorwise_static(
+        N.ptr(input),
+        N.dtype_code(input.dtype),
+        input.numel(),
+        N.ptr(out),
+        N.dtype_code(dest_dtype),
+        N.ptr(scale_in),
+        N.ptr(scale_inv),
+        None,
+        N.stream_of(input),
+    )
+    if status == N.PT_ERR_WORKSPACE:
+        # more streams in use on this device than the static scratch has slot sets
         ws = N.zeroed_workspace(input.device, lib.pt_quantize_fp8_tensorwise_workspace_bytes())
-    N.check(
-        lib.pt_quantize_fp8_tensorwise(
+        status = lib.pt_quantize_fp8_tensorwise(
             N.ptr(input),
             N.dtype_code(input.dtype),
             input.numel(),
@@ -79,10 +92,10 @@ def _quantize_fp8_tensorwise(input: torch.Tensor, dest_dtype: torch.dtype, scale
             N.ptr(scale_in),
             N.ptr(scale_inv),
             N.ptr(ws),
-            0 if ws is None else ws.numel(),
+            ws.numel(),
             N.stream_of(input),
         )
-    )
+    N.check(status)
     return [out, scale_inv]
 
 

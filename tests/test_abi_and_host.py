@@ -56,6 +56,10 @@ def test_argument_validation_without_gpu(native_lib):
     one = ctypes.c_float(0)
     assert lib.pt_quantize_fp8_tensorwise(1024, 0, 16, 2048, 3, None, ctypes.addressof(one), None, 0, None) == -3
     assert b"workspace" in lib.pt_last_error()
+    assert lib.pt_quantize_fp8_tensorwise_static(None, 9, 16, None, 3, None, None, None, None) == -1
+    assert lib.pt_quantize_fp8_tensorwise_static(1024, 0, 1 << 38, 2048, 3, None, ctypes.addressof(one), None, None) == -1
+    assert b"MAX_NUMEL" in lib.pt_last_error()
+    assert lib.pt_quantize_fp8_tensorwise_ex(1024, 0, 16, 2048, 3, None, ctypes.addressof(one), None, 0, None, 0, -1, None) == -1
     assert lib.pt_dequantize_fp8_tensorwise(None, 3, -1, None, None, 0, None) == -1
     assert lib.pt_quantize_fp8_rowwise(None, 0, 1, 1, 1, None, 7, None, None, None) == -1
     assert lib.pt_quantize_fp8_blockwise(None, 0, 8, 8, 3, None, None, None, None, None) == -1
