@@ -125,7 +125,7 @@ static int launch_vector_tiles(const GemmArgs &a, int tile_cfg, hipStream_t stre
     // tile_cfg: 0 = auto, 1 = 256x256, 2 = 256x128, 3 = 128x128
     if (tile_cfg == 0)
         tile_cfg = (a.M >= 2048 && a.N >= 2048) ? 1 : 3;
-    if (tile_cfg == 1)
+    if (tile_cfg == 1 || tile_cfg == 4)
         return launch_gemm_cfg<8, 8, SCALE_VECTOR, false, FA, FB>(a, stream);
     if (tile_cfg == 2)
         return launch_gemm_cfg<8, 4, SCALE_VECTOR, false, FA, FB>(a, stream);
@@ -208,7 +208,7 @@ int pt_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const void *b,
     PT_REQUIRE(scale_mode == SCALE_VECTOR || scale_mode == SCALE_BLOCK, "unknown scale mode");
     PT_REQUIRE(scale_mode != SCALE_BLOCK || ((sa_block == 1 || sa_block == 128) && (sb_block == 1 || sb_block == 128)),
                "sa_block / sb_block must be 1 or 128");
-    PT_REQUIRE(tile_cfg >= 0 && tile_cfg <= 3, "tile_cfg must be 0..3");
+    PT_REQUIRE(tile_cfg >= 0 && tile_cfg <= 4, "tile_cfg must be 0..4");
     if (M == 0 || N == 0)
         return PT_OK;
     PT_REQUIRE(a && b && c && a_scale && b_scale, "NULL tensor pointer");

@@ -3,15 +3,22 @@
 // input of VALU FMAs (the per-128-K-block scale is applied outside the matrix core), so this
 // translation unit is compiled with MFMA destinations in architectural VGPRs: results in
 // accumulation registers would cost one v_accvgpr_read per element on top of each FMA.
-#include "gemm_fp8_kernel.h"
+#include "gemm_fp8_block8.h"
 
 namespace pt {
 
 template <bool SB_VEC, int FA, int FB>
 static int launch_block_tiles(const GemmArgs &a, int tile_cfg, hipStream_t stream) {
-    // tile_cfg: 0 = auto, 1 = 256x256, 2 = 256x128, 3 = 128x128 (two workgroups per CU)
+    // tile_cfg: 0 = auto, 1 = 256x256, 2 = 256x128, 3 = 128x128 (two workgroups per CU),
+    // 4 = 256x256 with eight wavefronts (2-D B scales only)
     if (tile_cfg == 0)
         tile_cfg = (a.M >= 2048 && a.N >= 1024) ? 2 : 3;
+    if (tile_cfg == 4) {
+        if constexpr (SB_VEC)
+            tile_cfg = 2;
+        else
+            return launch_gemm_block8<FA, FB>(a, stream);
+    }
     if (tile_cfg == 3)
         return launch_gemm_cfg<4, 4, SCALE_BLOCK, SB_VEC, FA, FB>(a, stream);
     if (tile_cfg == 1)

@@ -19,7 +19,7 @@ from primus_turbo.pytorch.core.low_precision import ScalingGranularity
 _FP8 = (torch.float8_e4m3fn, torch.float8_e5m2)
 _OUT = (torch.bfloat16, torch.float16, torch.float32)
 
-TILE_CFG = 0  # 0 = automatic; tests and the benchmark may pin 1 (256x256), 2 (256x128), 3 (128x128)
+TILE_CFG = 0  # 0 = automatic; tests and the benchmark may pin 1 (256x256), 2 (256x128), 3 (128x128), 4 (256x256, eight wavefronts: block scales)
 
 
 def get_gemm_logical_shape(a: torch.Tensor, b: torch.Tensor, trans_a: bool, trans_b: bool) -> Tuple[int, int, int]:

@@ -38,7 +38,7 @@ def _deq_fp8(q: torch.Tensor, s: torch.Tensor, fmt):
 
 
 # ----------------------------------------------------------------------------- impl level
-@pytest.mark.parametrize("tile_cfg", [0, 1, 2, 3])
+@pytest.mark.parametrize("tile_cfg", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize(
     "M,N,K", [(256, 256, 128), (512, 384, 1024), (300, 200, 256), (1, 1, 128), (777, 130, 640), (4096, 4096, 512)]
 )
@@ -102,8 +102,42 @@ def test_layouts_rowwise(trans_a, trans_b, trans_c):
     _gate(ref, to_f32_np(c), f"layout {trans_a}{trans_b}{trans_c}")
 
 
+def test_blockwise_exact_small_integers():
+    """Block-scaled kernels on integer operands with power-of-two block scales: every product,
+    every scaled block sum and every partial sum is exact in fp32, so each tile configuration
+    has to give the integer result bit for bit (wrong row / block of a scale, a wrong fragment
+    or accumulator mapping, a slab applied twice or dropped at a tile change all show)."""
+    M, N, K = 768, 640, 1024
+    rng = np.random.default_rng(6)
+    a = torch.from_numpy(rng.integers(-4, 5, (M, K)).astype(np.float32))
+    b = torch.from_numpy(rng.integers(-4, 5, (N, K)).astype(np.float32))
+    sa = torch.from_numpy(np.exp2(rng.integers(-3, 4, (M, K // 128))).astype(np.float32))
+    sb = torch.from_numpy(np.exp2(rng.integers(-3, 4, ((N + 127) // 128, K // 128))).astype(np.float32))
+    ad = a * sa.repeat_interleave(128, dim=1)
+    bd = b * sb.repeat_interleave(128, dim=0)[:N].repeat_interleave(128, dim=1)
+    want = ad.double() @ bd.double().t()
+    assert want.abs().max() < 2**24
+    aq, bq = a.to(torch.float8_e4m3fn).cuda(), b.to(torch.float8_e4m3fn).cuda()
+    for cfg in (1, 2, 3, 4):
+        impl.TILE_CFG = cfg
+        try:
+            c = impl.gemm_fp8_impl(aq, sa.cuda(), False, bq, sb.cuda(), True, torch.float32, False, G.BLOCKWISE.value, 0)
+        finally:
+            impl.TILE_CFG = 0
+        assert torch.equal(c.cpu().double(), want), f"tile cfg {cfg}"
+
+
+@pytest.mark.parametrize("tile_cfg", [0, 4])
 @pytest.mark.parametrize("M,N,K", [(512, 384, 512), (300, 260, 256), (2048, 1024, 1024), (16384, 1024, 256)])
-def test_blockwise_nt_nn_tn(M, N, K):
+def test_blockwise_nt_nn_tn(M, N, K, tile_cfg):
+    impl.TILE_CFG = tile_cfg
+    try:
+        _blockwise_nt_nn_tn(M, N, K)
+    finally:
+        impl.TILE_CFG = 0
+
+
+def _blockwise_nt_nn_tn(M, N, K):
     a = bf16_randn((M, K), 35, outlier_frac=0.001)
     w = bf16_randn((N, K), 36)
     f8 = torch.float8_e4m3fn
