@@ -11,8 +11,12 @@ template <bool SB_VEC, int FA, int FB>
 static int launch_block_tiles(const GemmArgs &a, int tile_cfg, hipStream_t stream) {
     // tile_cfg: 0 = auto, 1 = 256x256, 2 = 256x128, 3 = 128x128 (two workgroups per CU),
     // 4 = 256x256 with eight wavefronts (2-D B scales only)
-    if (tile_cfg == 0)
+    if (tile_cfg == 0) {
         tile_cfg = (a.M >= 2048 && a.N >= 1024) ? 2 : 3;
+        // 256x256 with eight wavefronts once both dimensions fill the machine with such tiles
+        if (!SB_VEC && a.M >= 2048 && a.N >= 2048 && cdiv(a.M, 256) * cdiv(a.N, 256) >= device_cu_count())
+            tile_cfg = 4;
+    }
     if (tile_cfg == 4) {
         if constexpr (SB_VEC)
             tile_cfg = 2;
