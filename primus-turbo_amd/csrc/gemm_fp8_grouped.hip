@@ -7,7 +7,7 @@
 //                                   (forward and dgrad of a grouped linear layer)
 //   pt_grouped_gemm_fp8_variable_k  dW[g] = LHS_g^T . RHS_g over the rows of group g
 //                                   (wgrad; the reduction length differs per group)
-#include "gemm_fp8_kernel.h"
+#include "gemm_fp8_block8.h"
 
 
 
@@ -15,10 +15,20 @@ namespace pt {
 
 template <int GMODE, bool SB_VEC, int FA, int FB>
 static int launch_grouped_tiles(const GemmArgs &a, int tile_cfg, hipStream_t stream) {
-    // tile_cfg: 0 = auto, 1 / 2 = 256x128, 3 = 128x128 (two workgroups per CU)
+    // tile_cfg: 0 = auto, 1 / 2 = 256x128, 3 = 128x128 (two workgroups per CU), 4 = 256x256 with
+    // eight wavefronts (row groups only)
     // (the 256x128 tile leaves LDS for the tile prefix sums of 1024 groups only)
-    if (tile_cfg == 0) // 256-row tiles once the average group fills a couple of them
+    if (tile_cfg == 0) { // 256-row tiles once the average group fills a couple of them
         tile_cfg = ((GMODE == GROUP_K ? a.M >= 1024 : (a.G > 0 && a.M / a.G >= 512)) && a.N >= 1024) ? 2 : 3;
+        if (GMODE == GROUP_ROWS && !SB_VEC && tile_cfg == 2 && a.N >= 2048)
+            tile_cfg = 4;
+    }
+    if (tile_cfg == 4) {
+        if constexpr (GMODE == GROUP_ROWS && !SB_VEC)
+            return launch_gemm_block8<FA, FB, GROUP_ROWS>(a, stream);
+        else
+            tile_cfg = 2;
+    }
     if (a.G > 1024)
         tile_cfg = 3;
     if (tile_cfg == 3)
@@ -83,7 +93,7 @@ int pt_grouped_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const 
     PT_REQUIRE(is_fp8_dtype(a_dtype) && is_fp8_dtype(b_dtype), "operands must be e4m3 or e5m2");
     PT_REQUIRE(is_hp_dtype(c_dtype), "output must be bf16, fp16 or fp32");
     PT_REQUIRE(G >= 0 && M >= 0 && N >= 0 && K >= 0 && out_rows >= M, "bad dimensions");
-    PT_REQUIRE(tile_cfg >= 0 && tile_cfg <= 3, "tile_cfg must be 0..3");
+    PT_REQUIRE(tile_cfg >= 0 && tile_cfg <= 4, "tile_cfg must be 0..4");
     PT_REQUIRE(K < (1LL << 24), "K must be below 2^24");
     auto st = static_cast<hipStream_t>(stream);
     if (out_rows == 0 || N == 0)
@@ -172,7 +182,7 @@ int pt_grouped_gemm_fp8_variable_k(const void *lhs, int lhs_dtype, const float *
     PT_REQUIRE(is_fp8_dtype(lhs_dtype) && is_fp8_dtype(rhs_dtype), "operands must be e4m3 or e5m2");
     PT_REQUIRE(is_hp_dtype(c_dtype), "output must be bf16, fp16 or fp32");
     PT_REQUIRE(G >= 0 && Mp >= 0 && Ml >= 0 && Nr >= 0, "bad dimensions");
-    PT_REQUIRE(tile_cfg >= 0 && tile_cfg <= 3, "tile_cfg must be 0..3");
+    PT_REQUIRE(tile_cfg >= 0 && tile_cfg <= 4, "tile_cfg must be 0..4");
     PT_REQUIRE(Mp < (1LL << 24), "at most 2^24 rows");
     auto st = static_cast<hipStream_t>(stream);
     if (G == 0 || Ml == 0 || Nr == 0)

@@ -52,11 +52,21 @@ CASES = [
 ]
 
 
+@pytest.mark.parametrize("tile_cfg", [0, 4])
 @pytest.mark.parametrize("kind,G_,M,N,K", CASES)
 @pytest.mark.parametrize("trans_b", [True, False])
-def test_grouped_forward_product(kind, G_, M, N, K, trans_b):
+def test_grouped_forward_product(kind, G_, M, N, K, trans_b, tile_cfg):
     """out[rows of g] = A_g . W_g^T from the fused grouped quantizer's row output and 2-D-block
-    weights; both weight layouts; empty and ragged groups."""
+    weights; both weight layouts; empty and ragged groups; automatic tile choice and the pinned
+    eight-wavefront 256 x 256 tile."""
+    gimpl.TILE_CFG = tile_cfg
+    try:
+        _grouped_forward_product(kind, G_, M, N, K, trans_b)
+    finally:
+        gimpl.TILE_CFG = 0
+
+
+def _grouped_forward_product(kind, G_, M, N, K, trans_b):
     lens = group_lens(kind, G_, M, 31)
     gl, offs = _offs(lens)
     x = bf16_randn((M, K), seed=32)
