@@ -4,11 +4,15 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
 
 Prints ONE JSON line. A "step" is one pass of the hot path over one batch of
-synthetic input that is already resident in HBM. ``roofline`` prices the dominant
-kernel of the workload (algorithmic bytes or flops per launch / its average launch
-duration, timed with HIP events on the launch stream) against MI355X's published
-peak; ``cpu_baseline`` times the reference's own pure-PyTorch formulas
-(oracle/cpu_reference.py) on the host cores over a bounded sample.
+synthetic input that is already resident in HBM. The default workload is the 8192^3
+blockwise FP8 GEMM. Every time is the median of WINDOWS windows of K steps.
+``roofline`` prices the dominant kernel of the workload (algorithmic bytes or flops per
+launch / its launch duration, timed with HIP events on the launch stream) against MI355X's
+published peak; the HBM-bound workloads rotate their input through more than 512 MB of
+copies, so that the 256 MB Infinity Cache cannot serve the reads. ``cpu_baseline`` times the
+reference's own pure-PyTorch formulas (oracle/cpu_reference.py) on the host cores over a
+bounded sample. ``extra`` carries the same measurements for the other workloads of the
+configurations this path is quoted on (shorter runs, no CPU leg).
 """
 
 from __future__ import annotations
@@ -100,6 +104,13 @@ class QuantTensorwise:
         self.x = self.x_cpu.to(dev)
         self.n = self.x.numel()
         self.q, self.sinv = turbo.ops.quantize_fp8(self.x, turbo.float8_e4m3, G.TENSORWISE)
+        # 20 copies of the 32 MiB input (640 MiB): rotating through them keeps the reads in HBM
+        self._ring = [self.x] + [self.x.clone() for _ in range(19)]
+        self._pos = 0
+
+    def rotate(self):
+        self._pos = (self._pos + 1) % len(self._ring)
+        self.x = self._ring[self._pos]
 
     # bytes: quant reads 2 B + writes 1 B per element, dequant reads 1 B + writes 2 B
     def step_work(self):
@@ -113,20 +124,18 @@ class QuantTensorwise:
 
     def dominant(self):
         """One launch of the fused kernel through the C entry point with preallocated outputs: the
-        kernel runs ~15 us, less than the op's Python path takes to issue it."""
+        kernel runs ~13 us, less than the op's Python path takes to issue it."""
         from primus_turbo import _native as N
 
         if not hasattr(self, "_dom"):
             lib = N.lib()
             out = torch.empty_like(self.x, dtype=torch.float8_e4m3fn)
             sinv = torch.empty((), dtype=torch.float32, device=self.x.device)
-            ws = N.zeroed_workspace(self.x.device, lib.pt_quantize_fp8_tensorwise_workspace_bytes())
-            args = (N.ptr(self.x), N.dtype_code(self.x.dtype), self.x.numel(), N.ptr(out), N.dtype_code(out.dtype),
-                    None, N.ptr(sinv), N.ptr(ws), ws.numel(), N.stream_of(self.x))
-            self._dom = (lib.pt_quantize_fp8_tensorwise, args, out, sinv, ws)
-        fn, args = self._dom[0], self._dom[1]
-        N.check(fn(*args))
-        return self._dom[2]
+            self._dom = (lib.pt_quantize_fp8_tensorwise_static, out, sinv)
+        fn, out, sinv = self._dom
+        N.check(fn(N.ptr(self.x), N.dtype_code(self.x.dtype), self.x.numel(), N.ptr(out), N.dtype_code(out.dtype),
+                   None, N.ptr(sinv), None, N.stream_of(self.x)))
+        return out
 
     def dominant_work(self):
         return 3.0 * self.n  # bytes per launch
@@ -171,7 +180,92 @@ from bench_workloads import register as _register  # noqa: E402
 _register_quant(WORKLOADS)
 _register(WORKLOADS)
 
-DEFAULT_ORDER = ["gemm_fp8_rowwise", "quant_tensorwise"]
+DEFAULT_ORDER = ["gemm_fp8_blockwise_8192", "gemm_fp8_rowwise", "quant_tensorwise"]
+
+# the other workloads of the configurations the path is quoted on, reported under "extra"
+EXTRA_GEMM = ["gemm_fp8_rowwise", "gemm_fp8_blockwise", "gemm_fp8_blockwise_k7168", "grouped_gemm_fp8",
+              "grouped_gemm_fp8_down", "gemm_mxfp4", "gemm_mxfp4_n28672", "gemm_mxfp8", "gemm_mxfp8_n28672"]
+EXTRA_QUANT = ["quant_tensorwise", "quant_rowwise", "quant_blockwise", "quant_blockwise_dual", "quant_blockwise_weight",
+               "quant_grouped", "quant_mxfp8", "quant_mxfp8_dual", "quant_mxfp4", "quant_mxfp4_dual"]
+EXTRA_BUDGET_S = 400.0  # no further extra workload is started after this many seconds of run time
+
+
+def _median(xs):
+    xs = sorted(xs)
+    return xs[len(xs) // 2]
+
+
+def _rotating(wl, fn):
+    """``fn`` preceded by the workload's input rotation (HBM-bound workloads only)."""
+    rot = getattr(wl, "rotate", None)
+    if rot is None:
+        return fn
+
+    def call():
+        rot()
+        return fn()
+
+    return call
+
+
+def measure(wl, steps, warmup, windows):
+    """-> (ms_per_step, value, roofline dict, parity dict); every time a median of ``windows``."""
+    step = _rotating(wl, wl.step)
+    dominant = _rotating(wl, wl.dominant)
+    # Setup ends with the GPU busy: data generation ran on the host while the idle GPU dropped to
+    # its low power state, and a handful of sub-millisecond warm-up steps is over before the clocks
+    # are back up. (The parity check runs after the timed region for the same reason: its oracle
+    # leg keeps the GPU idle.)
+    t_spin = time.perf_counter()
+    while time.perf_counter() - t_spin < 0.3:
+        for _ in range(5):
+            step()
+        torch.cuda.synchronize()
+    for _ in range(warmup):
+        step()
+    wins = []
+    for _ in range(windows):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        wins.append((time.perf_counter() - t0) * 1e3 / steps)
+    ms_per_step = _median(wins)
+    scale = 1e12 if wl.unit == "TFLOP/s" else 1e9
+    value = wl.step_work() / (ms_per_step * 1e-3) / scale
+
+    # dominant kernel, HIP events on the launch stream
+    for _ in range(max(3, warmup)):
+        dominant()
+    timer = _graph_ms if getattr(wl, "graph_dominant", False) else _events_ms
+    dom_ms = _median([timer(dominant, max(steps, 20)) for _ in range(windows)])
+    achieved = wl.dominant_work() / (dom_ms * 1e-3) / scale
+    peak = {"hbm": HBM_PEAK_GBS, "mfma": getattr(wl, "peak", FP8_PEAK_TFLOPS)}[wl.bound]
+    roofline = dict(
+        bound=wl.bound,
+        achieved=round(achieved, 2),
+        peak=peak,
+        unit="GB/s" if wl.bound == "hbm" else "TFLOP/s",
+        frac=round(achieved / peak, 4),
+        traffic=getattr(wl, "traffic", None),
+        kernel=wl.dominant_name,
+        kernel_ms=round(dom_ms, 5),
+    )
+    if getattr(wl, "rotate", None) is not None:
+        roofline["inputs"] = "rotating through copies of the input (> 512 MB): reads come from HBM, not the Infinity Cache"
+    kernels = getattr(wl, "kernels", None)
+    if kernels is not None:  # further kernels of the step, each alone under HIP events
+        per = {}
+        for kname, fn, work in kernels():
+            for _ in range(3):
+                fn()
+            kms = _median([_events_ms(fn, max(steps, 20)) for _ in range(windows)])
+            per[kname] = dict(kernel_ms=round(kms, 5), achieved=round(work / (kms * 1e-3) / scale, 2),
+                              frac=round(work / (kms * 1e-3) / scale / peak, 4))
+        roofline["kernels"] = per
+    ok, what = wl.check()
+    return ms_per_step, value, roofline, dict(ok=ok, what=what)
 
 
 def main():
@@ -179,12 +273,16 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--windows", type=int, default=5, help="timed windows of --steps steps; the median is reported")
     ap.add_argument("--workload", default="auto", help="one of: auto, " + ", ".join(WORKLOADS))
+    ap.add_argument("--extra", default=None, choices=["all", "gemm", "none"],
+                    help="which other workloads to measure into 'extra' (default: all for the default workload, else none)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch one plain elementwise copy of 256 MiB (fp32 x + 0 -> y): the known-size "
                     "kernel that HBM traffic counters of a profiled run are scaled by")
     args = ap.parse_args()
+    t_start = time.perf_counter()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(
@@ -198,6 +296,7 @@ def main():
         sys.exit(3)
 
     name = args.workload
+    extra_mode = args.extra or ("all" if name == "auto" else "none")
     if name == "auto":
         name = next(w for w in DEFAULT_ORDER if w in WORKLOADS)
     dev = torch.device("cuda:0")
@@ -211,48 +310,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # Setup ends with the GPU busy: data generation above ran on the host while the idle GPU
-    # dropped to its low power state, and a handful of sub-millisecond warm-up steps is over before
-    # the clocks are back up. (The parity check runs after the timed region for the same reason: its
-    # oracle leg keeps the GPU idle.)
-    t_spin = time.perf_counter()
-    while time.perf_counter() - t_spin < 0.3:
-        for _ in range(5):
-            wl.step()
-        torch.cuda.synchronize()
-    for _ in range(args.warmup):
-        wl.step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        wl.step()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
-    scale = 1e12 if wl.unit == "TFLOP/s" else 1e9
-    value = wl.step_work() / (ms_per_step * 1e-3) / scale
-
-    # dominant kernel, HIP events on the launch stream
-    for _ in range(max(3, args.warmup)):
-        wl.dominant()
-    if getattr(wl, "graph_dominant", False):
-        dom_ms = _graph_ms(wl.dominant, max(args.steps, 20))
-    else:
-        dom_ms = _events_ms(wl.dominant, max(args.steps, 20))
-    achieved = wl.dominant_work() / (dom_ms * 1e-3) / scale
-    ok, what = wl.check()
-    peak = {"hbm": HBM_PEAK_GBS, "mfma": getattr(wl, "peak", FP8_PEAK_TFLOPS)}[wl.bound]
-    roofline = dict(
-        bound=wl.bound,
-        achieved=round(achieved, 2),
-        peak=peak,
-        unit="GB/s" if wl.bound == "hbm" else "TFLOP/s",
-        frac=round(achieved / peak, 4),
-        traffic=getattr(wl, "traffic", None),
-        kernel=wl.dominant_name,
-        kernel_ms=round(dom_ms, 5),
-    )
-
+    ms_per_step, value, roofline, parity = measure(wl, args.steps, args.warmup, args.windows)
     out = dict(
         metric=wl.metric,
         value=round(value, 2),
@@ -260,6 +318,7 @@ def main():
         n_gpus=1,
         steps=args.steps,
         warmup=args.warmup,
+        windows=args.windows,
         ms_per_step=round(ms_per_step, 5),
         higher_is_better=True,
         scaling="weak",
@@ -267,14 +326,32 @@ def main():
         dtype=wl.dtype,
         data="synthetic",
         config=dict(workload=wl.name),
-        parity=dict(ok=ok, what=what),
+        parity=parity,
         roofline=roofline,
     )
     if not args.no_cpu:
         out["cpu_baseline"] = wl.cpu_baseline()
-    extra = getattr(wl, "extra", None)
-    if extra:
-        out["extra"] = extra() if callable(extra) else extra
+    del wl
+    torch.cuda.empty_cache()
+
+    if extra_mode != "none":
+        keys = [k for k in EXTRA_GEMM + (EXTRA_QUANT if extra_mode == "all" else []) if k in WORKLOADS and k != name]
+        extra = {}
+        for key in keys:
+            if time.perf_counter() - t_start > EXTRA_BUDGET_S:
+                extra[key] = dict(skipped="time budget of the run spent")
+                continue
+            w = WORKLOADS[key](dev)
+            ms, val, roof, par = measure(w, max(10, args.steps // 2), max(3, args.warmup // 2), args.windows)
+            rec = dict(workload=w.name, ms=round(ms, 5), value=round(val, 2), unit=w.unit, bound=roof["bound"],
+                       frac=roof["frac"], achieved=roof["achieved"], kernel_ms=roof["kernel_ms"], parity_ok=par["ok"])
+            if "kernels" in roof:
+                rec["kernels"] = roof["kernels"]
+            extra[key] = rec
+            del w
+            torch.cuda.empty_cache()
+        out["extra"] = extra
+    out["run_seconds"] = round(time.perf_counter() - t_start, 1)
     print(json.dumps(out))
 
 

@@ -39,6 +39,21 @@ class _QuantBase:
     metric = "quantize GB/s (algorithmic bytes) & fraction of HBM peak"
     graph_dominant = True  # kernels of tens of microseconds: time replays of a captured batch
 
+    def rotate(self):
+        """Point ``self.x`` at the next of several identical copies of the input (at least 640 MiB
+        together): a kernel timed over the rotation reads from HBM; one that re-reads a single
+        tensor of up to 256 MB is served by the Infinity Cache."""
+        x = getattr(self, "x", None)
+        if x is None:
+            return
+        if not hasattr(self, "_ring"):
+            nbytes = x.numel() * x.element_size()
+            n = max(2, min(24, -(-(640 << 20) // nbytes)))
+            self._ring = [x] + [x.detach().clone().requires_grad_(x.requires_grad) for _ in range(n - 1)]
+            self._pos = 0
+        self._pos = (self._pos + 1) % len(self._ring)
+        self.x = self._ring[self._pos]
+
     def _cpu(self, fn, nbytes, what):
         fn()
         times = []

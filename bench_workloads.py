@@ -118,7 +118,7 @@ class GemmFp8Rowwise(_GemmBase):
         rel = OG.max_rel_err(ref_t, out[rows])
         cos = OG.cosine(out[rows], ref_t)
         ok = bool(same and rel <= 1e-2 and cos >= 0.9999)
-        return ok, f"quantized bytes bit-exact; 128 output rows vs oracle: max_rel_err={rel:.2e}, cosine={cos:.6f}"
+        return ok, f"quantized bytes bit-exact; 128 output rows vs oracle: max|err|/max|ref| (relative to the output range, not element-wise)={rel:.2e}, cosine={cos:.6f}"
 
     def cpu_baseline(self):
         """The reference's CPU formulas on an M-slice: rowwise quantize of the slice and of all of
@@ -200,7 +200,7 @@ class GemmFp8Blockwise(_GemmBase):
         rel = OG.max_rel_err(ref_t, out[rows])
         cos = OG.cosine(out[rows], ref_t)
         ok = bool(same and rel <= 1e-2 and cos >= 0.9999)
-        return ok, f"quantized bytes bit-exact; 128 output rows vs oracle: max_rel_err={rel:.2e}, cosine={cos:.6f}"
+        return ok, f"quantized bytes bit-exact; 128 output rows vs oracle: max|err|/max|ref| (relative to the output range, not element-wise)={rel:.2e}, cosine={cos:.6f}"
 
     def cpu_baseline(self):
         from oracle import cpu_reference as R
@@ -296,7 +296,7 @@ class GemmMx(_GemmBase):
         rel = OG.max_rel_err(ref_t, out[rows][:, :nb])
         cos = OG.cosine(out[rows][:, :nb], ref_t)
         ok = bool(same and rel <= 1e-2 and cos >= 0.9999)
-        return ok, f"codes and E8M0 bytes bit-exact: {same}; 128 x 2048 outputs vs oracle: max_rel_err={rel:.2e}, cosine={cos:.6f}"
+        return ok, f"codes and E8M0 bytes bit-exact: {same}; 128 x 2048 outputs vs oracle: max|err|/max|ref| (relative to the output range, not element-wise)={rel:.2e}, cosine={cos:.6f}"
 
     def cpu_baseline(self):
         """The oracle (numpy restatement of the reference's MX quantizer) plus an fp32 matmul on a
@@ -380,6 +380,32 @@ class GroupedGemmFp8(_GemmBase):
         return self.gg.grouped_gemm_fp8_impl(self.qr, self.wq, self.sr, self.ws, self.gl, self.offs, False, True,
                                              torch.bfloat16, self.G.BLOCKWISE.value, None, 0)
 
+    def kernels(self):
+        """The three GEMM launches of the step on pre-quantized operands, as the autograd function
+        issues them: (name, callable, flops)."""
+        qi, gg, gran = self.qi, self.gg, self.G.BLOCKWISE.value
+        f8 = torch.float8_e4m3fn
+        if not hasattr(self, "_bwd"):
+            x_row, x_col_t, x_srow, x_scol, _, _ = qi.quant_fp8_blockwise_segment_m_row_col_t_impl(
+                self.x.detach(), f8, 128, self.gl, self.offs)
+            g_row, g_col_t, g_srow, g_scol, vk_lens, vk_offs = qi.quant_fp8_blockwise_segment_m_row_col_t_impl(
+                self.dy, f8, 128, self.gl, self.offs)
+            wq, wq_t, ws = qi.quant_fp8_blockwise_for_weight_dual_impl(self.w.detach(), f8, block_size=128)
+            ws_t = ws.transpose(-2, -1).contiguous()
+            self._bwd = (x_col_t, x_scol, g_row, g_srow, g_col_t, g_scol, vk_lens, vk_offs, wq_t, ws_t)
+        x_col_t, x_scol, g_row, g_srow, g_col_t, g_scol, vk_lens, vk_offs, wq_t, ws_t = self._bwd
+        flops = 2.0 * self.M * self.N * self.K
+
+        def dgrad():
+            return gg.grouped_gemm_fp8_impl(g_row, wq_t, g_srow, ws_t, self.gl, self.offs, False, True, torch.bfloat16,
+                                            gran, None, 0)
+
+        def wgrad():
+            return gg.grouped_gemm_fp8_variable_k_impl(x_col_t, g_col_t, x_scol, g_scol, vk_lens, vk_offs, False, True,
+                                                       True, torch.bfloat16, gran, None, 0)
+
+        return [("forward", self.dominant, flops), ("dgrad", dgrad, flops), ("wgrad_variable_k", wgrad, flops)]
+
     def check(self):
         """Forward rows of the first and of the last non-empty expert (up to 64 each) against the
         oracle's de-quantized matmul; their quantized bytes bit-exact."""
@@ -404,7 +430,7 @@ class GroupedGemmFp8(_GemmBase):
             rel = max(rel, OG.max_rel_err(ref_t, out[r0:r1]))
             cos = min(cos, OG.cosine(out[r0:r1], ref_t))
         ok = bool(same and rel <= 1e-2 and cos >= 0.9999)
-        return ok, f"quantized bytes bit-exact: {same}; rows of two experts vs oracle: max_rel_err={rel:.2e}, cosine={cos:.6f}"
+        return ok, f"quantized bytes bit-exact: {same}; rows of two experts vs oracle: max|err|/max|ref| (relative to the output range, not element-wise)={rel:.2e}, cosine={cos:.6f}"
 
     def cpu_baseline(self):
         """The reference's CPU formulas (blockwise quantize, dequantize, per-expert fp32 matmul) for
@@ -506,7 +532,7 @@ class GroupedGemmMxfp8(_GemmBase):
             rel = max(rel, OG.max_rel_err(ref_t, out[r0 : r0 + n]))
             cos = min(cos, OG.cosine(out[r0 : r0 + n], ref_t))
         ok = bool(same and rel <= 1e-2 and cos >= 0.9999)
-        return ok, f"codes and E8M0 bytes bit-exact: {same}; rows of two experts vs oracle: max_rel_err={rel:.2e}, cosine={cos:.6f}"
+        return ok, f"codes and E8M0 bytes bit-exact: {same}; rows of two experts vs oracle: max|err|/max|ref| (relative to the output range, not element-wise)={rel:.2e}, cosine={cos:.6f}"
 
     def cpu_baseline(self):
         """The numpy oracle (MX quantize, de-quantize) plus an fp32 matmul for 256 tokens of the
