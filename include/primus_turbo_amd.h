@@ -503,6 +503,12 @@ PT_API int pt_glu_with_probs_bwd(const void *grad_out, const void *x, int x_dtyp
  * transpose used for tensorwise `.t()` copies, csrc/kernels/transpose/). */
 PT_API int pt_transpose_u8(const void *in, void *out, int64_t batch, int64_t R, int64_t C,
                            void *stream);
+/* The same for elements of 1, 2, 4 or 8 bytes. Replaces
+ * torch.ops.primus_turbo_cpp_extension.transpose_2d (csrc/pytorch/bindings_pytorch.cpp:44,
+ * csrc/pytorch/transpose/transpose.cpp:17-49: last two dimensions of a contiguous 2-D / 3-D
+ * tensor of any dtype). */
+PT_API int pt_transpose_2d(const void *in, void *out, int64_t batch, int64_t R, int64_t C,
+                           int elem_bytes, void *stream);
 
 /* Pre-shuffled MX operand layouts (the (16, 16) tile orders that the reference hands to AITER's
  * a4w4 GEMM). Replaces shuffle_weight / shuffle_e8m0_scale (csrc/include/primus_turbo/shuffle.h:26-32,

@@ -103,6 +103,30 @@ __global__ __launch_bounds__(256) void transpose_u8_tile128_kernel(const uint8_t
     }
 }
 
+// out[b, c, r] = in[b, r, c] for 2-, 4- and 8-byte elements through a padded 32 x 32 LDS tile
+// (coalesced rows on both sides).
+template <typename E>
+__global__ __launch_bounds__(256) void transpose_elem_kernel(const E *__restrict__ in, E *__restrict__ out, const int64_t R,
+                                                             const int64_t C) {
+    __shared__ E  t[32][33];
+    const int64_t r0 = static_cast<int64_t>(blockIdx.y) * 32, c0 = static_cast<int64_t>(blockIdx.x) * 32;
+    const int64_t b  = static_cast<int64_t>(blockIdx.z) * R * C;
+    const int     tx = threadIdx.x & 31, ty = threadIdx.x >> 5; // 32 x 8 threads
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int64_t r = r0 + ty + 8 * p, c = c0 + tx;
+        if (r < R && c < C)
+            t[ty + 8 * p][tx] = in[b + r * C + c];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int64_t c = c0 + ty + 8 * p, r = r0 + tx;
+        if (c < C && r < R)
+            out[b + c * R + r] = t[tx][ty + 8 * p];
+    }
+}
+
 void launch_transpose(const uint8_t *in, uint8_t *out, int64_t batch, int64_t R, int64_t C,
                       int64_t ldo, hipStream_t st) {
     if (batch <= 0 || C <= 0 || ldo <= 0)
@@ -280,6 +304,26 @@ int pt_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const void *b,
     if (scale_mode == SCALE_VECTOR)
         return launch_gemm_vector(g, fa, fb, tile_cfg, st);
     return launch_gemm_block(g, fa, fb, sb_block == 1, tile_cfg, st);
+}
+
+int pt_transpose_2d(const void *in, void *out, int64_t batch, int64_t R, int64_t C, int elem_bytes, void *stream) {
+    PT_REQUIRE(batch >= 0 && R >= 0 && C >= 0, "dimensions must be non-negative");
+    PT_REQUIRE(elem_bytes == 1 || elem_bytes == 2 || elem_bytes == 4 || elem_bytes == 8, "element size must be 1, 2, 4 or 8 bytes");
+    if (elem_bytes == 1)
+        return pt_transpose_u8(in, out, batch, R, C, stream);
+    if (batch * R * C == 0)
+        return PT_OK;
+    PT_REQUIRE(in && out, "NULL tensor pointer");
+    PT_REQUIRE(batch < 65536 && cdiv(R, 32) < 65536, "grid dimension out of range");
+    dim3 g(static_cast<unsigned>(cdiv(C, 32)), static_cast<unsigned>(cdiv(R, 32)), static_cast<unsigned>(batch));
+    auto st = static_cast<hipStream_t>(stream);
+    if (elem_bytes == 2)
+        transpose_elem_kernel<uint16_t><<<g, 256, 0, st>>>(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out), R, C);
+    else if (elem_bytes == 4)
+        transpose_elem_kernel<uint32_t><<<g, 256, 0, st>>>(static_cast<const uint32_t *>(in), static_cast<uint32_t *>(out), R, C);
+    else
+        transpose_elem_kernel<uint64_t><<<g, 256, 0, st>>>(static_cast<const uint64_t *>(in), static_cast<uint64_t *>(out), R, C);
+    return check_launch("transpose_elem_kernel");
 }
 
 int pt_transpose_u8(const void *in, void *out, int64_t batch, int64_t R, int64_t C, void *stream) {

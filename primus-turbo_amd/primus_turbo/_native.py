@@ -115,6 +115,7 @@ _SIGNATURES = {
         [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_i64, c_int, c_void_p],
     ),
     "pt_transpose_u8": (c_int, [c_void_p, c_void_p, c_i64, c_i64, c_i64, c_void_p]),
+    "pt_transpose_2d": (c_int, [c_void_p, c_void_p, c_i64, c_i64, c_i64, c_int, c_void_p]),
     "pt_moe_permute_workspace_bytes": (c_size_t, [c_i64, c_i64]),
     "pt_moe_permute_preprocess": (
         c_int,

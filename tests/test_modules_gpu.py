@@ -177,11 +177,24 @@ def test_grouped_linear(kind, B, M, N, K, balance, compiled):
         assert _snr(want, got) > gate, f"{kind} {name}: SNR {_snr(want, got):.1f} dB"
 
 
-def test_grouped_linear_needs_a_config():
+def test_grouped_linear_constructs_like_the_reference_and_needs_a_config_to_run():
+    """The reference's constructor signature (no config) constructs; ``forward`` asks for the
+    config; assigning one afterwards gives the same result as the constructor keyword."""
     from primus_turbo.pytorch.modules import GroupedLinear
 
+    mod = GroupedLinear(4, 128, 256, "cuda", dtype=torch.bfloat16)
+    assert tuple(mod.weight.shape) == (4, 256, 128)
+    x = torch.randn(64, 128, device="cuda", dtype=torch.bfloat16)
+    lens = torch.tensor([16, 0, 40, 8], dtype=torch.int64, device="cuda")
     with pytest.raises(NotImplementedError, match="Float8QuantConfig"):
-        GroupedLinear(4, 128, 128, "cuda", dtype=torch.bfloat16)
+        mod(x, lens)
+    cfg = Float8QuantConfig(granularity=G.BLOCKWISE, block_size=128)
+    mod.config = cfg
+    y = mod(x, lens)
+    mod2 = GroupedLinear(4, 128, 256, "cuda", dtype=torch.bfloat16, config=cfg)
+    with torch.no_grad():
+        mod2.weight.copy_(mod.weight)
+    assert torch.equal(y, mod2(x, lens))
 
 
 @pytest.mark.parametrize("kind", ["rowwise", "blockwise", "mxfp8"])
