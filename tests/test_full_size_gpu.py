@@ -153,6 +153,73 @@ def test_grouped_forward_full_config(N, K):
     assert torch.equal(solo, out[r0:r1])
 
 
+@pytest.mark.parametrize("N,K", [(4096, 7168), (7168, 2048)])
+def test_grouped_backward_full_config(N, K):
+    """dgrad and variable-K wgrad of the MoE configuration at full size (32 experts, 32768 Zipf
+    tokens, two experts empty), on the operands the autograd function hands them: sampled outputs
+    of sampled experts against float64 dot products of the de-quantized operands; an expert
+    without tokens gets an exactly zero weight gradient, and with beta = 1 its slice of the
+    accumulation buffer stays untouched bit for bit."""
+    Gn, M = 32, 32768
+    f8 = torch.float8_e4m3fn
+    lens = group_lens("zipf", Gn, M, 7)
+    assert (lens == 0).sum() >= 2
+    gl = torch.from_numpy(lens).cuda()
+    offs = torch.ops.primus_turbo_cpp_extension.grouped_gemm_compute_offs(gl)
+    x = bf16_randn((M, K), seed=211).cuda()
+    dy = bf16_randn((M, N), seed=212).cuda()
+    w = bf16_randn((Gn, N, K), seed=213).cuda()
+    _, x_col_t, _, x_scol, _, _ = qi.quant_fp8_blockwise_segment_m_row_col_t_impl(x, f8, 128, gl, offs)
+    g_row, g_col_t, g_srow, g_scol, vk_lens, vk_offs = qi.quant_fp8_blockwise_segment_m_row_col_t_impl(dy, f8, 128, gl, offs)
+    wq, wq_t, ws = qi.quant_fp8_blockwise_for_weight_dual_impl(w, f8, block_size=128)
+    ws_t = ws.transpose(-2, -1).contiguous()
+    del x, dy, w
+    starts = np.concatenate([[0], np.cumsum(lens)])
+    live = [g for g in range(Gn) if lens[g] > 0]
+    empty = [g for g in range(Gn) if lens[g] == 0]
+    rng = np.random.default_rng(9)
+
+    # ---- dgrad: dX[rows of g] = dY_g . W_g   ([M, N] x [N, K] -> [M, K]) ----
+    dx = gg.grouped_gemm_fp8_impl(g_row, wq_t, g_srow, ws_t, gl, offs, False, True, torch.bfloat16, G.BLOCKWISE.value, None, 0)
+    assert tuple(dx.shape) == (M, K)
+    gs_t = np.ascontiguousarray(to_f32_np(g_srow).T)  # [M, N / 128]
+    for g in live[::5]:
+        rows = np.sort(starts[g] + rng.choice(int(lens[g]), size=min(24, int(lens[g])), replace=False))
+        a_deq = Q.fp8_blockwise_dequant(codes_np(g_row)[rows], gs_t[rows], 1, "e4m3", 128)
+        # rows 128..383 of W_g^T [K, N] = output columns 128..383
+        wt_deq = Q.fp8_blockwise_weight_dequant(codes_np(wq_t[g])[128:384], to_f32_np(ws_t[g])[1:3], "e4m3", 128)
+        _sampled_gate(dx, a_deq, wt_deq, rows, np.arange(128, 384), f"dgrad expert {g}")
+
+    # ---- wgrad: dW[g] = dY_g^T . X_g over the group's 128-padded token range ----
+    dw = gg.grouped_gemm_fp8_variable_k_impl(x_col_t, g_col_t, x_scol, g_scol, vk_lens, vk_offs, False, True, True,
+                                             torch.bfloat16, G.BLOCKWISE.value, None, 0)
+    assert tuple(dw.shape) == (Gn, N, K)
+    vo = vk_offs.cpu().numpy()
+    xs_t = np.ascontiguousarray(to_f32_np(x_scol).T)  # [K, M_pad / 128]
+    gsc_t = np.ascontiguousarray(to_f32_np(g_scol).T)  # [N, M_pad / 128]
+    for g in empty:
+        assert torch.count_nonzero(dw[g]).item() == 0, f"expert {g} has no tokens: its weight gradient must be exactly zero"
+    ncols, krows = _pick(N, 48, 10), _pick(K, 40, 11)
+    for g in (live[0], live[len(live) // 2], int(np.argmax(lens))):
+        t0, t1 = int(vo[g]), int(vo[g + 1])
+        gy = Q.fp8_blockwise_dequant(codes_np(g_col_t)[ncols][:, t0:t1], gsc_t[ncols][:, t0 // 128 : t1 // 128], 1, "e4m3", 128)
+        gx = Q.fp8_blockwise_dequant(codes_np(x_col_t)[krows][:, t0:t1], xs_t[krows][:, t0 // 128 : t1 // 128], 1, "e4m3", 128)
+        _sampled_gate(dw[g], gy, gx, ncols, krows, f"wgrad expert {g}")
+
+    # ---- beta = 1: accumulate into an fp32 buffer; empty experts stay untouched ----
+    base = torch.empty((Gn, N, K), dtype=torch.float32, device="cuda").normal_(generator=torch.Generator("cuda").manual_seed(3))
+    keep = {g: base[g].clone() for g in empty}
+    g_big = int(np.argmax(lens))
+    before = base[g_big, :64].clone()
+    gg.grouped_gemm_fp8_variable_k_accum_impl(x_col_t, g_col_t, x_scol, g_scol, vk_lens, vk_offs, False, True, True,
+                                              torch.float32, G.BLOCKWISE.value, None, 0, base)
+    for g in empty:
+        assert torch.equal(base[g], keep[g]), f"beta = 1 touched the buffer of the empty expert {g}"
+    added = (base[g_big, :64] - before).float()
+    want = dw[g_big, :64].float()
+    assert (added - want).abs().max().item() <= 2e-2 * want.abs().max().item()  # bf16 rounding of dw + fp32 cancellation
+
+
 def test_tensorwise_quant_4096_exact_and_round_trip():
     x = bf16_randn((4096, 4096), seed=209, outlier_frac=0.001)
     q, sinv = turbo.ops.quantize_fp8(x.cuda(), turbo.float8_e4m3, G.TENSORWISE)
