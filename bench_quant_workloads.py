@@ -408,6 +408,83 @@ class SwigluWithProbs(_QuantBase):
         return self._cpu(fn, self.dominant_work() * 4096 / self.T, "forward of the first 4096 tokens in PyTorch")
 
 
+class GluQuantGrouped(_QuantBase):
+    """The step between the two grouped GEMMs of the MoE configuration in its fused form: fc1's
+    output [32768, 2 x 2048] bf16 is read once by the grouped blockwise quantizer, which applies
+    SwiGLU with the router probabilities on load and writes fc2's row codes, transposed
+    segment-padded column codes and both scale tensors. The step also times the two-step form
+    (activation kernel, then quantizer) whose extra 32768 x 2048 x 2 B write and re-read the fusion
+    removes."""
+
+    name = "swiglu_with_probs_fused_into_grouped_blockwise_quant_32768tokens_hidden2048_bf16"
+    metric = "fused activation + quantize GB/s (algorithmic bytes) & fraction of HBM peak"
+    dominant_name = "quant_block128_kernel<row + transposed column blocks, grouped, SiLU gate on load>"
+    dtype = "bf16 in, e4m3 out (fp32 arithmetic)"
+
+    def __init__(self, dev, tokens=32768, hidden=2048, groups=32):
+        import primus_turbo.pytorch as turbo
+        from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+        from bench_workloads import _zipf_group_lens
+
+        self.turbo, self.qi, self.T, self.H = turbo, qi, tokens, hidden
+        self.lens = _zipf_group_lens(groups, tokens, 7)
+        self.gl = torch.from_numpy(self.lens).to(dev)
+        self.offs = torch.ops.primus_turbo_cpp_extension.grouped_gemm_compute_offs(self.gl)
+        self.x_cpu = _randn_bf16((tokens, 2 * hidden), 31, 1.0)
+        g = torch.Generator().manual_seed(32)
+        self.p_cpu = torch.rand(tokens, generator=g, dtype=torch.float32)
+        self.x = self.x_cpu.to(dev)
+        self.p = self.p_cpu.to(dev)
+
+    def dominant_work(self):  # 2 H read (2 B each), H row codes + H column codes + scales written, + the probability
+        n = self.T * self.H
+        return 6.0 * n + 8.0 * n / 128 + 4.0 * self.T
+
+    step_work = dominant_work
+
+    def dominant(self):
+        return self.qi.glu_quant_fp8_blockwise_segment_m_row_col_impl(self.x, self.p, None, "silu", torch.float8_e4m3fn, 128,
+                                                                      self.gl, self.offs, True)
+
+    step = dominant
+
+    def two_step(self):
+        y = self.turbo.ops.swiglu_with_probs(self.x, self.p)
+        return self.qi.quant_fp8_blockwise_segment_m_row_col_t_impl(y, torch.float8_e4m3fn, 128, self.gl, self.offs)
+
+    def kernels(self):
+        n = self.T * self.H  # the two-step form moves 4 more bytes per element (bf16 activation out and in again)
+        return [("two_step_swiglu_then_quantize", self.two_step, self.dominant_work() + 4.0 * n)]
+
+    def check(self):
+        a, b = self.dominant(), self.two_step()
+        w = int(a[5][-1].item())
+        same = (torch.equal(a[0].view(torch.uint8), b[0].view(torch.uint8)) and torch.equal(a[2], b[2])
+                and torch.equal(a[1].view(torch.uint8)[:, :w], b[1].view(torch.uint8)[:, :w])
+                and torch.equal(a[3][: w // 128], b[3][: w // 128]))
+        from oracle import quantize as Q
+
+        y = self.turbo.ops.swiglu_with_probs(self.x[:1024], self.p[:1024]).float().cpu().numpy()
+        oq, os_ = Q.fp8_blockwise(y, 1, "e4m3", 128)
+        same = same and np.array_equal(_u8(a[0])[:1024], oq)
+        same = same and np.array_equal(_f32(a[2])[:, :1024].T.copy().view(np.int32), os_.view(np.int32))
+        return bool(same), "codes and scales bit-identical with the two-step form; row codes of 1024 tokens bit-exact vs the oracle"
+
+    def cpu_baseline(self):
+        from oracle import cpu_reference as R
+
+        rows = 2048
+
+        def fn():
+            a, b = self.x_cpu[:rows].float().chunk(2, dim=-1)
+            y = (torch.nn.functional.silu(a) * b * self.p_cpu[:rows, None]).to(torch.bfloat16)
+            R.quantize_fp8_blockwise_ref(y, torch.float8_e4m3fn, 1, 128)
+            R.quantize_fp8_blockwise_ref(y, torch.float8_e4m3fn, 128, 1)
+
+        return self._cpu(fn, self.dominant_work() * rows / self.T, f"first {rows} tokens: PyTorch SwiGLU, then row and column blockwise quantize")
+
+
 class MoePermute(_QuantBase):
     """MoE permute + unpermute around the expert bank of the MoE configuration: 4096 tokens with
     top-8 routing over 32 local experts (32768 routed rows), hidden 7168, bf16, rows padded per
@@ -478,6 +555,7 @@ class MoePermute(_QuantBase):
 def register(workloads):
     workloads["moe_permute"] = MoePermute
     workloads["swiglu_with_probs"] = SwigluWithProbs
+    workloads["glu_quant_grouped"] = GluQuantGrouped
     workloads["quant_rowwise"] = QuantRowwise
     workloads["quant_blockwise"] = lambda dev: QuantBlockwise(dev, False)
     workloads["quant_blockwise_dual"] = lambda dev: QuantBlockwise(dev, True)

@@ -229,6 +229,21 @@ PT_API int pt_quantize_fp8_blockwise_segment_m_row_col_t(
     const int64_t *padded_group_offs, int64_t num_groups, void *q_row, float *scale_inv_row,
     void *q_col_padded, void *q_col_t, int64_t ldt, float *scale_inv_col_padded, void *stream);
 
+/* Gated activation fused into the grouped quantizer above: x is the fc1 output [M, 2 N] (gate
+ * columns, then up columns) and what gets quantized is
+ *   y[m, n] = T( act(x[m, n]) * x[m, N + n] * probs[m] ),   zero where row_mask[m] == 0,
+ * act = 0 SiLU, 1 exact (erf) GELU, T = x's 16-bit type: the value swiglu_with_probs /
+ * geglu_with_probs would store (primus_turbo/triton/activation/swiglu_kernel.py:11-248) followed
+ * by quantize_fp8_blockwise_segment_m_row_col (csrc/kernels/quantization/quantization_blockwise.cu:
+ * 60-232), without y ever travelling through HBM. Bit-identical with running the two steps of
+ * this library one after the other. The reference has no fused form. probs is fp32 [M], row_mask
+ * optional int64 [M]; give q_col_padded and / or q_col_t (with ldt) as above. */
+PT_API int pt_glu_quantize_fp8_blockwise_segment_m_row_col(
+    const void *x, int x_dtype, const float *probs, const int64_t *row_mask, int act, int64_t M, int64_t N,
+    int q_dtype, const int64_t *group_offs, const int64_t *padded_group_offs, int64_t num_groups, void *q_row,
+    float *scale_inv_row, void *q_col_padded, void *q_col_t, int64_t ldt, float *scale_inv_col_padded,
+    void *stream);
+
 /* De-quantize with one fp32 scale per (block_m x block_n) block of a [B, M, N] tensor:
  *   y[b, m, n] = T(float(q[b, m, n]) * scale_inv[b, m / block_m, n / block_n]).
  * (1, 128) / (128, 1) replace primus_turbo::dequant_fp8_blockwise_impl, (128, 128)

@@ -10,18 +10,10 @@
 // are written as zeros (the reference leaves them unwritten), and the GELU gradient of the gate
 // is grad_out * probs * up * gelu'(gate) (the reference multiplies by grad_out once more, which
 // only agrees for grad_out = 1).
-#include "pt_common.h"
+#include "pt_activation.h"
 
 namespace pt {
 
-enum : int { ACT_SILU = 0, ACT_GELU = 1 };
-
-template <int ACT> __device__ __forceinline__ float act_fwd(float g) {
-    if constexpr (ACT == ACT_SILU)
-        return g / (1.0f + expf(-g));
-    else
-        return 0.5f * g * (1.0f + erff(g * 0.7071067811f));
-}
 // -> (act(g), act'(g))
 template <int ACT> __device__ __forceinline__ void act_both(float g, float &a, float &da) {
     if constexpr (ACT == ACT_SILU) {

@@ -14,7 +14,7 @@
 // from HBM once; all requested outputs come from the register copy. A tile row is
 // spread over the 16 lanes of one DPP row, so the 1 x 128 amax is four DPP steps;
 // column maxima meet through 8 KB of LDS.
-#include "pt_common.h"
+#include "pt_activation.h"
 
 namespace pt {
 
@@ -42,6 +42,10 @@ struct BlockQuantArgs {
     // codes (MODE_COL: [N, ldt]): the operand a GEMM reads when it reduces over the rows of x
     uint8_t *q_t;
     int64_t  ldt;
+    // gated-activation input (grouped row + column mode): x is [M, 2 N], gate columns first, and
+    // the tile quantized is T(act(gate) * up * probs[row]), zero where row_mask[row] == 0
+    const float   *probs;
+    const int64_t *row_mask;
 };
 
 // Eight consecutive elements of a tile row as they come from memory (16-bit inputs stay packed:
@@ -168,9 +172,13 @@ __device__ __forceinline__ void flush_transposed(const uint32_t *t, uint8_t *out
 // segment-padded row space and map back to input rows through the group offsets.
 // VEC8: N % 8 == 0 and all pointers 16-byte aligned (128-bit loads, 64-bit stores).
 // TRANS: also emit the transposed copy described at BlockQuantArgs::q_t.
-template <typename T, bool E5M2, int MODE, bool GROUPED, bool VEC8, bool TRANS = false>
+// GLU: 0 = x is the tile source itself; 1 + ACT_SILU / 1 + ACT_GELU = x holds gate and up halves
+// and the gated activation (rounded to T, as the stand-alone activation kernel stores it) is what
+// gets quantized, so that the activation never travels through HBM.
+template <typename T, bool E5M2, int MODE, bool GROUPED, bool VEC8, bool TRANS = false, int GLU = 0>
 __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArgs a) {
     static_assert(!TRANS || ((MODE & MODE_TILE) != 0) != ((MODE & MODE_COL) != 0), "one transposed output");
+    static_assert(GLU == 0 || (GROUPED && sizeof(T) == 2), "the gated input belongs to the grouped 16-bit quantizer");
     __shared__ uint32_t s_tr[TRANS ? BQ * BQ_TP : 1];
     const int     tid   = threadIdx.x;
     const int     cseg  = tid & 15; // which 8-column segment of the tile row
@@ -202,14 +210,47 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
 
     // phase 1: the whole tile share of this thread is requested before anything is used
     Held8<T> held[BQ_ROUNDS];
+    if constexpr (GLU == 0) {
 #pragma unroll
-    for (int r = 0; r < BQ_ROUNDS; ++r) {
-        const int64_t in_m  = in_m0 + tile_row_of(rslot, r);
-        const bool    valid = in_m < in_end;
-        if (valid && full)
-            held[r].load(x + in_m * N + gn);
-        else
-            held[r].load_checked(x + in_m * N + gn, [&](int i) { return valid && gn + i < N; });
+        for (int r = 0; r < BQ_ROUNDS; ++r) {
+            const int64_t in_m  = in_m0 + tile_row_of(rslot, r);
+            const bool    valid = in_m < in_end;
+            if (valid && full)
+                held[r].load(x + in_m * N + gn);
+            else
+                held[r].load_checked(x + in_m * N + gn, [&](int i) { return valid && gn + i < N; });
+        }
+    } else {
+        Held8<T> up[BQ_ROUNDS];
+        float    pr[BQ_ROUNDS];
+#pragma unroll
+        for (int r = 0; r < BQ_ROUNDS; ++r) {
+            const int64_t in_m  = in_m0 + tile_row_of(rslot, r);
+            const bool    valid = in_m < in_end;
+            const T      *g     = x + in_m * 2 * N + gn;
+            if (valid && full) {
+                held[r].load(g);
+                up[r].load(g + N);
+            } else {
+                held[r].load_checked(g, [&](int i) { return valid && gn + i < N; });
+                up[r].load_checked(g + N, [&](int i) { return valid && gn + i < N; });
+            }
+            pr[r] = (valid && (a.row_mask == nullptr || a.row_mask[in_m] != 0)) ? a.probs[in_m] : 0.f;
+        }
+#pragma unroll
+        for (int r = 0; r < BQ_ROUNDS; ++r) {
+            const int64_t in_m = in_m0 + tile_row_of(rslot, r);
+            const bool    live = in_m < in_end && (a.row_mask == nullptr || a.row_mask[in_m] != 0);
+            float         fg[8], fu[8];
+            held[r].get(fg);
+            up[r].get(fu);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) // (padding columns hold zeros: act(0) * 0 = 0)
+                fg[i] = live ? act_fwd<GLU - 1>(fg[i]) * fu[i] * pr[r] : 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                held[r].w[i] = pack2<T>(fg[2 * i], fg[2 * i + 1]);
+        }
     }
 
     float col_amax[BQ_PACK];
@@ -321,13 +362,27 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
     }
 }
 
-template <typename T, bool E5M2, int MODE, bool GROUPED>
+template <typename T, bool E5M2, int MODE, bool GROUPED, int GLU = 0>
 static int launch_block128(const BlockQuantArgs &a, int64_t tiles_m, int64_t tiles_n, int64_t batch,
                            bool vec, hipStream_t stream) {
     if (tiles_m * tiles_n * batch == 0)
         return PT_OK;
     dim3 g(static_cast<unsigned>(tiles_n), static_cast<unsigned>(tiles_m),
            static_cast<unsigned>(batch));
+    if constexpr (GLU != 0) {
+        if (a.q_t != nullptr) {
+            if (vec)
+                quant_block128_kernel<T, E5M2, MODE, GROUPED, true, true, GLU><<<g, 256, 0, stream>>>(a);
+            else
+                quant_block128_kernel<T, E5M2, MODE, GROUPED, false, true, GLU><<<g, 256, 0, stream>>>(a);
+        } else {
+            if (vec)
+                quant_block128_kernel<T, E5M2, MODE, GROUPED, true, false, GLU><<<g, 256, 0, stream>>>(a);
+            else
+                quant_block128_kernel<T, E5M2, MODE, GROUPED, false, false, GLU><<<g, 256, 0, stream>>>(a);
+        }
+        return check_launch("quant_block128_kernel");
+    }
     if constexpr (MODE == MODE_TILE || MODE == (MODE_ROW | MODE_COL)) {
         if (a.q_t != nullptr) {
             if (vec)
@@ -580,8 +635,11 @@ int pt_compute_group_offs(const int64_t *group_lens, int64_t num_groups, int64_t
 static int quantize_segment_m(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype, const int64_t *group_offs,
                               const int64_t *padded_group_offs, int64_t num_groups, void *q_row, float *scale_inv_row,
                               void *q_col_padded, void *q_col_t, int64_t ldt, float *scale_inv_col_padded,
-                              void *stream) {
+                              void *stream, int glu = 0, const float *probs = nullptr,
+                              const int64_t *row_mask = nullptr) {
     PT_REQUIRE(is_hp_dtype(x_dtype), "input must be bf16, fp16 or fp32");
+    PT_REQUIRE(glu == 0 || ((x_dtype == PT_DTYPE_BF16 || x_dtype == PT_DTYPE_F16) && probs != nullptr),
+               "the gated input must be bf16 or fp16 and needs the router probabilities");
     PT_REQUIRE(is_fp8_dtype(q_dtype), "output must be e4m3 or e5m2");
     PT_REQUIRE(M >= 0 && N >= 0 && num_groups >= 1, "bad dimensions");
     PT_REQUIRE(group_offs && padded_group_offs, "group offsets must not be NULL");
@@ -610,8 +668,22 @@ static int quantize_segment_m(const void *x, int x_dtype, int64_t M, int64_t N, 
     a.padded_offs = padded_group_offs;
     a.num_groups = static_cast<int>(num_groups);
     a.qmax = fp8_max_of(q_dtype);
+    a.probs    = probs;
+    a.row_mask = row_mask;
     auto       st  = static_cast<hipStream_t>(stream);
     const bool vec = vec_ok(a, 1);
+    if (glu != 0) {
+        const bool e5 = q_dtype == PT_DTYPE_E5M2;
+#define CALL_GLU(T, E5, ACT) return launch_block128<T, E5, MODE_ROW | MODE_COL, true, 1 + ACT>(a, tm, tn, 1, vec, st)
+        if (x_dtype == PT_DTYPE_BF16) {
+            if (glu == 1 + ACT_SILU) { if (e5) CALL_GLU(bf16_t, true, ACT_SILU); else CALL_GLU(bf16_t, false, ACT_SILU); }
+            else { if (e5) CALL_GLU(bf16_t, true, ACT_GELU); else CALL_GLU(bf16_t, false, ACT_GELU); }
+        } else {
+            if (glu == 1 + ACT_SILU) { if (e5) CALL_GLU(f16_t, true, ACT_SILU); else CALL_GLU(f16_t, false, ACT_SILU); }
+            else { if (e5) CALL_GLU(f16_t, true, ACT_GELU); else CALL_GLU(f16_t, false, ACT_GELU); }
+        }
+#undef CALL_GLU
+    }
 #define CALL(T, E5) return launch_block128<T, E5, MODE_ROW | MODE_COL, true>(a, tm, tn, 1, vec, st)
     PT_DISPATCH_T_E5(x_dtype, q_dtype, CALL);
 #undef CALL
@@ -636,6 +708,18 @@ int pt_quantize_fp8_blockwise_segment_m_row_col_t(const void *x, int x_dtype, in
     PT_REQUIRE(q_col_t != nullptr, "q_col_t must not be NULL");
     return quantize_segment_m(x, x_dtype, M, N, q_dtype, group_offs, padded_group_offs, num_groups, q_row, scale_inv_row,
                               q_col_padded, q_col_t, ldt, scale_inv_col_padded, stream);
+}
+
+int pt_glu_quantize_fp8_blockwise_segment_m_row_col(const void *x, int x_dtype, const float *probs,
+                                                    const int64_t *row_mask, int act, int64_t M, int64_t N, int q_dtype,
+                                                    const int64_t *group_offs, const int64_t *padded_group_offs,
+                                                    int64_t num_groups, void *q_row, float *scale_inv_row,
+                                                    void *q_col_padded, void *q_col_t, int64_t ldt,
+                                                    float *scale_inv_col_padded, void *stream) {
+    PT_REQUIRE(act == ACT_SILU || act == ACT_GELU, "act must be 0 (SiLU) or 1 (GELU)");
+    PT_REQUIRE(q_col_padded != nullptr || q_col_t != nullptr, "NULL output pointer");
+    return quantize_segment_m(x, x_dtype, M, N, q_dtype, group_offs, padded_group_offs, num_groups, q_row, scale_inv_row,
+                              q_col_padded, q_col_t, ldt, scale_inv_col_padded, stream, 1 + act, probs, row_mask);
 }
 
 int pt_dequantize_fp8_block(const void *q, int q_dtype, int64_t B, int64_t M, int64_t N,

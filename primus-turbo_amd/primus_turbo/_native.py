@@ -97,6 +97,11 @@ _SIGNATURES = {
         [c_void_p, c_int, c_i64, c_i64, c_int, c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_void_p, c_void_p, c_i64,
          c_void_p, c_void_p],
     ),
+    "pt_glu_quantize_fp8_blockwise_segment_m_row_col": (
+        c_int,
+        [c_void_p, c_int, c_void_p, c_void_p, c_int, c_i64, c_i64, c_int, c_void_p, c_void_p, c_i64, c_void_p, c_void_p,
+         c_void_p, c_void_p, c_i64, c_void_p, c_void_p],
+    ),
     "pt_compute_group_offs": (c_int, [c_void_p, c_i64, c_i64, c_void_p, c_void_p, c_void_p]),
     "pt_quantize_fp8_blockwise_segment_m_row_col": (
         c_int,

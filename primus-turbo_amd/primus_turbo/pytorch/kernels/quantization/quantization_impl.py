@@ -703,6 +703,69 @@ def _quant_fp8_blockwise_segment_m_row_col_t_impl_fake(x, dtype, block_size, gro
             torch.empty(G, dtype=torch.int64, device=dev), torch.empty(G + 1, dtype=torch.int64, device=dev))
 
 
+_GLU_ACT = {"silu": 0, "gelu": 1}
+
+
+@torch.library.custom_op("primus_turbo::glu_quant_fp8_blockwise_segment_m_row_col_impl", mutates_args=())
+def glu_quant_fp8_blockwise_segment_m_row_col_impl(
+    x: torch.Tensor, probs: torch.Tensor, row_mask: Optional[torch.Tensor], act: str, dtype: torch.dtype,
+    block_size: int, group_lens: torch.Tensor, group_offs: torch.Tensor, transposed_col: bool,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Gated activation fused into the grouped quantizer: ``x [M, 2 N]`` is the fc1 output of an MoE
+    expert MLP and the tensor quantized is ``y = T(act(x[:, :N]) * x[:, N:] * probs[:, None])`` (zero
+    rows where ``row_mask`` is 0), i.e. what ``swiglu_with_probs`` / ``geglu_with_probs`` would store,
+    which never travels through HBM here. Outputs as :func:`quant_fp8_blockwise_segment_m_row_col_impl`
+    (``transposed_col=False``) or :func:`quant_fp8_blockwise_segment_m_row_col_t_impl` (``True``), bit
+    for bit what those give on the stored activation. (No counterpart in the reference.)"""
+    N.require_cuda(x, probs, row_mask, group_lens, group_offs)
+    _check(act in _GLU_ACT, "act must be 'silu' or 'gelu'")
+    _check(x.dtype in (torch.bfloat16, torch.float16), "input must be bfloat16 or float16")
+    _check_fp8_out(dtype)
+    _check(x.dim() == 2 and x.is_contiguous() and x.shape[1] % 2 == 0, "input must be a contiguous [M, 2 N] tensor")
+    _need_block_128(block_size)
+    M, Nn = x.shape[0], x.shape[1] // 2
+    _check(probs.numel() == M, "probs must hold one value per row")
+    p32 = probs.reshape(-1).to(torch.float32).contiguous()
+    mask = None
+    if row_mask is not None:
+        _check(row_mask.numel() == M, "row_mask must hold one value per row")
+        mask = row_mask.reshape(-1).to(torch.int64).contiguous()
+    for t in (group_lens, group_offs):
+        _check(t.dtype == torch.int64 and t.is_contiguous(), "group_lens / group_offs must be contiguous int64")
+    G = group_lens.numel()
+    _check(group_offs.numel() == G + 1, "group_offs must have one more element than group_lens")
+    Mp, rs_shape, cs_shape = _segment_shapes(M, Nn, G, block_size)
+    ldt = _segment_t_pitch(M, G, block_size)
+    dev = x.device
+    padded_lens, padded_offs = _group_offs(group_lens, block_size, True)
+    q_row = torch.empty((M, Nn), dtype=dtype, device=dev)
+    q_col = torch.empty((Nn, ldt) if transposed_col else (Mp, Nn), dtype=dtype, device=dev)
+    s_row = torch.empty(rs_shape, dtype=torch.float32, device=dev)
+    s_col = torch.empty(cs_shape, dtype=torch.float32, device=dev)
+    N.check(
+        N.lib().pt_glu_quantize_fp8_blockwise_segment_m_row_col(
+            N.ptr(x), N.dtype_code(x.dtype), N.ptr(p32), N.ptr(mask), _GLU_ACT[act], M, Nn, N.dtype_code(dtype),
+            N.ptr(group_offs), N.ptr(padded_offs), G, N.ptr(q_row), N.ptr(s_row),
+            None if transposed_col else N.ptr(q_col), N.ptr(q_col) if transposed_col else None, ldt, N.ptr(s_col),
+            N.stream_of(x),
+        )
+    )
+    return q_row, q_col, s_row, s_col, padded_lens, padded_offs
+
+
+@glu_quant_fp8_blockwise_segment_m_row_col_impl.register_fake
+def _glu_quant_fp8_blockwise_segment_m_row_col_impl_fake(x, probs, row_mask, act, dtype, block_size, group_lens, group_offs,
+                                                         transposed_col):
+    M, Nn = x.shape[0], x.shape[1] // 2
+    G = group_lens.numel()
+    Mp, rs_shape, cs_shape = _segment_shapes(M, Nn, G, block_size)
+    dev = x.device
+    return (torch.empty((M, Nn), dtype=dtype, device=dev),
+            torch.empty((Nn, _segment_t_pitch(M, G, block_size)) if transposed_col else (Mp, Nn), dtype=dtype, device=dev),
+            torch.empty(rs_shape, dtype=torch.float32, device=dev), torch.empty(cs_shape, dtype=torch.float32, device=dev),
+            torch.empty(G, dtype=torch.int64, device=dev), torch.empty(G + 1, dtype=torch.int64, device=dev))
+
+
 # ---------------------------------------------------------------------------------------
 # MX quantizers (E8M0 scale per 32 elements): MXFP8 and MXFP4
 # reference: primus_turbo/pytorch/kernels/quantization/quantization_impl.py:496-569,814-835,

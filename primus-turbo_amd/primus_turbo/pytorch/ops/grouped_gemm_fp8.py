@@ -41,6 +41,7 @@ from primus_turbo.pytorch.kernels.grouped_gemm.grouped_gemm_fp8_impl import (
 from primus_turbo.pytorch.kernels.grouped_gemm.grouped_gemm_utils import group_offs_from_lens
 from primus_turbo.pytorch.kernels.quantization.quantization_impl import (
     grouped_quantize_mxfp8_impl,
+    glu_quant_fp8_blockwise_segment_m_row_col_impl,
     quant_fp8_blockwise_for_weight_dual_impl,
     quant_fp8_blockwise_for_weight_impl,
     quant_fp8_blockwise_segment_m_row_col_impl,
@@ -55,7 +56,7 @@ from primus_turbo.pytorch.ops.utils import (
     _setup_fused_grad_accum,
 )
 
-__all__ = ["grouped_gemm_fp8"]
+__all__ = ["grouped_gemm_fp8", "glu_grouped_gemm_fp8"]
 
 _NATIVE = BackendType.TRITON.value  # placeholder id: a single backend exists here
 
@@ -72,6 +73,56 @@ def _grouped_gemm_fp8_variable_k_impl_wrapper(a, b, a_scales, b_scales, group_le
     grouped_gemm_fp8_variable_k_accum_impl(a, b, a_scales, b_scales, group_lens, group_offs, trans_a, trans_b,
                                            trans_c, out.dtype, granularity, num_cu, default_backend, out)
     return _get_dummy_wgrad(out.shape, out_dtype)
+
+
+def _block_forward_product(a_fp8_row, a_scale_row, b, group_lens, group_offs, trans_b, out_dtype, config, num_cu, need_bwd):
+    """Quantize the BLOCKWISE weight (2-D blocks; with the transposed copy for the backward product
+    when it is needed and possible) and multiply -> ``(out, (weight codes, scales) for dgrad,
+    whether those are K-contiguous for dgrad already)``."""
+    bs = config.block_size
+    b_dtype = _get_fp8_dtype(config.format, True)
+    b_recipe = ScalingRecipe(use_2d_block=True)
+    b_fp8_t = None
+    if isinstance(b, QuantizedTensor):
+        check_quantized_tensor(b, config, scaling_recipe=b_recipe)
+        b_fp8, b_scale = b.qdata, b.scale_inv
+    elif (need_bwd or not trans_b) and b.size(-2) % 16 == 0:
+        b_fp8, b_fp8_t, b_scale = quant_fp8_blockwise_for_weight_dual_impl(b, b_dtype, block_size=bs)
+    else:
+        b_fp8, b_scale = quant_fp8_blockwise_for_weight_impl(b, b_dtype, block_size=bs)
+
+    # fwd reduces over b's last axis when trans_b, else over its middle axis
+    fwd_b, dgrad_b = (b_fp8, b_fp8_t) if trans_b else (b_fp8_t, b_fp8)
+    b_scale_t = b_scale.transpose(-2, -1).contiguous() if b_fp8_t is not None else None
+    fwd_s, dgrad_s = (b_scale, b_scale_t) if trans_b else (b_scale_t, b_scale)
+    if fwd_b is not None:
+        out = grouped_gemm_fp8_impl(a_fp8_row, fwd_b, a_scale_row, fwd_s, group_lens, group_offs, False, True,
+                                    out_dtype, config.granularity.value, num_cu, _NATIVE)
+    else:
+        out = grouped_gemm_fp8_impl(a_fp8_row, b_fp8, a_scale_row, b_scale, group_lens, group_offs, False, trans_b,
+                                    out_dtype, config.granularity.value, num_cu, _NATIVE)
+    if dgrad_b is not None:
+        return out, (dgrad_b, dgrad_s), True
+    return out, (b_fp8, b_scale), False
+
+
+def _block_backward_products(grad_out, a_fp8_col_t, a_scale_col, b_fp8, b_scale, group_lens, group_offs, trans_b, config,
+                             out_dtype, num_cu, b_ready, fuse_bgrad_accum, main_grad):
+    """dgrad and variable-K wgrad of the BLOCKWISE grouped layer -> ``(grad_a, grad_b)``."""
+    g_dtype = _get_fp8_dtype(config.format, False)
+    gran = config.granularity.value
+    g_row, g_col_t, g_scale_row, g_scale_col, var_k_lens, var_k_offs = quant_fp8_blockwise_segment_m_row_col_t_impl(
+        grad_out, g_dtype, config.block_size, group_lens, group_offs)
+    # grad_a = grad_out @ b^T: the saved weight copy is contiguous along the reduction already,
+    # or (caller-quantized weight) the forward operand read the other way round
+    grad_a = grouped_gemm_fp8_impl(g_row, b_fp8, g_scale_row, b_scale, group_lens, group_offs, False,
+                                   True if b_ready else not trans_b, out_dtype, gran, num_cu, _NATIVE)
+    # grad_b[g] = a_g^T @ grad_out_g over the padded token ranges, both operands K-major
+    grad_b = _grouped_gemm_fp8_variable_k_impl_wrapper(
+        a_fp8_col_t, g_col_t, a_scale_col, g_scale_col, var_k_lens, var_k_offs, False, True, trans_b, out_dtype, gran,
+        num_cu, _NATIVE, inplace_add_to_out=fuse_bgrad_accum, out=main_grad,
+    )
+    return grad_a, grad_b
 
 
 class FP8GroupedGemmBlockFunc(torch.autograd.Function):
@@ -104,32 +155,11 @@ class FP8GroupedGemmBlockFunc(torch.autograd.Function):
             a_fp8_row, _, a_scale_row, _, _, _ = quant_fp8_blockwise_segment_m_row_col_impl(
                 a.contiguous(), a_dtype, bs, group_lens, group_offs)
             a_fp8_col_t = a_scale_col = None
-        b_recipe = ScalingRecipe(use_2d_block=True)
-        b_fp8_t = None
-        if isinstance(b, QuantizedTensor):
-            check_quantized_tensor(b, config, scaling_recipe=b_recipe)
-            b_fp8, b_scale = b.qdata, b.scale_inv
-        elif (need_bwd or not trans_b) and b.size(-2) % 16 == 0:
-            b_fp8, b_fp8_t, b_scale = quant_fp8_blockwise_for_weight_dual_impl(b, b_dtype, block_size=bs)
-        else:
-            b_fp8, b_scale = quant_fp8_blockwise_for_weight_impl(b, b_dtype, block_size=bs)
-
-        # fwd reduces over b's last axis when trans_b, else over its middle axis
-        fwd_b, dgrad_b = (b_fp8, b_fp8_t) if trans_b else (b_fp8_t, b_fp8)
-        b_scale_t = b_scale.transpose(-2, -1).contiguous() if b_fp8_t is not None else None
-        fwd_s, dgrad_s = (b_scale, b_scale_t) if trans_b else (b_scale_t, b_scale)
-        if fwd_b is not None:
-            out = grouped_gemm_fp8_impl(a_fp8_row, fwd_b, a_scale_row, fwd_s, group_lens, group_offs, False, True,
-                                        out_dtype, config.granularity.value, num_cu, _NATIVE)
-        else:
-            out = grouped_gemm_fp8_impl(a_fp8_row, b_fp8, a_scale_row, b_scale, group_lens, group_offs, False, trans_b,
-                                        out_dtype, config.granularity.value, num_cu, _NATIVE)
+        out, saved_b, b_ready = _block_forward_product(a_fp8_row, a_scale_row, b, group_lens, group_offs, trans_b, out_dtype,
+                                                       config, num_cu, need_bwd)
         if need_bwd:
-            if dgrad_b is not None:
-                ctx.save_for_backward(a_fp8_col_t, a_scale_col, dgrad_b, dgrad_s, group_lens, group_offs)
-            else:
-                ctx.save_for_backward(a_fp8_col_t, a_scale_col, b_fp8, b_scale, group_lens, group_offs)
-        ctx.meta = (trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad, dgrad_b is not None)
+            ctx.save_for_backward(a_fp8_col_t, a_scale_col, saved_b[0], saved_b[1], group_lens, group_offs)
+        ctx.meta = (trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad, b_ready)
         return out
 
     @staticmethod
@@ -137,21 +167,49 @@ class FP8GroupedGemmBlockFunc(torch.autograd.Function):
         grad_out = _ensure_contiguous_grad_out(grad_out)
         a_fp8_col_t, a_scale_col, b_fp8, b_scale, group_lens, group_offs = ctx.saved_tensors
         trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad, b_ready = ctx.meta
-        g_dtype = _get_fp8_dtype(config.format, False)
-        gran = config.granularity.value
-
-        g_row, g_col_t, g_scale_row, g_scale_col, var_k_lens, var_k_offs = quant_fp8_blockwise_segment_m_row_col_t_impl(
-            grad_out, g_dtype, config.block_size, group_lens, group_offs)
-        # grad_a = grad_out @ b^T: the saved weight copy is contiguous along the reduction already,
-        # or (caller-quantized weight) the forward operand read the other way round
-        grad_a = grouped_gemm_fp8_impl(g_row, b_fp8, g_scale_row, b_scale, group_lens, group_offs, False,
-                                       True if b_ready else not trans_b, out_dtype, gran, num_cu, _NATIVE)
-        # grad_b[g] = a_g^T @ grad_out_g over the padded token ranges, both operands K-major
-        grad_b = _grouped_gemm_fp8_variable_k_impl_wrapper(
-            a_fp8_col_t, g_col_t, a_scale_col, g_scale_col, var_k_lens, var_k_offs, False, True, trans_b, out_dtype, gran,
-            num_cu, _NATIVE, inplace_add_to_out=fuse_bgrad_accum, out=main_grad,
-        )
+        grad_a, grad_b = _block_backward_products(grad_out, a_fp8_col_t, a_scale_col, b_fp8, b_scale, group_lens, group_offs,
+                                                  trans_b, config, out_dtype, num_cu, b_ready, fuse_bgrad_accum, main_grad)
         return grad_a, grad_b, None, None, None, None, None, None, None, None, None
+
+
+class FP8GluGroupedGemmBlockFunc(torch.autograd.Function):
+    """Gated activation -> BLOCKWISE grouped GEMM (fc2 of an MoE expert MLP) with the activation
+    fused into the quantizer of the GEMM's activation operand: the bf16 activation is neither
+    written nor re-read, forward or backward (wgrad uses the column codes saved by the fused
+    quantizer, the activation backward needs fc1's output only)."""
+
+    @staticmethod
+    def forward(ctx, x, probs, row_mask, act_type, b, group_lens, group_offs, trans_b, out_dtype, config, num_cu,
+                fuse_bgrad_accum_pattern=None):
+        fuse_bgrad_accum, main_grad = _setup_fused_grad_accum(b, fuse_bgrad_accum_pattern)
+        assert config.granularity == ScalingGranularity.BLOCKWISE and config.block_size in [128]
+        assert x.ndim == 2 and x.size(1) % 2 == 0, "x must be [tokens, 2 * hidden]"
+        assert b.ndim == 3 and group_lens.size(0) == b.size(0)
+        assert probs.dtype == torch.float32 and probs.numel() == x.size(0), "probs must be float32, one per token"
+        assert out_dtype in [torch.float16, torch.bfloat16]
+        need_bwd = any(ctx.needs_input_grad[i] for i in (0, 1, 4))
+        x2, p1 = x.contiguous(), probs.reshape(-1).contiguous()
+        a_fp8_row, a_col, a_scale_row, a_scale_col, _, _ = glu_quant_fp8_blockwise_segment_m_row_col_impl(
+            x2, p1, row_mask, act_type, _get_fp8_dtype(config.format, True), config.block_size, group_lens, group_offs,
+            need_bwd)
+        out, saved_b, b_ready = _block_forward_product(a_fp8_row, a_scale_row, b, group_lens, group_offs, trans_b, out_dtype,
+                                                       config, num_cu, need_bwd)
+        if need_bwd:
+            ctx.save_for_backward(x2, p1, row_mask, a_col, a_scale_col, saved_b[0], saved_b[1], group_lens, group_offs)
+        ctx.meta = (trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad, b_ready, act_type, probs.shape)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        from primus_turbo.pytorch.kernels.activation.glu_impl import ACT_GELU, ACT_SILU, glu_bwd_with_probs
+
+        grad_out = _ensure_contiguous_grad_out(grad_out)
+        x2, p1, row_mask, a_col_t, a_scale_col, b_fp8, b_scale, group_lens, group_offs = ctx.saved_tensors
+        trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad, b_ready, act_type, probs_shape = ctx.meta
+        grad_act, grad_b = _block_backward_products(grad_out, a_col_t, a_scale_col, b_fp8, b_scale, group_lens, group_offs,
+                                                    trans_b, config, x2.dtype, num_cu, b_ready, fuse_bgrad_accum, main_grad)
+        grad_x, grad_probs = glu_bwd_with_probs(grad_act, x2, p1, row_mask, ACT_SILU if act_type == "silu" else ACT_GELU)
+        return grad_x, grad_probs.view(probs_shape), None, None, grad_b, None, None, None, None, None, None, None
 
 
 def _quantize_plain(x, config, fwd: bool, axis: int):
@@ -363,3 +421,35 @@ def grouped_gemm_fp8(
     raise NotImplementedError(
         f"grouped_gemm_fp8: unknown granularity {config.granularity}"
     )
+
+
+def glu_grouped_gemm_fp8(
+    x: torch.Tensor,
+    probs: torch.Tensor,
+    b: Union[torch.Tensor, QuantizedTensor],
+    group_lens: torch.Tensor,
+    group_offs: Optional[torch.Tensor] = None,
+    trans_b: bool = True,
+    out_dtype: Optional[torch.dtype] = None,
+    config: Optional[Float8QuantConfig] = None,
+    num_cu: Optional[int] = None,
+    row_mask: Optional[torch.Tensor] = None,
+    act_type: str = "silu",
+    fuse_bgrad_accum_pattern: Optional[str] = None,
+) -> torch.Tensor:
+    """``grouped_gemm_fp8(swiglu_with_probs(x, probs, row_mask), b, group_lens, ...)`` (``act_type="gelu"``:
+    ``geglu_with_probs``) as one operation for the BLOCKWISE configuration: fc1's output ``x [tokens, 2 H]``
+    is read once by a quantizer that applies the gated activation on load, so the bf16 activation
+    never goes through HBM; results and gradients are bit-identical with the two-step form. (The
+    reference has the two steps only: ops/activation.py:21-83, ops/grouped_gemm_fp8.py:99-265.)"""
+    if config is None:
+        config = Float8QuantConfig(granularity=ScalingGranularity.BLOCKWISE, block_size=128)
+    if config.granularity != ScalingGranularity.BLOCKWISE:
+        raise NotImplementedError("glu_grouped_gemm_fp8: the fused quantizer exists for the BLOCKWISE configuration")
+    assert act_type in ("silu", "gelu"), f"Unsupported act_type: {act_type}"
+    if group_offs is None:
+        group_offs = group_offs_from_lens(group_lens)
+    if out_dtype is None:
+        out_dtype = torch.promote_types(x.dtype, b.dtype)
+    return FP8GluGroupedGemmBlockFunc.apply(x, probs, row_mask, act_type, b, group_lens, group_offs, trans_b, out_dtype,
+                                            config, num_cu, fuse_bgrad_accum_pattern)
