@@ -341,7 +341,9 @@ PT_API int pt_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const v
  * codes per byte, K counts codes). a_scale [M, >= K / 32] and b_scale [N, >= K / 32] are E8M0
  * bytes with row pitches sa_ld / sb_ld. K % 32 == 0; bytes of a row behind K must be zero
  * codes, as the MX quantizers leave them. Rows that are not whole 128-byte slabs (at least
- * four) are first copied into `workspace` (pt_gemm_mx_workspace_bytes, 16-byte aligned).
+ * four) are first copied into `workspace` (pt_gemm_mx_workspace_bytes, 16-byte aligned); for
+ * large problems the workspace also receives a copy of both scale arrays with the 32-bit words
+ * of one K position of all rows contiguous, which is what the kernel's scale copies then read.
  * accumulate != 0 adds into C (beta = 1). tile_cfg as for pt_gemm_fp8. */
 PT_API size_t pt_gemm_mx_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                                          int fp4);

@@ -54,8 +54,12 @@ struct GemmArgs {
     int64_t        lda, ldb;    // row pitch of A and B in bytes (>= K)
     // VECTOR: sA[m * sa_m], sB[n * sb_n]                      (stride 0 = one scalar)
     // BLOCK : sA[(m >> sa_shift) * sa_m + kb * sa_k], sB[(n >> sb_shift) * sb_n + kb * sb_k]
-    // MX    : sA / sB point at E8M0 bytes, byte[m * sa_m + kb] and byte[n * sb_n + kb]
+    // MX    : sA / sB point at E8M0 bytes, byte[m * sa_m + kb] and byte[n * sb_n + kb];
+    //         or, "word-major" (sa_wpitch, sb_wpitch != 0): the 32-bit word w of row m (its K blocks
+    //         4 w .. 4 w + 3) at byte m * 4 + w * sa_wpitch, i.e. the words of one K position of all
+    //         rows are contiguous and a scale copy fetches two cache lines instead of sixty-four
     int64_t sa_m, sa_k, sb_n, sb_k;
+    int64_t sa_wpitch, sb_wpitch;
     int     sa_shift, sb_shift; // 0 (one scale per row) or 7 (one per 128 rows)
     int     kb_valid;           // BLOCK / MX: K blocks the scale arrays hold (slabs beyond are zero padding)
     int     out_dtype;
@@ -544,6 +548,13 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     // the compiler would use to sink MFMAs -- and it does so after requesting the tile's last
     // slab, two steps before the MFMAs get there (the host guarantees KT > 2). Without
     // cross-tile pipelining it stops at the tile's last slab and keeps re-reading that one.
+    // scale addressing in bytes: from one row (column) to the next, and (MX) from one 32-bit word
+    // of a row to its next
+    [[maybe_unused]] const bool     mx_wordmajor = MODE == SCALE_MX && a.sa_wpitch != 0;
+    [[maybe_unused]] const uint32_t sa_rowp  = mx_wordmajor ? 4u : static_cast<uint32_t>(a.sa_m) * (MODE == SCALE_MX ? 1 : 4);
+    [[maybe_unused]] const uint32_t sb_rowp  = mx_wordmajor ? 4u : static_cast<uint32_t>(a.sb_n) * (MODE == SCALE_MX ? 1 : 4);
+    [[maybe_unused]] const uint32_t sa_wordp = mx_wordmajor ? static_cast<uint32_t>(a.sa_wpitch) : 4u;
+    [[maybe_unused]] const uint32_t sb_wordp = mx_wordmajor ? static_cast<uint32_t>(a.sb_wpitch) : 4u;
     uint32_t off[NL];
     {
         const int lrow = lane >> 3, pchk = lane & 7;
@@ -560,10 +571,11 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         for (int q = 0; q < NSC; ++q) {
             const int e = (q % (SC_ROWS / 64)) * 64 + lane;
             if (e < SC_A)
-                off[NLD + q] = static_cast<uint32_t>((wm * SC_A + e) >> a.sa_shift) * static_cast<uint32_t>(a.sa_m) * SC_ELT;
+                off[NLD + q] = static_cast<uint32_t>((wm * SC_A + e) >> a.sa_shift) * sa_rowp +
+                               (q / (SC_ROWS / 64)) * sa_wordp; // (+ the second scale word of an MXFP4 slab)
             else
-                off[NLD + q] = static_cast<uint32_t>((wn * SC_B + e - SC_A) >> a.sb_shift) * static_cast<uint32_t>(a.sb_n) * SC_ELT;
-            off[NLD + q] += (q / (SC_ROWS / 64)) * 4; // second scale word of an MXFP4 slab
+                off[NLD + q] = static_cast<uint32_t>((wn * SC_B + e - SC_A) >> a.sb_shift) * sb_rowp +
+                               (q / (SC_ROWS / 64)) * sb_wordp;
         }
     }
     const uint8_t *ld_ga, *ld_gb; // slab the loader points at
@@ -574,18 +586,18 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     // arrays (reads beyond return zero; they only ever meet rows that are never stored)
     [[maybe_unused]] const uint8_t *ld_sa = nullptr, *ld_sb = nullptr, *ld_sa_end = nullptr, *ld_sb_end = nullptr;
     [[maybe_unused]] const int64_t  sa_extent =
-        MODE == SCALE_MX ? (a.M - 1) * a.sa_m + a.kb_valid
+        MODE == SCALE_MX ? (mx_wordmajor ? static_cast<int64_t>((a.kb_valid + 3) / 4) * a.sa_wpitch : (a.M - 1) * a.sa_m + a.kb_valid)
                          : (((a.M - 1) >> a.sa_shift) * a.sa_m + (a.kb_valid - 1) * a.sa_k + 1) * 4;
     [[maybe_unused]] const int64_t sb_extent =
-        MODE == SCALE_MX ? (a.N - 1) * a.sb_n + a.kb_valid
+        MODE == SCALE_MX ? (mx_wordmajor ? static_cast<int64_t>((a.kb_valid + 3) / 4) * a.sb_wpitch : (a.N - 1) * a.sb_n + a.kb_valid)
                          : (((a.N - 1) >> a.sb_shift) * a.sb_n + (a.kb_valid - 1) * a.sb_k + 1) * 4;
-    [[maybe_unused]] const int64_t sa_step = MODE == SCALE_MX ? 4 * NW : a.sa_k * 4; // bytes per slab
-    [[maybe_unused]] const int64_t sb_step = MODE == SCALE_MX ? 4 * NW : a.sb_k * 4;
+    [[maybe_unused]] const int64_t sa_step = MODE == SCALE_MX ? static_cast<int64_t>(NW) * sa_wordp : a.sa_k * 4; // bytes per slab
+    [[maybe_unused]] const int64_t sb_step = MODE == SCALE_MX ? static_cast<int64_t>(NW) * sb_wordp : a.sb_k * 4;
     auto as_bytes = [](const float *p) { return reinterpret_cast<const uint8_t *>(p); };
     auto scales_to = [&](const TileCtx &t) {
         if constexpr (LDS_SC) {
-            ld_sa     = as_bytes(t.sA) + ((t.m0 >> a.sa_shift) * a.sa_m) * SC_ELT;
-            ld_sb     = as_bytes(t.sB) + ((t.n0 >> a.sb_shift) * a.sb_n) * SC_ELT;
+            ld_sa     = as_bytes(t.sA) + (t.m0 >> a.sa_shift) * sa_rowp;
+            ld_sb     = as_bytes(t.sB) + (t.n0 >> a.sb_shift) * sb_rowp;
             ld_sa_end = as_bytes(GMODE == GROUP_K ? a.sA : t.sA) + sa_extent;
             ld_sb_end = as_bytes(GMODE == GROUP_K ? a.sB : t.sB) + sb_extent;
         }
@@ -645,8 +657,8 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             ld_na = wrap ? nxt_t.rows_a * static_cast<uint32_t>(a.lda) : ld_na - KSTEP;
             ld_nb = wrap ? nxt_t.rows_b * static_cast<uint32_t>(a.ldb) : ld_nb - KSTEP;
             if constexpr (LDS_SC) {
-                const uint8_t *na = as_bytes(nxt_t.sA) + ((nxt_t.m0 >> a.sa_shift) * a.sa_m) * SC_ELT;
-                const uint8_t *nb = as_bytes(nxt_t.sB) + ((nxt_t.n0 >> a.sb_shift) * a.sb_n) * SC_ELT;
+                const uint8_t *na = as_bytes(nxt_t.sA) + (nxt_t.m0 >> a.sa_shift) * sa_rowp;
+                const uint8_t *nb = as_bytes(nxt_t.sB) + (nxt_t.n0 >> a.sb_shift) * sb_rowp;
                 ld_sa             = wrap ? na : ld_sa + sa_step;
                 ld_sb             = wrap ? nb : ld_sb + sb_step;
                 ld_sa_end         = wrap ? as_bytes(nxt_t.sA) + sa_extent : ld_sa_end;
@@ -945,7 +957,8 @@ static int launch_gemm_cfg(const GemmArgs &args_in, hipStream_t stream) {
     if (MODE == SCALE_BLOCK && ((!SB_VEC && a.sb_shift != 7) || (GMODE == GROUP_ROWS && a.sa_shift != 0)))
         return fail(PT_ERR_INVALID_ARGUMENT, "gemm_fp8: unsupported block-scale layout");
     // MX scale words are fetched as aligned 32-bit units
-    if (MODE == SCALE_MX && (a.sa_shift != 0 || a.sb_shift != 0 || a.sa_m % 4 != 0 || a.sb_n % 4 != 0 ||
+    if (MODE == SCALE_MX && (a.sa_shift != 0 || a.sb_shift != 0 || (a.sa_wpitch == 0 && (a.sa_m % 4 != 0 || a.sb_n % 4 != 0)) ||
+                             (a.sa_wpitch != 0) != (a.sb_wpitch != 0) || a.sa_wpitch % 4 != 0 || a.sb_wpitch % 4 != 0 ||
                              reinterpret_cast<uintptr_t>(a.sA) % 4 != 0 || reinterpret_cast<uintptr_t>(a.sB) % 4 != 0))
         return fail(PT_ERR_INVALID_ARGUMENT, "gemm_mx: scale rows must be 4-byte aligned");
     auto kern            = gemm_fp8_nt_kernel<TM, TN, MODE, SB_VEC, FA, FB, GMODE>;

@@ -16,6 +16,33 @@ template <int FA, int FB> static int launch_mx_tiles(const GemmArgs &a, int tile
     return launch_gemm_cfg<4, 4, SCALE_MX, false, FA, FB>(a, stream);
 }
 
+// out[w, r] = in[r * pitch + w] for w < W: the scale words of one K position of all rows made
+// contiguous (32 x 32 word tiles through LDS, coalesced on both sides)
+__global__ __launch_bounds__(256) void transpose_words_kernel(const uint32_t *__restrict__ in, uint32_t *__restrict__ out,
+                                                              const int64_t R, const int64_t W, const int64_t pitch) {
+    __shared__ uint32_t t[32][33];
+    const int64_t r0 = static_cast<int64_t>(blockIdx.y) * 32, w0 = static_cast<int64_t>(blockIdx.x) * 32;
+    const int     tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int64_t r = r0 + ty + 8 * p, w = w0 + tx;
+        if (r < R && w < W)
+            t[ty + 8 * p][tx] = in[r * pitch + w];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int64_t w = w0 + ty + 8 * p, r = r0 + tx;
+        if (w < W && r < R)
+            out[w * R + r] = t[tx][ty + 8 * p];
+    }
+}
+
+static void launch_transpose_words(const uint32_t *in, uint32_t *out, int64_t R, int64_t W, int64_t pitch, hipStream_t st) {
+    dim3 g(static_cast<unsigned>(cdiv(W, 32)), static_cast<unsigned>(cdiv(R, 32)));
+    transpose_words_kernel<<<g, 256, 0, st>>>(in, out, R, W, pitch);
+}
+
 } // namespace pt
 
 using namespace pt;
@@ -27,9 +54,21 @@ static int64_t mx_row_bytes(int64_t K, bool fp4) {
     return padded_k(fp4 ? cdiv(K, 2) : K);
 }
 
+// Word-major copy of a scale array: [rows, K / 128 words] 32-bit words transposed to [words, rows].
+// Done for problems whose scale traffic matters (large K loops over many rows): a few microseconds
+// on a few megabytes, against 64 separate cache lines per scale copy instruction in the GEMM.
+static bool mx_wordmajor_pays(int64_t M, int64_t N, int64_t K) {
+    return M >= 1024 && N >= 1024 && K >= 1024;
+}
+static int64_t mx_scale_words(int64_t K) {
+    return cdiv(K / 32, 4);
+}
+
 size_t pt_gemm_mx_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int fp4) {
     const int64_t need = mx_row_bytes(K, fp4 != 0);
     size_t        b    = 0;
+    if (mx_wordmajor_pays(M, N, K))
+        b += static_cast<size_t>(round_up(M * mx_scale_words(K) * 4, 256) + round_up(N * mx_scale_words(K) * 4, 256));
     if (lda != need)
         b += static_cast<size_t>(round_up(M * need, 256));
     if (ldb != need)
@@ -60,11 +99,25 @@ int pt_gemm_mx(const void *a, const void *a_scale, const void *b, const void *b_
     // that carry anything but zeros behind K, into zero-padded rows
     const int64_t  need = mx_row_bytes(K, fp4);
     const uint8_t *A = static_cast<const uint8_t *>(a), *B = static_cast<const uint8_t *>(b);
-    if (lda != need || ldb != need) {
+    // word-major scales need whole 32-bit words per row in the source
+    const bool     wordmajor = mx_wordmajor_pays(M, N, K) && sa_ld % 4 == 0 && sb_ld % 4 == 0 && aligned_to(a_scale, 4) &&
+                           aligned_to(b_scale, 4) && sa_ld >= mx_scale_words(K) * 4 && sb_ld >= mx_scale_words(K) * 4;
+    const void *sa_use = a_scale, *sb_use = b_scale;
+    if (lda != need || ldb != need || wordmajor) {
         const size_t want = pt_gemm_mx_workspace_bytes(M, N, K, lda, ldb, fp4);
         if (workspace == nullptr || workspace_bytes < want || !aligned_to(workspace, 16))
             return fail(PT_ERR_WORKSPACE, "pt_gemm_mx: workspace missing, too small or misaligned");
         uint8_t *ws = static_cast<uint8_t *>(workspace);
+        if (wordmajor) {
+            const int64_t W = mx_scale_words(K);
+            // in: [rows, sa_ld / 4] words (the first W of every row are used) -> out: [W, rows]
+            launch_transpose_words(static_cast<const uint32_t *>(a_scale), reinterpret_cast<uint32_t *>(ws), M, W, sa_ld / 4, st);
+            sa_use = ws;
+            ws += round_up(M * W * 4, 256);
+            launch_transpose_words(static_cast<const uint32_t *>(b_scale), reinterpret_cast<uint32_t *>(ws), N, W, sb_ld / 4, st);
+            sb_use = ws;
+            ws += round_up(N * W * 4, 256);
+        }
         if (lda != need) {
             launch_pad_rows2(A, ws, M, kbytes, lda, need, st);
             A = ws;
@@ -80,8 +133,10 @@ int pt_gemm_mx(const void *a, const void *a_scale, const void *b, const void *b_
     g.A          = A;
     g.B          = B;
     g.C          = c;
-    g.sA         = reinterpret_cast<const float *>(a_scale); // E8M0 bytes in this mode
-    g.sB         = reinterpret_cast<const float *>(b_scale);
+    g.sA         = reinterpret_cast<const float *>(sa_use); // E8M0 bytes in this mode
+    g.sB         = reinterpret_cast<const float *>(sb_use);
+    g.sa_wpitch  = wordmajor ? M * 4 : 0;
+    g.sb_wpitch  = wordmajor ? N * 4 : 0;
     g.M          = M;
     g.N          = N;
     g.K          = need;
