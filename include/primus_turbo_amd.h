@@ -315,7 +315,11 @@ PT_API int pt_dequantize_mx(const void *q, int q_dtype, const void *scale, int64
  *                            * b_scale[(n / sb_block) * sb_n + kb * sb_k]
  *     sa_block / sb_block are 1 (1 x 128 activation blocks) or 128 (128 x 128 tiles).
  * accumulate != 0 adds into C (beta = 1) instead of overwriting it.
- * tile_cfg: 0 = automatic, 1 = 256x256, 2 = 256x128, 3 = 128x128 workgroup tile.
+ * tile_cfg: 0 = automatic, 1 = 256x256, 2 = 256x128, 3 = 128x128 workgroup tile,
+ *           4 = 256x256 with eight wavefronts (block scales with 128 x 128 B blocks).
+ * For large problems the workspace also holds a [K / 128, M] copy of per-row block scales that
+ * arrive as [M, K / 128] (sa_block == 1, sa_k == 1): the kernel's scale copies then read
+ * contiguous memory. It is made only when the workspace has the size the function reports.
  * Requirements: a, b, c 16-byte aligned.
  */
 PT_API size_t pt_gemm_fp8_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans_a,

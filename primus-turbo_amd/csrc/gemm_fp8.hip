@@ -144,6 +144,33 @@ void launch_transpose(const uint8_t *in, uint8_t *out, int64_t batch, int64_t R,
     transpose_u8_kernel<<<g, 256, 0, st>>>(in, out, R, C, ldo);
 }
 
+// out[w, r] = in[r * pitch + w] for w < W: the scale words of one K position of all rows made
+// contiguous (32 x 32 word tiles through LDS, coalesced on both sides)
+__global__ __launch_bounds__(256) void transpose_words_kernel(const uint32_t *__restrict__ in, uint32_t *__restrict__ out,
+                                                              const int64_t R, const int64_t W, const int64_t pitch) {
+    __shared__ uint32_t t[32][33];
+    const int64_t r0 = static_cast<int64_t>(blockIdx.y) * 32, w0 = static_cast<int64_t>(blockIdx.x) * 32;
+    const int     tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int64_t r = r0 + ty + 8 * p, w = w0 + tx;
+        if (r < R && w < W)
+            t[ty + 8 * p][tx] = in[r * pitch + w];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int64_t w = w0 + ty + 8 * p, r = r0 + tx;
+        if (w < W && r < R)
+            out[w * R + r] = t[tx][ty + 8 * p];
+    }
+}
+
+void launch_transpose_words(const uint32_t *in, uint32_t *out, int64_t R, int64_t W, int64_t pitch, hipStream_t st) {
+    dim3 g(static_cast<unsigned>(cdiv(W, 32)), static_cast<unsigned>(cdiv(R, 32)));
+    transpose_words_kernel<<<g, 256, 0, st>>>(in, out, R, W, pitch);
+}
+
 template <int FA, int FB>
 static int launch_vector_tiles(const GemmArgs &a, int tile_cfg, hipStream_t stream) {
     // tile_cfg: 0 = auto, 1 = 256x256, 2 = 256x128, 3 = 128x128
@@ -208,12 +235,22 @@ using namespace pt;
 
 extern "C" {
 
+// Block-scale GEMMs whose A scales are stored one row of K blocks per matrix row ([M, K / 128],
+// the 1 x 128 activation quantizer's layout) get a copy with the scales of one K block of all rows
+// contiguous ([K / 128, M]): a scale copy of the kernel (64 rows per instruction) then reads two
+// cache lines instead of sixty-four.
+static bool block_scale_copy_pays(int64_t M, int64_t N, int64_t K) {
+    return M >= 1024 && N >= 1024 && K >= 1024;
+}
+
 size_t pt_gemm_fp8_workspace_bytes(int64_t M, int64_t N, int64_t K, int trans_a, int trans_b) {
     // An operand is copied into the workspace when its reduction axis is not contiguous
     // (transpose) or when K is not a multiple of 128 (zero padding of the K tail).
     const int64_t Kp    = padded_k(K);
     const bool    pad   = Kp != K;
     size_t        bytes = 0;
+    if (block_scale_copy_pays(M, N, K))
+        bytes += static_cast<size_t>(round_up(M * cdiv(K, 128) * 4, 256));
     if (trans_a || pad)
         bytes += static_cast<size_t>(round_up(M * Kp, 256));
     if (!trans_b || pad)
@@ -254,11 +291,22 @@ int pt_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const void *b,
     const bool     pad = Kp != K;
     const uint8_t *A   = static_cast<const uint8_t *>(a);
     const uint8_t *B   = static_cast<const uint8_t *>(b);
+    // workspace layout: [scale area of block_scale_copy_pays problems][operand copies]
+    const int64_t KB         = cdiv(K, 128);
+    const size_t  full       = pt_gemm_fp8_workspace_bytes(M, N, K, trans_a, trans_b);
+    const bool    have_ws    = workspace != nullptr && aligned_to(workspace, 16) && workspace_bytes >= full;
+    const size_t  scale_area = block_scale_copy_pays(M, N, K) ? static_cast<size_t>(round_up(M * KB * 4, 256)) : 0;
+    // per-row A scales stored [M, K / 128] (sa_k == 1): hand the kernel a [K / 128, M] copy
+    if (have_ws && scale_area != 0 && scale_mode == SCALE_BLOCK && sa_block == 1 && sa_k == 1 && sa_m >= KB) {
+        launch_transpose_words(reinterpret_cast<const uint32_t *>(a_scale), static_cast<uint32_t *>(workspace), M, KB, sa_m, st);
+        a_scale = static_cast<const float *>(workspace);
+        sa_m    = 1;
+        sa_k    = M;
+    }
     if (trans_a || !trans_b || pad) {
-        const size_t need = pt_gemm_fp8_workspace_bytes(M, N, K, trans_a, trans_b);
-        if (workspace == nullptr || workspace_bytes < need || !aligned_to(workspace, 16))
+        if (!have_ws)
             return fail(PT_ERR_WORKSPACE, "pt_gemm_fp8: workspace missing, too small or misaligned");
-        uint8_t *ws = static_cast<uint8_t *>(workspace);
+        uint8_t *ws = static_cast<uint8_t *>(workspace) + scale_area;
         if (trans_a || pad) {
             if (M * Kp > 0) {
                 if (trans_a) // stored [K, M] -> [M, Kp]

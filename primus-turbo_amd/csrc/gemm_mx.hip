@@ -16,33 +16,6 @@ template <int FA, int FB> static int launch_mx_tiles(const GemmArgs &a, int tile
     return launch_gemm_cfg<4, 4, SCALE_MX, false, FA, FB>(a, stream);
 }
 
-// out[w, r] = in[r * pitch + w] for w < W: the scale words of one K position of all rows made
-// contiguous (32 x 32 word tiles through LDS, coalesced on both sides)
-__global__ __launch_bounds__(256) void transpose_words_kernel(const uint32_t *__restrict__ in, uint32_t *__restrict__ out,
-                                                              const int64_t R, const int64_t W, const int64_t pitch) {
-    __shared__ uint32_t t[32][33];
-    const int64_t r0 = static_cast<int64_t>(blockIdx.y) * 32, w0 = static_cast<int64_t>(blockIdx.x) * 32;
-    const int     tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const int64_t r = r0 + ty + 8 * p, w = w0 + tx;
-        if (r < R && w < W)
-            t[ty + 8 * p][tx] = in[r * pitch + w];
-    }
-    __syncthreads();
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const int64_t w = w0 + ty + 8 * p, r = r0 + tx;
-        if (w < W && r < R)
-            out[w * R + r] = t[tx][ty + 8 * p];
-    }
-}
-
-static void launch_transpose_words(const uint32_t *in, uint32_t *out, int64_t R, int64_t W, int64_t pitch, hipStream_t st) {
-    dim3 g(static_cast<unsigned>(cdiv(W, 32)), static_cast<unsigned>(cdiv(R, 32)));
-    transpose_words_kernel<<<g, 256, 0, st>>>(in, out, R, W, pitch);
-}
-
 } // namespace pt
 
 using namespace pt;
