@@ -484,7 +484,12 @@ PT_API int pt_grouped_gemm_fp8_vec_variable_k(const void *lhs, int lhs_dtype, co
  * L [Ml, ld] and R [Nr, ld] (ld in elements) are transposed column-direction outputs of
  * pt_grouped_quantize_mx with scale bytes [rows, ld / 32]; p = the group offsets in elements,
  * padded to whole 128-byte slabs (128 elements, MXFP4: 256). An empty group yields C[g] = 0 (or
- * leaves it unchanged when accumulating). No workspace: both operands are read in place. */
+ * leaves it unchanged when accumulating). Both operands are read in place.
+ *
+ * workspace (both entry points; optional, NULL = none): room for word-major copies of the two
+ * scale arrays (pt_grouped_gemm_mx_workspace_bytes / ..._variable_k_workspace_bytes, 16-byte
+ * aligned), which turn the kernel's scale copies into contiguous reads; without it the scale
+ * arrays are read where they are. */
 PT_API int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype,
                                   const int64_t *group_offs, const int64_t *row_offs_padded,
                                   const int64_t *col_offs_padded, int64_t G, void *row_q,
@@ -494,13 +499,15 @@ PT_API int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, i
                               int64_t sa_ld, const void *b, int b_dtype, const void *b_scale,
                               int64_t ldb, int64_t sb_ld, void *c, int c_dtype,
                               const int64_t *group_offs, const int64_t *group_offs_out, int64_t G,
-                              int64_t a_rows, int64_t out_rows, int64_t N, int64_t K, int tile_cfg,
-                              void *stream);
+                              int64_t a_rows, int64_t out_rows, int64_t N, int64_t K, void *workspace,
+                              size_t workspace_bytes, int tile_cfg, void *stream);
+PT_API size_t pt_grouped_gemm_mx_workspace_bytes(int64_t G, int64_t a_rows, int64_t N, int64_t K);
+PT_API size_t pt_grouped_gemm_mx_variable_k_workspace_bytes(int64_t Ml, int64_t Nr, int64_t ld);
 PT_API int pt_grouped_gemm_mx_variable_k(const void *lhs, int lhs_dtype, const void *lhs_scale,
                                          const void *rhs, int rhs_dtype, const void *rhs_scale, void *c,
                                          int c_dtype, const int64_t *group_offs, int64_t G, int64_t Ml,
-                                         int64_t Nr, int64_t ld, int accumulate, int tile_cfg,
-                                         void *stream);
+                                         int64_t Nr, int64_t ld, int accumulate, void *workspace,
+                                         size_t workspace_bytes, int tile_cfg, void *stream);
 
 /* Gated activation of an MoE expert MLP with the router probability folded in -------------
  *

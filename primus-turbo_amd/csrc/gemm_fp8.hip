@@ -149,6 +149,8 @@ void launch_transpose(const uint8_t *in, uint8_t *out, int64_t batch, int64_t R,
 __global__ __launch_bounds__(256) void transpose_words_kernel(const uint32_t *__restrict__ in, uint32_t *__restrict__ out,
                                                               const int64_t R, const int64_t W, const int64_t pitch) {
     __shared__ uint32_t t[32][33];
+    in += static_cast<int64_t>(blockIdx.z) * R * pitch; // batch of matrices, each transposed on its own
+    out += static_cast<int64_t>(blockIdx.z) * W * R;
     const int64_t r0 = static_cast<int64_t>(blockIdx.y) * 32, w0 = static_cast<int64_t>(blockIdx.x) * 32;
     const int     tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
 #pragma unroll
@@ -166,8 +168,11 @@ __global__ __launch_bounds__(256) void transpose_words_kernel(const uint32_t *__
     }
 }
 
-void launch_transpose_words(const uint32_t *in, uint32_t *out, int64_t R, int64_t W, int64_t pitch, hipStream_t st) {
-    dim3 g(static_cast<unsigned>(cdiv(W, 32)), static_cast<unsigned>(cdiv(R, 32)));
+void launch_transpose_words(const uint32_t *in, uint32_t *out, int64_t R, int64_t W, int64_t pitch, hipStream_t st,
+                            int64_t batch) {
+    if (R * W * batch == 0)
+        return;
+    dim3 g(static_cast<unsigned>(cdiv(W, 32)), static_cast<unsigned>(cdiv(R, 32)), static_cast<unsigned>(batch));
     transpose_words_kernel<<<g, 256, 0, st>>>(in, out, R, W, pitch);
 }
 

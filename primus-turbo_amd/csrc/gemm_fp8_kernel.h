@@ -1009,8 +1009,9 @@ void launch_transpose(const uint8_t *in, uint8_t *out, int64_t batch, int64_t R,
 void launch_pad_rows(const uint8_t *in, uint8_t *out, int64_t R, int64_t C, int64_t ldo, hipStream_t st);
 // in[R, C] with row pitch ldi -> out[R, ldo] (columns [C, ldo) zero-filled)
 void launch_pad_rows2(const uint8_t *in, uint8_t *out, int64_t R, int64_t C, int64_t ldi, int64_t ldo, hipStream_t st);
-// out[w * R + r] = in[r * pitch + w] for w < W (32-bit words): a scale array made contiguous along its rows
-void launch_transpose_words(const uint32_t *in, uint32_t *out, int64_t R, int64_t W, int64_t pitch, hipStream_t st);
+// out[b][w * R + r] = in[b][r * pitch + w] for w < W (32-bit words): scale arrays made contiguous along their rows
+void launch_transpose_words(const uint32_t *in, uint32_t *out, int64_t R, int64_t W, int64_t pitch, hipStream_t st,
+                            int64_t batch = 1);
 int  launch_gemm_block(const GemmArgs &a, int fa, int fb, bool sb_vec, int tile_cfg, hipStream_t stream);
 
 } // namespace pt

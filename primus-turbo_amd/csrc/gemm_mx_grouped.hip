@@ -65,10 +65,26 @@ using namespace pt;
 
 extern "C" {
 
+// Word-major copies of the scale arrays (see pt_gemm_mx): worth a pre-pass when the K loop is long.
+static int64_t mxg_words(int64_t kblocks) {
+    return cdiv(kblocks, 4);
+}
+
+size_t pt_grouped_gemm_mx_workspace_bytes(int64_t G, int64_t a_rows, int64_t N, int64_t K) {
+    const int64_t W = mxg_words(K / 32);
+    return static_cast<size_t>(round_up(a_rows * W * 4, 256) + round_up(G * N * W * 4, 256));
+}
+
+size_t pt_grouped_gemm_mx_variable_k_workspace_bytes(int64_t Ml, int64_t Nr, int64_t ld) {
+    const int64_t W = mxg_words(ld / 32);
+    return static_cast<size_t>(round_up(Ml * W * 4, 256) + round_up(Nr * W * 4, 256));
+}
+
 int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, int64_t lda, int64_t sa_ld, const void *b,
                        int b_dtype, const void *b_scale, int64_t ldb, int64_t sb_ld, void *c, int c_dtype,
                        const int64_t *group_offs, const int64_t *group_offs_out, int64_t G, int64_t a_rows,
-                       int64_t out_rows, int64_t N, int64_t K, int tile_cfg, void *stream) {
+                       int64_t out_rows, int64_t N, int64_t K, void *workspace, size_t workspace_bytes, int tile_cfg,
+                       void *stream) {
     const bool fp4 = a_dtype == PT_DTYPE_E2M1X2;
     PT_REQUIRE(fp4 ? b_dtype == PT_DTYPE_E2M1X2 : (is_fp8_dtype(a_dtype) && is_fp8_dtype(b_dtype)),
                "operands must both be fp8 (e4m3 / e5m2) or both e2m1x2");
@@ -110,6 +126,21 @@ int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, int64_t 
         g.group_offs_out = group_offs_out;
         g.b_gstride      = N * ldb;
         g.sb_gstride     = N * sb_ld / 4; // the kernel steps a 4-byte pointer
+        // with a workspace: scale words of one K position of all rows contiguous (two cache lines
+        // per scale copy of the kernel instead of sixty-four)
+        const int64_t W = mxg_words(K / 32);
+        if (workspace != nullptr && aligned_to(workspace, 16) && aligned_to(a_scale, 4) && aligned_to(b_scale, 4) &&
+            workspace_bytes >= pt_grouped_gemm_mx_workspace_bytes(G, a_rows, N, K) && sa_ld >= 4 * W && sb_ld >= 4 * W) {
+            uint32_t *wa = static_cast<uint32_t *>(workspace);
+            uint32_t *wb = wa + round_up(a_rows * W * 4, 256) / 4;
+            launch_transpose_words(static_cast<const uint32_t *>(a_scale), wa, a_rows, W, sa_ld / 4, st);
+            launch_transpose_words(static_cast<const uint32_t *>(b_scale), wb, N, W, sb_ld / 4, st, G);
+            g.sA         = reinterpret_cast<const float *>(wa);
+            g.sB         = reinterpret_cast<const float *>(wb);
+            g.sa_wpitch  = a_rows * 4;
+            g.sb_wpitch  = N * 4;
+            g.sb_gstride = W * N;
+        }
         const int rc = launch_mxg<GROUP_ROWS>(g, fp4 ? 4 : a_dtype == PT_DTYPE_E5M2, b_dtype == PT_DTYPE_E5M2, tile_cfg, st);
         if (rc != PT_OK)
             return rc;
@@ -123,7 +154,8 @@ int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, int64_t 
 
 int pt_grouped_gemm_mx_variable_k(const void *lhs, int lhs_dtype, const void *lhs_scale, const void *rhs, int rhs_dtype,
                                   const void *rhs_scale, void *c, int c_dtype, const int64_t *group_offs, int64_t G,
-                                  int64_t Ml, int64_t Nr, int64_t ld, int accumulate, int tile_cfg, void *stream) {
+                                  int64_t Ml, int64_t Nr, int64_t ld, int accumulate, void *workspace,
+                                  size_t workspace_bytes, int tile_cfg, void *stream) {
     const bool fp4 = lhs_dtype == PT_DTYPE_E2M1X2;
     PT_REQUIRE(fp4 ? rhs_dtype == PT_DTYPE_E2M1X2 : (is_fp8_dtype(lhs_dtype) && is_fp8_dtype(rhs_dtype)),
                "operands must both be fp8 (e4m3 / e5m2) or both e2m1x2");
@@ -157,6 +189,21 @@ int pt_grouped_gemm_mx_variable_k(const void *lhs, int lhs_dtype, const void *lh
     g.G          = static_cast<int>(G);
     g.group_offs = group_offs;
     g.c_gstride  = Ml * Nr;
+    const int64_t W = mxg_words(ld / 32);
+    if (workspace != nullptr && aligned_to(workspace, 16) && aligned_to(lhs_scale, 4) && aligned_to(rhs_scale, 4) &&
+        workspace_bytes >= pt_grouped_gemm_mx_variable_k_workspace_bytes(Ml, Nr, ld) && (ld / 32) % 4 == 0) {
+        auto      st = static_cast<hipStream_t>(stream);
+        uint32_t *wa = static_cast<uint32_t *>(workspace);
+        uint32_t *wb = wa + round_up(Ml * W * 4, 256) / 4;
+        launch_transpose_words(static_cast<const uint32_t *>(lhs_scale), wa, Ml, W, ld / 32 / 4, st);
+        launch_transpose_words(static_cast<const uint32_t *>(rhs_scale), wb, Nr, W, ld / 32 / 4, st);
+        g.sA        = reinterpret_cast<const float *>(wa);
+        g.sB        = reinterpret_cast<const float *>(wb);
+        g.sa_wpitch = Ml * 4;
+        g.sb_wpitch = Nr * 4;
+        g.sa_k      = (fp4 ? 2 : 1) * Ml; // a slab's scale words of all rows, in steps of the kernel's 4-byte scale pointer
+        g.sb_k      = (fp4 ? 2 : 1) * Nr;
+    }
     return launch_mxg<GROUP_K>(g, fp4 ? 4 : lhs_dtype == PT_DTYPE_E5M2, rhs_dtype == PT_DTYPE_E5M2, tile_cfg,
                                static_cast<hipStream_t>(stream));
 }

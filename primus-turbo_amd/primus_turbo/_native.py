@@ -182,12 +182,14 @@ _SIGNATURES = {
     "pt_grouped_gemm_mx": (
         c_int,
         [c_void_p, c_int, c_void_p, c_i64, c_i64, c_void_p, c_int, c_void_p, c_i64, c_i64, c_void_p, c_int, c_void_p,
-         c_void_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_int, c_void_p],
+         c_void_p, c_i64, c_i64, c_i64, c_i64, c_i64, c_void_p, c_size_t, c_int, c_void_p],
     ),
+    "pt_grouped_gemm_mx_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64, c_i64]),
+    "pt_grouped_gemm_mx_variable_k_workspace_bytes": (c_size_t, [c_i64, c_i64, c_i64]),
     "pt_grouped_gemm_mx_variable_k": (
         c_int,
         [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_i64, c_i64, c_i64, c_i64, c_int,
-         c_int, c_void_p],
+         c_void_p, c_size_t, c_int, c_void_p],
     ),
     "pt_dequantize_fp8_block": (
         c_int,

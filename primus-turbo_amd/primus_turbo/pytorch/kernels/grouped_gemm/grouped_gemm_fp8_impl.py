@@ -156,11 +156,14 @@ def _grouped_mx(a, b, a_scales, b_scales, group_offs, group_offs_out, trans_a, t
     a, b = _mx_pitch(_u8(a), kb), _mx_pitch(_u8(b), kb)
     out = torch.empty((rows, Nn), dtype=out_dtype, device=a.device)
     oo = None if group_offs_out is None else group_offs_out.contiguous()
+    # word-major scale copies pay once the K loop is long (measured: MXFP8 from K = 4096, MXFP4 from K = 2048)
+    ws_bytes = N.lib().pt_grouped_gemm_mx_workspace_bytes(G, rows, Nn, K) if K >= (2048 if fp4 else 4096) else 0
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
     N.check(
         N.lib().pt_grouped_gemm_mx(
             N.ptr(a), da, N.ptr(a_s), a.shape[1], a_s.shape[1], N.ptr(b), db, N.ptr(b_s), b.shape[2], b_s.shape[2], N.ptr(out),
-            N.dtype_code(out.dtype), N.ptr(group_offs.contiguous()), N.ptr(oo), G, rows, rows, Nn, K, MX_TILE_CFG,
-            N.stream_of(a),
+            N.dtype_code(out.dtype), N.ptr(group_offs.contiguous()), N.ptr(oo), G, rows, rows, Nn, K, N.ptr(ws), ws_bytes,
+            MX_TILE_CFG, N.stream_of(a),
         )
     )
     return out
@@ -190,11 +193,13 @@ def _variable_k_mx(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans
     _check(tuple(out.shape) == (G, Ml, Nr) and out.is_contiguous(), f"out must be a contiguous {(G, Ml, Nr)} tensor")
     da, db = N.dtype_code(a.dtype), N.dtype_code(b.dtype)
     a, b = _u8(a), _u8(b)
+    ws_bytes = N.lib().pt_grouped_gemm_mx_variable_k_workspace_bytes(Ml, Nr, ld) if ld >= 1024 else 0
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
     N.check(
         N.lib().pt_grouped_gemm_mx_variable_k(
             N.ptr(a), da, N.ptr(a_s), N.ptr(b), db, N.ptr(b_s), N.ptr(out),
-            N.dtype_code(out.dtype), N.ptr(group_offs.contiguous()), G, Ml, Nr, ld, int(accumulate), MX_TILE_CFG,
-            N.stream_of(a),
+            N.dtype_code(out.dtype), N.ptr(group_offs.contiguous()), G, Ml, Nr, ld, int(accumulate), N.ptr(ws), ws_bytes,
+            MX_TILE_CFG, N.stream_of(a),
         )
     )
     return out
