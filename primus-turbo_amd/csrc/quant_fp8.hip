@@ -13,6 +13,12 @@
 
 #include <mutex>
 
+// Timing probes for kernel development: a test translation unit may define this macro to record
+// timestamps; in the library it expands to nothing.
+#ifndef PT_TW_TRACE_POINT
+#define PT_TW_TRACE_POINT(id)
+#endif
+
 namespace pt {
 
 // ===========================================================================
@@ -77,21 +83,35 @@ __device__ __forceinline__ float grid_max_exchange(float block_amax, const GridW
             slots[t] = 0ull;
     float v = 0.f;
     if (threadIdx.x < 64) {
+        // one wavefront polls: a lane takes four neighbouring slots and requests them together, so
+        // that a round of probes costs one memory round trip (not four in a row)
         bool bad = false;
-        for (uint32_t t = threadIdx.x; t < gw.wait_for; t += 64) {
-            uint32_t probes = 0;
-            uint64_t w;
-            while (static_cast<uint32_t>((w = __hip_atomic_load(&slots[t], __ATOMIC_RELAXED,
-                                                                __HIP_MEMORY_SCOPE_AGENT)) >>
-                                         32) != tag) {
+        for (uint32_t base = 0; base < gw.wait_for; base += 256) {
+            const uint32_t t0     = base + threadIdx.x * 4;
+            uint32_t       probes = 0;
+            uint64_t       w[4];
+            while (true) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    w[k] = t0 + k < gw.wait_for
+                               ? __hip_atomic_load(&slots[t0 + k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                               : static_cast<uint64_t>(tag) << 32;
+                bool all = true;
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    all = all && static_cast<uint32_t>(w[k] >> 32) == tag;
+                if (all)
+                    break;
                 if (++probes >= gw.max_probes) {
                     bad = true;
-                    w   = 0ull;
                     break;
                 }
                 __builtin_amdgcn_s_sleep(1);
             }
-            v = fmaxf(v, __uint_as_float(static_cast<uint32_t>(w) & 0x7fffffffu));
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (static_cast<uint32_t>(w[k] >> 32) == tag) // (a slot that never arrived contributes nothing)
+                    v = fmaxf(v, __uint_as_float(static_cast<uint32_t>(w[k]) & 0x7fffffffu));
         }
         if (bad)
             s_tag[1] = 1u; // same value from every lane that writes
@@ -194,6 +214,7 @@ __global__ __launch_bounds__(TW_THREADS) void quant_tensorwise_kernel(
     const int64_t    stride = static_cast<int64_t>(gridDim.x) * TW_THREADS;
     const int64_t    tid0   = static_cast<int64_t>(blockIdx.x) * TW_THREADS + threadIdx.x;
 
+    PT_TW_TRACE_POINT(0);
     if constexpr (VEC16) {
         const int64_t units = n / TW_VEC;
         const int64_t tail0 = units * TW_VEC; // first element of the scalar tail
@@ -219,7 +240,9 @@ __global__ __launch_bounds__(TW_THREADS) void quant_tensorwise_kernel(
             if (blockIdx.x == 0 && tail0 + threadIdx.x < n)
                 amax = fmaxf(amax, fabsf(HP<T>::to_f32(x[tail0 + threadIdx.x])));
             amax = block_max(amax, s_red);
+            PT_TW_TRACE_POINT(1);
             amax = grid_max_exchange(amax, gw, s_red, s_tag);
+            PT_TW_TRACE_POINT(2);
         }
         float scale;
         if constexpr (DYNAMIC)
@@ -245,6 +268,7 @@ __global__ __launch_bounds__(TW_THREADS) void quant_tensorwise_kernel(
         if (blockIdx.x == 0 && tail0 + threadIdx.x < n)
             q[tail0 + threadIdx.x] =
                 quant1<E5M2>(HP<T>::to_f32(x[tail0 + threadIdx.x]), scale, qmax);
+        PT_TW_TRACE_POINT(3);
     } else {
         float amax = 0.f;
         if constexpr (DYNAMIC) {
