@@ -418,9 +418,12 @@ __device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile, const 
             t.C += (a.group_offs_out[g] - lo) * a.N * (a.out_dtype == PT_DTYPE_F32 ? 4 : 2);
         t.KT    = static_cast<int>(a.K / KSTEP);
     } else {
+        // a group's tiles in XCD-contiguous order (workgroup i runs on XCD i % 8 and walks tiles
+        // i, i + grid, ...): every XCD works on a compact block of the group's output, so the
+        // group's operand panels are fetched into few L2s instead of all eight
         const int per = a.tiles_m * a.tiles_n;
         g             = tile / per;
-        tile_coords_local(tile - g * per, a.tiles_m, a.tiles_n, tm, tn);
+        tile_coords_local(xcd_contiguous_id(tile - g * per, per), a.tiles_m, a.tiles_n, tm, tn);
         // K ranges are given in elements; two E2M1 codes share a byte
         const int64_t lo = a.group_offs[g] >> (F4 ? 1 : 0), hi = a.group_offs[g + 1] >> (F4 ? 1 : 0);
         t.m0    = static_cast<int64_t>(tm) * BM;
@@ -786,6 +789,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         if constexpr (!XPIPE) {
             if (KT > 0)
                 take_first_slab(); // requested before the loop or before the previous tile's epilogue
+            PT_GEMM_TRACE_POINT(1);
         }
 
         // one K slab per iteration; the body must stay a single basic block (no branches), or
@@ -909,6 +913,7 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             advance_loader();
             buf = buf_n;
         }
+        PT_GEMM_TRACE_POINT(4);
         if constexpr (!XPIPE) {
             // the re-read copies of the last slab must have landed everywhere, and everyone must be
             // done reading the stages, before the next tile's first copies go into them

@@ -971,6 +971,13 @@ def _next_sr_seed(*flags: int) -> int:
     reference's quantizers keep one: reproducible for a fixed order of calls); 0 otherwise."""
     if not any(f & 4 for f in flags):
         return 0
+    # The seed is a launch argument: a captured graph would replay the same rounding noise on
+    # every step, which correlates the gradients' rounding errors. Refuse rather than do that.
+    if torch.cuda.is_available() and torch.cuda.is_current_stream_capturing():
+        raise RuntimeError(
+            "stochastic rounding (use_sr) cannot be captured into a HIP graph: its seed is a host-side launch "
+            "argument and every replay would reuse it; quantize with use_sr outside the captured region"
+        )
     _sr_counter[0] = (_sr_counter[0] + 1) & 0xFFFFFFFF
     return (_sr_counter[0] * 0x9E3779B1) & 0xFFFFFFFF
 

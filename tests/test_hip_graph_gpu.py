@@ -90,3 +90,33 @@ def test_graph_grouped_gemm_forward_backward(kind):
 
     _replay_check(fn, lambda seed: (bf16_randn((1024, 1024), seed=140 + seed), bf16_randn((4, 512, 1024), seed=150 + seed),
                                     bf16_randn((1024, 512), seed=160 + seed)), 3)
+
+
+def test_stochastic_rounding_refuses_graph_capture():
+    """The stochastic-rounding seed is a host-side launch argument: captured, every replay would
+    round with the same noise. The quantizer raises under capture instead (and works outside)."""
+    F4 = getattr(torch, "float4_e2m1fn_x2", None)
+    if F4 is None:
+        pytest.skip("torch without float4_e2m1fn_x2")
+    from primus_turbo.pytorch.core.low_precision import ScalingRecipe
+    from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+    x = bf16_randn((128, 256), seed=3).cuda()
+    sr = ScalingRecipe(use_sr=True)
+    qi.quantize_mxfp4_impl(x, F4, 1, 32, False, sr)  # eager: fine
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="cannot be captured"):
+        with torch.cuda.graph(graph, stream=side):
+            qi.quantize_mxfp4_impl(x, F4, 1, 32, False, sr)
+    torch.cuda.synchronize()
+    # round-to-nearest captures as before
+    g2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g2):
+        q, s = qi.quantize_mxfp4_impl(x, F4, 1, 32, False, ScalingRecipe())
+    g2.replay()
+    torch.cuda.synchronize()
+    q0, s0 = qi.quantize_mxfp4_impl(x, F4, 1, 32, False, ScalingRecipe())
+    assert torch.equal(q.view(torch.uint8), q0.view(torch.uint8)) and torch.equal(s.view(torch.uint8), s0.view(torch.uint8))
