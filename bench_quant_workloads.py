@@ -485,6 +485,59 @@ class GluQuantGrouped(_QuantBase):
         return self._cpu(fn, self.dominant_work() * rows / self.T, f"first {rows} tokens: PyTorch SwiGLU, then row and column blockwise quantize")
 
 
+class GluQuantGroupedMx(GluQuantGrouped):
+    """The same step for the MXFP8 recipe: the grouped MX quantizer applies SwiGLU with the router
+    probabilities on load and writes fc2's row codes (groups padded to 32 rows), transposed
+    column codes (groups padded to 128) and both E8M0 scale arrays."""
+
+    name = "swiglu_with_probs_fused_into_grouped_mxfp8_quant_32768tokens_hidden2048_bf16"
+    dominant_name = "mx_quant_kernel<e4m3, row + transposed column blocks, grouped, SiLU gate on load>"
+    dtype = "bf16 in, e4m3 + e8m0 out (fp32 arithmetic)"
+
+    def dominant_work(self):  # 2 H read (2 B each), H row codes + H column codes + a scale byte per 32 each, + the probability
+        n = self.T * self.H
+        return 6.0 * n + 2.0 * n / 32 + 4.0 * self.T
+
+    step_work = dominant_work
+
+    def dominant(self):
+        return self.qi.glu_grouped_quantize_mx_impl(self.x, self.p, None, "silu", torch.float8_e4m3fn, self.gl, self.offs, True)
+
+    step = dominant
+
+    def two_step(self):
+        y = self.turbo.ops.swiglu_with_probs(self.x, self.p)
+        return self.qi.grouped_quantize_mxfp8_impl(y, torch.float8_e4m3fn, None, 32, self.gl, self.offs, with_trans=True)
+
+    def check(self):
+        a, b = self.dominant(), self.two_step()
+        mr, mc = int(a[5][-1].item()), int(a[7][-1].item())
+        u8 = lambda t: t.view(torch.uint8)  # noqa: E731
+        same = (torch.equal(u8(a[0])[:mr], u8(b[0])[:mr]) and torch.equal(u8(a[1])[:mr], u8(b[1])[:mr])
+                and torch.equal(u8(a[2])[:, :mc], u8(b[2])[:, :mc]) and torch.equal(u8(a[3])[:, : mc // 32], u8(b[3])[:, : mc // 32]))
+        from oracle import quantize as Q
+
+        rows = int(self.lens[0])  # group 0 sits at the start of both layouts
+        if rows > 0:
+            y = self.turbo.ops.swiglu_with_probs(self.x[:rows], self.p[:rows]).float().cpu().numpy()
+            oq, os_ = Q.mx_quant_rowwise(y, "e4m3")
+            same = same and np.array_equal(_u8(a[0])[:rows], oq) and np.array_equal(_u8(a[1])[:rows], os_)
+        return bool(same), f"codes and scales bit-identical with the two-step form; row codes of group 0 ({rows} tokens) bit-exact vs the oracle"
+
+    def cpu_baseline(self):
+        from oracle import quantize as Q
+
+        rows = 512
+
+        def fn():
+            a, b = self.x_cpu[:rows].float().chunk(2, dim=-1)
+            y = (torch.nn.functional.silu(a) * b * self.p_cpu[:rows, None]).to(torch.bfloat16).float().numpy()
+            Q.mx_quant_rowwise(y, "e4m3")
+            Q.mx_quant_colwise(y, "e4m3")
+
+        return self._cpu(fn, self.dominant_work() * rows / self.T, f"first {rows} tokens: PyTorch SwiGLU, then the numpy MX oracle in both directions")
+
+
 class MoePermute(_QuantBase):
     """MoE permute + unpermute around the expert bank of the MoE configuration: 4096 tokens with
     top-8 routing over 32 local experts (32768 routed rows), hidden 7168, bf16, rows padded per
@@ -556,6 +609,7 @@ def register(workloads):
     workloads["moe_permute"] = MoePermute
     workloads["swiglu_with_probs"] = SwigluWithProbs
     workloads["glu_quant_grouped"] = GluQuantGrouped
+    workloads["glu_quant_grouped_mxfp8"] = GluQuantGroupedMx
     workloads["quant_rowwise"] = QuantRowwise
     workloads["quant_blockwise"] = lambda dev: QuantBlockwise(dev, False)
     workloads["quant_blockwise_dual"] = lambda dev: QuantBlockwise(dev, True)

@@ -495,6 +495,22 @@ PT_API int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t
                                   const int64_t *col_offs_padded, int64_t G, void *row_q,
                                   void *row_scale, int row_flags, void *col_q, void *col_scale,
                                   int col_flags, int64_t col_ld, uint32_t sr_seed, void *stream);
+/* Gated activation fused into pt_grouped_quantize_mx: x is the fc1 output [M, 2 N] (gate
+ * columns, then up columns) and what gets quantized is
+ *   y[m, n] = T( act(x[m, n]) * x[m, N + n] * probs[m] ),   zero where row_mask[m] == 0,
+ * act = 0 SiLU, 1 exact (erf) GELU, T = x's 16-bit type: the value swiglu_with_probs /
+ * geglu_with_probs would store (primus_turbo/triton/activation/swiglu_kernel.py:11-248) followed
+ * by grouped_quantize_mxfp8[_dual] / grouped_quantize_mxfp4[_dual] (quantization.cpp:971-1378),
+ * without y travelling through HBM; bit-identical with running the two steps of this library one
+ * after the other. The reference has no fused form. Round to nearest, 1-D blocks; row_q /
+ * row_scale are required (fc2's forward operand), col_q / col_scale (its wgrad operand) optional;
+ * col_flags: 0, or 2 = Hadamard-transformed column direction (MXFP4's wgrad recipe). probs is
+ * fp32 [M], row_mask optional int64 [M]. */
+PT_API int pt_glu_grouped_quantize_mx(const void *x, int x_dtype, const float *probs, const int64_t *row_mask,
+                                      int act, int64_t M, int64_t N, int q_dtype, const int64_t *group_offs,
+                                      const int64_t *row_offs_padded, const int64_t *col_offs_padded, int64_t G,
+                                      void *row_q, void *row_scale, void *col_q, void *col_scale, int col_flags,
+                                      int64_t col_ld, void *stream);
 PT_API int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, int64_t lda,
                               int64_t sa_ld, const void *b, int b_dtype, const void *b_scale,
                               int64_t ldb, int64_t sb_ld, void *c, int c_dtype,

@@ -15,6 +15,7 @@
 // quantized along rows (blocks of 32 columns) and/or along columns (blocks of 32 rows, output
 // transposed), so the dual quantizer reads HBM once. The "2-D block" variants share one
 // exponent per 32 x 32 tile.
+#include "pt_activation.h"
 #include "pt_common.h"
 
 namespace pt {
@@ -126,6 +127,10 @@ struct MxArgs {
     // MXFP4 stochastic rounding: bit 0 / bit 1 = row / column direction; one seed per launch
     int      sr_mask;
     uint32_t sr_seed;
+    // Gated input (the GLU kernels): x is [M, 2 N], gate half then up half of every row; the
+    // tile holds T(act(gate) * up * probs[m]), zeros for rows whose row_mask entry is 0.
+    const float   *probs;    // [M]
+    const int64_t *row_mask; // [M] or NULL
 };
 
 // The MXFP4 recipe's fixed 16-point Hadamard transform of v[base .. base + 16), in place:
@@ -161,10 +166,14 @@ __device__ __forceinline__ float abs_or_zero(float x) {
 
 // RHT: bit 0 / bit 1 = the row / column direction quantizes the Hadamard-transformed values
 // (16 consecutive elements along the direction; never together with 2-D blocks).
-template <typename T, int FMT, bool ROW, bool COL, bool ROW2D, bool COL2D, int RHT = 0>
+// GLU: 0 = x is the tile source itself; 1 + ACT_SILU / 1 + ACT_GELU = x holds gate and up halves
+// and the tile is the gated activation, rounded to T as the stand-alone activation kernel rounds
+// it (grouped mode only).
+template <typename T, int FMT, bool ROW, bool COL, bool ROW2D, bool COL2D, int RHT = 0, int GLU = 0>
 __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
     constexpr bool ANY2D = (ROW && ROW2D) || (COL && COL2D);
     static_assert(RHT == 0 || !ANY2D, "the Hadamard transform is not combined with 2-D blocks");
+    static_assert(GLU == 0 || !ANY2D, "the gated input is not combined with 2-D blocks");
     __shared__ __attribute__((aligned(16))) uint16_t tile[MX_TILE * MX_PITCH];
     __shared__ float                                 amax_rc[ANY2D ? MX_TILE * 4 : 1]; // [row][32-col block]
     __shared__ __attribute__((aligned(4))) uint8_t   sbytes[MX_TILE * 4]; // E8M0 bytes of the tile, [row or column][block]
@@ -197,7 +206,37 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
         const int     r = p * 16 + (tid >> 4), c = (tid & 15) * 8;
         const int64_t m = in_m0 + r, n = n0 + c;
         u32x4         v = u32x4{0u, 0u, 0u, 0u};
-        if (m < in_end && n < a.N) {
+        if constexpr (GLU != 0) {
+            if (m < in_end && n < a.N && (a.row_mask == nullptr || a.row_mask[m] != 0)) {
+                const uint16_t *gp = static_cast<const uint16_t *>(a.x) + m * 2 * a.N + n;
+                const float     pr = a.probs[m];
+                uint32_t        gw[4] = {0u, 0u, 0u, 0u}, uw[4] = {0u, 0u, 0u, 0u};
+                if (vec) {
+                    const u32x4 g4 = ld128(gp), u4 = ld128(gp + a.N);
+                    gw[0] = g4.x, gw[1] = g4.y, gw[2] = g4.z, gw[3] = g4.w;
+                    uw[0] = u4.x, uw[1] = u4.y, uw[2] = u4.z, uw[3] = u4.w;
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+                        if (n + k < a.N) {
+                            gw[k >> 1] |= static_cast<uint32_t>(gp[k]) << (16 * (k & 1));
+                            uw[k >> 1] |= static_cast<uint32_t>(gp[a.N + k]) << (16 * (k & 1));
+                        }
+                }
+                uint32_t o[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    float g0, g1, u0, u1;
+                    unpack2<T>(gw[k], g0, g1);
+                    unpack2<T>(uw[k], u0, u1);
+                    // columns behind N stay +0 whatever probs holds
+                    const float r0 = n + 2 * k < a.N ? act_fwd<GLU - 1>(g0) * u0 * pr : 0.f;
+                    const float r1 = n + 2 * k + 1 < a.N ? act_fwd<GLU - 1>(g1) * u1 * pr : 0.f;
+                    o[k]           = pack2<T>(r0, r1);
+                }
+                v = u32x4{o[0], o[1], o[2], o[3]};
+            }
+        } else if (m < in_end && n < a.N) {
             if (vec) {
                 v = ld128(x + m * a.N + n);
             } else {
@@ -415,6 +454,29 @@ template <typename T> static void launch_mx_rht(const MxArgs &a, bool row_rht, b
     }
 }
 
+// the gated-input quantizers: 1-D blocks, nearest rounding, both directions or rows only; MXFP4
+// may transform its column direction (the recipe of the wgrad operand)
+template <typename T, int FMT, int GLU> static void launch_mx_glu_dir(const MxArgs &a, bool col_rht, dim3 grid, hipStream_t st) {
+    if constexpr (FMT == MX_E2M1) {
+        if (a.col_q != nullptr && col_rht) {
+            mx_quant_kernel<T, FMT, true, true, false, false, 2, GLU><<<grid, 256, 0, st>>>(a);
+            return;
+        }
+    }
+    if (a.col_q != nullptr)
+        mx_quant_kernel<T, FMT, true, true, false, false, 0, GLU><<<grid, 256, 0, st>>>(a);
+    else
+        mx_quant_kernel<T, FMT, true, false, false, false, 0, GLU><<<grid, 256, 0, st>>>(a);
+}
+template <typename T, int GLU> static void launch_mx_glu(const MxArgs &a, int fmt, bool col_rht, dim3 grid, hipStream_t st) {
+    if (fmt == MX_E4M3)
+        launch_mx_glu_dir<T, MX_E4M3, GLU>(a, col_rht, grid, st);
+    else if (fmt == MX_E5M2)
+        launch_mx_glu_dir<T, MX_E5M2, GLU>(a, col_rht, grid, st);
+    else
+        launch_mx_glu_dir<T, MX_E2M1, GLU>(a, col_rht, grid, st);
+}
+
 template <typename T> static void launch_mx_fmt(const MxArgs &a, int fmt, bool row2d, bool col2d, dim3 grid, hipStream_t st) {
     if (fmt == MX_E4M3)
         launch_mx_dir<T, MX_E4M3>(a, row2d, col2d, grid, st);
@@ -608,6 +670,8 @@ int pt_quantize_mx(const void *x, int x_dtype, int64_t B, int64_t M, int64_t N, 
     a.col_s = static_cast<uint8_t *>(col_scale);
     a.group_offs = a.row_offs_pad = a.col_offs_pad = nullptr;
     a.G          = 0;
+    a.probs      = nullptr;
+    a.row_mask   = nullptr;
     a.sr_mask    = ((row_q && (row_flags & 4)) ? 1 : 0) | ((col_q && (col_flags & 4)) ? 2 : 0);
     a.sr_seed    = sr_seed;
     PT_REQUIRE(a.Mpad / 128 < 65536 && B < 65536, "grid dimension out of range");
@@ -626,10 +690,12 @@ int pt_quantize_mx(const void *x, int x_dtype, int64_t B, int64_t M, int64_t N, 
     return check_launch("mx_quant_kernel");
 }
 
-int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype, const int64_t *group_offs,
-                           const int64_t *row_offs_padded, const int64_t *col_offs_padded, int64_t G, void *row_q,
-                           void *row_scale, int row_flags, void *col_q, void *col_scale, int col_flags, int64_t col_ld,
-                           uint32_t sr_seed, void *stream) {
+// The shared body of the grouped quantizers; glu = 0 (x is [M, N]) or 1 + ACT_* (x is [M, 2 N]).
+static int grouped_quantize_mx(const void *x, int x_dtype, const float *probs, const int64_t *row_mask,
+                               int glu, int64_t M, int64_t N, int q_dtype, const int64_t *group_offs,
+                               const int64_t *row_offs_padded, const int64_t *col_offs_padded, int64_t G, void *row_q,
+                               void *row_scale, int row_flags, void *col_q, void *col_scale, int col_flags, int64_t col_ld,
+                               uint32_t sr_seed, void *stream) {
     PT_REQUIRE(x_dtype == PT_DTYPE_BF16 || x_dtype == PT_DTYPE_F16, "input must be bf16 or fp16");
     const int fmt = mx_fmt_of(q_dtype);
     PT_REQUIRE(fmt >= 0, "q_dtype must be e4m3, e5m2 or e2m1x2");
@@ -642,9 +708,15 @@ int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t N, int
     PT_REQUIRE(((row_flags | col_flags) & 1) == 0, "grouped MX quantization has no 2-D blocks");
     const bool rht = (((row_q ? row_flags : 0) | (col_q ? col_flags : 0)) & 2) != 0;
     PT_REQUIRE(col_ld % 128 == 0 && col_ld >= M, "col_ld must be a multiple of 128 that holds every padded group");
+    if (glu != 0) {
+        PT_REQUIRE(row_q != nullptr, "the gated quantizer produces the row direction (optionally the column direction too)");
+        PT_REQUIRE(((row_flags | col_flags) & 4) == 0 && (row_flags & 2) == 0,
+                   "the gated quantizer rounds to nearest; only its column direction may be Hadamard-transformed");
+    }
     if (M == 0 || N == 0)
         return PT_OK;
     PT_REQUIRE(x && group_offs && col_offs_padded, "NULL pointer");
+    PT_REQUIRE(glu == 0 || probs != nullptr, "NULL probs");
     PT_REQUIRE(aligned_to(row_q, 16) && aligned_to(col_q, 16), "outputs must be 16-byte aligned");
     PT_REQUIRE(aligned_to(row_scale, 4) && aligned_to(col_scale, 4), "scale outputs must be 4-byte aligned");
     MxArgs a;
@@ -664,10 +736,18 @@ int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t N, int
     a.G            = static_cast<int>(G);
     a.sr_mask      = ((row_q && (row_flags & 4)) ? 1 : 0) | ((col_q && (col_flags & 4)) ? 2 : 0);
     a.sr_seed      = sr_seed;
+    a.probs        = probs;
+    a.row_mask     = row_mask;
     PT_REQUIRE(col_ld / 128 < 65536, "grid dimension out of range");
     dim3 grid(static_cast<unsigned>(a.Npad / 128), static_cast<unsigned>(col_ld / 128), 1);
     auto st = static_cast<hipStream_t>(stream);
-    if (rht) {
+    if (glu != 0) {
+        const bool bf = x_dtype == PT_DTYPE_BF16;
+        if (glu == 1 + ACT_SILU)
+            bf ? launch_mx_glu<bf16_t, 1 + ACT_SILU>(a, fmt, rht, grid, st) : launch_mx_glu<f16_t, 1 + ACT_SILU>(a, fmt, rht, grid, st);
+        else
+            bf ? launch_mx_glu<bf16_t, 1 + ACT_GELU>(a, fmt, rht, grid, st) : launch_mx_glu<f16_t, 1 + ACT_GELU>(a, fmt, rht, grid, st);
+    } else if (rht) {
         if (x_dtype == PT_DTYPE_BF16)
             launch_mx_rht<bf16_t>(a, (row_flags & 2) != 0, (col_flags & 2) != 0, grid, st);
         else
@@ -678,6 +758,25 @@ int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t N, int
         launch_mx_fmt<f16_t>(a, fmt, false, false, grid, st);
     }
     return check_launch("mx_quant_kernel");
+}
+
+int pt_grouped_quantize_mx(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype, const int64_t *group_offs,
+                           const int64_t *row_offs_padded, const int64_t *col_offs_padded, int64_t G, void *row_q,
+                           void *row_scale, int row_flags, void *col_q, void *col_scale, int col_flags, int64_t col_ld,
+                           uint32_t sr_seed, void *stream) {
+    return grouped_quantize_mx(x, x_dtype, nullptr, nullptr, 0, M, N, q_dtype, group_offs,
+                               row_offs_padded, col_offs_padded, G, row_q, row_scale, row_flags, col_q, col_scale, col_flags,
+                               col_ld, sr_seed, stream);
+}
+
+int pt_glu_grouped_quantize_mx(const void *x, int x_dtype, const float *probs, const int64_t *row_mask, int act, int64_t M,
+                               int64_t N, int q_dtype, const int64_t *group_offs, const int64_t *row_offs_padded,
+                               const int64_t *col_offs_padded, int64_t G, void *row_q, void *row_scale, void *col_q,
+                               void *col_scale, int col_flags, int64_t col_ld, void *stream) {
+    PT_REQUIRE(act == ACT_SILU || act == ACT_GELU, "act must be 0 (SiLU) or 1 (GELU)");
+    return grouped_quantize_mx(x, x_dtype, probs, row_mask, 1 + act, M, N, q_dtype, group_offs,
+                               row_offs_padded, col_offs_padded, G, row_q, row_scale, 0, col_q, col_scale, col_flags, col_ld,
+                               0u, stream);
 }
 
 int pt_dequantize_mx(const void *q, int q_dtype, const void *scale, int64_t rows, int64_t cols, void *y, int y_dtype,

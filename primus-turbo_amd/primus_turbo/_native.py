@@ -179,6 +179,11 @@ _SIGNATURES = {
         [c_void_p, c_int, c_i64, c_i64, c_int, c_void_p, c_void_p, c_void_p, c_i64, c_void_p, c_void_p, c_int, c_void_p,
          c_void_p, c_int, c_i64, ctypes.c_uint32, c_void_p],
     ),
+    "pt_glu_grouped_quantize_mx": (
+        c_int,
+        [c_void_p, c_int, c_void_p, c_void_p, c_int, c_i64, c_i64, c_int, c_void_p, c_void_p, c_void_p, c_i64, c_void_p,
+         c_void_p, c_void_p, c_void_p, c_int, c_i64, c_void_p],
+    ),
     "pt_grouped_gemm_mx": (
         c_int,
         [c_void_p, c_int, c_void_p, c_i64, c_i64, c_void_p, c_int, c_void_p, c_i64, c_i64, c_void_p, c_int, c_void_p,

@@ -1256,6 +1256,72 @@ def _grouped_quantize_mx_op_fake(x, out_dtype, group_lens, group_offs, want_row,
             i64(0 if fp4 else G), i64(0 if fp4 else G + 1), i64(G), i64(G + 1))
 
 
+@torch.library.custom_op("primus_turbo::glu_grouped_quantize_mx", mutates_args=())
+def glu_grouped_quantize_mx_impl(
+    x: torch.Tensor, probs: torch.Tensor, row_mask: Optional[torch.Tensor], act: str, out_dtype: torch.dtype,
+    group_lens: torch.Tensor, group_offs: torch.Tensor, with_trans: bool, col_flags: int = 0,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Gated activation fused into the grouped MX quantizer: ``x [M, 2 N]`` is the fc1 output of an
+    MoE expert MLP and the tensor quantized is ``y = T(act(x[:, :N]) * x[:, N:] * probs[:, None])``
+    (zero rows where ``row_mask`` is 0), what ``swiglu_with_probs`` / ``geglu_with_probs`` would store,
+    which never travels through HBM here. Outputs as ``primus_turbo::grouped_quantize_mx`` on the
+    stored activation with round-to-nearest 1-D blocks, bit for bit: ``(row_q, row_scale, col_q,
+    col_scale, lens_row, offs_row, lens_col, offs_col)``, the column pair empty unless ``with_trans``,
+    row lens / offs empty for MXFP4 (its rows stay in place); ``col_flags=2`` transforms the MXFP4
+    column direction (``use_rht``). (No counterpart in the reference.)"""
+    N.require_cuda(x, probs, row_mask, group_lens, group_offs)
+    _check(act in _GLU_ACT, "act must be 'silu' or 'gelu'")
+    _check(x.dtype in (torch.bfloat16, torch.float16), "input must be bfloat16 or float16")
+    _check(x.dim() == 2 and x.is_contiguous() and x.shape[1] % 2 == 0, "input must be a contiguous [M, 2 N] tensor")
+    _check(group_lens.dtype == torch.int64 and group_offs.dtype == torch.int64, "group_lens / group_offs must be int64")
+    _check(group_lens.dim() == 1 and group_offs.dim() == 1 and group_offs.numel() == group_lens.numel() + 1,
+           "group_offs.size(0) must equal group_lens.size(0) + 1")
+    _check(group_lens.numel() >= 1, "must have at least one group")
+    fp4 = _FP4X2 is not None and out_dtype == _FP4X2
+    _check(fp4 or out_dtype in (torch.float8_e4m3fn, torch.float8_e5m2),
+           "Output must be Float8_e4m3fn, Float8_e5m2 or Float4_e2m1fn_x2")
+    M, Nn = x.shape[0], x.shape[1] // 2
+    _check(Nn % 32 == 0, f"N must be divisible by 32, got N={Nn}")
+    _check(probs.numel() == M, "probs must hold one value per row")
+    p32 = probs.reshape(-1).to(torch.float32).contiguous()
+    mask = None
+    if row_mask is not None:
+        _check(row_mask.numel() == M, "row_mask must hold one value per row")
+        mask = row_mask.reshape(-1).to(torch.int64).contiguous()
+    G = group_lens.numel()
+    pack = 2 if fp4 else 1
+    ra, ca, m_pad_row, m_pad_col, n_pad = _grouped_mx_dims(M, Nn, G, fp4)
+    dev = x.device
+    group_offs = group_offs.contiguous()
+    lens_row, offs_row = (group_lens, group_offs) if fp4 else _group_offs(group_lens, ra, True)
+    lens_col, offs_col = _group_offs(group_lens, ca, True)
+    row_q = torch.empty((m_pad_row, n_pad // pack), dtype=torch.uint8, device=dev)
+    row_s = torch.empty((m_pad_row, n_pad // 32), dtype=torch.uint8, device=dev)
+    col_q = col_s = None
+    if with_trans:
+        col_q = torch.empty((Nn, m_pad_col // pack), dtype=torch.uint8, device=dev)
+        col_s = torch.empty((Nn, m_pad_col // 32), dtype=torch.uint8, device=dev)
+    N.check(
+        N.lib().pt_glu_grouped_quantize_mx(
+            N.ptr(x), N.dtype_code(x.dtype), N.ptr(p32), N.ptr(mask), _GLU_ACT[act], M, Nn, N.dtype_code(out_dtype),
+            N.ptr(group_offs), None if fp4 else N.ptr(offs_row), N.ptr(offs_col), G, N.ptr(row_q), N.ptr(row_s),
+            N.ptr(col_q), N.ptr(col_s), int(col_flags) if with_trans else 0, m_pad_col, N.stream_of(x),
+        )
+    )
+    empty = lambda dt=torch.uint8: torch.empty(0, dtype=dt, device=dev)  # noqa: E731
+    view = lambda t, dt: (empty() if t is None else t).view(dt)  # noqa: E731
+    if fp4:
+        lens_row, offs_row = empty(torch.int64), empty(torch.int64)
+    return (view(row_q, out_dtype), view(row_s, _E8M0), view(col_q, out_dtype), view(col_s, _E8M0),
+            lens_row, offs_row, lens_col, offs_col)
+
+
+@glu_grouped_quantize_mx_impl.register_fake
+def _glu_grouped_quantize_mx_impl_fake(x, probs, row_mask, act, out_dtype, group_lens, group_offs, with_trans, col_flags=0):
+    half = x.new_empty((x.shape[0], x.shape[1] // 2))
+    return _grouped_quantize_mx_op_fake(half, out_dtype, group_lens, group_offs, True, with_trans, 0, 0)
+
+
 def grouped_quantize_mxfp8_impl(x, out_dtype, axis, block_size, group_lens, group_offs, with_trans=False,
                                 scaling_recipe=None, scaling_recipe_for_trans=None):
     """MXFP8 quantization of the packed rows of G groups, each virtually zero-padded along M.

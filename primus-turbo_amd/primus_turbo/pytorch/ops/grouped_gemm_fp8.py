@@ -40,8 +40,9 @@ from primus_turbo.pytorch.kernels.grouped_gemm.grouped_gemm_fp8_impl import (
 )
 from primus_turbo.pytorch.kernels.grouped_gemm.grouped_gemm_utils import group_offs_from_lens
 from primus_turbo.pytorch.kernels.quantization.quantization_impl import (
-    grouped_quantize_mxfp8_impl,
+    glu_grouped_quantize_mx_impl,
     glu_quant_fp8_blockwise_segment_m_row_col_impl,
+    grouped_quantize_mxfp8_impl,
     quant_fp8_blockwise_for_weight_dual_impl,
     quant_fp8_blockwise_for_weight_impl,
     quant_fp8_blockwise_segment_m_row_col_impl,
@@ -306,6 +307,48 @@ class FP8GroupedGemmTensorFunc(torch.autograd.Function):
         return grad_a, grad_b, None, None, None, None, None, None, None, None, None
 
 
+def _mx_weight_operands(b, b_t, config, need_bwd):
+    """The expert weights ``[G, N, K]`` as MXFP8 operands with 32 x 32 blocks: ``(row codes, row scales,
+    column codes, column scales)``, the column pair (the transposed quantization dgrad reads) only
+    when a backward pass will follow."""
+    fdt, bs, gran = _get_fp8_dtype(config.format, True), config.block_size, config.granularity
+    w_recipe = ScalingRecipe(use_2d_block=True)
+    b_col = b_col_s = None
+    if isinstance(b, QuantizedTensor):
+        check_quantized_tensor(b, config, axis=-1, scaling_recipe=w_recipe)
+        b_row, b_row_s = b.qdata, b.scale_inv
+        if need_bwd:
+            if b_t is None:
+                b_t = QuantizedTensor.quantize(b.dequantize(), b.real_dtype, gran, axis=-2, block_size=bs,
+                                               scaling_recipe=w_recipe)
+            assert isinstance(b_t, QuantizedTensor)
+            b_col, b_col_s = b_t.qdata, b_t.scale_inv
+    elif need_bwd:
+        b_row, b_row_s, b_col, b_col_s = quantize_mxfp8_impl(
+            b.contiguous(), fdt, None, bs, with_trans=True, scaling_recipe=w_recipe, scaling_recipe_for_trans=w_recipe)
+    else:
+        b_row, b_row_s = quantize_mxfp8_impl(b.contiguous(), fdt, 2, bs, scaling_recipe=w_recipe)
+    return b_row, b_row_s, b_col, b_col_s
+
+
+def _mx_backward_products(grad_out, a_col, a_col_s, b_col, b_col_s, group_lens, group_offs, config, dgrad_dtype,
+                          wgrad_dtype, num_cu, total_m, fuse_bgrad_accum, main_grad):
+    """dgrad and wgrad of the MXFP8 grouped product from the saved column-direction operands."""
+    gdt = _get_fp8_dtype(config.format, False)
+    gran = config.granularity.value
+    g_row, g_row_s, g_col, g_col_s, _, offs_row, lens_col, offs_col = grouped_quantize_mxfp8_impl(
+        grad_out, gdt, None, config.block_size, group_lens, group_offs, with_trans=True)
+    # dgrad: grad_a = grad_out @ b, as an NT product with the transposed weight quantization [G, K, N]
+    grad_a = grouped_gemm_fp8_impl(g_row, b_col, g_row_s, b_col_s, group_lens, offs_row, False, True, dgrad_dtype,
+                                   gran, num_cu, _NATIVE, False, group_offs)[:total_m]
+    # wgrad: grad_b[g] = grad_out_g^T @ a_g over the 128-padded segments -> [G, N, K]
+    grad_b = _grouped_gemm_fp8_variable_k_impl_wrapper(
+        g_col, a_col, g_col_s, a_col_s, lens_col, offs_col, False, False, False, wgrad_dtype, gran, num_cu, _NATIVE,
+        inplace_add_to_out=fuse_bgrad_accum, out=main_grad,
+    )
+    return grad_a, grad_b
+
+
 class FP8GroupedGemmMXFunc(torch.autograd.Function):
     """MX_BLOCKWISE (MXFP8) grouped GEMM autograd."""
 
@@ -322,8 +365,8 @@ class FP8GroupedGemmMXFunc(torch.autograd.Function):
         gran = config.granularity
         total_m = int(a.size(0))
         need_bwd = any(ctx.needs_input_grad[:2])
-        a_recipe, w_recipe = ScalingRecipe(), ScalingRecipe(use_2d_block=True)
-        a_col = a_col_s = b_col = b_col_s = None
+        a_recipe = ScalingRecipe()
+        a_col = a_col_s = None
         if isinstance(a, QuantizedTensor):
             # a grouped (packed rows, per-group padded) quantization made by the caller
             check_quantized_tensor(a, config, axis=-1, scaling_recipe=a_recipe)
@@ -339,20 +382,7 @@ class FP8GroupedGemmMXFunc(torch.autograd.Function):
                 a.contiguous(), fdt, None, bs, group_lens, group_offs, with_trans=True)
         else:
             a_row, a_row_s, _, offs_row = grouped_quantize_mxfp8_impl(a.contiguous(), fdt, 1, bs, group_lens, group_offs)
-        if isinstance(b, QuantizedTensor):
-            check_quantized_tensor(b, config, axis=-1, scaling_recipe=w_recipe)
-            b_row, b_row_s = b.qdata, b.scale_inv
-            if need_bwd:
-                if b_t is None:
-                    b_t = QuantizedTensor.quantize(b.dequantize(), b.real_dtype, gran, axis=-2, block_size=bs,
-                                                   scaling_recipe=w_recipe)
-                assert isinstance(b_t, QuantizedTensor)
-                b_col, b_col_s = b_t.qdata, b_t.scale_inv
-        elif need_bwd:
-            b_row, b_row_s, b_col, b_col_s = quantize_mxfp8_impl(
-                b.contiguous(), fdt, None, bs, with_trans=True, scaling_recipe=w_recipe, scaling_recipe_for_trans=w_recipe)
-        else:
-            b_row, b_row_s = quantize_mxfp8_impl(b.contiguous(), fdt, 2, bs, scaling_recipe=w_recipe)
+        b_row, b_row_s, b_col, b_col_s = _mx_weight_operands(b, b_t, config, need_bwd)
         # the padded row layout is read through offs_row, the result is packed by group_offs
         # into an output over-allocated to the padded rows
         out = grouped_gemm_fp8_impl(a_row, b_row, a_row_s, b_row_s, group_lens, offs_row, False, True, out_dtype,
@@ -367,19 +397,50 @@ class FP8GroupedGemmMXFunc(torch.autograd.Function):
         grad_out = _ensure_contiguous_grad_out(grad_out)
         a_col, a_col_s, b_col, b_col_s, group_lens, group_offs = ctx.saved_tensors
         config, out_dtype, num_cu, total_m, fuse_bgrad_accum, main_grad = ctx.meta
-        gdt = _get_fp8_dtype(config.format, False)
-        gran = config.granularity.value
-        g_row, g_row_s, g_col, g_col_s, _, offs_row, lens_col, offs_col = grouped_quantize_mxfp8_impl(
-            grad_out, gdt, None, config.block_size, group_lens, group_offs, with_trans=True)
-        # dgrad: grad_a = grad_out @ b, as an NT product with the transposed weight quantization [G, K, N]
-        grad_a = grouped_gemm_fp8_impl(g_row, b_col, g_row_s, b_col_s, group_lens, offs_row, False, True, out_dtype,
-                                       gran, num_cu, _NATIVE, False, group_offs)[:total_m]
-        # wgrad: grad_b[g] = grad_out_g^T @ a_g over the 128-padded segments -> [G, N, K]
-        grad_b = _grouped_gemm_fp8_variable_k_impl_wrapper(
-            g_col, a_col, g_col_s, a_col_s, lens_col, offs_col, False, False, False, out_dtype, gran, num_cu, _NATIVE,
-            inplace_add_to_out=fuse_bgrad_accum, out=main_grad,
-        )
+        grad_a, grad_b = _mx_backward_products(grad_out, a_col, a_col_s, b_col, b_col_s, group_lens, group_offs, config,
+                                               out_dtype, out_dtype, num_cu, total_m, fuse_bgrad_accum, main_grad)
         return grad_a, grad_b, None, None, None, None, None, None, None, None, None
+
+
+class FP8GluGroupedGemmMXFunc(torch.autograd.Function):
+    """Gated activation -> MXFP8 grouped GEMM (fc2 of an MoE expert MLP) with the activation fused
+    into the grouped MX quantizer of the GEMM's activation operand: the bf16 activation is neither
+    written nor re-read, forward or backward."""
+
+    @staticmethod
+    def forward(ctx, x, probs, row_mask, act_type, b, group_lens, group_offs, trans_b, out_dtype, config, num_cu,
+                fuse_bgrad_accum_pattern=None):
+        fuse_bgrad_accum, main_grad = _setup_fused_grad_accum(b, fuse_bgrad_accum_pattern)
+        assert config.granularity == ScalingGranularity.MX_BLOCKWISE and config.block_size == 32
+        assert x.ndim == 2 and x.size(1) % 2 == 0, "x must be [tokens, 2 * hidden]"
+        assert trans_b, "MXFP8 grouped GEMM only supports trans_b=True (NT layout)."
+        assert group_lens.size(0) == b.size(0), "group_lens size must match b size(0)."
+        assert probs.dtype == torch.float32 and probs.numel() == x.size(0), "probs must be float32, one per token"
+        total_m = int(x.size(0))
+        need_bwd = any(ctx.needs_input_grad[i] for i in (0, 1, 4))
+        x2, p1 = x.contiguous(), probs.reshape(-1).contiguous()
+        a_row, a_row_s, a_col, a_col_s, _, offs_row, _, _ = glu_grouped_quantize_mx_impl(
+            x2, p1, row_mask, act_type, _get_fp8_dtype(config.format, True), group_lens, group_offs, need_bwd)
+        b_row, b_row_s, b_col, b_col_s = _mx_weight_operands(b, None, config, need_bwd)
+        out = grouped_gemm_fp8_impl(a_row, b_row, a_row_s, b_row_s, group_lens, offs_row, False, True, out_dtype,
+                                    config.granularity.value, num_cu, _NATIVE, False, group_offs)[:total_m]
+        if need_bwd:
+            ctx.save_for_backward(x2, p1, row_mask, a_col, a_col_s, b_col, b_col_s, group_lens, group_offs)
+        ctx.meta = (config, out_dtype, num_cu, total_m, fuse_bgrad_accum, main_grad, act_type, probs.shape)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        from primus_turbo.pytorch.kernels.activation.glu_impl import ACT_GELU, ACT_SILU, glu_bwd_with_probs
+
+        grad_out = _ensure_contiguous_grad_out(grad_out)
+        x2, p1, row_mask, a_col, a_col_s, b_col, b_col_s, group_lens, group_offs = ctx.saved_tensors
+        config, out_dtype, num_cu, total_m, fuse_bgrad_accum, main_grad, act_type, probs_shape = ctx.meta
+        grad_act, grad_b = _mx_backward_products(grad_out, a_col, a_col_s, b_col, b_col_s, group_lens, group_offs, config,
+                                                 x2.dtype, out_dtype, num_cu, total_m, fuse_bgrad_accum, main_grad)
+        grad_x, grad_probs = glu_bwd_with_probs(grad_act.contiguous(), x2, p1, row_mask,
+                                                ACT_SILU if act_type == "silu" else ACT_GELU)
+        return grad_x, grad_probs.view(probs_shape), None, None, grad_b, None, None, None, None, None, None, None
 
 
 def grouped_gemm_fp8(
@@ -438,18 +499,22 @@ def glu_grouped_gemm_fp8(
     fuse_bgrad_accum_pattern: Optional[str] = None,
 ) -> torch.Tensor:
     """``grouped_gemm_fp8(swiglu_with_probs(x, probs, row_mask), b, group_lens, ...)`` (``act_type="gelu"``:
-    ``geglu_with_probs``) as one operation for the BLOCKWISE configuration: fc1's output ``x [tokens, 2 H]``
+    ``geglu_with_probs``) as one operation for the BLOCKWISE and MX_BLOCKWISE configurations: fc1's output ``x [tokens, 2 H]``
     is read once by a quantizer that applies the gated activation on load, so the bf16 activation
     never goes through HBM; results and gradients are bit-identical with the two-step form. (The
     reference has the two steps only: ops/activation.py:21-83, ops/grouped_gemm_fp8.py:99-265.)"""
     if config is None:
         config = Float8QuantConfig(granularity=ScalingGranularity.BLOCKWISE, block_size=128)
-    if config.granularity != ScalingGranularity.BLOCKWISE:
-        raise NotImplementedError("glu_grouped_gemm_fp8: the fused quantizer exists for the BLOCKWISE configuration")
+    if config.granularity not in (ScalingGranularity.BLOCKWISE, ScalingGranularity.MX_BLOCKWISE):
+        raise NotImplementedError(
+            "glu_grouped_gemm_fp8: the fused quantizer exists for the BLOCKWISE and MX_BLOCKWISE configurations")
     assert act_type in ("silu", "gelu"), f"Unsupported act_type: {act_type}"
     if group_offs is None:
         group_offs = group_offs_from_lens(group_lens)
     if out_dtype is None:
         out_dtype = torch.promote_types(x.dtype, b.dtype)
+    if config.granularity == ScalingGranularity.MX_BLOCKWISE:
+        return FP8GluGroupedGemmMXFunc.apply(x, probs, row_mask, act_type, b, group_lens, group_offs, trans_b, out_dtype,
+                                             config, num_cu, fuse_bgrad_accum_pattern)
     return FP8GluGroupedGemmBlockFunc.apply(x, probs, row_mask, act_type, b, group_lens, group_offs, trans_b, out_dtype,
                                             config, num_cu, fuse_bgrad_accum_pattern)

@@ -1,5 +1,5 @@
-"""The gated activation fused into the grouped blockwise quantizer, and the fused
-activation -> grouped GEMM operation built on it.
+"""The gated activation fused into the grouped quantizers (blockwise FP8, MXFP8, MXFP4), and the
+fused activation -> grouped GEMM operations built on them.
 
 Oracle = composition: ``oracle.activation`` (tolerance: floating point) -> the 16-bit rounding the
 stand-alone activation kernel stores -> ``oracle.quantize.fp8_blockwise_segment_m_row_col`` (bit-exact
@@ -19,9 +19,9 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture(scope="module", autouse=True)
 def _turbo(native_lib):
-    global turbo, qi, G, Float8QuantConfig
+    global turbo, qi, G, Float8QuantConfig, ScalingRecipe
     import primus_turbo.pytorch as turbo
-    from primus_turbo.pytorch.core.low_precision import Float8QuantConfig
+    from primus_turbo.pytorch.core.low_precision import Float8QuantConfig, ScalingRecipe
     from primus_turbo.pytorch.core.low_precision import ScalingGranularity as G
     from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
 
@@ -106,4 +106,85 @@ def test_fused_activation_grouped_gemm_equals_the_two_step_layer(act, trans_b):
     # inference (no gradient needed): the untransposed column output path
     with torch.no_grad():
         out = turbo.ops.glu_grouped_gemm_fp8(x, probs, w, gl, offs, trans_b=trans_b, config=cfg, row_mask=mask, act_type=act)
+    assert torch.equal(out, a[0])
+
+
+# ---- the grouped MX quantizers (MXFP8 / MXFP4) with the gated activation applied on load ----
+MX_CASES = [("balanced", 4, 1024, 512, False), ("ragged", 8, 3000, 384, True), ("zeros", 8, 2048, 256, False),
+            ("ragged", 3, 77, 96, True), ("zipf", 32, 8192, 2048, True)]
+
+
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e2m1"])
+@pytest.mark.parametrize("kind,G_,M,H,masked", MX_CASES)
+def test_fused_mx_quantizer_equals_the_two_steps_and_the_oracle(kind, G_, M, H, masked, fmt, dtype, act):
+    lens, gl, offs, x, probs, mask = _inputs(kind, G_, M, H, dtype, 181, masked)
+    fp4 = fmt == "e2m1"
+    qdt = {"e4m3": torch.float8_e4m3fn, "e5m2": torch.float8_e5m2, "e2m1": torch.float4_e2m1fn_x2}[fmt]
+    two = turbo.ops.swiglu_with_probs if act == "silu" else turbo.ops.geglu_with_probs
+    y = two(x, probs, mask)  # the stored activation of the two-step path (checked against its oracle above)
+    col_flags = 2 if fp4 else 0  # MXFP4's wgrad operand is Hadamard-transformed along the tokens
+    got = qi.glu_grouped_quantize_mx_impl(x, probs, mask, act, qdt, gl, offs, True, col_flags)
+    if fp4:
+        want = qi.grouped_quantize_mxfp4_impl(y, qdt, None, 32, gl, offs, with_trans=True, scaling_recipe=ScalingRecipe(),
+                                              scaling_recipe_for_trans=ScalingRecipe(use_rht=True))
+    else:
+        want = qi.grouped_quantize_mxfp8_impl(y, qdt, None, 32, gl, offs, with_trans=True)
+    torch.cuda.synchronize()
+    o = Q.mx_grouped_quant(to_f32_np(y), lens, fmt, row_align=1 if fp4 else 32, col_align=256 if fp4 else 128,
+                           col_rht=fp4)
+    mr, mc = int(o["row_offs"][-1]), int(o["col_offs"][-1])
+    pack = 2 if fp4 else 1
+    # bit for bit the two-step result ...
+    assert np.array_equal(codes_np(got[0])[:mr], codes_np(want[0])[:mr]), "row codes"
+    assert np.array_equal(codes_np(got[1])[:mr], codes_np(want[1])[:mr]), "row scales"
+    assert np.array_equal(codes_np(got[2])[:, : mc // pack], codes_np(want[2])[:, : mc // pack]), "column codes"
+    assert np.array_equal(codes_np(got[3])[:, : mc // 32], codes_np(want[3])[:, : mc // 32]), "column scales"
+    assert torch.equal(got[6], want[6]) and torch.equal(got[7], want[7])
+    if not fp4:
+        assert torch.equal(got[4], want[4]) and torch.equal(got[5], want[5])
+    # ... and the quantizer oracle on the stored activation
+    assert np.array_equal(codes_np(got[0])[:mr], o["row"]) and np.array_equal(codes_np(got[1])[:mr], o["row_scale"])
+    assert np.array_equal(codes_np(got[2])[:, : mc // pack], o["col"])
+    assert np.array_equal(codes_np(got[3])[:, : mc // 32], o["col_scale"])
+    # rows only (inference): the same row pair
+    r = qi.glu_grouped_quantize_mx_impl(x, probs, mask, act, qdt, gl, offs, False)
+    assert np.array_equal(codes_np(r[0])[:mr], o["row"]) and np.array_equal(codes_np(r[1])[:mr], o["row_scale"])
+    assert r[2].numel() == 0 and r[3].numel() == 0
+
+
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+@pytest.mark.parametrize("fp4", [False, True])
+def test_fused_activation_grouped_mx_gemm_equals_the_two_step_layer(act, fp4):
+    """fc2 of an expert MLP on MXFP8 / MXFP4 operands: the fused operation against
+    ``grouped_gemm_fp8/fp4(swiglu_with_probs(...))``, output and all three gradients, bit for bit."""
+    from primus_turbo.pytorch.core.low_precision import Float4QuantConfig, ScaleDtype
+
+    G_, M, H, N = 8, 2048, 512, 768
+    lens, gl, offs, x, probs, mask = _inputs("zipf", G_, M, H, torch.bfloat16, 191, True)
+    w = bf16_randn((G_, N, H), seed=195, scale=0.05).cuda()
+    dy = bf16_randn((M, N), seed=196).cuda()
+    if fp4:
+        cfg = Float4QuantConfig()
+        fused_op, plain_op = turbo.ops.glu_grouped_gemm_fp4, turbo.ops.grouped_gemm_fp4
+    else:
+        cfg = Float8QuantConfig(granularity=G.MX_BLOCKWISE, block_size=32, scale_dtype=ScaleDtype.E8M0)
+        fused_op, plain_op = turbo.ops.glu_grouped_gemm_fp8, turbo.ops.grouped_gemm_fp8
+
+    def run(fused):
+        xx, pp, ww = x.clone().requires_grad_(True), probs.clone().requires_grad_(True), w.clone().requires_grad_(True)
+        if fused:
+            out = fused_op(xx, pp, ww, gl, offs, config=cfg, row_mask=mask, act_type=act)
+        else:
+            two = turbo.ops.swiglu_with_probs if act == "silu" else turbo.ops.geglu_with_probs
+            out = plain_op(two(xx, pp, mask), ww, gl, offs, config=cfg)
+        out.backward(dy)
+        return out.detach(), xx.grad, pp.grad, ww.grad
+
+    a, b = run(True), run(False)
+    for name, u, v in zip(("out", "grad_x", "grad_probs", "grad_w"), a, b):
+        assert torch.equal(u, v), name
+    with torch.no_grad():
+        out = fused_op(x, probs, w, gl, offs, config=cfg, row_mask=mask, act_type=act)
     assert torch.equal(out, a[0])
