@@ -67,6 +67,57 @@ class _QuantBase:
                     sample=f"{what}, median of {len(times)} runs, {os.cpu_count()} logical CPUs visible")
 
 
+class HbmStream(_QuantBase):
+    """The yardstick of the HBM-bound kernels: what plain streaming kernels of the same traffic shape
+    reach on this GPU, measured by the same harness (rotating inputs, graph replays). The dominant
+    kernel reads a 16384 x 7168 bf16 tensor and writes one fp8-sized byte per element (the traffic
+    ratio of a quantizer, 3 bytes per element) with torch's elementwise cast; the other entries are
+    a same-size copy (2 + 2 bytes per element) and a read-only reduction."""
+
+    name = "hbm_streaming_yardstick_16384x7168_bf16 (torch elementwise cast to fp8, copy, abs-max)"
+    metric = "plain streaming GB/s & fraction of HBM peak"
+    dominant_name = "torch elementwise bf16 -> float8_e4m3fn cast (reads 2 B, writes 1 B per element)"
+    dtype = "bf16 (byte movement)"
+
+    def __init__(self, dev, M=16384, N=7168):
+        self.M, self.N = M, N
+        self.x_cpu = _randn_bf16((M, N), 5, 1.0)
+        self.x = self.x_cpu.to(dev)
+        self.q = torch.empty((M, N), dtype=torch.float8_e4m3fn, device=dev)
+        self.y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+
+    def dominant_work(self):
+        return 3.0 * self.M * self.N
+
+    step_work = dominant_work
+
+    def dominant(self):
+        self.q.copy_(self.x)
+        return self.q
+
+    step = dominant
+
+    def _copy(self):
+        self.y.copy_(self.x)
+        return self.y
+
+    def _amax(self):
+        return self.x.abs().amax()
+
+    def kernels(self):
+        n = float(self.M * self.N)
+        return [("copy_bf16_to_bf16", self._copy, 4.0 * n), ("abs_max_reduction_read_only", self._amax, 2.0 * n)]
+
+    def check(self):
+        ok = torch.equal(self._copy(), self.x) and torch.equal(self.dominant().float(), self.x.to(torch.float8_e4m3fn).float())
+        return bool(ok), "copy returns the input; cast equals torch's own cast (library kernels: nothing of this build is checked here)"
+
+    def cpu_baseline(self):
+        x = self.x_cpu[:2048]
+        y = torch.empty_like(x)
+        return self._cpu(lambda: y.copy_(x), 4.0 * x.numel(), "torch CPU copy of 2048 rows")
+
+
 class QuantRowwise(_QuantBase):
     """Rowwise FP8 quantize (last axis) + dequantize of an 8192 x 8192 bf16 GEMM operand."""
 
@@ -606,6 +657,7 @@ class MoePermute(_QuantBase):
 
 
 def register(workloads):
+    workloads["hbm_stream"] = HbmStream
     workloads["moe_permute"] = MoePermute
     workloads["swiglu_with_probs"] = SwigluWithProbs
     workloads["glu_quant_grouped"] = GluQuantGrouped

@@ -387,7 +387,9 @@ PT_API int pt_gemm_mx(const void *a, const void *a_scale, const void *b, const v
  * (or leaves it unchanged when accumulating). The workspace holds both transposed operands.
  * operands_kmajor != 0: LHS and RHS arrive transposed already, [Ml, Mp] and [Nr, Mp] (the
  * q_col_t output of pt_quantize_fp8_blockwise_segment_m_row_col_t, scales unchanged); no
- * workspace is used.
+ * workspace is used. tile_cfg 4 (the automatic choice for outputs of 1024 x 1024 and more) is a
+ * 256 x 256 tile with eight wavefronts that streams through the K ranges of consecutive groups
+ * without restarting its pipeline, writing one result tile per group on the way.
  */
 PT_API size_t pt_grouped_gemm_fp8_workspace_bytes(int64_t G, int64_t M, int64_t N, int64_t K,
                                                   int trans_b);

@@ -36,6 +36,8 @@
 #ifndef PT_GEMM_TRACE_POINT
 #define PT_GEMM_TRACE_DECL
 #define PT_GEMM_TRACE_POINT(id)
+#define PT_GEMM_TRACE_FLUSH
+#define PT_GEMM_TRACE_LDS_BYTES 0
 #endif
 namespace pt {
 

@@ -105,18 +105,29 @@ def test_grouped_forward_zero_tail_and_determinism():
 
 @pytest.mark.parametrize("kind,G_,M,N,K", CASES[:5])
 @pytest.mark.parametrize("trans_c", [True, False])
-def test_grouped_variable_k_product(kind, G_, M, N, K, trans_c):
+@pytest.mark.parametrize("tile_cfg", [0, 2, 4])
+def test_grouped_variable_k_product(kind, G_, M, N, K, trans_c, tile_cfg):
     """dW[g] = X_g^T . dY_g from the segment-padded column quantizations; an empty group gives
-    exactly zero; trans_c returns the transposed product."""
+    exactly zero; trans_c returns the transposed product. tile_cfg 4 is the eight-wavefront
+    256 x 256 kernel that streams through the groups of a chunk, 2 the 256 x 128 tile: the same
+    sums in the same order, so their results are identical."""
     lens = group_lens(kind, G_, M, 36)
     gl, offs = _offs(lens)
     x = bf16_randn((M, K), seed=37)
     dy = bf16_randn((M, N), seed=38)
     _, xc, _, xs, plens, poffs = qimpl.quant_fp8_blockwise_segment_m_row_col_impl(x.cuda(), torch.float8_e4m3fn, 128, gl, offs, N)
     _, gc, _, gs, _, _ = qimpl.quant_fp8_blockwise_segment_m_row_col_impl(dy.cuda(), torch.float8_e5m2, 128, gl, offs, K)
-    out = gimpl.grouped_gemm_fp8_variable_k_impl(xc, gc, xs, gs, plens, poffs, True, False, trans_c, torch.bfloat16,
-                                                 G.BLOCKWISE.value, None, 0)
+    gimpl.TILE_CFG = tile_cfg
+    try:
+        out = gimpl.grouped_gemm_fp8_variable_k_impl(xc, gc, xs, gs, plens, poffs, True, False, trans_c, torch.bfloat16,
+                                                     G.BLOCKWISE.value, None, 0)
+        gimpl.TILE_CFG = 3
+        out3 = gimpl.grouped_gemm_fp8_variable_k_impl(xc, gc, xs, gs, plens, poffs, True, False, trans_c, torch.bfloat16,
+                                                      G.BLOCKWISE.value, None, 0)
+    finally:
+        gimpl.TILE_CFG = 0
     torch.cuda.synchronize()
+    assert torch.equal(out, out3), "tile configurations differ"
     po = poffs.cpu().numpy()
     rows = int(po[-1])
     x_deq = Q.fp8_blockwise_dequant(codes_np(xc)[:rows], to_f32_np(xs)[: rows // 128], 0, "e4m3", 128)
@@ -131,7 +142,8 @@ def test_grouped_variable_k_product(kind, G_, M, N, K, trans_c):
     _gate(ref, got, f"{kind} G={G_} trans_c={trans_c}")
 
 
-def test_grouped_variable_k_accumulate():
+@pytest.mark.parametrize("tile_cfg", [0, 4])
+def test_grouped_variable_k_accumulate(tile_cfg):
     """beta = 1: the product is added to an fp32 buffer; empty groups leave theirs unchanged."""
     G_, M, N, K = 4, 1024, 256, 384
     lens = np.array([256, 0, 500, 268], dtype=np.int64)
@@ -142,10 +154,14 @@ def test_grouped_variable_k_accumulate():
     _, gc, _, gs, _, _ = qimpl.quant_fp8_blockwise_segment_m_row_col_impl(dy.cuda(), torch.float8_e4m3fn, 128, gl, offs, K)
     base = torch.randn((G_, N, K), generator=torch.Generator().manual_seed(41)).cuda()
     acc = base.clone()
-    fresh = gimpl.grouped_gemm_fp8_variable_k_impl(xc, gc, xs, gs, plens, poffs, True, False, True, torch.float32,
-                                                   G.BLOCKWISE.value, None, 0)
-    gimpl.grouped_gemm_fp8_variable_k_accum_impl(xc, gc, xs, gs, plens, poffs, True, False, True, torch.float32,
-                                                 G.BLOCKWISE.value, None, 0, acc)
+    gimpl.TILE_CFG = tile_cfg
+    try:
+        fresh = gimpl.grouped_gemm_fp8_variable_k_impl(xc, gc, xs, gs, plens, poffs, True, False, True, torch.float32,
+                                                       G.BLOCKWISE.value, None, 0)
+        gimpl.grouped_gemm_fp8_variable_k_accum_impl(xc, gc, xs, gs, plens, poffs, True, False, True, torch.float32,
+                                                     G.BLOCKWISE.value, None, 0, acc)
+    finally:
+        gimpl.TILE_CFG = 0
     torch.cuda.synchronize()
     assert torch.equal(acc[1], base[1])
     torch.testing.assert_close(acc, base + fresh, rtol=1e-6, atol=1e-5)
