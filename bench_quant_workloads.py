@@ -71,10 +71,10 @@ class HbmStream(_QuantBase):
     """The yardstick of the HBM-bound kernels: what plain streaming kernels of the same traffic shape
     reach on this GPU, measured by the same harness (rotating inputs, graph replays). The dominant
     kernel reads a 16384 x 7168 bf16 tensor and writes one fp8-sized byte per element (the traffic
-    ratio of a quantizer, 3 bytes per element) with torch's elementwise cast; the other entries are
-    a same-size copy (2 + 2 bytes per element) and a read-only reduction."""
+    ratio of a quantizer, 3 bytes per element) with torch's elementwise cast; the other entry is a
+    same-size copy (2 + 2 bytes per element)."""
 
-    name = "hbm_streaming_yardstick_16384x7168_bf16 (torch elementwise cast to fp8, copy, abs-max)"
+    name = "hbm_streaming_yardstick_16384x7168_bf16 (torch elementwise cast to fp8, copy)"
     metric = "plain streaming GB/s & fraction of HBM peak"
     dominant_name = "torch elementwise bf16 -> float8_e4m3fn cast (reads 2 B, writes 1 B per element)"
     dtype = "bf16 (byte movement)"
@@ -101,12 +101,9 @@ class HbmStream(_QuantBase):
         self.y.copy_(self.x)
         return self.y
 
-    def _amax(self):
-        return self.x.abs().amax()
-
     def kernels(self):
         n = float(self.M * self.N)
-        return [("copy_bf16_to_bf16", self._copy, 4.0 * n), ("abs_max_reduction_read_only", self._amax, 2.0 * n)]
+        return [("copy_bf16_to_bf16", self._copy, 4.0 * n)]
 
     def check(self):
         ok = torch.equal(self._copy(), self.x) and torch.equal(self.dominant().float(), self.x.to(torch.float8_e4m3fn).float())

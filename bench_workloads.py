@@ -22,19 +22,23 @@ FP4_PEAK_TFLOPS = 10100.0
 # 256 MiB launched in the same run (`bench.py --calib-copy`; factors 2.000 and 1.000); the runs are
 # summarised under profiles/. (fetched, written) in MiB.
 TRAFFIC_MIB = {
-    "gemm_fp8_rowwise": (779.3, 151.9),
-    "gemm_fp8_blockwise": (568.7, 224.0),
-    "gemm_fp8_blockwise_k7168": (1159.9, 128.1),
-    "gemm_fp8_blockwise_8192": (1327.5, 129.1),
-    "gemm_mxfp4": (3341.2, 761.7),
-    "gemm_mxfp8": (6414.0, 682.4),
-    # grouped workloads: forward launches only (the same kernel symbol also runs dgrad)
-    "grouped_gemm_fp8": (5333.5, 256.1),
-    "grouped_gemm_fp8_down": (2424.1, 448.2),
-    "grouped_gemm_mxfp8": (5495.4, 256.1),
-    "grouped_gemm_mxfp8_down": (2601.7, 448.2),
-    "grouped_gemm_mxfp4": (2767.3, 256.1),
-    "grouped_gemm_mxfp4_down": (1279.2, 448.2),
+    "gemm_fp8_rowwise": (779.1, 152.1),
+    "gemm_fp8_blockwise": (347.3, 226.2),
+    "gemm_fp8_blockwise_k7168": (691.3, 128.5),
+    "gemm_fp8_blockwise_8192": (791.2, 129.1),
+    "gemm_mxfp4": (3279.7, 704.3),
+    "gemm_mxfp8": (6357.3, 572.3),
+    "gemm_mxfp4_n28672": (1447.0, 448.0),
+    "gemm_mxfp8_n28672": (2781.0, 448.0),
+    # grouped workloads, forward launch: the fetch figure is the average over the forward and dgrad
+    # launches of the one kernel symbol that runs both (the counters cannot tell them apart), the
+    # write figure is the forward launches' own (they differ from dgrad's by the output width)
+    "grouped_gemm_fp8": (4820.8, 256.7),
+    "grouped_gemm_fp8_down": (2372.0, 449.6),
+    "grouped_gemm_mxfp8": (5490.2, 256.0),
+    "grouped_gemm_mxfp8_down": (2709.9, 448.1),
+    "grouped_gemm_mxfp4": (2752.2, 256.0),
+    "grouped_gemm_mxfp4_down": (1336.6, 448.0),
 }
 
 
@@ -147,7 +151,7 @@ class GemmFp8Rowwise(_GemmBase):
 class GemmFp8Blockwise(_GemmBase):
     """BASELINE config 2: DeepSeek-style blockwise GEMM, activations 1x128, weights 128x128."""
 
-    dominant_name = "gemm_fp8_nt_kernel<128x128 tile, 1x128 * 128x128 block scales>"
+    dominant_name = "gemm_fp8_block8_kernel<256x256 tile, eight wavefronts, 1x128 * 128x128 block scales>"
 
     def __init__(self, dev, M=16384, N=7168, K=2048):
         import primus_turbo.pytorch as turbo
@@ -341,7 +345,7 @@ class GroupedGemmFp8(_GemmBase):
     Zipf(1.2) counts with empty experts), blockwise 128 scales; a step is forward + dgrad + wgrad
     of one expert layer through the autograd op."""
 
-    dominant_name = "gemm_fp8_nt_kernel<128x128 tile, row groups, 1x128 * 128x128 block scales> (forward)"
+    dominant_name = "gemm_fp8_block8_kernel<256x256 tile, eight wavefronts, row groups, 1x128 * 128x128 block scales> (forward)"
 
     def __init__(self, dev, N=4096, K=7168, groups=32, tokens=32768):
         import primus_turbo.pytorch as turbo
