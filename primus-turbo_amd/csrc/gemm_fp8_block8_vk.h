@@ -29,7 +29,7 @@
 
 namespace pt {
 
-constexpr int B8V_MAX_CHUNKS = 16;
+constexpr int B8V_MAX_CHUNKS = VK_MAX_CHUNKS;
 
 template <int FA, int FB>
 __global__ __launch_bounds__(B8_THREADS) void gemm_fp8_block8_vk_kernel(const GemmArgs a, const int chunks) {
@@ -308,25 +308,6 @@ __global__ __launch_bounds__(B8_THREADS) void gemm_fp8_block8_vk_kernel(const Ge
     PT_GEMM_TRACE_FLUSH;
 }
 
-// chunks per output position: the smallest count (up to the group count) with which the units
-// fill whole rounds of the grid to within 5 %, else the best found
-static inline int b8v_pick_chunks(int64_t positions, int64_t grid, int64_t groups) {
-    int    best = 1;
-    double best_eff = 0.0;
-    const int64_t cmax = groups < B8V_MAX_CHUNKS ? groups : B8V_MAX_CHUNKS;
-    for (int c = 1; c <= cmax; ++c) {
-        const int64_t u = positions * c;
-        const double  eff = static_cast<double>(u) / static_cast<double>(cdiv(u, grid) * grid);
-        if (eff > best_eff + 1e-9) {
-            best     = c;
-            best_eff = eff;
-        }
-        if (eff >= 0.95)
-            break;
-    }
-    return best;
-}
-
 template <int FA, int FB> static int launch_gemm_block8_vk(const GemmArgs &args_in, hipStream_t stream) {
     constexpr int LDS = B8_NSTAGE * B8_STAGE + (B8V_MAX_CHUNKS + 2) * 4 + PT_GEMM_TRACE_LDS_BYTES;
     static_assert(LDS <= 160 * 1024, "tile configuration does not fit the LDS");
@@ -351,7 +332,7 @@ template <int FA, int FB> static int launch_gemm_block8_vk(const GemmArgs &args_
     }
     const int64_t positions = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
     const int64_t cus       = device_cu_count();
-    const int     chunks    = b8v_pick_chunks(positions, cus, a.G);
+    const int     chunks    = vk_pick_chunks(positions, cus, a.G);
     int64_t       grid      = positions * chunks < cus ? positions * chunks : cus;
     if (grid <= 0)
         return PT_OK;

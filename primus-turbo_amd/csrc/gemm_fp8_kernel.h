@@ -62,6 +62,9 @@ struct GemmArgs {
     //         rows are contiguous and a scale copy fetches two cache lines instead of sixty-four
     int64_t sa_m, sa_k, sb_n, sb_k;
     int64_t sa_wpitch, sb_wpitch;
+    // GROUP_K: the groups are cut into this many runs of about equal K length; a unit of work is one
+    // output position times one run (set by the launcher)
+    int vk_chunks;
     int     sa_shift, sb_shift; // 0 (one scale per row) or 7 (one per 128 rows)
     int     kb_valid;           // BLOCK / MX: K blocks the scale arrays hold (slabs beyond are zero padding)
     int     out_dtype;
@@ -379,6 +382,7 @@ struct TileCtx {
     const float   *sA, *sB; // scale arrays of the tile's matrix (BLOCK: at its first K block)
     uint8_t       *C;       // the tile's output matrix
     int            KT;      // K slabs of this tile
+    int            g0, g1;  // GROUP_K: the unit's groups [g0, g1) (KT = slabs of all of them)
 };
 
 // GROUP_ROWS: prefix[g] = number of tiles of the groups before g (in LDS), `g` is a search
@@ -386,7 +390,8 @@ struct TileCtx {
 template <int BM, int BN, int GMODE, bool F4 = false>
 __device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile, const int *prefix, int &g) {
     TileCtx t;
-    int     tm, tn;
+    t.g0 = t.g1 = 0;
+    int tm, tn;
     if constexpr (GMODE == GROUP_NONE) {
         tile_coords(tile, a.tiles_m, a.tiles_n, tm, tn);
         t.m0    = static_cast<int64_t>(tm) * BM;
@@ -420,21 +425,25 @@ __device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile, const 
             t.C += (a.group_offs_out[g] - lo) * a.N * (a.out_dtype == PT_DTYPE_F32 ? 4 : 2);
         t.KT    = static_cast<int>(a.K / KSTEP);
     } else {
-        // a group's tiles in XCD-contiguous order (workgroup i runs on XCD i % 8 and walks tiles
-        // i, i + grid, ...): every XCD works on a compact block of the group's output, so the
-        // group's operand panels are fetched into few L2s instead of all eight
-        const int per = a.tiles_m * a.tiles_n;
-        g             = tile / per;
-        tile_coords_local(xcd_contiguous_id(tile - g * per, per), a.tiles_m, a.tiles_n, tm, tn);
+        // unit = (chunk of consecutive groups, output position); the positions in XCD-contiguous
+        // order (workgroup i runs on XCD i % 8 and walks units i, i + grid, ...): every XCD works on a
+        // compact block of the output, so the chunk's operand panels are fetched into few L2s, and
+        // all workgroups are in the same chunk at the same time
+        const int per   = a.tiles_m * a.tiles_n;
+        const int chunk = tile / per;
+        tile_coords_local(xcd_contiguous_id(tile - chunk * per, per), a.tiles_m, a.tiles_n, tm, tn);
+        t.g0 = __builtin_amdgcn_readfirstlane(prefix[chunk]);
+        t.g1 = __builtin_amdgcn_readfirstlane(prefix[chunk + 1]);
+        g    = t.g0;
         // K ranges are given in elements; two E2M1 codes share a byte
-        const int64_t lo = a.group_offs[g] >> (F4 ? 1 : 0), hi = a.group_offs[g + 1] >> (F4 ? 1 : 0);
+        const int64_t lo = a.group_offs[t.g0] >> (F4 ? 1 : 0), hi = a.group_offs[t.g1] >> (F4 ? 1 : 0);
         t.m0    = static_cast<int64_t>(tm) * BM;
         t.m_end = a.M;
         t.Ag    = a.A + t.m0 * a.lda + lo;
         t.Bg    = a.B + lo;
         t.sA    = a.sA + (lo / KSTEP) * a.sa_k;
         t.sB    = a.sB + (lo / KSTEP) * a.sb_k;
-        t.C     = static_cast<uint8_t *>(a.C) + g * a.c_gstride * (a.out_dtype == PT_DTYPE_F32 ? 4 : 2);
+        t.C     = static_cast<uint8_t *>(a.C);
         t.KT    = static_cast<int>((hi - lo) / KSTEP);
     }
     t.n0     = static_cast<int64_t>(tn) * BN;
@@ -496,9 +505,12 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     constexpr int  NSB     = SB_VEC ? 4 : 1;
     static_assert(MODE != SCALE_BLOCK || SB_VEC || TN * 16 <= 128, "one B scale per wavefront and slab");
     [[maybe_unused]] uint32_t unit_scale = 0x7f7f7f7fu; // E8M0 1.0 for all four K blocks
-    // GROUP_K tiles have their own K extent (possibly none at all): they run the pipeline per
-    // tile instead of across tile boundaries; only the request for a tile's first two slabs is
-    // moved ahead of the previous tile's epilogue
+    // GROUP_K: a "tile" is a unit of work, one output position streaming through the K ranges of a
+    // chunk of consecutive groups (they lie side by side along K): the slab sequence continues
+    // across group boundaries, where the sums are written to the group's C and cleared. Units have
+    // their own K extent (possibly none at all), so the pipeline is restarted per unit instead of
+    // running across unit boundaries; only the request for a unit's first two slabs is moved
+    // ahead of the previous unit's last epilogue.
     constexpr bool XPIPE = GMODE != GROUP_K;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
@@ -513,7 +525,8 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     const uint32_t frag_off_hi = lm * KSTEP + (((4 + lg) ^ swz(lm)) << 4);
 
     // ---- tile list ----
-    int *prefix = reinterpret_cast<int *>(smem + NSTAGE * STAGE); // GROUP_ROWS: tiles before group g
+    // GROUP_ROWS: tiles before group g; GROUP_K: first group of chunk c
+    int *prefix = reinterpret_cast<int *>(smem + NSTAGE * STAGE);
     int  total;
     if constexpr (GMODE == GROUP_ROWS) {
         for (int g = tid; g < a.G; g += 256) {
@@ -533,7 +546,23 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         __syncthreads();
         total = __builtin_amdgcn_readfirstlane(prefix[a.G]);
     } else if constexpr (GMODE == GROUP_K) {
-        total = a.G * a.tiles_m * a.tiles_n;
+        // chunk c = groups [prefix[c], prefix[c + 1]): its first group is the first one that starts at
+        // or behind c / chunks of the total K length
+        const int     chunks  = a.vk_chunks;
+        const int64_t k_first = a.group_offs[0], k_total = a.group_offs[a.G] - k_first;
+        if (tid <= chunks)
+            prefix[tid] = a.G;
+        __syncthreads();
+        for (int g = tid; g < a.G; g += 256) {
+            const int64_t cum = a.group_offs[g] - k_first, prev = g > 0 ? a.group_offs[g - 1] - k_first : -1;
+            for (int c = 0; c < chunks; ++c) {
+                const int64_t thr = k_total * c / chunks;
+                if (cum >= thr && prev < thr)
+                    prefix[c] = g;
+            }
+        }
+        __syncthreads();
+        total = chunks * a.tiles_m * a.tiles_n;
     } else {
         total = a.tiles_m * a.tiles_n;
     }
@@ -796,7 +825,8 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
 
         // one K slab per iteration; the body must stay a single basic block (no branches), or
         // the compiler sinks the MFMAs behind them
-        for (int kt = 0; kt < KT; ++kt) {
+        auto run_slabs = [&](const int n_slabs) {
+        for (int kt = 0; kt < n_slabs; ++kt) {
             const int      buf_n = buf + 1 == NSTAGE ? 0 : buf + 1;
             const uint8_t *nxt   = smem + buf_n * STAGE;
             // where the slab two steps ahead goes: the current stage (after barrier X), or with
@@ -915,25 +945,50 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             advance_loader();
             buf = buf_n;
         }
-        PT_GEMM_TRACE_POINT(4);
-        if constexpr (!XPIPE) {
-            // the re-read copies of the last slab must have landed everywhere, and everyone must be
-            // done reading the stages, before the next tile's first copies go into them
-            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-            __builtin_amdgcn_s_barrier();
-            // the next tile's first slabs travel while this tile's result is written out
-            if (next_tile < total && nxt_t.KT > 0)
-                request_first_slabs(nxt_t);
-        }
-
-        // the epilogue reads the accumulators with hand-written instructions the compiler's
-        // hazard tracking does not see: let the last MFMA's write-back finish first
-        if constexpr (MODE != SCALE_BLOCK)
-            asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
-        PT_GEMM_TRACE_POINT(5);
+        };
         const int64_t wm_base = cur_t.m0 + wm * (TM * 16), wn_base = cur_t.n0 + wn * (TN * 16);
-        epilogue<TM, TN, MODE, MODE != SCALE_BLOCK>(a, acc, cur_t.C, cur_t.sA, cur_t.sB, cur_t.m_end, wm_base, wn_base,
-                                                     lane);
+        if constexpr (XPIPE) {
+            run_slabs(KT);
+            PT_GEMM_TRACE_POINT(4);
+            // the epilogue reads the accumulators with hand-written instructions the compiler's
+            // hazard tracking does not see: let the last MFMA's write-back finish first
+            if constexpr (MODE != SCALE_BLOCK)
+                asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+            PT_GEMM_TRACE_POINT(5);
+            epilogue<TM, TN, MODE, MODE != SCALE_BLOCK>(a, acc, cur_t.C, cur_t.sA, cur_t.sB, cur_t.m_end, wm_base, wn_base,
+                                                         lane);
+        } else {
+            const int ES     = a.out_dtype == PT_DTYPE_F32 ? 4 : 2;
+            int64_t   g_lo   = a.group_offs[cur_t.g0] >> (F4 ? 1 : 0);
+            for (int g = cur_t.g0; g < cur_t.g1; ++g) {
+                const int64_t g_hi = a.group_offs[g + 1] >> (F4 ? 1 : 0);
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+                run_slabs(static_cast<int>((g_hi - g_lo) / KSTEP));
+                g_lo = g_hi;
+                PT_GEMM_TRACE_POINT(4);
+                if (g + 1 == cur_t.g1) {
+                    // the re-read copies of the unit's last slab must have landed everywhere, and
+                    // everyone must be done reading the stages, before the next unit's first copies go
+                    // into them
+                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                    __builtin_amdgcn_s_barrier();
+                    // the next unit's first slabs travel while this unit's last result is written out
+                    if (next_tile < total && nxt_t.KT > 0)
+                        request_first_slabs(nxt_t);
+                }
+                if constexpr (MODE != SCALE_BLOCK)
+                    asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+                PT_GEMM_TRACE_POINT(5);
+                uint8_t *Cg = cur_t.C + static_cast<int64_t>(g) * a.c_gstride * ES;
+                epilogue<TM, TN, MODE, MODE != SCALE_BLOCK>(a, acc, Cg, cur_t.sA, cur_t.sB, cur_t.m_end, wm_base, wn_base, lane);
+            }
+            if (cur_t.g0 >= cur_t.g1 && next_tile < total && nxt_t.KT > 0)
+                request_first_slabs(nxt_t); // (an empty chunk: nothing was in flight)
+        }
 
         PT_GEMM_TRACE_POINT(6);
         if (next_tile >= total)
@@ -945,6 +1000,26 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+// GROUP_K: chunks of consecutive groups per output position: the smallest count (up to the group
+// count) with which the units fill whole rounds of the grid to within 5 %, else the best found
+constexpr int VK_MAX_CHUNKS = 16;
+static inline int vk_pick_chunks(int64_t positions, int64_t grid, int64_t groups) {
+    int           best     = 1;
+    double        best_eff = 0.0;
+    const int64_t cmax     = groups < VK_MAX_CHUNKS ? groups : VK_MAX_CHUNKS;
+    for (int c = 1; c <= cmax; ++c) {
+        const int64_t u   = positions * c;
+        const double  eff = static_cast<double>(u) / static_cast<double>((u + grid - 1) / grid * grid);
+        if (eff > best_eff + 1e-9) {
+            best     = c;
+            best_eff = eff;
+        }
+        if (eff >= 0.95)
+            break;
+    }
+    return best;
+}
+
 // Upper bound on the number of tiles (exact for the ungrouped case): GROUP_ROWS cannot know
 // the per-group row counts on the host, but every group adds at most one partial tile row.
 template <int TM, int TN, int MODE, bool SB_VEC, int FA, int FB, int GMODE = GROUP_NONE>
@@ -953,7 +1028,7 @@ static int launch_gemm_cfg(const GemmArgs &args_in, hipStream_t stream) {
     constexpr int STAGES  = gemm_stages(TM, TN, FA == 4) * gemm_stage_bytes(TM, TN, MODE, FA == 4);
     // groups whose tile prefix sums fit into the LDS next to the stages
     constexpr int MAX_G   = (160 * 1024 - STAGES) / 4 - 2 < 2048 ? 1024 : 2048;
-    constexpr int LDS_MAX = STAGES + (GMODE == GROUP_ROWS ? (MAX_G + 2) * 4 : 0);
+    constexpr int LDS_MAX = STAGES + (GMODE == GROUP_ROWS ? (MAX_G + 2) * 4 : GMODE == GROUP_K ? (VK_MAX_CHUNKS + 2) * 4 : 0);
     static_assert(LDS_MAX <= 160 * 1024, "tile configuration does not fit the LDS");
     GemmArgs a = args_in;
     a.gmode    = GMODE;
@@ -981,17 +1056,20 @@ static int launch_gemm_cfg(const GemmArgs &args_in, hipStream_t stream) {
             return fail(PT_ERR_LAUNCH, "gemm_fp8: cannot raise the dynamic LDS limit");
         attr_set.fetch_or(dev_bit, std::memory_order_release);
     }
-    const int lds = STAGES + (GMODE == GROUP_ROWS ? (a.G + 2) * 4 : 0);
+    const int lds = STAGES + (GMODE == GROUP_ROWS ? (a.G + 2) * 4 : GMODE == GROUP_K ? (VK_MAX_CHUNKS + 2) * 4 : 0);
     // persistent grid: as many workgroups as fit on the machine at once (LDS-limited)
     const int per_cu = (160 * 1024) / lds;
+    int64_t   grid   = static_cast<int64_t>(device_cu_count()) * (per_cu < 1 ? 1 : per_cu);
     int64_t   total;
-    if (GMODE == GROUP_ROWS)
+    if (GMODE == GROUP_ROWS) {
         total = (static_cast<int64_t>(a.tiles_m) + a.G) * a.tiles_n;
-    else if (GMODE == GROUP_K)
-        total = static_cast<int64_t>(a.G) * a.tiles_m * a.tiles_n;
-    else
+    } else if (GMODE == GROUP_K) {
+        const int64_t positions = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
+        a.vk_chunks             = vk_pick_chunks(positions, grid, a.G);
+        total                   = positions * a.vk_chunks;
+    } else {
         total = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
-    int64_t grid = static_cast<int64_t>(device_cu_count()) * (per_cu < 1 ? 1 : per_cu);
+    }
     if (grid > total)
         grid = total;
     if (grid <= 0)
