@@ -33,12 +33,12 @@ TRAFFIC_MIB = {
     # grouped workloads, forward launch: the fetch figure is the average over the forward and dgrad
     # launches of the one kernel symbol that runs both (the counters cannot tell them apart), the
     # write figure is the forward launches' own (they differ from dgrad's by the output width)
-    "grouped_gemm_fp8": (4820.8, 256.7),
-    "grouped_gemm_fp8_down": (2372.0, 449.6),
-    "grouped_gemm_mxfp8": (5490.2, 256.0),
-    "grouped_gemm_mxfp8_down": (2709.9, 448.1),
-    "grouped_gemm_mxfp4": (2752.2, 256.0),
-    "grouped_gemm_mxfp4_down": (1336.6, 448.0),
+    "grouped_gemm_fp8": (4810.3, 256.6),
+    "grouped_gemm_fp8_down": (2372.3, 449.4),
+    "grouped_gemm_mxfp8": (5354.8, 256.0),
+    "grouped_gemm_mxfp8_down": (2653.8, 448.0),
+    "grouped_gemm_mxfp4": (2752.3, 256.0),
+    "grouped_gemm_mxfp4_down": (1335.2, 448.0),
 }
 
 
