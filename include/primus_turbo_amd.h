@@ -348,7 +348,8 @@ PT_API int pt_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const v
  * four) are first copied into `workspace` (pt_gemm_mx_workspace_bytes, 16-byte aligned); for
  * large problems the workspace also receives a copy of both scale arrays with the 32-bit words
  * of one K position of all rows contiguous, which is what the kernel's scale copies then read.
- * accumulate != 0 adds into C (beta = 1). tile_cfg as for pt_gemm_fp8. */
+ * accumulate != 0 adds into C (beta = 1). tile_cfg as for pt_gemm_fp8; 4 = 256 x 256 tile with
+ * eight wavefronts (the automatic choice for MXFP4 with M, N >= 2048), bit-identical results. */
 PT_API size_t pt_gemm_mx_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                                          int fp4);
 PT_API int pt_gemm_mx(const void *a, const void *a_scale, const void *b, const void *b_scale,

@@ -73,11 +73,52 @@ def test_mxfp4_gemm_matches_dequantized_matmul(M, N, K):
     _gate(ref, to_f32_np(out), f"mxfp4 {M}x{N}x{K}")
 
 
-def test_mx_gemm_exact_on_integers():
+@pytest.mark.parametrize("M,N,K", SHAPES + [(2048, 2304, 4224)])
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e2m1"])
+def test_mx_gemm_eight_wavefront_tile(M, N, K, fmt):
+    """tile_cfg 4 (256 x 256 tile, eight wavefronts, gemm_mx8.h) against the oracle and against the
+    automatic configuration: the same products added in the same order, so the bits are the same.
+    Exact-integer operands on the same path in the next test."""
+    if fmt == "e2m1" and FP4 is None:
+        pytest.skip("torch has no float4_e2m1fn_x2")
+    a = bf16_randn((M, K), seed=71, outlier_frac=0.002).cuda()
+    b = bf16_randn((N, K), seed=72).cuda()
+    if fmt == "e2m1":
+        aq, as_ = qi.quantize_mxfp4_impl(a, FP4, 1, 32)
+        bq, bs = qi.quantize_mxfp4_impl(b, FP4, 1, 32, scaling_recipe=ScalingRecipe(use_2d_block=True))
+        run = lambda: g4.gemm_fp4_impl(aq, as_, False, bq, bs, True, torch.float32, False, G.MX_BLOCKWISE.value, 0)  # noqa: E731
+    else:
+        dt = torch.float8_e4m3fn if fmt == "e4m3" else torch.float8_e5m2
+        aq, as_ = qi.quantize_mxfp8_impl(a, dt, 1, 32)
+        bq, bs = qi.quantize_mxfp8_impl(b, torch.float8_e4m3fn, 1, 32, scaling_recipe=ScalingRecipe(use_2d_block=True))
+        run = lambda: gi.gemm_fp8_impl(aq, as_, False, bq, bs, True, torch.bfloat16, False, G.MX_BLOCKWISE.value, 0)  # noqa: E731
+    auto = run()
+    gi.TILE_CFG = 4
+    try:
+        got = run()
+    finally:
+        gi.TILE_CFG = 0
+    torch.cuda.synchronize()
+    assert torch.equal(got, auto), "tile configurations differ"
+    ref = OG.gemm_dequantized(Q.mx_dequant(codes_np(aq), codes_np(as_), fmt),
+                              Q.mx_dequant(codes_np(bq), codes_np(bs), "e2m1" if fmt == "e2m1" else "e4m3"))
+    _gate(ref, to_f32_np(got), f"mx8 {fmt} {M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("tile_cfg", [0, 4])
+def test_mx_gemm_exact_on_integers(tile_cfg):
+    gi.TILE_CFG = tile_cfg
+    try:
+        _exact_on_integers((128, 128, 512) if tile_cfg == 0 else (384, 320, 1024))
+    finally:
+        gi.TILE_CFG = 0
+
+
+def _exact_on_integers(shape):
     """Operands whose codes and block scales make every partial product an exact small integer
     times a power of two: the fp32 result must equal the exact value, which fails for any
     mismatch between scale bytes and the rows / K blocks they belong to."""
-    M, N, K = 128, 128, 512
+    M, N, K = shape
     rng = np.random.default_rng(64)
     # values k * 2^e with k in {-3..3} and a per (row, 32-block) exponent e in {-2..2}
     ea = rng.integers(-2, 3, size=(M, K // 32))
