@@ -142,6 +142,55 @@ def test_grouped_variable_k_product(kind, G_, M, N, K, trans_c, tile_cfg):
     _gate(ref, got, f"{kind} G={G_} trans_c={trans_c}")
 
 
+@pytest.mark.parametrize("kind,G_,M", [("balanced", 1, 1500), ("zipf", 5, 3000), ("zeros", 64, 6000), ("zipf", 40, 9000)])
+@pytest.mark.parametrize("out_dtype,accumulate", [(torch.bfloat16, False), (torch.float32, False), (torch.float32, True)])
+def test_grouped_variable_k_streaming_tile_mid_size(kind, G_, M, out_dtype, accumulate):
+    """Outputs of 1024 x 1280 (the automatic choice is the eight-wavefront streaming tile; 1280 is
+    not a whole number of 256-column tiles, so edge tiles take the checked store path) with one
+    group, few groups, more groups than chunks and many empty ones: identical with the 128 x 128
+    four-wavefront tile, within the gate of the oracle, empty groups exactly zero / untouched."""
+    N, K = 1280, 1024  # dW is [G, N, K] with trans_c
+    lens = group_lens(kind, G_, M, 136)
+    gl, offs = _offs(lens)
+    x = bf16_randn((M, K), seed=137)
+    dy = bf16_randn((M, N), seed=138)
+    _, xc, _, xs, plens, poffs = qimpl.quant_fp8_blockwise_segment_m_row_col_impl(x.cuda(), torch.float8_e4m3fn, 128, gl, offs, N)
+    _, gc, _, gs, _, _ = qimpl.quant_fp8_blockwise_segment_m_row_col_impl(dy.cuda(), torch.float8_e5m2, 128, gl, offs, K)
+
+    def run(cfg):
+        gimpl.TILE_CFG = cfg
+        try:
+            if accumulate:
+                base = torch.full((G_, N, K), 0.5, dtype=torch.float32, device="cuda")
+                gimpl.grouped_gemm_fp8_variable_k_accum_impl(xc, gc, xs, gs, plens, poffs, True, False, True, out_dtype,
+                                                             G.BLOCKWISE.value, None, 0, base)
+                return base - 0.5
+            return gimpl.grouped_gemm_fp8_variable_k_impl(xc, gc, xs, gs, plens, poffs, True, False, True, out_dtype,
+                                                          G.BLOCKWISE.value, None, 0)
+        finally:
+            gimpl.TILE_CFG = 0
+
+    auto, small = run(0), run(3)
+    torch.cuda.synchronize()
+    if accumulate:  # (x + 0.5) - 0.5 rounds differently from x for small x: compare within fp32 noise
+        torch.testing.assert_close(auto, small, rtol=0, atol=1e-5)
+    else:
+        assert torch.equal(auto, small), "tile configurations differ"
+    po = poffs.cpu().numpy()
+    rows = int(po[-1])
+    x_deq = Q.fp8_blockwise_dequant(codes_np(xc)[:rows], to_f32_np(xs)[: rows // 128], 0, "e4m3", 128)
+    g_deq = Q.fp8_blockwise_dequant(codes_np(gc)[:rows], to_f32_np(gs)[: rows // 128], 0, "e5m2", 128)
+    ref = np.ascontiguousarray(OG.grouped_gemm_variable_k_dequantized(x_deq, g_deq, np.diff(po)).transpose(0, 2, 1))
+    got = to_f32_np(auto)
+    for g in range(G_):
+        if lens[g] == 0:
+            assert not got[g].any(), f"group {g} is empty: its dW must be exactly zero (or untouched)"
+    if accumulate:
+        assert OG.cosine(ref, got) >= MIN_COS
+    else:
+        _gate(ref, got, f"{kind} G={G_}")
+
+
 @pytest.mark.parametrize("tile_cfg", [0, 4])
 def test_grouped_variable_k_accumulate(tile_cfg):
     """beta = 1: the product is added to an fp32 buffer; empty groups leave theirs unchanged."""
