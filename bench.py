@@ -184,8 +184,9 @@ DEFAULT_ORDER = ["gemm_fp8_blockwise_8192", "gemm_fp8_rowwise", "quant_tensorwis
 
 # the other workloads of the configurations the path is quoted on, reported under "extra"
 EXTRA_GEMM = ["gemm_fp8_rowwise", "gemm_fp8_blockwise", "gemm_fp8_blockwise_k7168", "grouped_gemm_fp8",
-              "grouped_gemm_fp8_down", "gemm_mxfp4", "gemm_mxfp4_n28672", "gemm_mxfp8", "gemm_mxfp8_n28672"]
-EXTRA_QUANT = ["hbm_stream", "quant_tensorwise", "quant_rowwise", "quant_blockwise", "quant_blockwise_dual", "quant_blockwise_weight",
+              "grouped_gemm_fp8_down", "gemm_mxfp4", "gemm_mxfp4_n28672", "gemm_mxfp8", "gemm_mxfp8_n28672",
+              "grouped_gemm_mxfp8", "grouped_gemm_mxfp8_down", "grouped_gemm_mxfp4", "grouped_gemm_mxfp4_down"]
+EXTRA_QUANT = ["hbm_stream", "swiglu_with_probs", "moe_permute", "quant_tensorwise", "quant_rowwise", "quant_blockwise", "quant_blockwise_dual", "quant_blockwise_weight",
                "quant_grouped", "glu_quant_grouped", "glu_quant_grouped_mxfp8", "quant_mxfp8", "quant_mxfp8_dual", "quant_mxfp4", "quant_mxfp4_dual"]
 EXTRA_BUDGET_S = 400.0  # no further extra workload is started after this many seconds of run time
 

@@ -509,6 +509,44 @@ class GroupedGemmMxfp8(_GemmBase):
         return self.gg.grouped_gemm_fp8_impl(self.qr, self.wq, self.sr, self.ws, self.gl, self.offs_row, False, True,
                                              torch.bfloat16, self.G.MX_BLOCKWISE.value, None, 0, False, self.offs)
 
+    def _backward_operands(self):
+        """(grad row codes / scales, grad column codes / scales, activation column codes / scales,
+        transposed weight codes / scales, padded row offsets, padded column lens / offsets) as
+        the autograd function prepares them."""
+        from primus_turbo.pytorch.core.low_precision import ScalingRecipe
+
+        qi, f8 = self.qi, torch.float8_e4m3fn
+        _, _, a_col, a_col_s, _, _, _, _ = qi.grouped_quantize_mxfp8_impl(self.x.detach(), f8, None, 32, self.gl, self.offs,
+                                                                          with_trans=True)
+        g_row, g_row_s, g_col, g_col_s, _, offs_row, lens_col, offs_col = qi.grouped_quantize_mxfp8_impl(
+            self.dy, f8, None, 32, self.gl, self.offs, with_trans=True)
+        r2 = ScalingRecipe(use_2d_block=True)
+        _, _, b_col, b_col_s = qi.quantize_mxfp8_impl(self.w.detach(), f8, None, 32, with_trans=True, scaling_recipe=r2,
+                                                      scaling_recipe_for_trans=r2)
+        return g_row, g_row_s, g_col, g_col_s, a_col, a_col_s, b_col, b_col_s, offs_row, lens_col, offs_col
+
+    def _impls(self):
+        return self.gg.grouped_gemm_fp8_impl, self.gg.grouped_gemm_fp8_variable_k_impl
+
+    def kernels(self):
+        """The three GEMM launches of the step on pre-quantized operands, as the autograd function
+        issues them: (name, callable, flops)."""
+        if not hasattr(self, "_bwd"):
+            self._bwd = self._backward_operands()
+        g_row, g_row_s, g_col, g_col_s, a_col, a_col_s, b_col, b_col_s, offs_row, lens_col, offs_col = self._bwd
+        rows_impl, vk_impl = self._impls()
+        gran, flops = self.G.MX_BLOCKWISE.value, 2.0 * self.M * self.N * self.K
+
+        def dgrad():
+            return rows_impl(g_row, b_col, g_row_s, b_col_s, self.gl, offs_row, False, True, torch.bfloat16, gran, None, 0,
+                             False, self.offs)
+
+        def wgrad():
+            return vk_impl(g_col, a_col, g_col_s, a_col_s, lens_col, offs_col, False, False, False, torch.bfloat16, gran,
+                           None, 0)
+
+        return [("forward", self.dominant, flops), ("dgrad", dgrad, flops), ("wgrad_variable_k", wgrad, flops)]
+
     def check(self):
         """Forward rows of the first and of the last non-empty expert (up to 64 each) against the
         oracle's de-quantized matmul; their codes and E8M0 bytes bit-exact."""
@@ -603,6 +641,24 @@ class GroupedGemmMxfp4(GroupedGemmMxfp8):
     def dominant(self):
         return self.gg.grouped_gemm_fp4_impl(self.qr, self.wq, self.sr, self.ws, self.gl, self.offs_row, False, True,
                                              torch.bfloat16, self.G.MX_BLOCKWISE.value, None, 0, False, self.offs)
+
+    def _backward_operands(self):
+        from primus_turbo.pytorch.core.low_precision import ScalingRecipe, float4_e2m1fn_x2 as f4
+
+        qi = self.qi
+        plain, rht = ScalingRecipe(), ScalingRecipe(use_rht=True)
+        _, _, a_col, a_col_s, _, _, _, _ = qi.grouped_quantize_mxfp4_impl(self.x.detach(), f4, None, 32, self.gl, self.offs,
+                                                                          with_trans=True, scaling_recipe=plain,
+                                                                          scaling_recipe_for_trans=rht)
+        g_row, g_row_s, g_col, g_col_s, _, _, lens_col, offs_col = qi.grouped_quantize_mxfp4_impl(
+            self.dy, f4, None, 32, self.gl, self.offs, with_trans=True, scaling_recipe=plain, scaling_recipe_for_trans=rht)
+        r2 = ScalingRecipe(use_2d_block=True)
+        _, _, b_col, b_col_s = qi.quantize_mxfp4_impl(self.w.detach(), f4, None, 32, with_trans=True, scaling_recipe=r2,
+                                                      scaling_recipe_for_trans=r2)
+        return g_row, g_row_s, g_col, g_col_s, a_col, a_col_s, b_col, b_col_s, self.offs, lens_col, offs_col
+
+    def _impls(self):
+        return self.gg.grouped_gemm_fp4_impl, self.gg.grouped_gemm_fp4_variable_k_impl
 
 
 def _keyed(key, make):
