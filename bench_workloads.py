@@ -115,6 +115,7 @@ class GemmFp8Rowwise(_GemmBase):
         aq, asi = Q.fp8_rowwise(a, -1, "e4m3")
         bq, bsi = Q.fp8_rowwise(b, -1, "e4m3")
         same = np.array_equal(self.aq.cpu().view(torch.uint8).numpy()[rows], aq)
+        same = same and np.array_equal(np.ascontiguousarray(self.as_inv.cpu().numpy()[rows]).view(np.int32), np.ascontiguousarray(asi).view(np.int32))
         same = same and np.array_equal(self.bq.cpu().view(torch.uint8).numpy(), bq)
         ref = OG.gemm_dequantized(Q.fp8_dequant(aq, asi, "e4m3"), Q.fp8_dequant(bq, bsi, "e4m3"), trans_b=True)
         # the product is rounded to bf16: compare against the bf16-rounded oracle
@@ -122,7 +123,7 @@ class GemmFp8Rowwise(_GemmBase):
         rel = OG.max_rel_err(ref_t, out[rows])
         cos = OG.cosine(out[rows], ref_t)
         ok = bool(same and rel <= 1e-2 and cos >= 0.9999)
-        return ok, f"quantized bytes bit-exact; 128 output rows vs oracle: max|err|/max|ref| (relative to the output range, not element-wise)={rel:.2e}, cosine={cos:.6f}"
+        return ok, f"quantized bytes and activation scales bit-exact; 128 output rows vs oracle: max|err|/max|ref| (relative to the output range, not element-wise)={rel:.2e}, cosine={cos:.6f}"
 
     def cpu_baseline(self):
         """The reference's CPU formulas on an M-slice: rowwise quantize of the slice and of all of
@@ -163,7 +164,7 @@ class GemmFp8Blockwise(_GemmBase):
         from primus_turbo.pytorch.kernels.gemm.gemm_fp8_impl import gemm_fp8_impl
         from primus_turbo.pytorch.kernels.quantization.quantization_impl import (
             quant_fp8_blockwise_for_weight_impl,
-            quant_fp8_blockwise_impl,
+            quant_fp8_blockwise_kmajor_impl,
         )
 
         self.turbo, self.G = turbo, ScalingGranularity
@@ -174,7 +175,9 @@ class GemmFp8Blockwise(_GemmBase):
         self.b_cpu = _randn_bf16((N, K), 4, 1.0)
         self.a, self.b = self.a_cpu.to(dev), self.b_cpu.to(dev)
         self._impl = gemm_fp8_impl
-        self.aq, self.as_inv = quant_fp8_blockwise_impl(self.a, turbo.float8_e4m3, -1, 128)
+        # the operands as the op's forward hands them to the kernel: row scales of A block-major
+        self.aq, as_kmajor, _, _ = quant_fp8_blockwise_kmajor_impl(self.a, turbo.float8_e4m3, 128, False)
+        self.as_inv = as_kmajor.t()
         self.bq, self.bs_inv = quant_fp8_blockwise_for_weight_impl(self.b, turbo.float8_e4m3, 128)
 
     def step(self):

@@ -179,6 +179,17 @@ PT_API int pt_quantize_fp8_blockwise_t(const void *x, int x_dtype, int64_t M, in
                                        void *q_row, float *scale_inv_row, void *q_col,
                                        void *q_col_t, int64_t ldt, float *scale_inv_col,
                                        void *stream);
+/* The row direction of the above with its scales stored block-major, scale_inv_row_kmajor
+ * [N / 128, M] (the value of row m and block kb at kb * M + m): the layout the block-scaled GEMM
+ * reads per K slab, so that no transposition of the scale array precedes the product, and the one
+ * in which the 128 scale values a workgroup produces per tile are contiguous (whole cache lines
+ * instead of 128 masked 4-byte writes). q_col_t / ldt / scale_inv_col as for
+ * pt_quantize_fp8_blockwise_t, or NULL / 0 / NULL for the row direction alone. Codes and scale
+ * values are those of pt_quantize_fp8_blockwise; the reference has the [M, N / 128] layout only
+ * (quantization_impl.py quant_fp8_blockwise_impl). */
+PT_API int pt_quantize_fp8_blockwise_kmajor(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype,
+                                            void *q_row, float *scale_inv_row_kmajor, void *q_col_t,
+                                            int64_t ldt, float *scale_inv_col, void *stream);
 
 /* Replaces torch.ops.primus_turbo_cpp_extension.quantize_fp8_blockwise_for_weight
  * (bindings_pytorch.cpp:52-93, csrc/pytorch/quantization/quantization.cpp:1443-1480,

@@ -525,7 +525,7 @@ extern "C" {
 
 static int quantize_blocks(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype, void *q_row,
                            float *scale_inv_row, void *q_col, void *q_col_t, int64_t ldt, float *scale_inv_col,
-                           void *stream) {
+                           void *stream, bool row_scales_kmajor = false) {
     PT_REQUIRE(is_hp_dtype(x_dtype), "input must be bf16, fp16 or fp32");
     PT_REQUIRE(is_fp8_dtype(q_dtype), "output must be e4m3 or e5m2");
     PT_REQUIRE(M >= 0 && N >= 0, "dimensions must be non-negative");
@@ -551,8 +551,8 @@ static int quantize_blocks(const void *x, int x_dtype, int64_t M, int64_t N, int
     a.ldt = ldt;
     a.M = M;
     a.N = N;
-    a.rs_m = tn;
-    a.rs_n = 1;
+    a.rs_m = row_scales_kmajor ? 1 : tn; // [M, N / 128], or block-major [N / 128, M]
+    a.rs_n = row_scales_kmajor ? M : 1;
     a.qmax = fp8_max_of(q_dtype);
     auto       st  = static_cast<hipStream_t>(stream);
     const bool vec = vec_ok(a, 1);
@@ -579,6 +579,14 @@ int pt_quantize_fp8_blockwise_t(const void *x, int x_dtype, int64_t M, int64_t N
                                 void *stream) {
     PT_REQUIRE(q_col_t != nullptr || M * N == 0, "q_col_t must not be NULL");
     return quantize_blocks(x, x_dtype, M, N, q_dtype, q_row, scale_inv_row, q_col, q_col_t, ldt, scale_inv_col, stream);
+}
+
+int pt_quantize_fp8_blockwise_kmajor(const void *x, int x_dtype, int64_t M, int64_t N, int q_dtype, void *q_row,
+                                     float *scale_inv_row_kmajor, void *q_col_t, int64_t ldt, float *scale_inv_col,
+                                     void *stream) {
+    PT_REQUIRE(q_row != nullptr || M * N == 0, "q_row must not be NULL");
+    return quantize_blocks(x, x_dtype, M, N, q_dtype, q_row, scale_inv_row_kmajor, nullptr, q_col_t, ldt, scale_inv_col, stream,
+                           true);
 }
 
 static int quantize_weight_tiles(const void *w, int w_dtype, int64_t B, int64_t M, int64_t N, void *q, void *q_t,

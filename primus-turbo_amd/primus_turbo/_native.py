@@ -84,6 +84,10 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_int, c_i64, c_i64, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_i64, c_void_p, c_void_p],
     ),
+    "pt_quantize_fp8_blockwise_kmajor": (
+        c_int,
+        [c_void_p, c_int, c_i64, c_i64, c_int, c_void_p, c_void_p, c_void_p, c_i64, c_void_p, c_void_p],
+    ),
     "pt_quantize_fp8_blockwise_weight": (
         c_int,
         [c_void_p, c_int, c_i64, c_i64, c_i64, c_void_p, c_int, c_void_p, c_void_p],

@@ -114,11 +114,21 @@ def _launch(a, a_scale_inv, trans_a, b, b_scale_inv, trans_b, out, trans_c, gran
     _check(out.dtype in _OUT, "out_dtype must be bfloat16, float16 or float32")
     _check(a_scale_inv.dtype == torch.float32 and b_scale_inv.dtype == torch.float32, "scales must be float32")
     a, b = a.contiguous(), b.contiguous()
-    a_scale_inv, b_scale_inv = a_scale_inv.contiguous(), b_scale_inv.contiguous()
+    # per-row block scales of A may arrive as the [M, K/128] view of a block-major [K/128, M] tensor
+    # (quant_fp8_blockwise_kmajor_impl(...)[1].t()): the kernel reads that layout in place
+    a_kmajor = (granularity == ScalingGranularity.BLOCKWISE and not trans_a and a_scale_inv.dim() == 2
+                and a_scale_inv.shape[1] > 1 and a_scale_inv.stride() == (1, a_scale_inv.shape[0]))
+    if not a_kmajor:
+        a_scale_inv = a_scale_inv.contiguous()
+    b_scale_inv = b_scale_inv.contiguous()
     M, Nn, K = get_gemm_logical_shape(a, b, trans_a, trans_b)
     mode, sa_m, sa_k, sb_n, sb_k, sa_blk, sb_blk = _scale_desc(
         granularity, a_scale_inv, b_scale_inv, trans_a, trans_b, M, Nn, K
     )
+    if a_kmajor and (sa_m, sa_k, sa_blk) == ((K + 127) // 128, 1, 1):
+        sa_m, sa_k = 1, M
+    elif a_kmajor:
+        a_scale_inv = a_scale_inv.contiguous()
     if trans_c:
         # C^T = op(B)^T . op(A)^T: swap the operand roles, the kernel always writes row-major [M', N']
         a, b = b, a

@@ -382,6 +382,50 @@ def _quant_fp8_blockwise_dual_t_impl_fake(x, dtype, block_size=128):
     )
 
 
+@torch.library.custom_op("primus_turbo::quant_fp8_blockwise_kmajor_impl", mutates_args=())
+def quant_fp8_blockwise_kmajor_impl(
+    x: torch.Tensor, dtype: torch.dtype, block_size: int, with_col_t: bool
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """The row direction of :func:`quant_fp8_blockwise_impl` with its scales stored block-major,
+    ``scales_row_kmajor [N/b, M]`` (``.t()`` of it is the reference's ``[M, N/b]`` tensor, value for
+    value): the layout the block-scaled GEMM reads, so no transposition pass precedes the product,
+    and the quantizer writes whole cache lines of scales. ``with_col_t`` adds the transposed column
+    codes and their scales as :func:`quant_fp8_blockwise_dual_t_impl` (empty tensors otherwise).
+    ``(x_fp8_row, scales_row_kmajor, x_fp8_col_t, scales_col)``. (No counterpart in the reference.)"""
+    N.require_cuda(x)
+    _check(x.dtype in _HP_DTYPES, "input must be bfloat16, float16 or float32")
+    _check_fp8_out(dtype)
+    _check(x.dim() == 2 and x.is_contiguous(), "Input must be 2D and contiguous")
+    _need_block_128(block_size)
+    M, Nn = x.shape
+    Mp = ceil_div(M, block_size) * block_size
+    dev = x.device
+    q_row = torch.empty((M, Nn), dtype=dtype, device=dev)
+    s_row = torch.empty((ceil_div(Nn, block_size), M), dtype=torch.float32, device=dev)
+    q_col_t = torch.empty((Nn, Mp) if with_col_t else (0,), dtype=dtype, device=dev)
+    s_col = torch.empty((ceil_div(M, block_size), Nn) if with_col_t else (0,), dtype=torch.float32, device=dev)
+    N.check(
+        N.lib().pt_quantize_fp8_blockwise_kmajor(
+            N.ptr(x), N.dtype_code(x.dtype), M, Nn, N.dtype_code(dtype), N.ptr(q_row), N.ptr(s_row),
+            N.ptr(q_col_t) if with_col_t else None, Mp if with_col_t else 0, N.ptr(s_col) if with_col_t else None,
+            N.stream_of(x),
+        )
+    )
+    return q_row, s_row, q_col_t, s_col
+
+
+@quant_fp8_blockwise_kmajor_impl.register_fake
+def _quant_fp8_blockwise_kmajor_impl_fake(x, dtype, block_size, with_col_t):
+    M, Nn = x.shape
+    dev = x.device
+    return (
+        torch.empty((M, Nn), dtype=dtype, device=dev),
+        torch.empty((ceil_div(Nn, block_size), M), dtype=torch.float32, device=dev),
+        torch.empty((Nn, ceil_div(M, block_size) * block_size) if with_col_t else (0,), dtype=dtype, device=dev),
+        torch.empty((ceil_div(M, block_size), Nn) if with_col_t else (0,), dtype=torch.float32, device=dev),
+    )
+
+
 # quantize_fp8_blockwise_for_weight(Tensor input, ScalarType dest_dtype, int block_size) -> Tensor[]
 _ext.define("quantize_fp8_blockwise_for_weight(Tensor input, ScalarType dest_dtype, int block_size) -> Tensor[]")
 

@@ -36,6 +36,7 @@ from primus_turbo.pytorch.core.quantized_tensor import (
 from primus_turbo.pytorch.kernels.gemm.gemm_fp8_impl import gemm_fp8_accum_impl, gemm_fp8_impl
 from primus_turbo.pytorch.kernels.quantization.quantization_impl import (
     quant_fp8_blockwise_dual_t_impl,
+    quant_fp8_blockwise_kmajor_impl,
     quant_fp8_blockwise_for_weight_dual_impl,
 )
 from primus_turbo.pytorch.ops.quantization import dequantize_fp8, quantize_fp8, quantize_fp8_with_trans
@@ -174,11 +175,13 @@ class FP8GemmBlockFunction(torch.autograd.Function):
                 if a_t is None:
                     a_t = QuantizedTensor.quantize(a.dequantize(), fdt, gran, axis=-2, block_size=bs)
                 a_col, a_col_s = a_t.qdata, a_t.scale_inv
-        elif need_bwd:
-            a_row, a_row_s, a_col, a_col_s = quant_fp8_blockwise_dual_t_impl(a.contiguous(), fdt, bs)
-            a_kmajor = True
+        elif a.dim() == 2:
+            # row scales block-major, as the GEMM reads them; the column-direction copy of `a` only
+            # feeds wgrad: skipped when nothing asks for a gradient
+            a_row, a_row_s_km, a_col, a_col_s = quant_fp8_blockwise_kmajor_impl(a.contiguous(), fdt, bs, need_bwd)
+            a_row_s = a_row_s_km.t()
+            a_kmajor = need_bwd
         else:
-            # the column-direction copy of `a` only feeds wgrad: skip it when nothing asks for a gradient
             a_row, a_row_s = quantize_fp8(a, fdt, gran, axis=-1, block_size=bs)
         w_recipe = ScalingRecipe(use_2d_block=True)  # weight tiles serve forward and backward unchanged
         b_q_t = None
@@ -210,7 +213,8 @@ class FP8GemmBlockFunction(torch.autograd.Function):
         gdt = _get_fp8_dtype(config.format, False)
         g = grad_out.contiguous()
         if a_kmajor:
-            g_row, g_row_s, g_col_t, g_col_s = quant_fp8_blockwise_dual_t_impl(g, gdt, config.block_size)
+            g_row, g_row_s_km, g_col_t, g_col_s = quant_fp8_blockwise_kmajor_impl(g, gdt, config.block_size, True)
+            g_row_s = g_row_s_km.t()
         else:
             g_row, g_row_s, g_col, g_col_s = quantize_fp8_with_trans(g, gdt, gran, block_size=config.block_size)
         grad_a = _gemm(g_row, g_row_s, False, b_q, b_s, True if b_ready else not trans_b, out_dtype, False, gran)

@@ -188,3 +188,39 @@ def test_blockwise_dual_transposed_column_output(shape, dtype):
     assert qct.shape == (N, Mp)
     assert torch.equal(qct.view(torch.uint8)[:, :M], qc.view(torch.uint8).t().contiguous())
     assert not bool(qct.view(torch.uint8)[:, M:].any())
+
+
+@pytest.mark.parametrize("shape", [(256, 384), (130, 257), (1000, 512), (16384, 2048), (77, 96), (1, 1)])
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+@pytest.mark.parametrize("with_col_t", [False, True])
+def test_blockwise_row_scales_block_major(shape, dtype, with_col_t):
+    """The quantizer that stores its row scales block-major ([N/128, M], the layout the block-scaled
+    GEMM reads): codes and scale values bit for bit those of the oracle, the optional transposed
+    column output that of the dual quantizer; and the GEMM gives identical bits whether it gets the
+    [M, N/128] view of these scales or a contiguous copy of it."""
+    from primus_turbo.pytorch.kernels.gemm import gemm_fp8_impl as gi
+    from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+    M, N = shape
+    x = bf16_randn(shape, seed=27, outlier_frac=0.001)
+    xf, f = to_f32_np(x), FMT[dtype]
+    q, s_km, q_t, s_col = qi.quant_fp8_blockwise_kmajor_impl(x.cuda(), dtype, 128, with_col_t)
+    torch.cuda.synchronize()
+    oq, os_ = Q.fp8_blockwise(xf, 1, f)
+    assert np.array_equal(codes_np(q), oq)
+    assert s_km.is_contiguous() and tuple(s_km.shape) == (os_.shape[1], M)
+    _eq_scales(s_km.t().contiguous(), os_)
+    if with_col_t:
+        oqc, osc = Q.fp8_blockwise(xf, 0, f)
+        assert np.array_equal(codes_np(q_t)[:, :M], oqc.T) and not codes_np(q_t)[:, M:].any()
+        _eq_scales(s_col, osc)
+    else:
+        assert q_t.numel() == 0 and s_col.numel() == 0
+    if N >= 256 and M >= 77:
+        w = bf16_randn((192, N), seed=28).cuda()
+        wq, ws = qi.quant_fp8_blockwise_for_weight_impl(w, torch.float8_e4m3fn, 128)
+        a = gi.gemm_fp8_impl(q, s_km.t(), False, wq, ws, True, torch.bfloat16, False, G.BLOCKWISE.value, 0)
+        b = gi.gemm_fp8_impl(q, s_km.t().contiguous(), False, wq, ws, True, torch.bfloat16, False, G.BLOCKWISE.value, 0)
+        c = gi.gemm_fp8_impl(q, s_km.t(), False, wq, ws, True, torch.bfloat16, True, G.BLOCKWISE.value, 0)
+        torch.cuda.synchronize()
+        assert torch.equal(a, b) and torch.equal(c, a.t().contiguous())
