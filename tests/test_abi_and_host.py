@@ -64,6 +64,14 @@ def test_argument_validation_without_gpu(native_lib):
     assert lib.pt_quantize_fp8_rowwise(None, 0, 1, 1, 1, None, 7, None, None, None) == -1
     assert lib.pt_quantize_fp8_blockwise(None, 0, 8, 8, 3, None, None, None, None, None) == -1
     assert b"at least one" in lib.pt_last_error()
+    assert lib.pt_quantize_fp8_blockwise_kmajor(1024, 0, 8, 8, 3, None, None, None, 0, None, None) == -1
+    assert b"q_row" in lib.pt_last_error()
+    # the gated grouped MX quantizer: act out of range, no row output, a Hadamard-transformed row direction
+    assert lib.pt_glu_grouped_quantize_mx(1024, 0, 1024, None, 7, 8, 64, 3, 1024, None, 1024, 1, 1024, 1024, None, None, 0, 128, None) == -1
+    assert b"act" in lib.pt_last_error()
+    assert lib.pt_glu_grouped_quantize_mx(1024, 0, 1024, None, 0, 8, 64, 3, 1024, None, 1024, 1, None, None, 1024, 1024, 0, 128, None) == -1
+    assert b"row direction" in lib.pt_last_error()
+    assert lib.pt_glu_grouped_quantize_mx(1024, 0, 1024, None, 0, 8, 64, 3, 1024, None, 1024, 1, 1024, 1024, 1024, 1024, 4, 128, None) == -1
     assert lib.pt_dequantize_fp8_block(None, 3, 1, 8, 8, None, 0, 128, None, 0, None) == -1
     assert lib.pt_compute_group_offs(None, -1, 1, None, None, None) == -1
     assert lib.pt_quantize_fp8_tensorwise_workspace_bytes() >= 64
