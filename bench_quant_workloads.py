@@ -337,7 +337,8 @@ class QuantMx(_QuantBase):
         kind = "mxfp4_e2m1" if fp4 else "mxfp8_e4m3"
         self.fmt = "e2m1" if fp4 else "e4m3"
         self.name = f"{kind}_{'row+col_dual' if dual else 'row'}_quant_{M}x{N}_bf16" + ("" if dual else " (+ dequantize)")
-        self.dominant_name = "mx_quant_kernel (128x128 tile through LDS, E8M0 exponent from the amax bits)"
+        self.dominant_name = ("mx_quant_kernel (128x128 tile through LDS, E8M0 exponent from the amax bits)" if dual else
+                              "mx_quant_rows_kernel (stream without LDS: 8 elements per lane, block amax over four lanes)")
         self.qdt = torch.float4_e2m1fn_x2 if fp4 else torch.float8_e4m3fn
         self._q = qi.quantize_mxfp4_impl if fp4 else qi.quantize_mxfp8_impl
         self._dq = qi.dequantize_mxfp4_impl if fp4 else qi.dequantize_mxfp8_impl

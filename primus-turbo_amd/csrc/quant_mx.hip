@@ -105,6 +105,11 @@ __device__ __forceinline__ void mx_encode32_fp4_sr(const float (&v)[32], float i
     }
 }
 
+// A build for timing studies may define this to record a time stamp per workgroup and phase
+#ifndef PT_MX_TRACE
+#define PT_MX_TRACE(id)
+#endif
+
 constexpr int MX_TILE  = 128;
 constexpr int MX_PITCH = MX_TILE + 8; // 16-bit elements per LDS row (272 B: 16-byte aligned rows)
 
@@ -199,6 +204,7 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
         row_cnt  = (a.row_offs_pad != nullptr ? a.row_offs_pad[g + 1] - a.row_offs_pad[g] : in_end - a.group_offs[g]) - done;
     }
 
+    PT_MX_TRACE(0);
     // ---- tile -> LDS (zeros outside the matrix) ----
     const bool vec = (a.N & 7) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
 #pragma unroll
@@ -250,7 +256,9 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
         }
         *reinterpret_cast<u32x4 *>(&tile[r * MX_PITCH + c]) = v;
     }
+    PT_MX_TRACE(1);
     __syncthreads();
+    PT_MX_TRACE(2);
 
     auto elem = [&](uint16_t raw) -> float {
         T t;
@@ -334,6 +342,7 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
                 *reinterpret_cast<const uint32_t *>(&sbytes[tid * 4]);
     }
 
+    PT_MX_TRACE(3);
     // ---- column direction: task = (column n, 32-row block rb); output transposed ----
     // The codes go back through the LDS (over the input tile, once everybody has read it) so that
     // they leave as whole 128-byte (FP4: 64-byte) rows of the transposed output.
@@ -386,7 +395,9 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
             }
             sbytes[c * 4 + rb] = static_cast<uint8_t>(e + 127);
         }
+        PT_MX_TRACE(4);
         __syncthreads(); // everybody is done with the input tile
+        PT_MX_TRACE(5);
         uint8_t *stage = reinterpret_cast<uint8_t *>(tile);
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
@@ -397,6 +408,7 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
                 *reinterpret_cast<u32x4 *>(d + 16) = u32x4{code[p][4], code[p][5], code[p][6], code[p][7]};
         }
         __syncthreads();
+        PT_MX_TRACE(6);
         constexpr int CHUNKS = CROW / 16; // 16-byte chunks per output row
 #pragma unroll
         for (int p = 0; p < MX_TILE * CHUNKS / 256; ++p) {
@@ -412,6 +424,124 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
             *reinterpret_cast<uint32_t *>(a.col_s + (b * a.N + n0 + tid) * (a.Mpad >> 5) + (m0 >> 5)) =
                 *reinterpret_cast<const uint32_t *>(&sbytes[tid * 4]);
     }
+    PT_MX_TRACE(7);
+}
+
+// Row direction only, 1-D blocks, nearest or stochastic rounding, rows of whole 16-byte pieces: a
+// plain stream without LDS, same bytes as the tile kernel. The padded rows are cut into runs of
+// 512 columns; a wavefront takes four consecutive runs, a lane 8 consecutive elements of each (a
+// quarter of a block: the block's abs-max is a reduction over four neighbouring lanes). The 64
+// scale bytes of a wavefront leave as 16 words.
+template <typename T, int FMT>
+__global__ __launch_bounds__(256) void mx_quant_rows_kernel(const MxArgs a, const int64_t rows, const int64_t runs_per_row) {
+    const int     lane  = threadIdx.x & 63;
+    const int64_t total = rows * runs_per_row;
+    const int64_t u0    = (static_cast<int64_t>(blockIdx.x) * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6)) * 4;
+    if (u0 >= total)
+        return;
+    const uint16_t *x = static_cast<const uint16_t *>(a.x);
+    int64_t         row[4], run[4];
+    row[0] = u0 / runs_per_row;
+    run[0] = u0 - row[0] * runs_per_row;
+#pragma unroll
+    for (int k = 1; k < 4; ++k) {
+        const bool wrap = run[k - 1] + 1 == runs_per_row;
+        row[k]          = wrap ? row[k - 1] + 1 : row[k - 1];
+        run[k]          = wrap ? 0 : run[k - 1] + 1;
+    }
+    u32x4 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int64_t n = run[k] * 512 + lane * 8;
+        v[k]            = (u0 + k < total && n < a.N) ? ld128(x + row[k] * a.N + n) : u32x4{0u, 0u, 0u, 0u};
+    }
+    uint32_t ebytes = 0; // byte k: the scale byte of this lane's block in run k
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const uint32_t ww[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+        float          f[8];
+        float          am = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            unpack2<T>(ww[i], f[2 * i], f[2 * i + 1]);
+            am = fmaxf(am, fmaxf(abs_or_zero(f[2 * i]), abs_or_zero(f[2 * i + 1])));
+        }
+        am = fmaxf(am, dpp_f32<0xB1>(am)); // quad_perm [1,0,3,2]
+        am = fmaxf(am, dpp_f32<0x4E>(am)); // quad_perm [2,3,0,1]
+        const int   e   = mx_exponent<FMT>(am);
+        const float inv = mx_inv_scale(e);
+        ebytes |= static_cast<uint32_t>(e + 127) << (8 * k);
+        constexpr float Q = MxFmt<FMT>::QMAX;
+        const int64_t   n = run[k] * 512 + lane * 8;
+        const bool      in = u0 + k < total && n < a.Npad;
+        if constexpr (FMT == MX_E2M1) {
+            uint32_t w = 0;
+            if (a.sr_mask & 1) {
+                // the seeds of the tile kernel: tile (batch, row tile, column tile), task 4 r + c
+                // of the tile, then one step per pair of the block
+                const int64_t  m  = row[k] % a.M, bt = row[k] / a.M, nb = n >> 5;
+                const uint32_t id = static_cast<uint32_t>((bt * (a.Mpad >> 7) + (m >> 7)) * (a.Npad >> 7) + (nb >> 2));
+                const uint32_t t  = static_cast<uint32_t>((m & 127) * 4 + (nb & 3));
+                uint32_t seed = sr_hash(a.sr_seed ^ (id * 512u + t)) + 4u * (lane & 3) * 0x9E3779B9u;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const f32x2_t pair = {scale_clamp(f[2 * i], inv, Q), scale_clamp(f[2 * i + 1], inv, Q)};
+                    seed += 0x9E3779B9u;
+                    w |= (__builtin_amdgcn_cvt_scalef32_sr_pk_fp4_f32(0u, pair, seed, 1.0f, 0) & 0xffu) << (8 * i);
+                }
+            } else {
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp(f[0], inv, Q), scale_clamp(f[1], inv, Q), 1.0f, 0);
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp(f[2], inv, Q), scale_clamp(f[3], inv, Q), 1.0f, 1);
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp(f[4], inv, Q), scale_clamp(f[5], inv, Q), 1.0f, 2);
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp(f[6], inv, Q), scale_clamp(f[7], inv, Q), 1.0f, 3);
+            }
+            if (in)
+                *reinterpret_cast<uint32_t *>(a.row_q + row[k] * (a.Npad >> 1) + (n >> 1)) = w;
+        } else {
+            const uint32_t c0 = cvt4_fp8<FMT == MX_E5M2>(scale_clamp(f[0], inv, Q), scale_clamp(f[1], inv, Q),
+                                                         scale_clamp(f[2], inv, Q), scale_clamp(f[3], inv, Q));
+            const uint32_t c1 = cvt4_fp8<FMT == MX_E5M2>(scale_clamp(f[4], inv, Q), scale_clamp(f[5], inv, Q),
+                                                         scale_clamp(f[6], inv, Q), scale_clamp(f[7], inv, Q));
+            if (in)
+                *reinterpret_cast<u32x2 *>(a.row_q + row[k] * a.Npad + n) = u32x2{c0, c1};
+        }
+    }
+    // lane L < 16 writes scale word L & 3 of run L >> 2: the bytes of the blocks 4 (L & 3) .. + 3 of
+    // that run, which the lanes 16 (L & 3) + 4 j hold
+    uint32_t word = 0;
+    const int k_of = (lane >> 2) & 3, j0 = lane & 3;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t wj = static_cast<uint32_t>(__shfl(static_cast<int>(ebytes), 16 * j0 + 4 * j, 64));
+        word |= ((wj >> (8 * k_of)) & 0xffu) << (8 * j);
+    }
+    if (lane < 16) {
+        int64_t r = row[0], c = run[0];
+#pragma unroll
+        for (int k = 1; k < 4; ++k)
+            if (k_of == k)
+                r = row[k], c = run[k];
+        const int64_t sb = c * 16 + j0 * 4; // scale byte index in the padded row
+        if (u0 + k_of < total && sb < (a.Npad >> 5))
+            *reinterpret_cast<uint32_t *>(a.row_s + r * (a.Npad >> 5) + sb) = word;
+    }
+}
+
+// The streaming row kernel serves an ungrouped launch when only the row direction is asked for,
+// with 1-D blocks and no transform, and the rows are whole 16-byte pieces.
+static bool mx_rows_stream_ok(const MxArgs &a, bool row2d, bool rht) {
+    return a.col_q == nullptr && a.row_q != nullptr && !row2d && !rht && (a.N & 7) == 0 &&
+           (reinterpret_cast<uintptr_t>(a.x) & 15) == 0 && a.group_offs == nullptr;
+}
+template <typename T> static void launch_mx_rows(const MxArgs &a, int fmt, hipStream_t st) {
+    const int64_t rows = a.B * a.M, runs = cdiv(a.Npad, 512);
+    const dim3    grid(static_cast<unsigned>(cdiv(rows * runs, 16)));
+    if (fmt == MX_E4M3)
+        mx_quant_rows_kernel<T, MX_E4M3><<<grid, 256, 0, st>>>(a, rows, runs);
+    else if (fmt == MX_E5M2)
+        mx_quant_rows_kernel<T, MX_E5M2><<<grid, 256, 0, st>>>(a, rows, runs);
+    else
+        mx_quant_rows_kernel<T, MX_E2M1><<<grid, 256, 0, st>>>(a, rows, runs);
 }
 
 template <typename T, int FMT, bool ROW, bool COL>
@@ -677,6 +807,14 @@ int pt_quantize_mx(const void *x, int x_dtype, int64_t B, int64_t M, int64_t N, 
     PT_REQUIRE(a.Mpad / 128 < 65536 && B < 65536, "grid dimension out of range");
     dim3 grid(static_cast<unsigned>(a.Npad / 128), static_cast<unsigned>(a.Mpad / 128), static_cast<unsigned>(B));
     auto st = static_cast<hipStream_t>(stream);
+    if (mx_rows_stream_ok(a, (row_flags & 1) != 0, rht)) {
+        PT_REQUIRE(cdiv(B * M * cdiv(a.Npad, 512), 16) < (1LL << 31), "too many rows");
+        if (x_dtype == PT_DTYPE_BF16)
+            launch_mx_rows<bf16_t>(a, fmt, st);
+        else
+            launch_mx_rows<f16_t>(a, fmt, st);
+        return check_launch("mx_quant_rows_kernel");
+    }
     if (rht) {
         if (x_dtype == PT_DTYPE_BF16)
             launch_mx_rht<bf16_t>(a, (row_flags & 2) != 0, (col_flags & 2) != 0, grid, st);

@@ -74,6 +74,53 @@ def test_mx_single_direction_and_mixed_recipes(fmt, dt, axis):
 
 
 @pytest.mark.parametrize("fmt,dt", FMTS)
+@pytest.mark.parametrize("shape,dtype", [((128, 128), torch.bfloat16), ((200, 96), torch.bfloat16),
+                                         ((33, 32), torch.float16), ((1000, 2080), torch.bfloat16),
+                                         ((7, 4096), torch.bfloat16), ((3, 160, 192), torch.float16),
+                                         ((2, 50, 544), torch.bfloat16)])
+def test_mx_row_direction_alone(fmt, dt, shape, dtype):
+    """Rows only with 1-D blocks (the streaming kernel): codes, the zero codes of the pad columns
+    and the scale bytes bit-exact against the oracle, batches and rows shorter than a
+    wavefront's share included."""
+    x = bf16_randn(shape, seed=58, outlier_frac=0.002, dtype=dtype)
+    q, s = _fn(fmt)(x.cuda(), dt, x.ndim - 1, 32)
+    torch.cuda.synchronize()
+    xs = x if x.ndim == 3 else x[None]
+    qs, ss = (q, s) if x.ndim == 3 else (q[None], s[None])
+    for b in range(xs.shape[0]):
+        oq, os_ = Q.mx_quant_rowwise(to_f32_np(xs[b]), fmt)
+        assert codes_np(qs[b]).shape == oq.shape and codes_np(ss[b]).shape == os_.shape
+        assert np.array_equal(codes_np(ss[b]), os_), "row scale bytes"
+        assert np.array_equal(codes_np(qs[b]), oq), "row codes"
+
+
+@pytest.mark.skipif(FP4 is None, reason="torch has no float4_e2m1fn_x2")
+@pytest.mark.parametrize("shape", [(256, 128), (3, 200, 608)])
+def test_mxfp4_stochastic_rounding_same_noise_alone_and_dual(shape):
+    """With one seed the row direction draws the same rounding noise whether it is quantized
+    alone (streaming kernel) or together with the column direction (tile kernel)."""
+    from primus_turbo import _native as N
+
+    x = bf16_randn(shape, seed=59).cuda()
+    B = shape[0] if len(shape) == 3 else 1
+    M, Nn = shape[-2:]
+    Mp, Np = -(-M // 128) * 128, -(-Nn // 128) * 128
+    outs = []
+    for dual in (False, True):
+        rq = torch.zeros((B, M, Np // 2), dtype=torch.uint8, device="cuda")
+        rs = torch.zeros((B, M, Np // 32), dtype=torch.uint8, device="cuda")
+        cq = torch.zeros((B, Nn, Mp // 2), dtype=torch.uint8, device="cuda") if dual else None
+        cs = torch.zeros((B, Nn, Mp // 32), dtype=torch.uint8, device="cuda") if dual else None
+        N.check(N.lib().pt_quantize_mx(N.ptr(x), N.dtype_code(x.dtype), B, M, Nn, N.dtype_code(FP4), N.ptr(rq), N.ptr(rs), 4,
+                                       N.ptr(cq), N.ptr(cs), 0, 0x1234ABCD, N.stream_of(x)))
+        torch.cuda.synchronize()
+        outs.append((rq, rs))
+    assert torch.equal(outs[0][1], outs[1][1]) and torch.equal(outs[0][0], outs[1][0])
+    q0, _ = qi.quantize_mxfp4_impl(x, FP4, x.ndim - 1, 32)
+    assert not torch.equal(outs[0][0], q0.view(torch.uint8).reshape(outs[0][0].shape)), "the noise is there"
+
+
+@pytest.mark.parametrize("fmt,dt", FMTS)
 def test_mx_batched_and_fp16(fmt, dt):
     x = bf16_randn((3, 160, 192), seed=52, dtype=torch.float16)
     rq, rs, cq, cs = _fn(fmt)(x.cuda(), dt, None, 32, with_trans=True)
@@ -109,6 +156,8 @@ def test_mx_special_values(fmt, dt):
     oq, os_ = Q.mx_quant_colwise(xf, fmt)
     assert np.array_equal(codes_np(cs), os_) and np.array_equal(codes_np(cq), oq)
     assert codes_np(rs)[8:, :].max() == 0  # untouched rows: all-zero blocks
+    q1, s1 = _fn(fmt)(xb.cuda(), dt, 1, 32)  # the row direction alone: same bytes
+    assert torch.equal(q1.view(torch.uint8), rq.view(torch.uint8)) and torch.equal(s1.view(torch.uint8), rs.view(torch.uint8))
 
 
 @pytest.mark.parametrize("fmt,dt", FMTS)
