@@ -208,45 +208,81 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
     const int64_t gn   = tn * BQ + cseg * BQ_PACK;
     const bool    full = VEC8 && (gn + BQ_PACK <= N);
 
-    // phase 1: the whole tile share of this thread is requested before anything is used
+    // phase 1: the whole tile share of this thread is requested before anything is used. With
+    // whole 16-byte pieces no branch may separate the loads (the compiler would wait for each one
+    // in turn): a piece outside the matrix reads the matrix's first bytes and is zeroed afterwards.
     Held8<T> held[BQ_ROUNDS];
     if constexpr (GLU == 0) {
+        if constexpr (VEC8) {
+            bool ok[BQ_ROUNDS];
 #pragma unroll
-        for (int r = 0; r < BQ_ROUNDS; ++r) {
-            const int64_t in_m  = in_m0 + tile_row_of(rslot, r);
-            const bool    valid = in_m < in_end;
-            if (valid && full)
-                held[r].load(x + in_m * N + gn);
-            else
+            for (int r = 0; r < BQ_ROUNDS; ++r) {
+                const int64_t in_m = in_m0 + tile_row_of(rslot, r);
+                ok[r]              = in_m < in_end && gn < N;
+                held[r].load(x + (ok[r] ? in_m * N + gn : 0));
+            }
+#pragma unroll
+            for (int r = 0; r < BQ_ROUNDS; ++r)
+#pragma unroll
+                for (int i = 0; i < Held8<T>::WORDS; ++i)
+                    held[r].w[i] = ok[r] ? held[r].w[i] : 0u;
+        } else {
+#pragma unroll
+            for (int r = 0; r < BQ_ROUNDS; ++r) {
+                const int64_t in_m  = in_m0 + tile_row_of(rslot, r);
+                const bool    valid = in_m < in_end;
                 held[r].load_checked(x + in_m * N + gn, [&](int i) { return valid && gn + i < N; });
+            }
         }
     } else {
         Held8<T> up[BQ_ROUNDS];
         float    pr[BQ_ROUNDS];
+        bool     live[BQ_ROUNDS]; // the row exists and is not masked out
+        if constexpr (VEC8) {
+            int64_t ms[BQ_ROUNDS];
 #pragma unroll
-        for (int r = 0; r < BQ_ROUNDS; ++r) {
-            const int64_t in_m  = in_m0 + tile_row_of(rslot, r);
-            const bool    valid = in_m < in_end;
-            const T      *g     = x + in_m * 2 * N + gn;
-            if (valid && full) {
+            for (int r = 0; r < BQ_ROUNDS; ++r) {
+                const int64_t in_m = in_m0 + tile_row_of(rslot, r);
+                live[r]            = in_m < in_end;
+                const bool ok      = live[r] && gn < N;
+                ms[r]              = live[r] ? in_m : 0;
+                const T *g         = x + (ok ? in_m * 2 * N + gn : 0);
                 held[r].load(g);
                 up[r].load(g + N);
-            } else {
+                pr[r] = a.probs[ms[r]];
+            }
+            if (a.row_mask != nullptr) {
+                int64_t keep[BQ_ROUNDS];
+#pragma unroll
+                for (int r = 0; r < BQ_ROUNDS; ++r)
+                    keep[r] = a.row_mask[ms[r]];
+#pragma unroll
+                for (int r = 0; r < BQ_ROUNDS; ++r)
+                    live[r] = live[r] && keep[r] != 0;
+            }
+#pragma unroll
+            for (int r = 0; r < BQ_ROUNDS; ++r)
+                live[r] = live[r] && gn < N;
+        } else {
+#pragma unroll
+            for (int r = 0; r < BQ_ROUNDS; ++r) {
+                const int64_t in_m  = in_m0 + tile_row_of(rslot, r);
+                const bool    valid = in_m < in_end;
+                const T      *g     = x + in_m * 2 * N + gn;
                 held[r].load_checked(g, [&](int i) { return valid && gn + i < N; });
                 up[r].load_checked(g + N, [&](int i) { return valid && gn + i < N; });
+                live[r] = valid && (a.row_mask == nullptr || a.row_mask[in_m] != 0);
+                pr[r]   = live[r] ? a.probs[in_m] : 0.f;
             }
-            pr[r] = (valid && (a.row_mask == nullptr || a.row_mask[in_m] != 0)) ? a.probs[in_m] : 0.f;
         }
 #pragma unroll
         for (int r = 0; r < BQ_ROUNDS; ++r) {
-            const int64_t in_m = in_m0 + tile_row_of(rslot, r);
-            const bool    live = in_m < in_end && (a.row_mask == nullptr || a.row_mask[in_m] != 0);
-            float         fg[8], fu[8];
+            float fg[8], fu[8];
             held[r].get(fg);
             up[r].get(fu);
 #pragma unroll
             for (int i = 0; i < 8; ++i) // (padding columns hold zeros: act(0) * 0 = 0)
-                fg[i] = live ? act_fwd<GLU - 1>(fg[i]) * fu[i] * pr[r] : 0.f;
+                fg[i] = live[r] ? act_fwd<GLU - 1>(fg[i]) * fu[i] * pr[r] : 0.f;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
                 held[r].w[i] = pack2<T>(fg[2 * i], fg[2 * i + 1]);

@@ -52,14 +52,38 @@ __device__ __forceinline__ float mx_inv_scale(int e) {
     return __uint_as_float(static_cast<uint32_t>(127 - e) << 23);
 }
 
-// 32 scaled values -> packed codes. FP8: 8 dwords, FP4: 4 dwords.
-template <int FMT> __device__ __forceinline__ void mx_encode32(const float (&v)[32], float inv, uint32_t (&out)[8]) {
+// clamp(x * scale, +-qmax) in two instructions for an x that is not NaN (same value as scale_clamp)
+__device__ __forceinline__ float scale_clamp_no_nan(float x, float scale, float qmax) {
+    return __builtin_amdgcn_fmed3f(x * scale, -qmax, qmax);
+}
+
+// N scaled values (N = 8 or 32) -> packed codes. FP8: N / 4 dwords, FP4: N / 8 dwords. `no_nan`: the
+// caller knows that no value is NaN (the short clamp serves).
+template <int FMT, int N, int W> __device__ __forceinline__ void mx_encode(const float (&v)[N], float inv, uint32_t (&out)[W], bool no_nan) {
     constexpr float Q = MxFmt<FMT>::QMAX;
+    if (no_nan) {
+        if constexpr (FMT == MX_E2M1) {
+#pragma unroll
+            for (int d = 0; d < N / 8; ++d) {
+                uint32_t w = 0;
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp_no_nan(v[8 * d + 0], inv, Q), scale_clamp_no_nan(v[8 * d + 1], inv, Q), 1.0f, 0);
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp_no_nan(v[8 * d + 2], inv, Q), scale_clamp_no_nan(v[8 * d + 3], inv, Q), 1.0f, 1);
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp_no_nan(v[8 * d + 4], inv, Q), scale_clamp_no_nan(v[8 * d + 5], inv, Q), 1.0f, 2);
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp_no_nan(v[8 * d + 6], inv, Q), scale_clamp_no_nan(v[8 * d + 7], inv, Q), 1.0f, 3);
+                out[d] = w;
+            }
+        } else {
+#pragma unroll
+            for (int d = 0; d < N / 4; ++d)
+                out[d] = cvt4_fp8<FMT == MX_E5M2>(scale_clamp_no_nan(v[4 * d], inv, Q), scale_clamp_no_nan(v[4 * d + 1], inv, Q),
+                                                  scale_clamp_no_nan(v[4 * d + 2], inv, Q), scale_clamp_no_nan(v[4 * d + 3], inv, Q));
+        }
+        return;
+    }
     if constexpr (FMT == MX_E2M1) {
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
+        for (int d = 0; d < N / 8; ++d) {
             uint32_t w = 0;
-            // byte k of the dword holds elements 8 d + 2 k (low nibble) and 8 d + 2 k + 1
             w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp(v[8 * d + 0], inv, Q), scale_clamp(v[8 * d + 1], inv, Q), 1.0f, 0);
             w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp(v[8 * d + 2], inv, Q), scale_clamp(v[8 * d + 3], inv, Q), 1.0f, 1);
             w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp(v[8 * d + 4], inv, Q), scale_clamp(v[8 * d + 5], inv, Q), 1.0f, 2);
@@ -68,10 +92,30 @@ template <int FMT> __device__ __forceinline__ void mx_encode32(const float (&v)[
         }
     } else {
 #pragma unroll
-        for (int d = 0; d < 8; ++d)
+        for (int d = 0; d < N / 4; ++d)
             out[d] = cvt4_fp8<FMT == MX_E5M2>(scale_clamp(v[4 * d], inv, Q), scale_clamp(v[4 * d + 1], inv, Q),
                                               scale_clamp(v[4 * d + 2], inv, Q), scale_clamp(v[4 * d + 3], inv, Q));
     }
+}
+
+// The abs-max of 16-bit floats taken on their bit patterns, two at a time: with the sign bit
+// cleared, floats order like unsigned integers. A NaN shows as a value above the infinity
+// pattern; the caller then takes the abs-max that ignores NaN from the float values.
+template <typename T> struct Bits16;
+template <> struct Bits16<bf16_t> {
+    static constexpr uint32_t INF = 0x7F80u;
+    static __device__ __forceinline__ float to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+};
+template <> struct Bits16<f16_t> {
+    static constexpr uint32_t INF = 0x7C00u;
+    static __device__ __forceinline__ float to_f32(uint32_t b) {
+        return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(b)));
+    }
+};
+__device__ __forceinline__ uint32_t pk_absmax16(uint32_t acc, uint32_t w) {
+    typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, acc),
+                                                                  __builtin_bit_cast(u16x2, w & 0x7FFF7FFFu)));
 }
 
 // Stochastic rounding (MXFP4 gradients): the hardware converter adds the seed's bits below the
@@ -206,46 +250,96 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
 
     PT_MX_TRACE(0);
     // ---- tile -> LDS (zeros outside the matrix) ----
-    const bool vec = (a.N & 7) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
-#pragma unroll
-    for (int p = 0; p < 8; ++p) {
-        const int     r = p * 16 + (tid >> 4), c = (tid & 15) * 8;
-        const int64_t m = in_m0 + r, n = n0 + c;
-        u32x4         v = u32x4{0u, 0u, 0u, 0u};
+    // Whole 16-byte pieces (the common case) are all requested before the first is used: a piece
+    // outside the matrix reads the matrix's first bytes instead and is replaced by zeros, so that
+    // no branch separates the loads.
+    const bool vec = (a.N & 7) == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15) == 0;
+    if (vec) {
+        u32x4 piece[8];
+        bool  inside[8];
         if constexpr (GLU != 0) {
-            if (m < in_end && n < a.N && (a.row_mask == nullptr || a.row_mask[m] != 0)) {
-                const uint16_t *gp = static_cast<const uint16_t *>(a.x) + m * 2 * a.N + n;
-                const float     pr = a.probs[m];
-                uint32_t        gw[4] = {0u, 0u, 0u, 0u}, uw[4] = {0u, 0u, 0u, 0u};
-                if (vec) {
-                    const u32x4 g4 = ld128(gp), u4 = ld128(gp + a.N);
-                    gw[0] = g4.x, gw[1] = g4.y, gw[2] = g4.z, gw[3] = g4.w;
-                    uw[0] = u4.x, uw[1] = u4.y, uw[2] = u4.z, uw[3] = u4.w;
-                } else {
+            u32x4   up[8];
+            float   pr[8];
+            int64_t ms[8];
+#pragma unroll
+            for (int p = 0; p < 8; ++p) {
+                const int     r = p * 16 + (tid >> 4), c = (tid & 15) * 8;
+                const int64_t m = in_m0 + r, n = n0 + c;
+                inside[p]       = m < in_end && n < a.N;
+                ms[p]           = inside[p] ? m : 0;
+                const uint16_t *gp = static_cast<const uint16_t *>(a.x) + ms[p] * 2 * a.N + (inside[p] ? n : 0);
+                piece[p]           = ld128(gp);
+                up[p]              = ld128(gp + a.N);
+                pr[p]              = a.probs[ms[p]];
+            }
+            if (a.row_mask != nullptr) {
+                int64_t keep[8];
+#pragma unroll
+                for (int p = 0; p < 8; ++p)
+                    keep[p] = a.row_mask[ms[p]];
+#pragma unroll
+                for (int p = 0; p < 8; ++p)
+                    inside[p] = inside[p] && keep[p] != 0;
+            }
+#pragma unroll
+            for (int p = 0; p < 8; ++p) {
+                const uint32_t gw[4] = {piece[p].x, piece[p].y, piece[p].z, piece[p].w};
+                const uint32_t uw[4] = {up[p].x, up[p].y, up[p].z, up[p].w};
+                uint32_t       o[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    float g0, g1, u0, u1;
+                    unpack2<T>(gw[k], g0, g1);
+                    unpack2<T>(uw[k], u0, u1);
+                    o[k] = pack2<T>(act_fwd<GLU - 1>(g0) * u0 * pr[p], act_fwd<GLU - 1>(g1) * u1 * pr[p]);
+                }
+                piece[p] = u32x4{o[0], o[1], o[2], o[3]};
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < 8; ++p) {
+                const int     r = p * 16 + (tid >> 4), c = (tid & 15) * 8;
+                const int64_t m = in_m0 + r, n = n0 + c;
+                inside[p]       = m < in_end && n < a.N;
+                piece[p]        = ld128(x + (inside[p] ? m * a.N + n : 0));
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+            const int r = p * 16 + (tid >> 4), c = (tid & 15) * 8;
+            *reinterpret_cast<u32x4 *>(&tile[r * MX_PITCH + c]) = inside[p] ? piece[p] : u32x4{0u, 0u, 0u, 0u};
+        }
+    } else {
+#pragma unroll 1
+        for (int p = 0; p < 8; ++p) {
+            const int     r = p * 16 + (tid >> 4), c = (tid & 15) * 8;
+            const int64_t m = in_m0 + r, n = n0 + c;
+            u32x4         v = u32x4{0u, 0u, 0u, 0u};
+            if constexpr (GLU != 0) {
+                if (m < in_end && n < a.N && (a.row_mask == nullptr || a.row_mask[m] != 0)) {
+                    const uint16_t *gp = static_cast<const uint16_t *>(a.x) + m * 2 * a.N + n;
+                    const float     pr = a.probs[m];
+                    uint32_t        gw[4] = {0u, 0u, 0u, 0u}, uw[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
                     for (int k = 0; k < 8; ++k)
                         if (n + k < a.N) {
                             gw[k >> 1] |= static_cast<uint32_t>(gp[k]) << (16 * (k & 1));
                             uw[k >> 1] |= static_cast<uint32_t>(gp[a.N + k]) << (16 * (k & 1));
                         }
-                }
-                uint32_t o[4];
+                    uint32_t o[4];
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    float g0, g1, u0, u1;
-                    unpack2<T>(gw[k], g0, g1);
-                    unpack2<T>(uw[k], u0, u1);
-                    // columns behind N stay +0 whatever probs holds
-                    const float r0 = n + 2 * k < a.N ? act_fwd<GLU - 1>(g0) * u0 * pr : 0.f;
-                    const float r1 = n + 2 * k + 1 < a.N ? act_fwd<GLU - 1>(g1) * u1 * pr : 0.f;
-                    o[k]           = pack2<T>(r0, r1);
+                    for (int k = 0; k < 4; ++k) {
+                        float g0, g1, u0, u1;
+                        unpack2<T>(gw[k], g0, g1);
+                        unpack2<T>(uw[k], u0, u1);
+                        // columns behind N stay +0 whatever probs holds
+                        const float r0 = n + 2 * k < a.N ? act_fwd<GLU - 1>(g0) * u0 * pr : 0.f;
+                        const float r1 = n + 2 * k + 1 < a.N ? act_fwd<GLU - 1>(g1) * u1 * pr : 0.f;
+                        o[k]           = pack2<T>(r0, r1);
+                    }
+                    v = u32x4{o[0], o[1], o[2], o[3]};
                 }
-                v = u32x4{o[0], o[1], o[2], o[3]};
-            }
-        } else if (m < in_end && n < a.N) {
-            if (vec) {
-                v = ld128(x + m * a.N + n);
-            } else {
+            } else if (m < in_end && n < a.N) {
                 uint16_t e[8];
 #pragma unroll
                 for (int k = 0; k < 8; ++k)
@@ -253,42 +347,41 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
                 v = u32x4{e[0] | (uint32_t(e[1]) << 16), e[2] | (uint32_t(e[3]) << 16), e[4] | (uint32_t(e[5]) << 16),
                           e[6] | (uint32_t(e[7]) << 16)};
             }
+            *reinterpret_cast<u32x4 *>(&tile[r * MX_PITCH + c]) = v;
         }
-        *reinterpret_cast<u32x4 *>(&tile[r * MX_PITCH + c]) = v;
     }
     PT_MX_TRACE(1);
     __syncthreads();
     PT_MX_TRACE(2);
 
-    auto elem = [&](uint16_t raw) -> float {
-        T t;
-        __builtin_memcpy(&t, &raw, 2);
-        return HP<T>::to_f32(t);
-    };
-
     // ---- row direction: task = (row r, 32-column block c) ----
     float rv[2][32];
     float ram[2];
+    bool  rnan[2] = {true, true}; // false: the task's 32 input values are known to hold no NaN
     if constexpr (ROW || ANY2D) {
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
             const int t = tid + 256 * p, r = t >> 2, c = t & 3;
-            float     am = 0.f;
+            uint32_t  m2 = 0;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const u32x4    w    = *reinterpret_cast<const u32x4 *>(&tile[r * MX_PITCH + c * 32 + q * 8]);
                 const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    const float lo = elem(static_cast<uint16_t>(ww[k] & 0xffffu)), hi = elem(static_cast<uint16_t>(ww[k] >> 16));
-                    rv[p][q * 8 + 2 * k]     = lo;
-                    rv[p][q * 8 + 2 * k + 1] = hi;
-                    am = fmaxf(am, fmaxf(abs_or_zero(lo), abs_or_zero(hi)));
+                    unpack2<T>(ww[k], rv[p][q * 8 + 2 * k], rv[p][q * 8 + 2 * k + 1]);
+                    m2 = pk_absmax16(m2, ww[k]);
                 }
             }
+            const uint32_t m16 = max(m2 & 0xffffu, m2 >> 16);
+            rnan[p]            = m16 > Bits16<T>::INF;
+            float am           = Bits16<T>::to_f32(m16);
             if constexpr ((RHT & 1) != 0) {
                 hadamard16(rv[p], 0);
                 hadamard16(rv[p], 16);
+                rnan[p] = true; // the transformed values are not looked at
+            }
+            if (rnan[p]) {
                 am = 0.f;
 #pragma unroll
                 for (int k = 0; k < 32; ++k)
@@ -320,7 +413,7 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
                 const uint32_t id = (static_cast<uint32_t>(blockIdx.z) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
                 mx_encode32_fp4_sr(rv[p], mx_inv_scale(e), sr_hash(a.sr_seed ^ (id * 512u + t)), code);
             } else {
-                mx_encode32<FMT>(rv[p], mx_inv_scale(e), code);
+                mx_encode<FMT>(rv[p], mx_inv_scale(e), code, !rnan[p]);
             }
             sbytes[r * 4 + c] = static_cast<uint8_t>(e + 127);
             if (r < row_cnt) {
@@ -358,23 +451,26 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
         // serves both (task p: column c, numbered t = 128 rb + c as the seeds of stochastic rounding expect)
         const int rb = tid >> 6, c0 = (tid & 63) * 2;
         float     v2[2][32];
+        uint32_t  m2 = 0; // low half: column c0, high half: column c0 + 1
 #pragma unroll
         for (int i = 0; i < 32; ++i) {
             const uint32_t w = *reinterpret_cast<const uint32_t *>(&tile[(rb * 32 + i) * MX_PITCH + c0]);
-            v2[0][i]         = elem(static_cast<uint16_t>(w & 0xffffu));
-            v2[1][i]         = elem(static_cast<uint16_t>(w >> 16));
+            unpack2<T>(w, v2[0][i], v2[1][i]);
+            m2 = pk_absmax16(m2, w);
         }
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
             const int c = c0 + p, t = 128 * rb + c;
             float (&v)[32] = v2[p];
-            float am = 0.f;
-#pragma unroll
-            for (int i = 0; i < 32; ++i)
-                am = fmaxf(am, abs_or_zero(v[i]));
+            const uint32_t m16 = p == 0 ? (m2 & 0xffffu) : (m2 >> 16);
+            bool           cnan = m16 > Bits16<T>::INF;
+            float          am   = Bits16<T>::to_f32(m16);
             if constexpr ((RHT & 2) != 0) {
                 hadamard16(v, 0);
                 hadamard16(v, 16);
+                cnan = true; // the transformed values are not looked at
+            }
+            if (cnan) {
                 am = 0.f;
 #pragma unroll
                 for (int i = 0; i < 32; ++i)
@@ -391,7 +487,7 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
                 const uint32_t id = (static_cast<uint32_t>(blockIdx.z) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
                 mx_encode32_fp4_sr(v, mx_inv_scale(e), sr_hash(a.sr_seed ^ 0x5BD1E995u ^ (id * 512u + t)), code[p]);
             } else {
-                mx_encode32<FMT>(v, mx_inv_scale(e), code[p]);
+                mx_encode<FMT>(v, mx_inv_scale(e), code[p], !cnan);
             }
             sbytes[c * 4 + rb] = static_cast<uint8_t>(e + 127);
         }
@@ -460,14 +556,26 @@ __global__ __launch_bounds__(256) void mx_quant_rows_kernel(const MxArgs a, cons
     for (int k = 0; k < 4; ++k) {
         const uint32_t ww[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
         float          f[8];
-        float          am = 0.f;
+        uint32_t       m2 = 0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             unpack2<T>(ww[i], f[2 * i], f[2 * i + 1]);
-            am = fmaxf(am, fmaxf(abs_or_zero(f[2 * i]), abs_or_zero(f[2 * i + 1])));
+            m2 = pk_absmax16(m2, ww[i]);
         }
-        am = fmaxf(am, dpp_f32<0xB1>(am)); // quad_perm [1,0,3,2]
-        am = fmaxf(am, dpp_f32<0x4E>(am)); // quad_perm [2,3,0,1]
+        // the block's abs-max: over the four lanes of the quad (quad_perm [1,0,3,2], then [2,3,0,1])
+        uint32_t m16 = max(m2 & 0xffffu, m2 >> 16);
+        m16          = max(m16, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, m16, 0xB1, 0xf, 0xf, true)));
+        m16          = max(m16, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, m16, 0x4E, 0xf, 0xf, true)));
+        const bool nan = m16 > Bits16<T>::INF; // somewhere in the block
+        float      am  = Bits16<T>::to_f32(m16);
+        if (nan) {
+            am = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                am = fmaxf(am, abs_or_zero(f[i]));
+            am = fmaxf(am, dpp_f32<0xB1>(am));
+            am = fmaxf(am, dpp_f32<0x4E>(am));
+        }
         const int   e   = mx_exponent<FMT>(am);
         const float inv = mx_inv_scale(e);
         ebytes |= static_cast<uint32_t>(e + 127) << (8 * k);
@@ -490,20 +598,17 @@ __global__ __launch_bounds__(256) void mx_quant_rows_kernel(const MxArgs a, cons
                     w |= (__builtin_amdgcn_cvt_scalef32_sr_pk_fp4_f32(0u, pair, seed, 1.0f, 0) & 0xffu) << (8 * i);
                 }
             } else {
-                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp(f[0], inv, Q), scale_clamp(f[1], inv, Q), 1.0f, 0);
-                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp(f[2], inv, Q), scale_clamp(f[3], inv, Q), 1.0f, 1);
-                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp(f[4], inv, Q), scale_clamp(f[5], inv, Q), 1.0f, 2);
-                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, scale_clamp(f[6], inv, Q), scale_clamp(f[7], inv, Q), 1.0f, 3);
+                uint32_t c[1];
+                mx_encode<FMT>(f, inv, c, !nan);
+                w = c[0];
             }
             if (in)
                 *reinterpret_cast<uint32_t *>(a.row_q + row[k] * (a.Npad >> 1) + (n >> 1)) = w;
         } else {
-            const uint32_t c0 = cvt4_fp8<FMT == MX_E5M2>(scale_clamp(f[0], inv, Q), scale_clamp(f[1], inv, Q),
-                                                         scale_clamp(f[2], inv, Q), scale_clamp(f[3], inv, Q));
-            const uint32_t c1 = cvt4_fp8<FMT == MX_E5M2>(scale_clamp(f[4], inv, Q), scale_clamp(f[5], inv, Q),
-                                                         scale_clamp(f[6], inv, Q), scale_clamp(f[7], inv, Q));
+            uint32_t c[2];
+            mx_encode<FMT>(f, inv, c, !nan);
             if (in)
-                *reinterpret_cast<u32x2 *>(a.row_q + row[k] * a.Npad + n) = u32x2{c0, c1};
+                *reinterpret_cast<u32x2 *>(a.row_q + row[k] * a.Npad + n) = u32x2{c[0], c[1]};
         }
     }
     // lane L < 16 writes scale word L & 3 of run L >> 2: the bytes of the blocks 4 (L & 3) .. + 3 of
