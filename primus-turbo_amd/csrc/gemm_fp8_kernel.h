@@ -235,20 +235,33 @@ __device__ __forceinline__ void epilogue_inner(T *row, int64_t step, bool accu, 
     static_for<0, TM>([&](auto ic) {
         constexpr int i = ic;
         if constexpr (sizeof(T) == 4) {
-            static_for<0, TN>([&](auto jc) {
-                constexpr int j = jc;
-                f32x4         v = read_acc<ACC_IN_AGPR>(acc[i][j]);
-                if constexpr (MODE == SCALE_VECTOR) {
+            // accumulating: the old values of four tiles are requested together, then used (one
+            // load at a time would pay the memory latency TN times per row)
+            constexpr int JB = TN < 4 ? TN : 4;
+            static_for<0, TN / JB>([&](auto jbc) {
+                constexpr int j0 = JB * jbc;
+                f32x4         old[JB];
+                if (accu) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        v[e] = v[e] * sa[i] * sb[j][e];
+                    for (int jj = 0; jj < JB; ++jj)
+                        old[jj] = *reinterpret_cast<const f32x4 *>(row + (j0 + jj) * 16);
                 }
-                T *q = row + j * 16;
-                if (accu)
-                    v += *reinterpret_cast<const f32x4 *>(q);
-                *reinterpret_cast<f32x4 *>(q) = v;
-                // keep each accumulator's read next to its store (register pressure)
                 __builtin_amdgcn_sched_barrier(0);
+                static_for<0, JB>([&](auto jjc) {
+                    constexpr int j = j0 + jjc;
+                    f32x4         v = read_acc<ACC_IN_AGPR>(acc[i][j]);
+                    if constexpr (MODE == SCALE_VECTOR) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            v[e] = v[e] * sa[i] * sb[j][e];
+                    }
+                    T *q = row + j * 16;
+                    if (accu)
+                        v += old[j - j0];
+                    *reinterpret_cast<f32x4 *>(q) = v;
+                    // keep each accumulator's read next to its store (register pressure)
+                    __builtin_amdgcn_sched_barrier(0);
+                });
             });
         } else {
             static_for<0, TN / 2>([&](auto jc) {
