@@ -172,7 +172,8 @@ class QuantBlockwise(_QuantBase):
 
         self.qi, self.dual, self.M, self.N = qi, dual, M, N
         self.name = f"fp8_e4m3_blockwise_{'1x128+128x1_dual' if dual else '1x128'}_quant_{M}x{N}_bf16"
-        self.dominant_name = "quant_block128_kernel (one 128x128 tile per workgroup, " + ("row and column blocks)" if dual else "row blocks)")
+        self.dominant_name = ("quant_block128_kernel (one 128x128 tile per workgroup, row and column blocks)" if dual else
+                              "quant_rows128_kernel (stream without LDS: 16 lanes per 1x128 block, four blocks of four rows per wavefront)")
         self.x_cpu = _randn_bf16((M, N), 12)
         self.x = self.x_cpu.to(dev)
 

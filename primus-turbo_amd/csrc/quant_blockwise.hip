@@ -398,6 +398,73 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
     }
 }
 
+// Row blocks alone, rows of whole 16-byte pieces: a stream without LDS, same bytes as the tile
+// kernel. A workgroup takes 16 rows of four neighbouring 128-column blocks, a wavefront four of
+// those rows (runs of 1 KB): 16 lanes quantize one row of one block, a load covers one block of
+// the four rows, and all four loads of a lane are requested before the first is used. The 16
+// scales of a wavefront leave as 16 bytes per row (row-major scales, [M, N / 128]) or as 16 bytes
+// per block (block-major scales, [N / 128, M]).
+template <typename T, bool E5M2>
+__global__ __launch_bounds__(256) void quant_rows128_kernel(const BlockQuantArgs a, const int64_t col_groups) {
+    const int     lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int     cseg = lane & 15, g = lane >> 4;
+    const int64_t cg = blockIdx.x % col_groups, rg = blockIdx.x / col_groups;
+    const bool    block_major = a.rs_n != 1;
+    const T      *x = static_cast<const T *>(a.x);
+    Held8<T>      held[4];
+    bool          ok[4];
+    int64_t       row[4], tn[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        row[k]           = rg * 16 + 4 * wave + g;
+        tn[k]            = cg * 4 + k;
+        const int64_t gn = tn[k] * BQ + cseg * BQ_PACK;
+        ok[k]            = gn < a.N && row[k] < a.M; // (N is a multiple of 8: a piece is inside or outside as a whole)
+        held[k].load(x + (ok[k] ? row[k] * a.N + gn : 0));
+    }
+    float inv[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        float vals[BQ_PACK];
+        held[k].get(vals);
+        float amax = 0.f;
+#pragma unroll
+        for (int i = 0; i < BQ_PACK; ++i) {
+            vals[i] = ok[k] ? vals[i] : 0.f;
+            amax    = fmaxf(amax, fabsf(vals[i]));
+        }
+        amax              = row16_max(amax); // the 16 lanes of this row's block
+        const float scale = a.qmax / fmaxf(amax, BQ_EPS);
+        inv[k]            = 1.0f / scale;
+        if (ok[k]) {
+            const float s[8] = {scale, scale, scale, scale, scale, scale, scale, scale};
+            *reinterpret_cast<u32x2 *>(a.q_row + row[k] * a.N + tn[k] * BQ + cseg * BQ_PACK) = quant8<E5M2>(vals, s, a.qmax);
+        }
+    }
+    if (block_major) {
+        // lane L < 16 writes the scale of block L >> 2 and row L & 3, which the lanes 16 (L & 3) .. hold
+        float mine = 0.f;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float v = __shfl(inv[k], 16 * (lane & 3), 64);
+            mine          = (lane >> 2) == k ? v : mine;
+        }
+        const int64_t r = rg * 16 + 4 * wave + (lane & 3), t = cg * 4 + (lane >> 2);
+        if (lane < 16 && r < a.M && t * BQ < a.N)
+            a.s_row[r * a.rs_m + t * a.rs_n] = mine;
+    } else if (cseg == 0 && row[0] < a.M) {
+        float *p = a.s_row + row[0] * a.rs_m + tn[0];
+        if ((tn[3] + 1) * BQ - BQ < a.N && (reinterpret_cast<uintptr_t>(p) & 15) == 0) {
+            st128(p, u32x4{__float_as_uint(inv[0]), __float_as_uint(inv[1]), __float_as_uint(inv[2]), __float_as_uint(inv[3])});
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (tn[k] * BQ < a.N)
+                    p[k] = inv[k];
+        }
+    }
+}
+
 template <typename T, bool E5M2, int MODE, bool GROUPED, int GLU = 0>
 static int launch_block128(const BlockQuantArgs &a, int64_t tiles_m, int64_t tiles_n, int64_t batch,
                            bool vec, hipStream_t stream) {
@@ -592,6 +659,18 @@ static int quantize_blocks(const void *x, int x_dtype, int64_t M, int64_t N, int
     a.qmax = fp8_max_of(q_dtype);
     auto       st  = static_cast<hipStream_t>(stream);
     const bool vec = vec_ok(a, 1);
+    if (row && !col && vec) {
+        const int64_t col_groups = cdiv(tn, 4), row_groups = cdiv(M, 16);
+        PT_REQUIRE(col_groups * row_groups < (1LL << 31), "too many blocks");
+        const dim3 grid(static_cast<unsigned>(col_groups * row_groups));
+#define CALL(T, E5)                                                                                \
+    do {                                                                                           \
+        quant_rows128_kernel<T, E5><<<grid, 256, 0, st>>>(a, col_groups);                          \
+        return check_launch("quant_rows128_kernel");                                               \
+    } while (0)
+        PT_DISPATCH_T_E5(x_dtype, q_dtype, CALL);
+#undef CALL
+    }
 #define CALL(T, E5)                                                                                \
     do {                                                                                           \
         if (row && col)                                                                            \

@@ -71,6 +71,9 @@ def test_blockwise_other_sources(src):
     assert np.array_equal(codes_np(qr), oqr) and np.array_equal(codes_np(qc), oqc)
     _eq_scales(sr, osr)
     _eq_scales(sc, osc)
+    q, s = turbo.ops.quantize_fp8(x.cuda(), torch.float8_e4m3fn, G.BLOCKWISE, block_size=128, axis=1)  # rows alone
+    assert np.array_equal(codes_np(q), oqr)
+    _eq_scales(s, osr)
 
 
 @pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
