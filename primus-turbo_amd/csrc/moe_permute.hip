@@ -199,13 +199,28 @@ __global__ __launch_bounds__(256) void moe_permute_kernel(const uint8_t *__restr
     if (n == 0)
         return;
     const u32x4 zero{0u, 0u, 0u, 0u};
-    for (int64_t j = threadIdx.x * 16L; j < hidden_bytes; j += 256 * 16L) {
-        const u32x4 v = is_pad ? zero : ld128(tokens + token * hidden_bytes + j);
+    // four 16-byte pieces per thread and round, all requested before the first is stored (a piece
+    // behind the row's end re-reads the thread's first piece: no branch between the loads)
+    for (int64_t j0 = threadIdx.x * 16L; j0 < hidden_bytes; j0 += 4 * 256 * 16L) {
+        u32x4 v[4] = {zero, zero, zero, zero};
+        if (!is_pad) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int64_t j = j0 + q * 256 * 16L;
+                v[q]            = ld128(tokens + token * hidden_bytes + (j < hidden_bytes ? j : j0));
+            }
+        }
         for (int i = 0; i < n; ++i) {
             const int     d = row[i];
             const int64_t r = d > 0 ? d - 1 : -static_cast<int64_t>(d) - 1;
-            if (d != 0 && r < out_rows) // a map made for a larger output never writes past this one
-                st128_nt(out + r * hidden_bytes + j, d > 0 ? v : zero);
+            if (d != 0 && r < out_rows) { // a map made for a larger output never writes past this one
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int64_t j = j0 + q * 256 * 16L;
+                    if (j < hidden_bytes)
+                        st128_nt(out + r * hidden_bytes + j, d > 0 ? v[q] : zero);
+                }
+            }
         }
     }
     if (sf != nullptr)
@@ -243,16 +258,26 @@ __global__ __launch_bounds__(256) void moe_unpermute_kernel(const T *__restrict_
     const int     n     = row[2 * E];
     for (int64_t c = threadIdx.x * 8L; c < H; c += 256 * 8L) {
         float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        for (int i = 0; i < n; ++i) {
-            const int s = row[i];
-            if (s <= 0 || s > in_rows)
-                continue;
-            const u32x4 w = ld128(permuted + (s - 1) * H + c);
-            float       f0, f1;
-            unpack2<T>(w.x, f0, f1); acc[0] += f0; acc[1] += f1;
-            unpack2<T>(w.y, f0, f1); acc[2] += f0; acc[3] += f1;
-            unpack2<T>(w.z, f0, f1); acc[4] += f0; acc[5] += f1;
-            unpack2<T>(w.w, f0, f1); acc[6] += f0; acc[7] += f1;
+        // the copies of four map entries are requested together, then added in the map's order
+        // (an entry that names no row reads this thread's own output piece and is not added)
+        for (int i0 = 0; i0 < n; i0 += 4) {
+            u32x4 w[4];
+            bool  ok[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int s = i0 + q < n ? row[i0 + q] : 0;
+                ok[q]       = s > 0 && s <= in_rows;
+                w[q]        = ld128(ok[q] ? permuted + (s - 1) * H + c : out + token * H + c);
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (ok[q]) {
+                    float f0, f1;
+                    unpack2<T>(w[q].x, f0, f1); acc[0] += f0; acc[1] += f1;
+                    unpack2<T>(w[q].y, f0, f1); acc[2] += f0; acc[3] += f1;
+                    unpack2<T>(w[q].z, f0, f1); acc[4] += f0; acc[5] += f1;
+                    unpack2<T>(w[q].w, f0, f1); acc[6] += f0; acc[7] += f1;
+                }
         }
         st128_nt(out + token * H + c, u32x4{pack2<T>(acc[0], acc[1]), pack2<T>(acc[2], acc[3]), pack2<T>(acc[4], acc[5]),
                                            pack2<T>(acc[6], acc[7])});

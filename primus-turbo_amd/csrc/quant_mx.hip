@@ -783,46 +783,61 @@ __global__ __launch_bounds__(256) void mx_dequant_kernel(const uint8_t *__restri
     }
 }
 
-// Row-direction data with 16-byte aligned pointers: a plain stream. A thread takes 16 consecutive
-// elements of a row (half a 32-element block, one scale byte): 16 (FP4: 8) code bytes in, 32 or
-// 64 bytes out, whole lines per wavefront on both sides.
+// Row-direction data with 16-byte aligned pointers: a plain stream. A thread takes 8 consecutive
+// elements of a row (a quarter of a block, one scale byte): 8 (FP4: 4) code bytes in, 16 or 32
+// bytes out, whole lines per wavefront on both sides; four such pieces per round, all of them
+// requested before the first is used. `per_row_shift`: log2 of the pieces per row, or -1.
 template <typename T, int FMT>
 __global__ __launch_bounds__(256) void mx_dequant_stream_kernel(const uint8_t *__restrict__ q, const uint8_t *__restrict__ s,
-                                                                T *__restrict__ y, const int64_t rows, const int64_t cols) {
-    const int64_t per_row = cols >> 4, units = rows * per_row;
+                                                                T *__restrict__ y, const int64_t rows, const int64_t cols,
+                                                                const int per_row_shift) {
+    const int64_t per_row = cols >> 3, units = rows * per_row;
     const int64_t stride  = static_cast<int64_t>(gridDim.x) * 256;
-    for (int64_t u = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; u < units; u += stride) {
-        const int64_t r = u / per_row, c = u - r * per_row;
-        const float   sc = __uint_as_float(static_cast<uint32_t>(s[r * (cols >> 5) + (c >> 1)]) << 23);
-        float         f[16];
-        if constexpr (FMT == MX_E2M1) {
-            const u32x2    w     = *reinterpret_cast<const u32x2 *>(q + (u << 3));
-            const uint32_t ww[2] = {w.x, w.y};
+    for (int64_t u0 = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; u0 < units; u0 += 4 * stride) {
+        uint32_t code[4][2];
+        uint32_t sbyte[4];
 #pragma unroll
-            for (int k = 0; k < 16; ++k)
-                f[k] = e2m1_to_f32(ww[k >> 3] >> (4 * (k & 7))) * sc;
-        } else {
-            const u32x4    w     = ld128(q + (u << 4));
-            const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                f[4 * k + 0] = fp8_to_f32<FMT == MX_E5M2>(ww[k], 0) * sc;
-                f[4 * k + 1] = fp8_to_f32<FMT == MX_E5M2>(ww[k], 1) * sc;
-                f[4 * k + 2] = fp8_to_f32<FMT == MX_E5M2>(ww[k], 2) * sc;
-                f[4 * k + 3] = fp8_to_f32<FMT == MX_E5M2>(ww[k], 3) * sc;
+        for (int k = 0; k < 4; ++k) {
+            const int64_t u = u0 + k * stride < units ? u0 + k * stride : u0; // (a piece behind the end re-reads the first)
+            const int64_t r = per_row_shift >= 0 ? u >> per_row_shift : u / per_row, c = u - r * per_row;
+            sbyte[k]        = s[r * (cols >> 5) + (c >> 2)];
+            if constexpr (FMT == MX_E2M1) {
+                code[k][0] = *reinterpret_cast<const uint32_t *>(q + (u << 2));
+                code[k][1] = 0;
+            } else {
+                const u32x2 w = *reinterpret_cast<const u32x2 *>(q + (u << 3));
+                code[k][0] = w.x, code[k][1] = w.y;
             }
         }
-        char *dst = reinterpret_cast<char *>(y + (u << 4));
-        if constexpr (sizeof(T) == 4) {
 #pragma unroll
-            for (int k = 0; k < 4; ++k)
-                st128(dst + 16 * k, u32x4{__float_as_uint(f[4 * k]), __float_as_uint(f[4 * k + 1]),
-                                          __float_as_uint(f[4 * k + 2]), __float_as_uint(f[4 * k + 3])});
-        } else {
+        for (int k = 0; k < 4; ++k) {
+            const int64_t u = u0 + k * stride;
+            if (u >= units)
+                break;
+            const float sc = __uint_as_float(sbyte[k] << 23);
+            float       f[8];
+            if constexpr (FMT == MX_E2M1) {
 #pragma unroll
-            for (int k = 0; k < 2; ++k)
-                st128(dst + 16 * k, u32x4{pack2<T>(f[8 * k], f[8 * k + 1]), pack2<T>(f[8 * k + 2], f[8 * k + 3]),
-                                          pack2<T>(f[8 * k + 4], f[8 * k + 5]), pack2<T>(f[8 * k + 6], f[8 * k + 7])});
+                for (int i = 0; i < 8; ++i)
+                    f[i] = e2m1_to_f32(code[k][0] >> (4 * i)) * sc;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    f[4 * i + 0] = fp8_to_f32<FMT == MX_E5M2>(code[k][i], 0) * sc;
+                    f[4 * i + 1] = fp8_to_f32<FMT == MX_E5M2>(code[k][i], 1) * sc;
+                    f[4 * i + 2] = fp8_to_f32<FMT == MX_E5M2>(code[k][i], 2) * sc;
+                    f[4 * i + 3] = fp8_to_f32<FMT == MX_E5M2>(code[k][i], 3) * sc;
+                }
+            }
+            char *dst = reinterpret_cast<char *>(y + (u << 3));
+            if constexpr (sizeof(T) == 4) {
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                    st128(dst + 16 * i, u32x4{__float_as_uint(f[4 * i]), __float_as_uint(f[4 * i + 1]),
+                                              __float_as_uint(f[4 * i + 2]), __float_as_uint(f[4 * i + 3])});
+            } else {
+                st128(dst, u32x4{pack2<T>(f[0], f[1]), pack2<T>(f[2], f[3]), pack2<T>(f[4], f[5]), pack2<T>(f[6], f[7])});
+            }
         }
     }
 }
@@ -831,11 +846,15 @@ template <typename T, int FMT>
 static void launch_mx_dequant_t(const uint8_t *q, const uint8_t *s, T *y, int64_t rows, int64_t cols, int transpose,
                                 hipStream_t st) {
     if (!transpose && aligned_to(q, 16) && aligned_to(y, 16)) {
-        const int64_t units = rows * (cols >> 4);
-        int64_t       grid  = cdiv(units, 256);
+        const int64_t units = rows * (cols >> 3), per_row = cols >> 3;
+        int64_t       grid  = cdiv(units, 4 * 256);
         const int64_t cap   = 32L * device_cu_count();
         grid                = grid > cap ? cap : grid;
-        mx_dequant_stream_kernel<T, FMT><<<static_cast<unsigned>(grid), 256, 0, st>>>(q, s, y, rows, cols);
+        int shift = -1;
+        if ((per_row & (per_row - 1)) == 0)
+            for (shift = 0; (int64_t{1} << shift) < per_row; ++shift) {
+            }
+        mx_dequant_stream_kernel<T, FMT><<<static_cast<unsigned>(grid), 256, 0, st>>>(q, s, y, rows, cols, shift);
         return;
     }
     dim3 grid(static_cast<unsigned>(cdiv(cols, 64)), static_cast<unsigned>(cdiv(rows, 64)));
