@@ -196,6 +196,16 @@ __device__ __forceinline__ void st128(void *p, u32x4 v) {
 __device__ __forceinline__ void st128_nt(void *p, u32x4 v) {
     __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p));
 }
+__device__ __forceinline__ void st64_nt(void *p, u32x2 v) {
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x2 *>(p));
+}
+__device__ __forceinline__ void st32_nt(void *p, uint32_t v) {
+    __builtin_nontemporal_store(v, reinterpret_cast<uint32_t *>(p));
+}
+// streaming load: input is read once by this kernel
+__device__ __forceinline__ u32x4 ld128_nt(const void *p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+}
 
 __device__ __forceinline__ float bf16lo(uint32_t w) {
     return __uint_as_float(w << 16);

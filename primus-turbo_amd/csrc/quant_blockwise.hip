@@ -53,11 +53,11 @@ struct BlockQuantArgs {
 template <typename T> struct Held8 {
     static constexpr int WORDS = sizeof(T) == 4 ? 8 : 4;
     uint32_t             w[WORDS];
-    __device__ __forceinline__ void load(const T *p) {
-        const u32x4 a = ld128(p);
+    template <bool STREAM = false> __device__ __forceinline__ void load(const T *p) {
+        const u32x4 a = STREAM ? ld128_nt(p) : ld128(p);
         w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w;
         if constexpr (sizeof(T) == 4) {
-            const u32x4 b = ld128(p + 4);
+            const u32x4 b = STREAM ? ld128_nt(p + 4) : ld128(p + 4);
             w[4] = b.x; w[5] = b.y; w[6] = b.z; w[7] = b.w;
         }
     }
@@ -420,7 +420,7 @@ __global__ __launch_bounds__(256) void quant_rows128_kernel(const BlockQuantArgs
         tn[k]            = cg * 4 + k;
         const int64_t gn = tn[k] * BQ + cseg * BQ_PACK;
         ok[k]            = gn < a.N && row[k] < a.M; // (N is a multiple of 8: a piece is inside or outside as a whole)
-        held[k].load(x + (ok[k] ? row[k] * a.N + gn : 0));
+        held[k].template load<true>(x + (ok[k] ? row[k] * a.N + gn : 0));
     }
     float inv[4];
 #pragma unroll
@@ -438,7 +438,7 @@ __global__ __launch_bounds__(256) void quant_rows128_kernel(const BlockQuantArgs
         inv[k]            = 1.0f / scale;
         if (ok[k]) {
             const float s[8] = {scale, scale, scale, scale, scale, scale, scale, scale};
-            *reinterpret_cast<u32x2 *>(a.q_row + row[k] * a.N + tn[k] * BQ + cseg * BQ_PACK) = quant8<E5M2>(vals, s, a.qmax);
+            st64_nt(a.q_row + row[k] * a.N + tn[k] * BQ + cseg * BQ_PACK, quant8<E5M2>(vals, s, a.qmax));
         }
     }
     if (block_major) {

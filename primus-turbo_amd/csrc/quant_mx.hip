@@ -549,7 +549,7 @@ __global__ __launch_bounds__(256) void mx_quant_rows_kernel(const MxArgs a, cons
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const int64_t n = run[k] * 512 + lane * 8;
-        v[k]            = (u0 + k < total && n < a.N) ? ld128(x + row[k] * a.N + n) : u32x4{0u, 0u, 0u, 0u};
+        v[k]            = (u0 + k < total && n < a.N) ? ld128_nt(x + row[k] * a.N + n) : u32x4{0u, 0u, 0u, 0u};
     }
     uint32_t ebytes = 0; // byte k: the scale byte of this lane's block in run k
 #pragma unroll
@@ -603,12 +603,12 @@ __global__ __launch_bounds__(256) void mx_quant_rows_kernel(const MxArgs a, cons
                 w = c[0];
             }
             if (in)
-                *reinterpret_cast<uint32_t *>(a.row_q + row[k] * (a.Npad >> 1) + (n >> 1)) = w;
+                st32_nt(a.row_q + row[k] * (a.Npad >> 1) + (n >> 1), w);
         } else {
             uint32_t c[2];
             mx_encode<FMT>(f, inv, c, !nan);
             if (in)
-                *reinterpret_cast<u32x2 *>(a.row_q + row[k] * a.Npad + n) = u32x2{c[0], c[1]};
+                st64_nt(a.row_q + row[k] * a.Npad + n, u32x2{c[0], c[1]});
         }
     }
     // lane L < 16 writes scale word L & 3 of run L >> 2: the bytes of the blocks 4 (L & 3) .. + 3 of
