@@ -414,10 +414,16 @@ constexpr int RW_THREADS = 256;
 template <typename T> struct Vec8 {
     static constexpr int DW = 8 * sizeof(T) / 4; // 4 or 8 dwords
     u32x4                v[DW / 4];
+    // (streaming loads: a row is read once, or re-read only when it is longer than the registers hold)
     __device__ __forceinline__ void load(const T *p) {
 #pragma unroll
         for (int i = 0; i < DW / 4; ++i)
-            v[i] = ld128(reinterpret_cast<const char *>(p) + 16 * i);
+            v[i] = ld128_nt(reinterpret_cast<const char *>(p) + 16 * i);
+    }
+    __device__ __forceinline__ void keep_if(bool ok) {
+#pragma unroll
+        for (int i = 0; i < DW / 4; ++i)
+            v[i] = ok ? v[i] : u32x4{0u, 0u, 0u, 0u};
     }
     __device__ __forceinline__ void zero() {
 #pragma unroll
@@ -476,17 +482,19 @@ __global__ __launch_bounds__(RW_THREADS) void quant_rowwise_inner_kernel(
         Vec8<T>       held[HOLD];
         if constexpr (DYNAMIC) {
             float amax = 0.f;
+            // all pieces are requested before the first is used: a piece behind the row's end
+            // re-reads the row's first piece and is zeroed (a branch between the loads would
+            // make each wait for the one before)
 #pragma unroll
             for (int it = 0; it < HOLD; ++it) {
                 const int64_t u = threadIdx.x + it * RW_THREADS;
-                if (u < units)
-                    held[it].load(xr + u * 8);
-                else
-                    held[it].zero();
+                held[it].load(xr + (u < units ? u : 0) * 8);
             }
 #pragma unroll
-            for (int it = 0; it < HOLD; ++it)
+            for (int it = 0; it < HOLD; ++it) {
+                held[it].keep_if(threadIdx.x + it * RW_THREADS < units);
                 amax = fmaxf(amax, held[it].amax());
+            }
             for (int64_t u = threadIdx.x + HOLD * RW_THREADS; u < units; u += RW_THREADS) {
                 Vec8<T> t;
                 t.load(xr + u * 8);
@@ -500,8 +508,7 @@ __global__ __launch_bounds__(RW_THREADS) void quant_rowwise_inner_kernel(
             for (int it = 0; it < HOLD; ++it) {
                 const int64_t u = threadIdx.x + it * RW_THREADS;
                 if (u < units)
-                    *reinterpret_cast<u32x2 *>(qr + u * 8) =
-                        held[it].template quant<E5M2>(scale, qmax);
+                    st64_nt(qr + u * 8, held[it].template quant<E5M2>(scale, qmax));
             }
         } else {
             scale = scale_in[row];
@@ -512,7 +519,7 @@ __global__ __launch_bounds__(RW_THREADS) void quant_rowwise_inner_kernel(
              u += RW_THREADS) {
             Vec8<T> t;
             t.load(xr + u * 8);
-            *reinterpret_cast<u32x2 *>(qr + u * 8) = t.template quant<E5M2>(scale, qmax);
+            st64_nt(qr + u * 8, t.template quant<E5M2>(scale, qmax));
         }
     } else {
         if constexpr (DYNAMIC) {
