@@ -181,6 +181,37 @@ __device__ __forceinline__ float block_max(float v, float *smem) {
 }
 
 // ---------------------------------------------------------------------------
+// Tile order of the tiled quantizers. Workgroups go to the eight XCDs (each with its own L2)
+// round-robin in launch order. The tile grid (gridDim.x by gridDim.y, per blockIdx.z) is walked
+// in blocks of 8 x 8 tiles, and in every aligned run of 512 workgroups each XCD gets one whole
+// block: the 4-byte scale words of eight tiles side by side or on top of each other then fill
+// whole 32-byte units in one L2 instead of leaving eight L2s as masked partial writes. Grids
+// that are no multiple of 8 tiles in a direction keep the launch order, with eight tiles of a
+// row per XCD where that fits.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void xcd_block_tile(uint32_t &tile_x, uint32_t &tile_y) {
+    const uint32_t gx = gridDim.x, gy = gridDim.y, per_z = gx * gy;
+    const uint32_t wg0 = blockIdx.y * gx + blockIdx.x;
+    tile_x = blockIdx.x;
+    tile_y = blockIdx.y;
+    if ((gx & 7) == 0 && (gy & 7) == 0) {
+        uint32_t blk = wg0 >> 6, j = wg0 & 63;
+        if ((wg0 | 511u) < per_z) {
+            const uint32_t r = wg0 & 511u;
+            blk              = ((wg0 >> 9) << 3) + (r & 7u);
+            j                = r >> 3;
+        }
+        const uint32_t nbx = gx >> 3;
+        tile_x             = (blk % nbx) * 8 + (j & 7u);
+        tile_y             = (blk / nbx) * 8 + (j >> 3);
+    } else if ((gx & 7) == 0 && (wg0 | 63u) < per_z) {
+        const uint32_t t = (wg0 & ~63u) + ((wg0 & 7u) << 3) + ((wg0 >> 3) & 7u);
+        tile_x           = t % gx;
+        tile_y           = t / gx;
+    }
+}
+
+// ---------------------------------------------------------------------------
 // 128-bit global memory helpers
 // ---------------------------------------------------------------------------
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));

@@ -183,7 +183,9 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
     const int     tid   = threadIdx.x;
     const int     cseg  = tid & 15; // which 8-column segment of the tile row
     const int     rslot = tid >> 4; // row within a round
-    const int64_t tn = blockIdx.x, tm = blockIdx.y, batch = blockIdx.z;
+    uint32_t tile_x, tile_y; // (tile order: blocks of 8 x 8 tiles per XCD, see xcd_block_tile)
+    xcd_block_tile(tile_x, tile_y);
+    const int64_t tn = tile_x, tm = tile_y, batch = blockIdx.z;
     const int64_t M = a.M, N = a.N;
     const float   qmax = a.qmax;
 

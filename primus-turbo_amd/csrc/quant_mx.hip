@@ -227,8 +227,13 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
     __shared__ float                                 amax_rc[ANY2D ? MX_TILE * 4 : 1]; // [row][32-col block]
     __shared__ __attribute__((aligned(4))) uint8_t   sbytes[MX_TILE * 4]; // E8M0 bytes of the tile, [row or column][block]
     const int     tid = threadIdx.x;
-    const int64_t n0 = static_cast<int64_t>(blockIdx.x) * MX_TILE, m0 = static_cast<int64_t>(blockIdx.y) * MX_TILE;
-    const int64_t b  = blockIdx.z;
+    // (tile order: blocks of 8 x 8 tiles per XCD, see xcd_block_tile)
+    uint32_t tile_x, tile_y;
+    xcd_block_tile(tile_x, tile_y);
+    const uint32_t tile_z = blockIdx.z, gx = gridDim.x, gy = gridDim.y;
+    const uint32_t wg = (tile_z * gy + tile_y) * gx + tile_x; // the tile's number (batch, row tile, column tile)
+    const int64_t  n0 = static_cast<int64_t>(tile_x) * MX_TILE, m0 = static_cast<int64_t>(tile_y) * MX_TILE;
+    const int64_t  b  = tile_z;
     const uint16_t *x = static_cast<const uint16_t *>(a.x) + b * a.M * a.N;
     // tile row r holds input row in_m0 + r (while below in_end) and goes to row row_dst0 + r of
     // the row-direction output (while r < row_cnt: in the padded layout that includes the zero
@@ -410,7 +415,7 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
             uint32_t  code[8];
             if (FMT == MX_E2M1 && (a.sr_mask & 1)) {
                 // a seed per 32-element block: launch seed, tile and task mixed
-                const uint32_t id = (static_cast<uint32_t>(blockIdx.z) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+                const uint32_t id = wg; // the tile's number (batch, row tile, column tile)
                 mx_encode32_fp4_sr(rv[p], mx_inv_scale(e), sr_hash(a.sr_seed ^ (id * 512u + t)), code);
             } else {
                 mx_encode<FMT>(rv[p], mx_inv_scale(e), code, !rnan[p]);
@@ -484,7 +489,7 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
             }
             const int e = mx_exponent<FMT>(am);
             if (FMT == MX_E2M1 && (a.sr_mask & 2)) {
-                const uint32_t id = (static_cast<uint32_t>(blockIdx.z) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+                const uint32_t id = wg; // the tile's number (batch, row tile, column tile)
                 mx_encode32_fp4_sr(v, mx_inv_scale(e), sr_hash(a.sr_seed ^ 0x5BD1E995u ^ (id * 512u + t)), code[p]);
             } else {
                 mx_encode<FMT>(v, mx_inv_scale(e), code[p], !cnan);
