@@ -181,6 +181,25 @@ __device__ __forceinline__ float block_max(float v, float *smem) {
 }
 
 // ---------------------------------------------------------------------------
+// The group g with offs[g] <= pos < offs[g + 1] (offs ascending, G + 1 entries; empty groups are
+// never returned; 0 when no group holds pos). Every lane of the calling wavefront must take part;
+// lane i looks at group i (+ 64, + 128, ...), so the offsets arrive in one round trip per 64
+// groups instead of one per group.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ int find_group(const int64_t *__restrict__ offs, int G, int64_t pos) {
+    const int lane = threadIdx.x & 63;
+    int       g    = 0;
+    for (int base = 0; base < G; base += 64) {
+        const int  i   = base + lane;
+        const bool hit = i < G && pos >= offs[i < G ? i : 0] && pos < offs[i < G ? i + 1 : 1];
+        const unsigned long long m = __ballot(hit);
+        if (m != 0)
+            g = base + __builtin_ctzll(m);
+    }
+    return __builtin_amdgcn_readfirstlane(g);
+}
+
+// ---------------------------------------------------------------------------
 // Tile order of the tiled quantizers. Workgroups go to the eight XCDs (each with its own L2)
 // round-robin in launch order. The tile grid (gridDim.x by gridDim.y, per blockIdx.z) is walked
 // in blocks of 8 x 8 tiles, and in every aligned run of 512 workgroups each XCD gets one whole

@@ -198,10 +198,7 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
         const int64_t pad_start_tile = tm * BQ;
         if (pad_start_tile >= M_out)
             return;
-        int g = 0;
-        for (int i = 0; i < a.num_groups; ++i)
-            if (pad_start_tile >= a.padded_offs[i] && pad_start_tile < a.padded_offs[i + 1])
-                g = i;
+        const int g = find_group(a.padded_offs, a.num_groups, pad_start_tile);
         const int64_t o0 = a.group_offs[g], o1 = a.group_offs[g + 1];
         in_m0  = o0 + (pad_start_tile - a.padded_offs[g]);
         in_end = o1 < M ? o1 : M;

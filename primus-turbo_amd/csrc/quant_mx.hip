@@ -242,10 +242,7 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
     if (a.group_offs != nullptr) {
         if (m0 >= a.col_offs_pad[a.G])
             return;
-        int g = 0;
-        for (int i = 0; i < a.G; ++i)
-            if (m0 >= a.col_offs_pad[i] && m0 < a.col_offs_pad[i + 1])
-                g = i;
+        const int g = find_group(a.col_offs_pad, a.G, m0);
         in_m0    = a.group_offs[g] + (m0 - a.col_offs_pad[g]);
         in_end   = a.group_offs[g + 1];
         const int64_t done = in_m0 - a.group_offs[g]; // rows of the group in earlier tiles
