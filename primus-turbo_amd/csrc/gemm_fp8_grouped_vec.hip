@@ -58,10 +58,7 @@ __global__ __launch_bounds__(256) void transpose_grouped_pad_kernel(const uint8_
     const int64_t       p0 = static_cast<int64_t>(blockIdx.y) * 128, c0 = static_cast<int64_t>(blockIdx.x) * 128;
     if (p0 >= padded[G])
         return;
-    int g = 0;
-    for (int i = 0; i < G; ++i)
-        if (p0 >= padded[i] && p0 < padded[i + 1])
-            g = i;
+    const int g = find_group(padded, G, p0);
     const int64_t in0 = offs[g] + (p0 - padded[g]), in_end = offs[g + 1];
     const int     tid = threadIdx.x;
     const bool    vec = (C & 15) == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0;
@@ -69,14 +66,25 @@ __global__ __launch_bounds__(256) void transpose_grouped_pad_kernel(const uint8_
         const int     cc = tid & 7, rg = tid >> 3;
         const int64_t gc = c0 + cc * 16;
         u32x4         a[4];
+        if (vec) {
+            // the four pieces are requested together (a piece outside the group re-reads the first
+            // bytes of the matrix and is zeroed: no branch between the loads)
+            bool ok[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int64_t gr = in0 + rg * 4 + e;
-            a[e]             = u32x4{0, 0, 0, 0};
-            if (gr < in_end && gc < C) {
-                if (vec) {
-                    a[e] = *reinterpret_cast<const u32x4 *>(in + gr * C + gc);
-                } else {
+            for (int e = 0; e < 4; ++e) {
+                const int64_t gr = in0 + rg * 4 + e;
+                ok[e]            = gr < in_end && gc < C;
+                a[e]             = *reinterpret_cast<const u32x4 *>(in + (ok[e] ? gr * C + gc : 0));
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                a[e] = ok[e] ? a[e] : u32x4{0, 0, 0, 0};
+        } else {
+#pragma unroll 1
+            for (int e = 0; e < 4; ++e) {
+                const int64_t gr = in0 + rg * 4 + e;
+                a[e]             = u32x4{0, 0, 0, 0};
+                if (gr < in_end && gc < C) {
                     uint32_t w[4] = {0, 0, 0, 0};
                     for (int k = 0; k < 16; ++k)
                         if (gc + k < C)
