@@ -65,8 +65,8 @@ __global__ __launch_bounds__(256) void glu_fwd_kernel(const T *__restrict__ x, c
                 float r[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
                 if (live) {
                     float fg[8], fu[8];
-                    unpack8<T>(ld128(g + c), fg);
-                    unpack8<T>(ld128(u + c), fu);
+                    unpack8<T>(ld128_nt(g + c), fg);
+                    unpack8<T>(ld128_nt(u + c), fu);
 #pragma unroll
                     for (int k = 0; k < 8; ++k)
                         r[k] = act_fwd<ACT>(fg[k]) * fu[k] * p;
@@ -98,9 +98,9 @@ __global__ __launch_bounds__(256) void glu_bwd_kernel(const T *__restrict__ grad
                 float rg[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, ru[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
                 if (live) {
                     float fg[8], fu[8], fo[8];
-                    unpack8<T>(ld128(g + c), fg);
-                    unpack8<T>(ld128(u + c), fu);
-                    unpack8<T>(ld128(go + c), fo);
+                    unpack8<T>(ld128_nt(g + c), fg);
+                    unpack8<T>(ld128_nt(u + c), fu);
+                    unpack8<T>(ld128_nt(go + c), fo);
 #pragma unroll
                     for (int k = 0; k < 8; ++k) {
                         float a, da;

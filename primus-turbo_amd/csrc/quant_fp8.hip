@@ -334,6 +334,46 @@ static int launch_quant_tensorwise(const void *x, int64_t n, void *q, const floa
     return check_launch("quant_tensorwise_kernel");
 }
 
+// y[8 u .. 8 u + 7] = T(fp8(q[8 u ..]) * s) for the pieces u = first, first + step, ... below
+// `units`: 8 code bytes in, 16 or 32 bytes out per lane (whole lines per wavefront on both sides),
+// four pieces per round requested together, streaming accesses (nothing here is read twice).
+template <typename T, bool E5M2>
+__device__ __forceinline__ void dequant_pieces8(const uint8_t *__restrict__ q, T *__restrict__ y, const float s,
+                                                const int64_t first, const int64_t step, const int64_t units) {
+    for (int64_t u0 = first; u0 < units; u0 += 4 * step) {
+        u32x2 w[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int64_t u = u0 + k * step;
+            w[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(q + 8 * (u < units ? u : u0)));
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int64_t u = u0 + k * step;
+            if (u >= units)
+                break;
+            const uint32_t ww[2] = {w[k].x, w[k].y};
+            float          f[8];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                f[4 * i + 0] = fp8_to_f32<E5M2>(ww[i], 0) * s;
+                f[4 * i + 1] = fp8_to_f32<E5M2>(ww[i], 1) * s;
+                f[4 * i + 2] = fp8_to_f32<E5M2>(ww[i], 2) * s;
+                f[4 * i + 3] = fp8_to_f32<E5M2>(ww[i], 3) * s;
+            }
+            char *dst = reinterpret_cast<char *>(y + u * 8);
+            if constexpr (sizeof(T) == 4) {
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                    st128_nt(dst + 16 * i, u32x4{__float_as_uint(f[4 * i]), __float_as_uint(f[4 * i + 1]),
+                                                 __float_as_uint(f[4 * i + 2]), __float_as_uint(f[4 * i + 3])});
+            } else {
+                st128_nt(dst, u32x4{pack2<T>(f[0], f[1]), pack2<T>(f[2], f[3]), pack2<T>(f[4], f[5]), pack2<T>(f[6], f[7])});
+            }
+        }
+    }
+}
+
 // ===========================================================================
 // Tensorwise dequantize
 // ===========================================================================
@@ -345,35 +385,9 @@ __global__ __launch_bounds__(256) void dequant_tensorwise_kernel(
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     const int64_t tid0   = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if constexpr (VEC16) {
-        const int64_t units = n / 16;
-        for (int64_t u = tid0; u < units; u += stride) {
-            const u32x4    w     = ld128(q + u * 16);
-            const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
-            float          f[16];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                f[4 * i + 0] = fp8_to_f32<E5M2>(ww[i], 0) * s;
-                f[4 * i + 1] = fp8_to_f32<E5M2>(ww[i], 1) * s;
-                f[4 * i + 2] = fp8_to_f32<E5M2>(ww[i], 2) * s;
-                f[4 * i + 3] = fp8_to_f32<E5M2>(ww[i], 3) * s;
-            }
-            char *dst = reinterpret_cast<char *>(y + u * 16);
-            if constexpr (sizeof(T) == 4) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    st128(dst + 16 * i,
-                          u32x4{__float_as_uint(f[4 * i]), __float_as_uint(f[4 * i + 1]),
-                                __float_as_uint(f[4 * i + 2]), __float_as_uint(f[4 * i + 3])});
-            } else {
-#pragma unroll
-                for (int i = 0; i < 2; ++i)
-                    st128(dst + 16 * i,
-                          u32x4{pack2<T>(f[8 * i], f[8 * i + 1]), pack2<T>(f[8 * i + 2], f[8 * i + 3]),
-                                pack2<T>(f[8 * i + 4], f[8 * i + 5]),
-                                pack2<T>(f[8 * i + 6], f[8 * i + 7])});
-            }
-        }
-        const int64_t tail0 = units * 16;
+        const int64_t units = n / 8;
+        dequant_pieces8<T, E5M2>(q, y, s, tid0, stride, units);
+        const int64_t tail0 = units * 8;
         if (blockIdx.x == 0 && tail0 + threadIdx.x < n)
             y[tail0 + threadIdx.x] =
                 HP<T>::from_f32(fp8_to_f32<E5M2>(q[tail0 + threadIdx.x], 0) * s);
@@ -387,7 +401,7 @@ template <typename T, bool E5M2>
 static int launch_dequant_tensorwise(const void *q, int64_t n, const float *scale_inv, void *y,
                                      hipStream_t stream) {
     const bool    vec   = aligned_to(q, 16) && aligned_to(y, 16);
-    const int64_t units = vec ? n / 16 : n;
+    const int64_t units = vec ? cdiv(n / 8, 4) : n; // work items of a thread: four 8-byte pieces, or one element
     const int     cus   = device_cu_count();
     int64_t       grid  = cdiv(units, 256);
     if (grid < 1)
@@ -699,36 +713,7 @@ __global__ __launch_bounds__(256) void dequant_rowwise_inner_vec_kernel(
     const int64_t inner) {
     const int64_t row   = blockIdx.x;
     const float   s     = scale_inv[row];
-    const int64_t units = inner / 16;
-    const uint8_t *qr   = q + row * inner;
-    T             *yr   = y + row * inner;
-    for (int64_t u = threadIdx.x; u < units; u += 256) {
-        const u32x4    w     = ld128(qr + u * 16);
-        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
-        float          f[16];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            f[4 * i + 0] = fp8_to_f32<E5M2>(ww[i], 0) * s;
-            f[4 * i + 1] = fp8_to_f32<E5M2>(ww[i], 1) * s;
-            f[4 * i + 2] = fp8_to_f32<E5M2>(ww[i], 2) * s;
-            f[4 * i + 3] = fp8_to_f32<E5M2>(ww[i], 3) * s;
-        }
-        char *dst = reinterpret_cast<char *>(yr + u * 16);
-        if constexpr (sizeof(T) == 4) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                st128(dst + 16 * i,
-                      u32x4{__float_as_uint(f[4 * i]), __float_as_uint(f[4 * i + 1]),
-                            __float_as_uint(f[4 * i + 2]), __float_as_uint(f[4 * i + 3])});
-        } else {
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-                st128(dst + 16 * i,
-                      u32x4{pack2<T>(f[8 * i], f[8 * i + 1]), pack2<T>(f[8 * i + 2], f[8 * i + 3]),
-                            pack2<T>(f[8 * i + 4], f[8 * i + 5]),
-                            pack2<T>(f[8 * i + 6], f[8 * i + 7])});
-        }
-    }
+    dequant_pieces8<T, E5M2>(q + row * inner, y + row * inner, s, threadIdx.x, 256, inner / 8);
 }
 
 template <typename T, bool E5M2>
