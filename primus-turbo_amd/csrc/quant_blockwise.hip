@@ -533,7 +533,7 @@ __global__ __launch_bounds__(256) void dequant_block_vec_kernel(
          u += stride) {
         const int64_t  i = u * 16;
         const int64_t  n = i % N, m = (i / N) % M, b = i / (M * N);
-        const u32x4    w = ld128(q + i);
+        const u32x4    w = ld128_nt(q + i);
         const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
         float          f[16];
         if constexpr (PER_COL) { // bn == 1: sixteen different scales
@@ -559,13 +559,13 @@ __global__ __launch_bounds__(256) void dequant_block_vec_kernel(
         if constexpr (sizeof(T) == 4) {
 #pragma unroll
             for (int k = 0; k < 4; ++k)
-                st128(dst + 16 * k,
+                st128_nt(dst + 16 * k,
                       u32x4{__float_as_uint(f[4 * k]), __float_as_uint(f[4 * k + 1]),
                             __float_as_uint(f[4 * k + 2]), __float_as_uint(f[4 * k + 3])});
         } else {
 #pragma unroll
             for (int k = 0; k < 2; ++k)
-                st128(dst + 16 * k,
+                st128_nt(dst + 16 * k,
                       u32x4{pack2<T>(f[8 * k], f[8 * k + 1]), pack2<T>(f[8 * k + 2], f[8 * k + 3]),
                             pack2<T>(f[8 * k + 4], f[8 * k + 5]),
                             pack2<T>(f[8 * k + 6], f[8 * k + 7])});

@@ -804,10 +804,10 @@ __global__ __launch_bounds__(256) void mx_dequant_stream_kernel(const uint8_t *_
             const int64_t r = per_row_shift >= 0 ? u >> per_row_shift : u / per_row, c = u - r * per_row;
             sbyte[k]        = s[r * (cols >> 5) + (c >> 2)];
             if constexpr (FMT == MX_E2M1) {
-                code[k][0] = *reinterpret_cast<const uint32_t *>(q + (u << 2));
+                code[k][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(q + (u << 2)));
                 code[k][1] = 0;
             } else {
-                const u32x2 w = *reinterpret_cast<const u32x2 *>(q + (u << 3));
+                const u32x2 w = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(q + (u << 3)));
                 code[k][0] = w.x, code[k][1] = w.y;
             }
         }
@@ -835,10 +835,10 @@ __global__ __launch_bounds__(256) void mx_dequant_stream_kernel(const uint8_t *_
             if constexpr (sizeof(T) == 4) {
 #pragma unroll
                 for (int i = 0; i < 2; ++i)
-                    st128(dst + 16 * i, u32x4{__float_as_uint(f[4 * i]), __float_as_uint(f[4 * i + 1]),
+                    st128_nt(dst + 16 * i, u32x4{__float_as_uint(f[4 * i]), __float_as_uint(f[4 * i + 1]),
                                               __float_as_uint(f[4 * i + 2]), __float_as_uint(f[4 * i + 3])});
             } else {
-                st128(dst, u32x4{pack2<T>(f[0], f[1]), pack2<T>(f[2], f[3]), pack2<T>(f[4], f[5]), pack2<T>(f[6], f[7])});
+                st128_nt(dst, u32x4{pack2<T>(f[0], f[1]), pack2<T>(f[2], f[3]), pack2<T>(f[4], f[5]), pack2<T>(f[6], f[7])});
             }
         }
     }
