@@ -474,8 +474,8 @@ PT_API int pt_grouped_gemm_fp8_vec_variable_k(const void *lhs, int lhs_dtype, co
  * With q_dtype e2m1x2 it is the grouped MXFP4 quantizer (grouped_quantize_mxfp4[_dual],
  * quantization.cpp:1209-1378; default dispatch flydsl/quantization/mxfp4_grouped_quant.py:320-349):
  * two codes per byte, rows kept tight (row_offs_padded NULL) and column groups padded to 256;
- * row_flags / col_flags / sr_seed as for pt_quantize_mx (bits 1 and 2: grouped data have no 2-D
- * blocks).
+ * row_flags / col_flags / sr_seed as for pt_quantize_mx; a direction's 32 x 32 blocks (bit 0) are
+ * counted from its group's first row, the rows behind the group's end being zeros.
  *
  * pt_grouped_gemm_mx replaces primus_turbo::grouped_gemm_fp8_impl for MX_BLOCKWISE
  * (kernels/grouped_gemm/grouped_gemm_fp8_impl.py:888-930 with group_offs_out; caller

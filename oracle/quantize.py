@@ -372,7 +372,7 @@ def mx_quant_colwise(x: np.ndarray, fmt, use_2d_block: bool = False, pad: int = 
 
 
 def mx_grouped_quant(x: np.ndarray, group_lens: np.ndarray, fmt, row_align: int = 32, col_align: int = 128,
-                     row_rht: bool = False, col_rht: bool = False):
+                     row_rht: bool = False, col_rht: bool = False, row_2d: bool = False, col_2d: bool = False):
     """Grouped MX quantizer of a packed-M activation ``x [M, N]`` (layout rules of
     /root/reference/csrc/pytorch/quantization/quantization.cpp:971-1100 and
     /root/reference/primus_turbo/pytorch/kernels/quantization/quantization_impl.py:572-700:
@@ -380,7 +380,8 @@ def mx_grouped_quant(x: np.ndarray, group_lens: np.ndarray, fmt, row_align: int 
     and to ``col_align`` rows for the column direction; per-block numerics are those of the
     dense MX quantizer; the grouped MXFP4 quantizer, quantization_impl.py:657-811 with the layout
     of /root/reference/primus_turbo/flydsl/quantization/mxfp4_grouped_quant.py:320-349, is
-    ``row_align=1, col_align=256``). Composition of ``mx_quant_rowwise`` / ``mx_quant_colwise`` per group
+    ``row_align=1, col_align=256``; ``row_2d`` / ``col_2d``: 32 x 32 blocks counted from the
+    group's first row, rows behind the group's end being zeros). Composition of ``mx_quant_rowwise`` / ``mx_quant_colwise`` per group
     (pinned there); the padded placement is pinned by the round trip through ``mx_dequant``
     against the dense quantizer of each group.
 
@@ -409,10 +410,15 @@ def mx_grouped_quant(x: np.ndarray, group_lens: np.ndarray, fmt, row_align: int 
         if n == 0:
             continue
         seg = x[offs[g] : offs[g] + n]
-        q, sc = mx_quant_rowwise(seg, fmt, use_rht=row_rht)
-        row[ro[g] : ro[g] + n] = q
-        row_scale[ro[g] : ro[g] + n] = sc
-        q, sc = mx_quant_colwise(seg, fmt, pad=col_align, use_rht=col_rht)
+        # the pad rows are zero rows of the group: code 0 and scale byte 0 with 1-D blocks, the
+        # exponent of their 32 x 32 block with 2-D blocks
+        n_r = int(rl[g])
+        seg_r = np.zeros((n_r, N), dtype=F32)
+        seg_r[:n] = seg
+        q, sc = mx_quant_rowwise(seg_r, fmt, use_2d_block=row_2d, use_rht=row_rht)
+        row[ro[g] : ro[g] + n_r] = q
+        row_scale[ro[g] : ro[g] + n_r] = sc
+        q, sc = mx_quant_colwise(seg, fmt, use_2d_block=col_2d, pad=col_align, use_rht=col_rht)
         col[:, co[g] // cpb : co[g + 1] // cpb] = q
         col_scale[:, co[g] // 32 : co[g + 1] // 32] = sc
     return dict(row=row, row_scale=row_scale, col=col, col_scale=col_scale, row_lens=rl, row_offs=ro, col_lens=cl,

@@ -969,13 +969,13 @@ static int grouped_quantize_mx(const void *x, int x_dtype, const float *probs, c
     PT_REQUIRE(row_q || col_q, "nothing to produce");
     if (const int rc = check_mx_flags(fmt, row_q ? row_flags : 0, col_q ? col_flags : 0))
         return rc;
-    PT_REQUIRE(((row_flags | col_flags) & 1) == 0, "grouped MX quantization has no 2-D blocks");
     const bool rht = (((row_q ? row_flags : 0) | (col_q ? col_flags : 0)) & 2) != 0;
     PT_REQUIRE(col_ld % 128 == 0 && col_ld >= M, "col_ld must be a multiple of 128 that holds every padded group");
     if (glu != 0) {
         PT_REQUIRE(row_q != nullptr, "the gated quantizer produces the row direction (optionally the column direction too)");
         PT_REQUIRE(((row_flags | col_flags) & 4) == 0 && (row_flags & 2) == 0,
                    "the gated quantizer rounds to nearest; only its column direction may be Hadamard-transformed");
+        PT_REQUIRE(((row_flags | col_flags) & 1) == 0, "the gated quantizer has no 2-D blocks");
     }
     if (M == 0 || N == 0)
         return PT_OK;
@@ -1017,9 +1017,9 @@ static int grouped_quantize_mx(const void *x, int x_dtype, const float *probs, c
         else
             launch_mx_rht<f16_t>(a, (row_flags & 2) != 0, (col_flags & 2) != 0, grid, st);
     } else if (x_dtype == PT_DTYPE_BF16) {
-        launch_mx_fmt<bf16_t>(a, fmt, false, false, grid, st);
+        launch_mx_fmt<bf16_t>(a, fmt, row_q && (row_flags & 1), col_q && (col_flags & 1), grid, st);
     } else {
-        launch_mx_fmt<f16_t>(a, fmt, false, false, grid, st);
+        launch_mx_fmt<f16_t>(a, fmt, row_q && (row_flags & 1), col_q && (col_flags & 1), grid, st);
     }
     return check_launch("mx_quant_kernel");
 }

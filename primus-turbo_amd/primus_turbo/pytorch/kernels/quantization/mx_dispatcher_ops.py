@@ -252,8 +252,17 @@ def _grouped_meta(fp4: bool, dual: bool):
         mk = lambda shp, dt: torch.empty(shp, dtype=torch.uint8, device=dev).view(dt)  # noqa: E731
         lens = lambda: torch.empty(G, dtype=torch.int64, device=dev)  # noqa: E731
         offs = lambda: torch.empty(G + 1, dtype=torch.int64, device=dev)  # noqa: E731
-        row = [mk((m_pad_row, n_pad // pack), dest_dtype), mk((m_pad_row, n_pad // 32), _E8M0)]
-        col = [mk((Nn, m_pad_col // pack), dest_dtype), mk((Nn, m_pad_col // 32), _E8M0)]
+        # the shuffle_scale arguments of the MXFP8 schemas (the MXFP4 ones have none)
+        if fp4:
+            shuf_row = shuf_col = False
+        elif dual:
+            shuf_row, shuf_col = (bool(rest[2]) if len(rest) > 2 else False), (bool(rest[4]) if len(rest) > 4 else False)
+        else:
+            shuf_row = shuf_col = bool(rest[3]) if len(rest) > 3 else False
+        rs_shape = Q._scale_pad(m_pad_row, n_pad // 32) if shuf_row else (m_pad_row, n_pad // 32)
+        cs_shape = Q._scale_pad(Nn, m_pad_col // 32) if shuf_col else (Nn, m_pad_col // 32)
+        row = [mk((m_pad_row, n_pad // pack), dest_dtype), mk(rs_shape, _E8M0)]
+        col = [mk((Nn, m_pad_col // pack), dest_dtype), mk(cs_shape, _E8M0)]
         if dual:
             return row + col + [lens(), offs(), lens(), offs()]
         axis = rest[0]

@@ -1377,14 +1377,21 @@ def grouped_quantize_mxfp8_impl(x, out_dtype, axis, block_size, group_lens, grou
     ``M_pad_row`` / ``M_pad_col`` = ``total_M + G * align`` rounded up to ``align``; what lies
     beyond ``offs_padded[G]`` is unspecified."""
     assert block_size == 32, "The block size must be 32 for MXFP8 quantization"
-    for r in (scaling_recipe, scaling_recipe_for_trans):
-        if r is not None and (r.use_2d_block or getattr(r, "shuffle_scale", False) or getattr(r, "shuffle_out", False)):
-            raise NotImplementedError("grouped MXFP8 quantization: 2-D blocks and shuffled layouts are not implemented")
+    r, rt = _mx_recipes(with_trans, scaling_recipe, scaling_recipe_for_trans, "MXFP8")
     if with_trans:
-        return _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, True, True)
+        rq, rs, cq, cs, lr, orow, lc, ocol = _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, True, True,
+                                                                  _mx_flags(r), _mx_flags(rt))
+        rq, rs = _apply_mx_shuffles(rq, rs, r, "rowwise")
+        cq, cs = _apply_mx_shuffles(cq, cs, rt, "colwise")
+        return rq, rs, cq, cs, lr, orow, lc, ocol
     assert axis in (0, 1), "The axis must be 0 or 1"
-    rq, rs, cq, cs, lr, orow, lc, ocol = _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, axis == 1, axis == 0)
-    return (rq, rs, lr, orow) if axis == 1 else (cq, cs, lc, ocol)
+    rq, rs, cq, cs, lr, orow, lc, ocol = _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, axis == 1, axis == 0,
+                                                              _mx_flags(r), _mx_flags(r))
+    if axis == 1:
+        rq, rs = _apply_mx_shuffles(rq, rs, r, "rowwise")
+        return rq, rs, lr, orow
+    cq, cs = _apply_mx_shuffles(cq, cs, r, "colwise")
+    return cq, cs, lc, ocol
 
 
 def grouped_dequantize_mxfp8_impl(x, out_dtype, axis, block_size, scale_inv, group_offs, group_offs_padded,
@@ -1417,18 +1424,23 @@ def grouped_quantize_mxfp4_impl(x, out_dtype, axis, block_size, group_lens, grou
     256 G`` rounded up to 256. Otherwise ``(q, scale, lens_padded, offs_padded)`` of the direction
     ``axis`` asks for (1 = rows, 0 = transposed columns). ``use_rht`` in a recipe applies the fixed
     16-point Hadamard transform along that direction (within each group's padded rows for the
-    column direction), ``use_sr`` rounds the codes stochastically. 2-D blocks and shuffled layouts
-    raise."""
+    column direction), ``use_sr`` rounds the codes stochastically, ``use_2d_block`` shares one
+    exponent per 32 x 32 block counted from the group's first row, ``shuffle_out`` /
+    ``shuffle_scale`` give the pre-shuffled forms of the outputs (a pass over the plain ones)."""
     assert block_size == 32, "The block size must be 32 for MXFP4 quantization"
     assert _FP4X2 is not None and out_dtype == _FP4X2, "The out_dtype must be float4_e2m1fn_x2 for MXFP4 quantization"
-    for r in (scaling_recipe, scaling_recipe_for_trans):
-        if r is not None and (r.use_2d_block or r.shuffle_scale or r.shuffle_out):
-            raise NotImplementedError("grouped MXFP4 quantization: 2-D blocks and shuffled layouts are not implemented")
-    rf = _mx_flags(scaling_recipe)
+    r, rt = _mx_recipes(with_trans, scaling_recipe, scaling_recipe_for_trans, "MXFP4")
     if with_trans:
-        cf = _mx_flags(scaling_recipe_for_trans)
-        return _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, True, True, rf, cf)
+        rq, rs, cq, cs, lr, orow, lc, ocol = _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, True, True,
+                                                                  _mx_flags(r), _mx_flags(rt))
+        rq, rs = _apply_mx_shuffles(rq, rs, r, "rowwise")
+        cq, cs = _apply_mx_shuffles(cq, cs, rt, "colwise")
+        return rq, rs, cq, cs, lr, orow, lc, ocol
     assert axis in (0, 1), "The axis must be 0 (colwise) or 1 (rowwise) when with_trans is False."
     rq, rs, cq, cs, lr, orow, lc, ocol = _grouped_mx_quantize(x, out_dtype, group_lens, group_offs, axis == 1, axis == 0,
-                                                              rf, rf)
-    return (rq, rs, lr, orow) if axis == 1 else (cq, cs, lc, ocol)
+                                                              _mx_flags(r), _mx_flags(r))
+    if axis == 1:
+        rq, rs = _apply_mx_shuffles(rq, rs, r, "rowwise")
+        return rq, rs, lr, orow
+    cq, cs = _apply_mx_shuffles(cq, cs, r, "colwise")
+    return cq, cs, lc, ocol

@@ -78,6 +78,56 @@ def test_grouped_mx_quantizer_bit_exact(kind, G_, M, N, dtype):
         del starts
 
 
+@pytest.mark.parametrize("kind,G_,M,N", [("ragged", 8, 1000, 384), ("zeros", 8, 640, 128), ("zipf", 32, 4096, 512), ("ragged", 3, 77, 96)])
+@pytest.mark.parametrize("row_2d,col_2d", [(True, True), (True, False), (False, True)])
+def test_grouped_mx_quantizer_2d_blocks_bit_exact(kind, G_, M, N, row_2d, col_2d):
+    """32 x 32 blocks in the grouped quantizer: counted from each group's first row (the rows
+    behind a group's end are zeros), one exponent replicated into the scale slot of each row."""
+    lens = group_lens(kind, G_, M, 51)
+    gl, offs = _offs(lens)
+    x = bf16_randn((M, N), seed=52, outlier_frac=0.002)
+    dtype = torch.float8_e4m3fn
+    rq, rs, cq, cs, lr, orow, lc, ocol = qimpl.grouped_quantize_mxfp8_impl(
+        x.cuda(), dtype, None, 32, gl, offs, with_trans=True, scaling_recipe=ScalingRecipe(use_2d_block=row_2d),
+        scaling_recipe_for_trans=ScalingRecipe(use_2d_block=col_2d))
+    o = Q.mx_grouped_quant(x.float().numpy(), lens, "e4m3", row_2d=row_2d, col_2d=col_2d)
+    mr, mc = int(o["row_offs"][-1]), int(o["col_offs"][-1])
+    assert np.array_equal(codes_np(rs)[:mr], o["row_scale"]) and np.array_equal(codes_np(rq)[:mr], o["row"])
+    assert np.array_equal(codes_np(cs)[:, : mc // 32], o["col_scale"]) and np.array_equal(codes_np(cq)[:, :mc], o["col"])
+    # one direction alone gives the same tensors
+    q1, s1, _, _ = qimpl.grouped_quantize_mxfp8_impl(x.cuda(), dtype, 1, 32, gl, offs, scaling_recipe=ScalingRecipe(use_2d_block=row_2d))
+    q0, s0, _, _ = qimpl.grouped_quantize_mxfp8_impl(x.cuda(), dtype, 0, 32, gl, offs, scaling_recipe=ScalingRecipe(use_2d_block=col_2d))
+    assert np.array_equal(codes_np(q1)[:mr], o["row"]) and np.array_equal(codes_np(s1)[:mr], o["row_scale"])
+    assert np.array_equal(codes_np(q0)[:, :mc], o["col"]) and np.array_equal(codes_np(s0)[:, : mc // 32], o["col_scale"])
+
+
+def test_grouped_mx_quantizer_shuffled_outputs():
+    """``shuffle_out`` / ``shuffle_scale`` in the grouped quantizer: the pre-shuffled forms of the
+    plain outputs (the same pass as behind the dense quantizers), undone by the inverse ops."""
+    lens = group_lens("ragged", 8, 1000, 53)
+    gl, offs = _offs(lens)
+    x = bf16_randn((1000, 384), seed=54).cuda()
+    dtype = torch.float8_e4m3fn
+    plain = qimpl.grouped_quantize_mxfp8_impl(x, dtype, None, 32, gl, offs, with_trans=True)
+    rec = ScalingRecipe(shuffle_scale=True, shuffle_out=True)
+    shuf = qimpl.grouped_quantize_mxfp8_impl(x, dtype, None, 32, gl, offs, with_trans=True, scaling_recipe=rec,
+                                             scaling_recipe_for_trans=rec)
+    mr, mc = int(plain[5][-1]), int(plain[7][-1])
+    for qi_, si_, rows in ((0, 1, mr), (2, 3, 384)):
+        q, s = shuf[qi_], shuf[si_]
+        assert q.shape == plain[qi_].shape and s.shape[0] % 256 == 0 and s.shape[1] % 8 == 0
+        assert not torch.equal(q.view(torch.uint8), plain[qi_].view(torch.uint8))
+        back, sback = qimpl.mx_plain_layout(q, s, True, True)
+        back = back.view(torch.uint8)
+        if qi_ == 0:
+            assert torch.equal(back[:rows], plain[0].view(torch.uint8)[:rows])
+            assert torch.equal(sback.view(torch.uint8)[:rows], plain[1].view(torch.uint8)[:rows])
+        else:
+            assert torch.equal(back[:, :mc], plain[2].view(torch.uint8)[:, :mc])
+            assert torch.equal(sback.view(torch.uint8)[:, : mc // 32], plain[3].view(torch.uint8)[:, : mc // 32])
+    assert all(torch.equal(a, b) for a, b in zip(shuf[4:], plain[4:]))
+
+
 GCASES = [("balanced", 4, 1024, 512, 512), ("ragged", 8, 3000, 384, 1024), ("zeros", 8, 2048, 256, 512),
           ("zipf", 32, 8192, 1024, 768), ("ragged", 3, 77, 96, 640), ("zipf", 16, 4096, 2048, 512)]
 

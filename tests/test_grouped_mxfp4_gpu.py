@@ -72,6 +72,23 @@ def test_grouped_mxfp4_quantizer_bit_exact(kind, G_, M, N, dtype):
     assert torch.equal(o1, offs) and torch.equal(o0, ocol) and torch.equal(l1, gl) and torch.equal(l0, lc)
 
 
+@pytest.mark.parametrize("kind,G_,M,N", [("ragged", 8, 1000, 384), ("zeros", 8, 640, 128), ("ragged", 3, 77, 96)])
+def test_grouped_mxfp4_quantizer_2d_blocks_bit_exact(kind, G_, M, N):
+    """32 x 32 blocks in the grouped MXFP4 quantizer, counted from each group's first row (row
+    direction: rows stay where they are; column direction: groups padded to 256)."""
+    lens = group_lens(kind, G_, M, 63)
+    gl, offs = _offs(lens)
+    x = bf16_randn((M, N), seed=64, outlier_frac=0.002)
+    rec = ScalingRecipe(use_2d_block=True)
+    rq, rs, cq, cs, _, _, _, ocol = qimpl.grouped_quantize_mxfp4_impl(x.cuda(), FP4, None, 32, gl, offs, with_trans=True,
+                                                                      scaling_recipe=rec, scaling_recipe_for_trans=rec)
+    o = Q.mx_grouped_quant(to_f32_np(x), lens, "e2m1", row_align=1, col_align=256, row_2d=True, col_2d=True)
+    mc = int(o["col_offs"][-1])
+    assert np.array_equal(ocol.cpu().numpy(), o["col_offs"])
+    assert np.array_equal(codes_np(rs), o["row_scale"]) and np.array_equal(codes_np(rq), o["row"])
+    assert np.array_equal(codes_np(cs)[:, : mc // 32], o["col_scale"]) and np.array_equal(codes_np(cq)[:, : mc // 2], o["col"])
+
+
 # (kind, G, M, N, K): includes N / K that are multiples of 32 only and K below four slabs
 GCASES = [("balanced", 4, 1024, 512, 1024), ("ragged", 8, 3000, 384, 2048), ("zeros", 8, 2048, 256, 1024),
           ("zipf", 32, 8192, 1024, 1536), ("ragged", 3, 77, 96, 160), ("zipf", 16, 4096, 2048, 1408),
@@ -211,9 +228,9 @@ def test_grouped_quantize_fp4_ops_surface():
     mc = int(oc[-1])  # what lies beyond the last padded group is unspecified
     assert torch.equal(out[7], oc) and torch.equal(out[2].view(torch.uint8)[:, : mc // 2], qc.view(torch.uint8)[:, : mc // 2])
     assert int(oc[-1]) % 256 == 0 and bool((lc % 256 == 0).all())
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(NotImplementedError):  # the Hadamard transform is not combined with 2-D blocks
         turbo.ops.grouped_quantize_fp4(x, FP4, G.MX_BLOCKWISE, gl, offs, block_size=32, axis=1,
-                                       scaling_recipe=ScalingRecipe(use_2d_block=True))
+                                       scaling_recipe=ScalingRecipe(use_2d_block=True, use_rht=True))
 
 
 @pytest.mark.parametrize("kind,G_,M,N", [("ragged", 8, 1000, 384), ("zeros", 8, 640, 128), ("zipf", 32, 4096, 512),

@@ -18,8 +18,9 @@ E8 = getattr(torch, "float8_e8m0fnu", torch.uint8)
 
 @pytest.fixture(scope="module", autouse=True)
 def _ext(native_lib):
-    global ext
+    global ext, Qi
     import primus_turbo.pytorch  # noqa: F401  (registers the operators)
+    from primus_turbo.pytorch.kernels.quantization import quantization_impl as Qi
 
     ext = torch.ops.primus_turbo_cpp_extension
 
@@ -121,8 +122,19 @@ def test_grouped_quantize_mxfp8_names():
     src = np.concatenate([np.arange(lens[g]) + offs_r[g] for g in range(G_)]).astype(np.int64)
     assert np.array_equal(y.cpu().numpy(), ref[src][:, :N])
     _same_meta(ext.grouped_dequantize_mxfp8, (rq, rs, offs, orow, 1, 32, torch.float32, M), y)
-    with pytest.raises(NotImplementedError):
-        ext.grouped_quantize_mxfp8(x, gl, offs, dt, 1, 128, True)  # 2-D blocks: dense quantizers only
+    # 2-D blocks and the pre-shuffled forms, by the reference's argument names
+    want2 = Q.mx_grouped_quant(to_f32_np(x), lens, "e4m3", row_2d=True, col_2d=True)
+    two = ext.grouped_quantize_mxfp8(x, gl, offs, dt, 1, 128, True)
+    assert np.array_equal(codes_np(two[0])[:nr], want2["row"][:nr]) and np.array_equal(codes_np(two[1])[:nr], want2["row_scale"][:nr])
+    _same_meta(ext.grouped_quantize_mxfp8, (x, gl, offs, dt, 1, 128, True), two)
+    shuf = ext.grouped_quantize_mxfp8_dual(x, gl, offs, dt, False, True, True, True, True, False)
+    back, sback = Qi.mx_plain_layout(shuf[0], shuf[1], True, True)
+    assert torch.equal(back.view(torch.uint8)[:nr], rq.view(torch.uint8)[:nr])
+    assert torch.equal(sback.view(torch.uint8)[:nr], rs.view(torch.uint8)[:nr])
+    assert np.array_equal(codes_np(shuf[2])[:, :nc], want2["col"][:, :nc])  # column codes: 2-D blocks, not shuffled
+    assert np.array_equal(codes_np(ext.unshuffle_scale(shuf[3], cs.shape[0], cs.shape[1]))[:, : nc // 32],
+                          want2["col_scale"][:, : nc // 32])
+    _same_meta(ext.grouped_quantize_mxfp8_dual, (x, gl, offs, dt, False, True, True, True, True, False), shuf)
 
 
 @pytest.mark.skipif(F4 is None, reason="torch without float4_e2m1fn_x2")

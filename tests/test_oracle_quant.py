@@ -277,6 +277,32 @@ def test_mx_grouped_layout(lens, fmt, ra, ca):
         assert not o["col_scale"][:, (c0 + n + 31) // 32 : c1 // 32].any()
 
 
+def test_mx_grouped_2d_blocks():
+    """32 x 32 blocks in the grouped quantizer are counted from each group's first row: a group's
+    slice equals the dense 2-D quantizer of that group's rows, its pad rows are zero codes that
+    carry the exponent of their block, and every block de-quantizes with one exponent."""
+    lens = np.array([40, 0, 64, 7], dtype=np.int64)
+    M, N = int(lens.sum()), 96
+    rng = np.random.default_rng(6)
+    x = (rng.standard_normal((M, N)) * np.exp(rng.standard_normal((M, 1)))).astype(np.float32)
+    o = Q.mx_grouped_quant(x, lens, "e4m3", row_2d=True, col_2d=True)
+    starts = np.concatenate([[0], np.cumsum(lens)])
+    for g, n in enumerate(lens):
+        if n == 0:
+            continue
+        r0, r1, c0 = o["row_offs"][g], o["row_offs"][g + 1], o["col_offs"][g]
+        seg = x[starts[g] : starts[g] + n]
+        q, s = Q.mx_quant_rowwise(seg, "e4m3", True)
+        assert np.array_equal(o["row"][r0 : r0 + n], q) and np.array_equal(o["row_scale"][r0 : r0 + n], s)
+        assert not o["row"][r0 + n : r1].any()
+        blk = o["row_scale"][r0:r1].reshape((r1 - r0) // 32, 32, -1)
+        assert np.all(blk == blk[:, :1]), "one exponent per 32 x 32 block, pad rows included"
+        qc, sc = Q.mx_quant_colwise(seg, "e4m3", True)
+        assert np.array_equal(o["col"][:, c0 : c0 + qc.shape[1]], qc) and np.array_equal(o["col_scale"][:, c0 // 32 : c0 // 32 + sc.shape[1]], sc)
+        # the exponent of a block is that of its abs-max: the row and the column direction agree on it
+        assert np.array_equal(s[::32, : N // 32], sc[::32, : -(-n // 32)].T[: -(-n // 32)][:, : N // 32])
+
+
 def test_hadamard16_is_the_orthonormal_sylvester_matrix():
     """``hadamard16`` against scipy's Sylvester construction where fp32 arithmetic is exact (small
     integers), its involution, norm preservation, and what the recipe relies on: the transform
