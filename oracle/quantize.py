@@ -39,7 +39,10 @@ What each function follows, and what pins it (tests/test_oracle_*.py):
   /root/reference/csrc/pytorch/quantization/quantization.cpp:971-1100 (rows of a group padded
   to 32 / 128 with zero data); pinned by the group-by-group round trip against the dense
   quantizer and by the zero-pad invariants (same PARITY UNPINNED remark for bit-identity
-  with the reference's own kernels).
+  with the reference's own kernels). Its 2-D blocks are counted from each group's first row,
+  pad rows carrying their block's exponent: the reference's grouped kernels are absent, so
+  this placement is PARITY UNPINNED; pinned is that each group's slice equals the dense 2-D
+  quantizer of that group's rows.
 """
 
 from __future__ import annotations
