@@ -251,6 +251,9 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
     }
 
     PT_MX_TRACE(0);
+    // (the row direction is taken from the registers of the loads where that is possible)
+    constexpr bool EARLY_ROW = ROW && !ANY2D && (RHT & 1) == 0;
+    bool           row_done  = false;
     // ---- tile -> LDS (zeros outside the matrix) ----
     // Whole 16-byte pieces (the common case) are all requested before the first is used: a piece
     // outside the matrix reads the matrix's first bytes instead and is replaced by zeros, so that
@@ -307,9 +310,75 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
             }
         }
 #pragma unroll
-        for (int p = 0; p < 8; ++p) {
-            const int r = p * 16 + (tid >> 4), c = (tid & 15) * 8;
-            *reinterpret_cast<u32x4 *>(&tile[r * MX_PITCH + c]) = inside[p] ? piece[p] : u32x4{0u, 0u, 0u, 0u};
+        for (int p = 0; p < 8; ++p)
+            piece[p] = inside[p] ? piece[p] : u32x4{0u, 0u, 0u, 0u};
+        // The row direction with 1-D blocks needs no transposition: it is encoded straight from the
+        // registers the loads arrived in (a lane holds a quarter of a block, the block's abs-max is
+        // a reduction over four neighbouring lanes), 8 code bytes per lane and 128 per row segment.
+        if constexpr (EARLY_ROW) {
+#pragma unroll
+            for (int p = 0; p < 8; ++p) {
+                const int      r = p * 16 + (tid >> 4), cb = (tid & 15) >> 2; // tile row, 32-column block
+                const uint32_t ww[4] = {piece[p].x, piece[p].y, piece[p].z, piece[p].w};
+                float          f[8];
+                uint32_t       m2 = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    unpack2<T>(ww[i], f[2 * i], f[2 * i + 1]);
+                    m2 = pk_absmax16(m2, ww[i]);
+                }
+                uint32_t m16 = max(m2 & 0xffffu, m2 >> 16);
+                m16          = max(m16, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, m16, 0xB1, 0xf, 0xf, true)));
+                m16          = max(m16, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, m16, 0x4E, 0xf, 0xf, true)));
+                const bool nan = m16 > Bits16<T>::INF; // somewhere in the block
+                float      am  = Bits16<T>::to_f32(m16);
+                if (nan) {
+                    am = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i)
+                        am = fmaxf(am, abs_or_zero(f[i]));
+                    am = fmaxf(am, dpp_f32<0xB1>(am));
+                    am = fmaxf(am, dpp_f32<0x4E>(am));
+                }
+                const int   e   = mx_exponent<FMT>(am);
+                const float inv = mx_inv_scale(e);
+                if ((tid & 3) == 0)
+                    sbytes[r * 4 + cb] = static_cast<uint8_t>(e + 127);
+                const int64_t n = n0 + (tid & 15) * 8;
+                if constexpr (FMT == MX_E2M1) {
+                    uint32_t w = 0;
+                    if (a.sr_mask & 1) {
+                        // the seeds of the LDS row pass: task 4 r + cb of this tile, one step per pair
+                        constexpr float Q = MxFmt<MX_E2M1>::QMAX;
+                        uint32_t seed = sr_hash(a.sr_seed ^ (wg * 512u + static_cast<uint32_t>(r * 4 + cb))) + 4u * (tid & 3) * 0x9E3779B9u;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const f32x2_t pair = {scale_clamp(f[2 * i], inv, Q), scale_clamp(f[2 * i + 1], inv, Q)};
+                            seed += 0x9E3779B9u;
+                            w |= (__builtin_amdgcn_cvt_scalef32_sr_pk_fp4_f32(0u, pair, seed, 1.0f, 0) & 0xffu) << (8 * i);
+                        }
+                    } else {
+                        uint32_t c[1];
+                        mx_encode<FMT>(f, inv, c, !nan);
+                        w = c[0];
+                    }
+                    if (r < row_cnt)
+                        *reinterpret_cast<uint32_t *>(a.row_q + (row_dst0 + r) * (a.Npad >> 1) + (n >> 1)) = w;
+                } else {
+                    uint32_t c[2];
+                    mx_encode<FMT>(f, inv, c, !nan);
+                    if (r < row_cnt)
+                        *reinterpret_cast<u32x2 *>(a.row_q + (row_dst0 + r) * a.Npad + n) = u32x2{c[0], c[1]};
+                }
+            }
+            row_done = true;
+        }
+        if constexpr (COL || !EARLY_ROW) {
+#pragma unroll
+            for (int p = 0; p < 8; ++p) {
+                const int r = p * 16 + (tid >> 4), c = (tid & 15) * 8;
+                *reinterpret_cast<u32x4 *>(&tile[r * MX_PITCH + c]) = piece[p];
+            }
         }
     } else {
 #pragma unroll 1
@@ -361,6 +430,7 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
     float ram[2];
     bool  rnan[2] = {true, true}; // false: the task's 32 input values are known to hold no NaN
     if constexpr (ROW || ANY2D) {
+        if (!row_done) {
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
             const int t = tid + 256 * p, r = t >> 2, c = t & 3;
@@ -393,10 +463,12 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
             if constexpr (ANY2D)
                 amax_rc[r * 4 + c] = am;
         }
+        } // the row pass through the LDS
     }
     if constexpr (ANY2D)
         __syncthreads();
     if constexpr (ROW) {
+        if (!row_done) {
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
             const int     t = tid + 256 * p, r = t >> 2, c = t & 3;
@@ -431,6 +503,7 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
             }
         }
         __syncthreads();
+        } // the row pass through the LDS
         // the four scale bytes of a tile row leave as one word (Npad / 32 is a multiple of 4)
         if (tid < MX_TILE && tid < row_cnt)
             *reinterpret_cast<uint32_t *>(a.row_s + (row_dst0 + tid) * (a.Npad >> 5) + (n0 >> 5)) =
