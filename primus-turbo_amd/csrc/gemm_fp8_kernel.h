@@ -808,6 +808,13 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
         for (int i = 0; i < TM; ++i)
             fa[i] = ldfrag(smem + a_part, i);
     };
+    // Stores of the result tile a wavefront has just written that may still be in flight (0, or the
+    // count of the straight-line epilogue for 16-bit / fp32 outputs). They are younger than the
+    // copies the first slab of the next tile waits for and older than that slab's own copies;
+    // memory operations retire in order, so the first slab's waits leave that many more
+    // operations outstanding instead of waiting for the stores to be acknowledged.
+    constexpr int ST16 = TM * TN / 2, ST32 = TM * TN;
+    int           pending = 0;
     PT_GEMM_TRACE_DECL;
     PT_GEMM_TRACE_POINT(0);
     if constexpr (XPIPE) {
@@ -937,14 +944,53 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                     // my reads of the current stage are done (they were issued a column ago) and my
                     // copies of the next slab's B part have landed; younger copies may be in flight
                     PT_GEMM_TRACE_POINT(2);
-                    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LA + issued_before(COL)) : "memory");
+                    // (the case distinction on `pending` lives inside the asm statement so that the
+                    // slab stays one basic block for the compiler; the counter field holds 63 at most)
+                    {
+                        constexpr int W = LA + issued_before(COL);
+                        asm volatile("s_cmp_eq_u32 %0, 0\n\t"
+                                     "s_cbranch_scc1 .Lx0_%=\n\t"
+                                     "s_cmp_eq_u32 %0, %4\n\t"
+                                     "s_cbranch_scc1 .Lx16_%=\n\t"
+                                     "s_waitcnt vmcnt(%3) lgkmcnt(0)\n\t"
+                                     "s_branch .Lxe_%=\n"
+                                     ".Lx16_%=:\n\t"
+                                     "s_waitcnt vmcnt(%2) lgkmcnt(0)\n\t"
+                                     "s_branch .Lxe_%=\n"
+                                     ".Lx0_%=:\n\t"
+                                     "s_waitcnt vmcnt(%1) lgkmcnt(0)\n"
+                                     ".Lxe_%=:"
+                                     :
+                                     : "s"(pending), "n"(W), "n"(W + ST16 > 63 ? 63 : W + ST16),
+                                       "n"(W + ST32 > 63 ? 63 : W + ST32), "n"(ST16)
+                                     : "memory", "scc");
+                    }
                     __builtin_amdgcn_s_barrier();
                     PT_GEMM_TRACE_POINT(3);
                     read_scales(nxt);
                 }
                 if constexpr (j == JY - 1) {
                     // ---- barrier Y: the next slab's A part has landed ----
-                    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(issued_before(JY * COL)) : "memory");
+                    {
+                        constexpr int W = issued_before(JY * COL);
+                        asm volatile("s_cmp_eq_u32 %0, 0\n\t"
+                                     "s_cbranch_scc1 .Ly0_%=\n\t"
+                                     "s_cmp_eq_u32 %0, %4\n\t"
+                                     "s_cbranch_scc1 .Ly16_%=\n\t"
+                                     "s_waitcnt vmcnt(%3)\n\t"
+                                     "s_branch .Lye_%=\n"
+                                     ".Ly16_%=:\n\t"
+                                     "s_waitcnt vmcnt(%2)\n\t"
+                                     "s_branch .Lye_%=\n"
+                                     ".Ly0_%=:\n\t"
+                                     "s_waitcnt vmcnt(%1)\n"
+                                     ".Lye_%=:"
+                                     :
+                                     : "s"(pending), "n"(W), "n"(W + ST16 > 63 ? 63 : W + ST16),
+                                       "n"(W + ST32 > 63 ? 63 : W + ST32), "n"(ST16)
+                                     : "memory", "scc");
+                    }
+                    pending = 0; // from the next slab on every wait is for copies younger than the stores
                     __builtin_amdgcn_s_barrier();
                 }
                 fb[j] = ldfrag(nxt + b_part, j); // column j is done: refill from the next slab
@@ -970,6 +1016,10 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             PT_GEMM_TRACE_POINT(5);
             epilogue<TM, TN, MODE, MODE != SCALE_BLOCK>(a, acc, cur_t.C, cur_t.sA, cur_t.sB, cur_t.m_end, wm_base, wn_base,
                                                          lane);
+            // (the same test as the epilogue's: its straight-line path issues exactly this many stores)
+            const bool fast = wm_base + TM * 16 <= cur_t.m_end && wn_base + TN * 16 <= a.N && (a.N & 7) == 0 &&
+                              (reinterpret_cast<uintptr_t>(cur_t.C) & 15) == 0;
+            pending = __builtin_amdgcn_readfirstlane(fast ? (a.out_dtype == PT_DTYPE_F32 ? ST32 : ST16) : 0);
         } else {
             const int ES     = a.out_dtype == PT_DTYPE_F32 ? 4 : 2;
             int64_t   g_lo   = a.group_offs[cur_t.g0] >> (F4 ? 1 : 0);
