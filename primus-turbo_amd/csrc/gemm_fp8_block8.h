@@ -196,13 +196,23 @@ __global__ __launch_bounds__(B8_THREADS) void gemm_fp8_block8_kernel(const GemmA
     const uint32_t a_part = wm * (TM * 16) * KSTEP;
     const uint32_t b_part = A_BYTES + wn * (TN * 16) * KSTEP;
 
-    // ---- pipeline start: slab 0 whole, first part of slab 1 ----
+    // ---- pipeline start: slabs 0 and 1 ----
+    // (the loader steps past slab 1 here: with two slabs per tile that is the next tile already)
+    if (tile + static_cast<int>(gridDim.x) < total)
+        nxt_t = make_tile<BM, BN, GMODE>(a, tile + gridDim.x, prefix, g_nxt);
     loader_to(cur_t);
     static_for<0, NL>([&](auto c) { issue_nth(c, 0); });
     advance_loader();
-    static_for<0, B8_P1>([&](auto c) { issue_nth(c, 1); });
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(B8_P1) : "memory");
+    static_for<0, NL>([&](auto c) { issue_nth(c, 1); });
+    advance_loader();
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
     __builtin_amdgcn_s_barrier();
+    // Stores of the result tile this wavefront has just written that may still be in flight (0, or
+    // the count of the epilogue's straight-line path). All copies of a slab are issued a slab
+    // ahead, so behind an epilogue those stores are the only memory operations younger than the
+    // copies the next barrier waits for: memory operations retire in order, and leaving that many
+    // outstanding waits for the copies without waiting for the stores to be acknowledged.
+    int pending = 0;
     read_scales(smem);
 #pragma unroll
     for (int j = 0; j < TN; ++j)
@@ -245,7 +255,24 @@ __global__ __launch_bounds__(B8_THREADS) void gemm_fp8_block8_kernel(const GemmA
                 if constexpr (i == 6) {
                     // ---- the slab's barrier: my copies of the next slab have landed (nothing
                     // younger is in flight) and my reads of the current stage are complete ----
-                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                    // (the case distinction lives inside the asm statement so that the slab stays
+                    // one basic block for the compiler)
+                    asm volatile("s_cmp_eq_u32 %0, 16\n\t"
+                                 "s_cbranch_scc1 .Lb16_%=\n\t"
+                                 "s_cmp_eq_u32 %0, 32\n\t"
+                                 "s_cbranch_scc1 .Lb32_%=\n\t"
+                                 "s_waitcnt vmcnt(0) lgkmcnt(0)\n\t"
+                                 "s_branch .Lbend_%=\n"
+                                 ".Lb16_%=:\n\t"
+                                 "s_waitcnt vmcnt(16) lgkmcnt(0)\n\t"
+                                 "s_branch .Lbend_%=\n"
+                                 ".Lb32_%=:\n\t"
+                                 "s_waitcnt vmcnt(32) lgkmcnt(0)\n"
+                                 ".Lbend_%=:"
+                                 :
+                                 : "s"(pending)
+                                 : "memory", "scc");
+                    pending = 0;
                     __builtin_amdgcn_s_barrier();
                     read_scales(nxt);
                 }
@@ -263,20 +290,18 @@ __global__ __launch_bounds__(B8_THREADS) void gemm_fp8_block8_kernel(const GemmA
                     __builtin_amdgcn_sched_barrier(0);
                     if constexpr (i == TM - 1)
                         fb[j] = ldfrag(nxt + b_part, j); // dead from here on: refill from the next slab
-                    // second part (A rows) of the next slab's copies: row groups 0..3, into the next stage
-                    if constexpr (i < LA && j == 1)
-                        issue_nth(std::integral_constant<int, B8_P1 + i>{}, buf ^ 1);
-                    // first part (B rows, scales) of the slab after next: row groups 6 and 7, into the
-                    // stage the barrier has just freed
+                    // all copies of the slab after next: row groups 6 and 7, into the stage the
+                    // barrier has just freed (nine copies in eight MFMA slots)
                     if constexpr (i >= 6) {
                         constexpr int s = (i - 6) * TN + j; // 0..7
-                        if constexpr (s >= 1 && s <= B8_P1)
-                            issue_nth(std::integral_constant<int, s - 1>{}, buf);
+                        issue_nth(std::integral_constant<int, s>{}, buf);
+                        if constexpr (s == 7) {
+                            issue_nth(std::integral_constant<int, 8>{}, buf);
+                            advance_loader();
+                        }
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 });
-                if constexpr (i == LA)
-                    advance_loader(); // the next slab is requested in full: on to the one after
             });
 #pragma unroll
             for (int t = TILES - DEPTH; t < TILES; ++t)
@@ -286,6 +311,13 @@ __global__ __launch_bounds__(B8_THREADS) void gemm_fp8_block8_kernel(const GemmA
 
         const int64_t wm_base = cur_t.m0 + wm * (TM * 16), wn_base = cur_t.n0 + wn * (TN * 16);
         epilogue<TM, TN, SCALE_BLOCK, false>(a, acc, cur_t.C, cur_t.sA, cur_t.sB, cur_t.m_end, wm_base, wn_base, lane);
+        // the straight-line store path (the condition of `epilogue`) issues one 16-byte store per pair
+        // of MFMA tiles (16-bit outputs) or per tile (fp32); other paths are not counted on
+        {
+            const bool fast = wm_base + TM * 16 <= cur_t.m_end && wn_base + TN * 16 <= a.N && (a.N & 7) == 0 &&
+                              (reinterpret_cast<uintptr_t>(cur_t.C) & 15) == 0;
+            pending = __builtin_amdgcn_readfirstlane(fast ? (a.out_dtype == PT_DTYPE_F32 ? TM * TN : TM * TN / 2) : 0);
+        }
 
         if (next_tile >= total)
             break;
