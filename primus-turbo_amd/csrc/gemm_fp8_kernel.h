@@ -946,7 +946,11 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                     PT_GEMM_TRACE_POINT(2);
                     // (the case distinction on `pending` lives inside the asm statement so that the
                     // slab stays one basic block for the compiler; the counter field holds 63 at most)
-                    {
+                    if constexpr (GMODE == GROUP_NONE) {
+                        // (dense problems: few tiles per workgroup, and the case distinction costs
+                        // about 1 % of a long K loop: the plain wait)
+                        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LA + issued_before(COL)) : "memory");
+                    } else {
                         constexpr int W = LA + issued_before(COL);
                         asm volatile("s_cmp_eq_u32 %0, 0\n\t"
                                      "s_cbranch_scc1 .Lx0_%=\n\t"
@@ -971,7 +975,9 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                 }
                 if constexpr (j == JY - 1) {
                     // ---- barrier Y: the next slab's A part has landed ----
-                    {
+                    if constexpr (GMODE == GROUP_NONE) {
+                        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(issued_before(JY * COL)) : "memory");
+                    } else {
                         constexpr int W = issued_before(JY * COL);
                         asm volatile("s_cmp_eq_u32 %0, 0\n\t"
                                      "s_cbranch_scc1 .Ly0_%=\n\t"
