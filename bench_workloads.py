@@ -22,23 +22,23 @@ FP4_PEAK_TFLOPS = 10100.0
 # 256 MiB launched in the same run (`bench.py --calib-copy`; factors 2.000 and 1.000); the runs are
 # summarised under profiles/. (fetched, written) in MiB.
 TRAFFIC_MIB = {
-    "gemm_fp8_rowwise": (777.2, 151.2),
-    "gemm_fp8_blockwise": (347.3, 226.1),
-    "gemm_fp8_blockwise_k7168": (690.9, 128.7),
-    "gemm_fp8_blockwise_8192": (788.6, 129.4),
-    "gemm_mxfp4": (3270.4, 522.4),
-    "gemm_mxfp8": (6362.4, 578.6),
-    "gemm_mxfp4_n28672": (1433.9, 455.2),
-    "gemm_mxfp8_n28672": (2779.3, 448.0),
+    "gemm_fp8_rowwise": (777.2, 151.0),
+    "gemm_fp8_blockwise": (349.4, 225.9),
+    "gemm_fp8_blockwise_k7168": (696.1, 129.0),
+    "gemm_fp8_blockwise_8192": (799.3, 136.3),
+    "gemm_mxfp4": (3270.7, 522.8),
+    "gemm_mxfp8": (6358.4, 572.4),
+    "gemm_mxfp4_n28672": (1434.2, 455.4),
+    "gemm_mxfp8_n28672": (2780.0, 448.0),
     # grouped workloads, forward launch: the fetch figure is the average over the forward and dgrad
     # launches of the one kernel symbol that runs both (the counters cannot tell them apart), the
     # write figure is the forward launches' own (they differ from dgrad's by the output width)
-    "grouped_gemm_fp8": (4815.6, 256.5),
-    "grouped_gemm_fp8_down": (2374.5, 449.3),
-    "grouped_gemm_mxfp8": (5506.2, 256.0),
-    "grouped_gemm_mxfp8_down": (2713.4, 448.0),
-    "grouped_gemm_mxfp4": (2769.0, 256.0),
-    "grouped_gemm_mxfp4_down": (1354.5, 448.0),
+    "grouped_gemm_fp8": (4658.7, 256.3),
+    "grouped_gemm_fp8_down": (2411.5, 448.8),
+    "grouped_gemm_mxfp8": (5354.7, 256.0),
+    "grouped_gemm_mxfp8_down": (2650.7, 448.0),
+    "grouped_gemm_mxfp4": (2752.2, 256.0),
+    "grouped_gemm_mxfp4_down": (1345.3, 448.0),
 }
 
 
