@@ -63,6 +63,24 @@ def test_blockwise_row_col_dual(shape, dtype):
         assert np.all(blocks[amax >= 1e-4] == top)
 
 
+def test_blockwise_rows_alone_random_shapes():
+    """Forty random shapes (columns a multiple of 8): the row blocks quantized alone (streaming
+    kernel), in both scale layouts, give the bytes and scales of the dual quantizer's row output."""
+    from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+    rng = np.random.default_rng(61)
+    for k in range(40):
+        M, N = int(rng.integers(1, 701)), 8 * int(rng.integers(1, 601))
+        src = (torch.bfloat16, torch.float16, torch.float32)[k % 3]
+        x = bf16_randn((M, N), seed=700 + k, outlier_frac=0.001, dtype=src).cuda()
+        dt = torch.float8_e5m2 if k % 4 == 3 else torch.float8_e4m3fn
+        qr, sr, _, _ = turbo.ops.quantize_fp8_with_trans(x, dt, G.BLOCKWISE, block_size=128)
+        q, s = turbo.ops.quantize_fp8(x, dt, G.BLOCKWISE, block_size=128, axis=1)
+        assert torch.equal(q.view(torch.uint8), qr.view(torch.uint8)) and torch.equal(s, sr), (M, N, src)
+        q2, s_km, _, _ = qi.quant_fp8_blockwise_kmajor_impl(x, dt, 128, False)
+        assert torch.equal(q2.view(torch.uint8), qr.view(torch.uint8)) and torch.equal(s_km.t().contiguous(), sr), (M, N, src)
+
+
 @pytest.mark.parametrize("src", [torch.float16, torch.float32])
 def test_blockwise_other_sources(src):
     x = bf16_randn((300, 520), 22, dtype=src)

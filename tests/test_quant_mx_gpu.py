@@ -94,6 +94,20 @@ def test_mx_row_direction_alone(fmt, dt, shape, dtype):
         assert np.array_equal(codes_np(qs[b]), oq), "row codes"
 
 
+@pytest.mark.parametrize("fmt,dt", FMTS)
+def test_mx_row_direction_alone_random_shapes(fmt, dt):
+    """Forty random shapes (rows 1 .. 700, columns a multiple of 32 up to 4800, a few batched):
+    the row direction quantized alone gives the bytes of the dual quantizer's row output."""
+    rng = np.random.default_rng(60)
+    for k in range(40):
+        M, N = int(rng.integers(1, 701)), 32 * int(rng.integers(1, 151))
+        shape = (int(rng.integers(2, 4)), M, N) if k % 8 == 7 else (M, N)
+        x = bf16_randn(shape, seed=600 + k, outlier_frac=0.001, dtype=torch.float16 if k % 5 == 4 else torch.bfloat16).cuda()
+        q, s = _fn(fmt)(x, dt, x.ndim - 1, 32)
+        rq, rs, _, _ = _fn(fmt)(x, dt, None, 32, with_trans=True)
+        assert torch.equal(q.view(torch.uint8), rq.view(torch.uint8)) and torch.equal(s.view(torch.uint8), rs.view(torch.uint8)), shape
+
+
 @pytest.mark.skipif(FP4 is None, reason="torch has no float4_e2m1fn_x2")
 @pytest.mark.parametrize("shape", [(256, 128), (3, 200, 608)])
 def test_mxfp4_stochastic_rounding_same_noise_alone_and_dual(shape):
