@@ -8,8 +8,8 @@ csrc/pytorch/transpose/transpose.cpp:17-49) as thin adapters over this library's
 so that callers of the reference's extension module keep working. Each has a Meta implementation
 for tracing.
 
-Not offered (they raise ``NotImplementedError``): 2-D blocks and pre-shuffled outputs of the
-GROUPED quantizers; a ``padding_align_size`` other than 128.
+Not offered (they raise ``NotImplementedError``): a ``padding_align_size`` other than 128, and the
+Hadamard transform together with 2-D blocks.
 """
 
 from __future__ import annotations
