@@ -35,8 +35,9 @@ constexpr int TW_VEC     = 16; // elements per thread per unit (16 fp8 bytes = o
 //   [WS_GAVE_UP]   tag of the last launch in which a workgroup gave up waiting
 //   [WS_SLOTS + b] slot of workgroup b: (tag << 32) | abs-max bits
 // A launch takes tag = g + 1 (never 0). Thread 0 of every workgroup reads g BEFORE it
-// publishes (the published word depends on the value read, so the two cannot swap) and
-// hands the tag to its workgroup through LDS; wavefront 0 then polls the slots of all
+// publishes (the published word depends on the value read, so the two cannot swap); it asks
+// for g when the kernel starts (grid_generation), so that this round trip passes under the loads
+// of the tensor, and hands the tag to its workgroup through LDS; wavefront 0 then polls the slots of all
 // workgroups until each carries the tag. Slots of earlier launches carry older tags and
 // need no clearing; workgroup 0 zeroes the slots this launch does not use, so a stale tag
 // can never be 2^32 launches old. Workgroup 0 stores g = tag once its own poll is over,
@@ -60,15 +61,22 @@ struct GridWait {
     uint32_t  wait_for;   // number of slots to wait for (the grid size; tests pass more)
 };
 
-// Returns the grid-wide abs-max. s_tag[1] != 0 afterwards when this workgroup's poll ended at
-// the probe bound (the value returned is then only a partial maximum) or, in workgroup 0,
-// when any workgroup of the launch is known to have given up.
-__device__ __forceinline__ float grid_max_exchange(float block_amax, const GridWait &gw,
+// The generation word as thread 0 sees it when the kernel starts (other threads: 0, not used).
+// The launch that wrote it has completed (launches that share a workspace are ordered), and
+// workgroup 0 of this launch replaces it only after every workgroup has published, i.e. used it.
+__device__ __forceinline__ uint32_t grid_generation(const GridWait &gw) {
+    return threadIdx.x == 0
+               ? static_cast<uint32_t>(__hip_atomic_load(&gw.ws[WS_GEN], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+               : 0u;
+}
+
+// Returns the grid-wide abs-max; g = grid_generation() of this launch. s_tag[1] != 0 afterwards
+// when this workgroup's poll ended at the probe bound (the value returned is then only a partial
+// maximum) or, in workgroup 0, when any workgroup of the launch is known to have given up.
+__device__ __forceinline__ float grid_max_exchange(float block_amax, uint32_t g, const GridWait &gw,
                                                    float *s_red, uint32_t *s_tag) {
     uint64_t *slots = gw.ws + WS_SLOTS;
     if (threadIdx.x == 0) {
-        const uint32_t g =
-            static_cast<uint32_t>(__hip_atomic_load(&gw.ws[WS_GEN], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
         const uint32_t tag = (g + 1u == 0u) ? 1u : g + 1u;
         s_tag[0]           = tag;
         s_tag[1]           = 0u;
@@ -215,6 +223,9 @@ __global__ __launch_bounds__(TW_THREADS) void quant_tensorwise_kernel(
     const int64_t    tid0   = static_cast<int64_t>(blockIdx.x) * TW_THREADS + threadIdx.x;
 
     PT_TW_TRACE_POINT(0);
+    [[maybe_unused]] uint32_t gen = 0u;
+    if constexpr (DYNAMIC)
+        gen = grid_generation(gw);
     if constexpr (VEC16) {
         const int64_t units = n / TW_VEC;
         const int64_t tail0 = units * TW_VEC; // first element of the scalar tail
@@ -241,7 +252,7 @@ __global__ __launch_bounds__(TW_THREADS) void quant_tensorwise_kernel(
                 amax = fmaxf(amax, fabsf(HP<T>::to_f32(x[tail0 + threadIdx.x])));
             amax = block_max(amax, s_red);
             PT_TW_TRACE_POINT(1);
-            amax = grid_max_exchange(amax, gw, s_red, s_tag);
+            amax = grid_max_exchange(amax, gen, gw, s_red, s_tag);
             PT_TW_TRACE_POINT(2);
         }
         float scale;
@@ -275,7 +286,7 @@ __global__ __launch_bounds__(TW_THREADS) void quant_tensorwise_kernel(
             for (int64_t i = tid0; i < n; i += stride)
                 amax = fmaxf(amax, fabsf(HP<T>::to_f32(x[i])));
             amax = block_max(amax, s_red);
-            amax = grid_max_exchange(amax, gw, s_red, s_tag);
+            amax = grid_max_exchange(amax, gen, gw, s_red, s_tag);
         }
         float scale;
         if constexpr (DYNAMIC)
