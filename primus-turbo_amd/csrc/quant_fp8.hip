@@ -53,6 +53,11 @@ constexpr int WS_WORDS = WS_SLOTS + WS_MAX_BLOCKS;
 // raises *status (when given) and WS_GAVE_UP; workgroup 0 then writes NaN into scale_inv,
 // so the failure travels with the data: everything de-quantized from it is NaN.
 constexpr uint32_t GRID_WAIT_MAX_PROBES = 1u << 21;
+// Wavefronts of a workgroup that poll, and how far each starts behind the one before (units of
+// s_sleep, 64 clocks). Measured on a 4096 x 4096 launch: one wavefront 14.5 us, two 1280 clocks
+// apart 13.1, two 640 apart 13.7, four 640 apart 14.6, eight 320 apart 15.3 (more probes in
+// flight delay the slots they wait for).
+constexpr int GRID_POLL_WAVES = 2, GRID_POLL_STEP = 20;
 
 struct GridWait {
     uint64_t *ws;         // workspace words
@@ -80,6 +85,7 @@ __device__ __forceinline__ float grid_max_exchange(float block_amax, uint32_t g,
         const uint32_t tag = (g + 1u == 0u) ? 1u : g + 1u;
         s_tag[0]           = tag;
         s_tag[1]           = 0u;
+        s_tag[2]           = 0u;
         __hip_atomic_store(&slots[blockIdx.x],
                            (static_cast<uint64_t>(tag) << 32) | __float_as_uint(block_amax),
                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -90,19 +96,28 @@ __device__ __forceinline__ float grid_max_exchange(float block_amax, uint32_t g,
         for (uint32_t t = gw.wait_for + threadIdx.x; t < WS_MAX_BLOCKS; t += blockDim.x)
             slots[t] = 0ull;
     float v = 0.f;
-    if (threadIdx.x < 64) {
-        // one wavefront polls: a lane takes four neighbouring slots and requests them together, so
-        // that a round of probes costs one memory round trip (not four in a row)
-        bool bad = false;
+    if (threadIdx.x < 64 * GRID_POLL_WAVES) {
+        // GRID_POLL_WAVES wavefronts poll, each a part of a round trip behind the one before, so
+        // that a slot that arrives just after a probe has left is seen by the next wavefront's
+        // probe instead of a whole round trip later. A lane takes four slots, 64 apart, and
+        // requests them together (one memory round trip per round of probes, not four in a row;
+        // each of the four requests of the wavefront covers 512 consecutive bytes: every
+        // workgroup polls the same few lines, and their number is what the poll costs).
+        // The first wavefront that has seen every slot raises s_tag[2] and the others stop: what
+        // they have seen so far are valid amax values and join the block's maximum.
+        for (uint32_t i = 0; i < (threadIdx.x >> 6); ++i)
+            __builtin_amdgcn_s_sleep(GRID_POLL_STEP);
+        const uint32_t lane = threadIdx.x & 63;
+        bool           bad = false, whole = true; // whole: this lane has seen all of its slots tagged
         for (uint32_t base = 0; base < gw.wait_for; base += 256) {
-            const uint32_t t0     = base + threadIdx.x * 4;
+            const uint32_t t0     = base + lane;
             uint32_t       probes = 0;
             uint64_t       w[4];
             while (true) {
 #pragma unroll
                 for (int k = 0; k < 4; ++k)
-                    w[k] = t0 + k < gw.wait_for
-                               ? __hip_atomic_load(&slots[t0 + k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                    w[k] = t0 + 64 * k < gw.wait_for
+                               ? __hip_atomic_load(&slots[t0 + 64 * k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
                                : static_cast<uint64_t>(tag) << 32;
                 bool all = true;
 #pragma unroll
@@ -110,8 +125,13 @@ __device__ __forceinline__ float grid_max_exchange(float block_amax, uint32_t g,
                     all = all && static_cast<uint32_t>(w[k] >> 32) == tag;
                 if (all)
                     break;
+                if (__hip_atomic_load(&s_tag[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 0u) {
+                    whole = false; // another wavefront has the whole picture
+                    break;
+                }
                 if (++probes >= gw.max_probes) {
-                    bad = true;
+                    whole = false;
+                    bad   = true;
                     break;
                 }
                 __builtin_amdgcn_s_sleep(1);
@@ -121,6 +141,8 @@ __device__ __forceinline__ float grid_max_exchange(float block_amax, uint32_t g,
                 if (static_cast<uint32_t>(w[k] >> 32) == tag) // (a slot that never arrived contributes nothing)
                     v = fmaxf(v, __uint_as_float(static_cast<uint32_t>(w[k]) & 0x7fffffffu));
         }
+        if (__all(whole) && lane == 0)
+            __hip_atomic_store(&s_tag[2], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         if (bad)
             s_tag[1] = 1u; // same value from every lane that writes
     }
@@ -218,7 +240,7 @@ __global__ __launch_bounds__(TW_THREADS) void quant_tensorwise_kernel(
     const float *__restrict__ scale_in, float *__restrict__ scale_inv_out, const GridWait gw,
     const float qmax) {
     __shared__ float    s_red[TW_THREADS / 64];
-    __shared__ uint32_t s_tag[2];
+    __shared__ uint32_t s_tag[3];
     const int64_t    stride = static_cast<int64_t>(gridDim.x) * TW_THREADS;
     const int64_t    tid0   = static_cast<int64_t>(blockIdx.x) * TW_THREADS + threadIdx.x;
 
