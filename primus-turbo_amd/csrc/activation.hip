@@ -111,8 +111,8 @@ __global__ __launch_bounds__(256) void glu_bwd_kernel(const T *__restrict__ grad
                         rg[k]          = gp * (fu[k] * da);
                     }
                 }
-                st128(dg + c, pack8<T>(rg));
-                st128(du + c, pack8<T>(ru));
+                st128_nt(dg + c, pack8<T>(rg)); // (streaming stores: the step's 198 -> 179 us; the forward
+                st128_nt(du + c, pack8<T>(ru)); //  output keeps plain stores, its reader follows at once)
             }
         } else {
             for (int64_t c = threadIdx.x; c < H; c += 256) {

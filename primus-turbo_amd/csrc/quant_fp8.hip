@@ -289,14 +289,14 @@ __global__ __launch_bounds__(TW_THREADS) void quant_tensorwise_kernel(
 #pragma unroll
             for (int it = 0; it < RET; ++it) {
                 const int64_t u = tid0 + it * stride;
-                if (u < units)
-                    st128(q + u * TW_VEC, held[it].template quant<E5M2>(scale, qmax));
+                if (u < units) // (streaming stores: 13.1 -> 11.3 us at 4096 x 4096; streaming loads cost 0.8 us)
+                    st128_nt(q + u * TW_VEC, held[it].template quant<E5M2>(scale, qmax));
             }
         }
         for (int64_t u = tid0 + (DYNAMIC ? RET : 0) * stride; u < units; u += stride) {
             Unit16<T> t;
             t.load(x + u * TW_VEC);
-            st128(q + u * TW_VEC, t.template quant<E5M2>(scale, qmax));
+            st128_nt(q + u * TW_VEC, t.template quant<E5M2>(scale, qmax));
         }
         if (blockIdx.x == 0 && tail0 + threadIdx.x < n)
             q[tail0 + threadIdx.x] =
