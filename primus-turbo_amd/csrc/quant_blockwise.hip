@@ -180,6 +180,9 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
     static_assert(!TRANS || ((MODE & MODE_TILE) != 0) != ((MODE & MODE_COL) != 0), "one transposed output");
     static_assert(GLU == 0 || (GROUPED && sizeof(T) == 2), "the gated input belongs to the grouped 16-bit quantizer");
     __shared__ uint32_t s_tr[TRANS ? BQ * BQ_TP : 1];
+    // the weight quantizer (tile scales, no transposed copy) is a plain stream: non-temporal loads
+    // and stores (0.506 -> 0.462 ms on 32 x 4096 x 7168)
+    constexpr bool WSTREAM = MODE == MODE_TILE && !TRANS;
     const int     tid   = threadIdx.x;
     const int     cseg  = tid & 15; // which 8-column segment of the tile row
     const int     rslot = tid >> 4; // row within a round
@@ -218,7 +221,7 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
             for (int r = 0; r < BQ_ROUNDS; ++r) {
                 const int64_t in_m = in_m0 + tile_row_of(rslot, r);
                 ok[r]              = in_m < in_end && gn < N;
-                held[r].load(x + (ok[r] ? in_m * N + gn : 0));
+                held[r].template load<WSTREAM>(x + (ok[r] ? in_m * N + gn : 0));
             }
 #pragma unroll
             for (int r = 0; r < BQ_ROUNDS; ++r)
@@ -338,8 +341,12 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
             float         vals[BQ_PACK];
             held[r].get(vals);
             const u32x2 code = quant8<E5M2>(vals, s, qmax); // rows beyond the matrix hold zeros: code 0
-            if (in_m < in_end)
-                store8(a.q_row + batch * M * N + in_m * N + gn, code, full, gn, N);
+            if (in_m < in_end) {
+                if (WSTREAM && full)
+                    st64_nt(a.q_row + batch * M * N + in_m * N + gn, code);
+                else
+                    store8(a.q_row + batch * M * N + in_m * N + gn, code, full, gn, N);
+            }
             if constexpr (TRANS) {
                 code4[r & 3] = code;
                 if ((r & 3) == 3)
