@@ -110,9 +110,13 @@ __device__ __forceinline__ u32x2 quant8(const float (&f)[8], const float (&s)[8]
     return o;
 }
 
-__device__ __forceinline__ void store8(uint8_t *p, u32x2 v, bool vec, int64_t gn, int64_t N) {
+// STREAM: a whole piece leaves as a non-temporal store
+template <bool STREAM> __device__ __forceinline__ void store8(uint8_t *p, u32x2 v, bool vec, int64_t gn, int64_t N) {
     if (vec) {
-        *reinterpret_cast<u32x2 *>(p) = v;
+        if constexpr (STREAM)
+            st64_nt(p, v);
+        else
+            *reinterpret_cast<u32x2 *>(p) = v;
     } else {
         const uint32_t w[2] = {v.x, v.y};
 #pragma unroll
@@ -180,9 +184,10 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
     static_assert(!TRANS || ((MODE & MODE_TILE) != 0) != ((MODE & MODE_COL) != 0), "one transposed output");
     static_assert(GLU == 0 || (GROUPED && sizeof(T) == 2), "the gated input belongs to the grouped 16-bit quantizer");
     __shared__ uint32_t s_tr[TRANS ? BQ * BQ_TP : 1];
-    // the weight quantizer (tile scales, no transposed copy) is a plain stream: non-temporal loads
-    // and stores (0.506 -> 0.462 ms on 32 x 4096 x 7168)
-    constexpr bool WSTREAM = MODE == MODE_TILE && !TRANS;
+    // The input is read once and nobody reads the row output soon: non-temporal loads and row
+    // stores (weight quantizer, 32 x 4096 x 7168: 0.506 -> 0.459 ms, with the transposed copy
+    // 0.707 -> 0.656 ms; row + column outputs of 16384 x 7168: 98 -> 90 us). The transposed and
+    // column outputs keep plain stores: with the hint they are slower (92 us).
     const int     tid   = threadIdx.x;
     const int     cseg  = tid & 15; // which 8-column segment of the tile row
     const int     rslot = tid >> 4; // row within a round
@@ -221,7 +226,7 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
             for (int r = 0; r < BQ_ROUNDS; ++r) {
                 const int64_t in_m = in_m0 + tile_row_of(rslot, r);
                 ok[r]              = in_m < in_end && gn < N;
-                held[r].template load<WSTREAM>(x + (ok[r] ? in_m * N + gn : 0));
+                held[r].template load<true>(x + (ok[r] ? in_m * N + gn : 0));
             }
 #pragma unroll
             for (int r = 0; r < BQ_ROUNDS; ++r)
@@ -249,8 +254,8 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
                 const bool ok      = live[r] && gn < N;
                 ms[r]              = live[r] ? in_m : 0;
                 const T *g         = x + (ok ? in_m * 2 * N + gn : 0);
-                held[r].load(g);
-                up[r].load(g + N);
+                held[r].template load<true>(g);
+                up[r].template load<true>(g + N);
                 pr[r] = a.probs[ms[r]];
             }
             if (a.row_mask != nullptr) {
@@ -319,8 +324,7 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
             const float scale = qmax / fmaxf(amax, BQ_EPS);
             if (valid) {
                 const float s[8] = {scale, scale, scale, scale, scale, scale, scale, scale};
-                store8(a.q_row + batch * M * N + in_m * N + gn, quant8<E5M2>(vals, s, qmax),
-                       full, gn, N);
+                store8<true>(a.q_row + batch * M * N + in_m * N + gn, quant8<E5M2>(vals, s, qmax), full, gn, N);
                 if (cseg == 0)
                     a.s_row[in_m * a.rs_m + tn * a.rs_n] = 1.0f / scale;
             }
@@ -341,12 +345,8 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
             float         vals[BQ_PACK];
             held[r].get(vals);
             const u32x2 code = quant8<E5M2>(vals, s, qmax); // rows beyond the matrix hold zeros: code 0
-            if (in_m < in_end) {
-                if (WSTREAM && full)
-                    st64_nt(a.q_row + batch * M * N + in_m * N + gn, code);
-                else
-                    store8(a.q_row + batch * M * N + in_m * N + gn, code, full, gn, N);
-            }
+            if (in_m < in_end)
+                store8<true>(a.q_row + batch * M * N + in_m * N + gn, code, full, gn, N);
             if constexpr (TRANS) {
                 code4[r & 3] = code;
                 if ((r & 3) == 3)
@@ -390,7 +390,7 @@ __global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArg
             held[r].get(vals);
             const u32x2 code = quant8<E5M2>(vals, s, qmax); // grouped: pad rows carry zeros -> code 0
             if (a.q_col != nullptr && out_m < M_out)
-                store8(a.q_col + out_m * N + gn, code, full, gn, N);
+                store8<false>(a.q_col + out_m * N + gn, code, full, gn, N);
             if constexpr (TRANS) {
                 code4[r & 3] = code;
                 if ((r & 3) == 3)

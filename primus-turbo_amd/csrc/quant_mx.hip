@@ -273,8 +273,8 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
                 inside[p]       = m < in_end && n < a.N;
                 ms[p]           = inside[p] ? m : 0;
                 const uint16_t *gp = static_cast<const uint16_t *>(a.x) + ms[p] * 2 * a.N + (inside[p] ? n : 0);
-                piece[p]           = ld128(gp);
-                up[p]              = ld128(gp + a.N);
+                piece[p]           = ld128_nt(gp);
+                up[p]              = ld128_nt(gp + a.N);
                 pr[p]              = a.probs[ms[p]];
             }
             if (a.row_mask != nullptr) {
@@ -306,7 +306,7 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
                 const int     r = p * 16 + (tid >> 4), c = (tid & 15) * 8;
                 const int64_t m = in_m0 + r, n = n0 + c;
                 inside[p]       = m < in_end && n < a.N;
-                piece[p]        = ld128(x + (inside[p] ? m * a.N + n : 0));
+                piece[p]        = ld128_nt(x + (inside[p] ? m * a.N + n : 0));
             }
         }
 #pragma unroll
@@ -363,12 +363,12 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
                         w = c[0];
                     }
                     if (r < row_cnt)
-                        *reinterpret_cast<uint32_t *>(a.row_q + (row_dst0 + r) * (a.Npad >> 1) + (n >> 1)) = w;
+                        st32_nt(a.row_q + (row_dst0 + r) * (a.Npad >> 1) + (n >> 1), w);
                 } else {
                     uint32_t c[2];
                     mx_encode<FMT>(f, inv, c, !nan);
                     if (r < row_cnt)
-                        *reinterpret_cast<u32x2 *>(a.row_q + (row_dst0 + r) * a.Npad + n) = u32x2{c[0], c[1]};
+                        st64_nt(a.row_q + (row_dst0 + r) * a.Npad + n, u32x2{c[0], c[1]});
                 }
             }
             row_done = true;
