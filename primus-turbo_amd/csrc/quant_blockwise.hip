@@ -180,7 +180,7 @@ __device__ __forceinline__ void flush_transposed(const uint32_t *t, uint8_t *out
 // and the gated activation (rounded to T, as the stand-alone activation kernel stores it) is what
 // gets quantized, so that the activation never travels through HBM.
 template <typename T, bool E5M2, int MODE, bool GROUPED, bool VEC8, bool TRANS = false, int GLU = 0>
-__global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArgs a) {
+__device__ __forceinline__ void quant_block128_tile(const BlockQuantArgs &a) {
     static_assert(!TRANS || ((MODE & MODE_TILE) != 0) != ((MODE & MODE_COL) != 0), "one transposed output");
     static_assert(GLU == 0 || (GROUPED && sizeof(T) == 2), "the gated input belongs to the grouped 16-bit quantizer");
     __shared__ uint32_t s_tr[TRANS ? BQ * BQ_TP : 1];
@@ -471,6 +471,20 @@ __global__ __launch_bounds__(256) void quant_rows128_kernel(const BlockQuantArgs
     }
 }
 
+template <typename T, bool E5M2, int MODE, bool GROUPED, bool VEC8, bool TRANS = false, int GLU = 0>
+__global__ __launch_bounds__(256) void quant_block128_kernel(const BlockQuantArgs a) {
+    quant_block128_tile<T, E5M2, MODE, GROUPED, VEC8, TRANS, GLU>(a);
+}
+// The same tile with the registers capped for four workgroups per CU (the compiler takes 155 when
+// left alone, three workgroups). Measured per form: the grouped row + column quantizer without the
+// transposed copy gains (32768 x 7168: 188 -> 173 us), with the copy it makes no difference (146
+// against 147 us), the dense row + column form loses (91 -> 95 us) and so does the gated one
+// (93 -> 100 us): only the first is launched this way.
+template <typename T, bool E5M2, int MODE, bool VEC8>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void quant_block128_occ4_kernel(const BlockQuantArgs a) {
+    quant_block128_tile<T, E5M2, MODE, true, VEC8, false, 0>(a);
+}
+
 template <typename T, bool E5M2, int MODE, bool GROUPED, int GLU = 0>
 static int launch_block128(const BlockQuantArgs &a, int64_t tiles_m, int64_t tiles_n, int64_t batch,
                            bool vec, hipStream_t stream) {
@@ -500,6 +514,13 @@ static int launch_block128(const BlockQuantArgs &a, int64_t tiles_m, int64_t til
                 quant_block128_kernel<T, E5M2, MODE, GROUPED, false, true><<<g, 256, 0, stream>>>(a);
             return check_launch("quant_block128_kernel");
         }
+    }
+    if constexpr (GROUPED && MODE == (MODE_ROW | MODE_COL)) {
+        if (vec)
+            quant_block128_occ4_kernel<T, E5M2, MODE, true><<<g, 256, 0, stream>>>(a);
+        else
+            quant_block128_occ4_kernel<T, E5M2, MODE, false><<<g, 256, 0, stream>>>(a);
+        return check_launch("quant_block128_kernel");
     }
     if (vec)
         quant_block128_kernel<T, E5M2, MODE, GROUPED, true><<<g, 256, 0, stream>>>(a);
