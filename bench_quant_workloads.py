@@ -263,7 +263,7 @@ class QuantGrouped(_QuantBase):
     """Fused grouped row + column blockwise quantize of the routed tokens [32768, 7168], 32 experts."""
 
     name = "fp8_e4m3_grouped_row+col_blockwise_quant_32768x7168_bf16_32experts_zipf1.2"
-    dominant_name = "quant_block128_kernel (grouped: row blocks + segment-padded column blocks from one read)"
+    dominant_name = "quant_block128_occ4_kernel (grouped: row blocks + segment-padded column blocks from one read)"
     graph_dominant = False
 
     def __init__(self, dev, M=32768, N=7168, groups=32):
