@@ -101,8 +101,7 @@ __device__ __forceinline__ float grid_max_exchange(float block_amax, uint32_t g,
         // that a slot that arrives just after a probe has left is seen by the next wavefront's
         // probe instead of a whole round trip later. A lane takes four slots, 64 apart, and
         // requests them together (one memory round trip per round of probes, not four in a row;
-        // each of the four requests of the wavefront covers 512 consecutive bytes: every
-        // workgroup polls the same few lines, and their number is what the poll costs).
+        // each of the four requests of the wavefront covers 512 consecutive bytes).
         // The first wavefront that has seen every slot raises s_tag[2] and the others stop: what
         // they have seen so far are valid amax values and join the block's maximum.
         for (uint32_t i = 0; i < (threadIdx.x >> 6); ++i)
