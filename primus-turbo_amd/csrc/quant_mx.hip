@@ -225,6 +225,7 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
     static_assert(GLU == 0 || !ANY2D, "the gated input is not combined with 2-D blocks");
     __shared__ __attribute__((aligned(16))) uint16_t tile[MX_TILE * MX_PITCH];
     __shared__ float                                 amax_rc[ANY2D ? MX_TILE * 4 : 1]; // [row][32-col block]
+    __shared__ float                                 amax_blk[ROW && ROW2D ? 16 : 1];  // [32-row block][32-col block]
     __shared__ __attribute__((aligned(4))) uint8_t   sbytes[MX_TILE * 4]; // E8M0 bytes of the tile, [row or column][block]
     const int     tid = threadIdx.x;
     // (tile order: blocks of 8 x 8 tiles per XCD, see xcd_block_tile)
@@ -252,7 +253,7 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
 
     PT_MX_TRACE(0);
     // (the row direction is taken from the registers of the loads where that is possible)
-    constexpr bool EARLY_ROW = ROW && !ANY2D && (RHT & 1) == 0;
+    constexpr bool EARLY_ROW = ROW && (RHT & 1) == 0;
     bool           row_done  = false;
     // ---- tile -> LDS (zeros outside the matrix) ----
     // Whole 16-byte pieces (the common case) are all requested before the first is used: a piece
@@ -316,31 +317,60 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
         // registers the loads arrived in (a lane holds a quarter of a block, the block's abs-max is
         // a reduction over four neighbouring lanes), 8 code bytes per lane and 128 per row segment.
         if constexpr (EARLY_ROW) {
+            float am8[8];  // abs-max of this lane's block in piece p (the same in the four lanes of a block)
+            bool  nan8[8]; // a NaN somewhere in that block
+#pragma unroll
+            for (int p = 0; p < 8; ++p) {
+                const uint32_t ww[4] = {piece[p].x, piece[p].y, piece[p].z, piece[p].w};
+                uint32_t       m2 = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    m2 = pk_absmax16(m2, ww[i]);
+                uint32_t m16 = max(m2 & 0xffffu, m2 >> 16);
+                m16          = max(m16, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, m16, 0xB1, 0xf, 0xf, true)));
+                m16          = max(m16, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, m16, 0x4E, 0xf, 0xf, true)));
+                nan8[p]      = m16 > Bits16<T>::INF;
+                float am     = Bits16<T>::to_f32(m16);
+                if (nan8[p]) {
+                    am = 0.f;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        float f0, f1;
+                        unpack2<T>(ww[i], f0, f1);
+                        am = fmaxf(am, fmaxf(abs_or_zero(f0), abs_or_zero(f1)));
+                    }
+                    am = fmaxf(am, dpp_f32<0xB1>(am));
+                    am = fmaxf(am, dpp_f32<0x4E>(am));
+                }
+                am8[p] = am;
+                if constexpr (ANY2D)
+                    if ((tid & 3) == 0)
+                        amax_rc[(p * 16 + (tid >> 4)) * 4 + ((tid & 15) >> 2)] = am;
+            }
+            if constexpr (ROW2D) {
+                // the 16 blocks of 32 x 32: sixteen lanes reduce the 32 row values of one block
+                __syncthreads();
+                {
+                    const int blk = tid >> 4, rb = blk >> 2, cb = blk & 3, i = (tid & 15) * 2;
+                    const float m = row16_max(fmaxf(amax_rc[(rb * 32 + i) * 4 + cb], amax_rc[(rb * 32 + i + 1) * 4 + cb]));
+                    if ((tid & 15) == 0)
+                        amax_blk[blk] = m;
+                }
+                __syncthreads();
+#pragma unroll
+                for (int p = 0; p < 8; ++p)
+                    am8[p] = amax_blk[((p * 16 + (tid >> 4)) >> 5) * 4 + ((tid & 15) >> 2)];
+            }
 #pragma unroll
             for (int p = 0; p < 8; ++p) {
                 const int      r = p * 16 + (tid >> 4), cb = (tid & 15) >> 2; // tile row, 32-column block
                 const uint32_t ww[4] = {piece[p].x, piece[p].y, piece[p].z, piece[p].w};
                 float          f[8];
-                uint32_t       m2 = 0;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
+                for (int i = 0; i < 4; ++i)
                     unpack2<T>(ww[i], f[2 * i], f[2 * i + 1]);
-                    m2 = pk_absmax16(m2, ww[i]);
-                }
-                uint32_t m16 = max(m2 & 0xffffu, m2 >> 16);
-                m16          = max(m16, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, m16, 0xB1, 0xf, 0xf, true)));
-                m16          = max(m16, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, m16, 0x4E, 0xf, 0xf, true)));
-                const bool nan = m16 > Bits16<T>::INF; // somewhere in the block
-                float      am  = Bits16<T>::to_f32(m16);
-                if (nan) {
-                    am = 0.f;
-#pragma unroll
-                    for (int i = 0; i < 8; ++i)
-                        am = fmaxf(am, abs_or_zero(f[i]));
-                    am = fmaxf(am, dpp_f32<0xB1>(am));
-                    am = fmaxf(am, dpp_f32<0x4E>(am));
-                }
-                const int   e   = mx_exponent<FMT>(am);
+                const bool  nan = nan8[p];
+                const int   e   = mx_exponent<FMT>(am8[p]);
                 const float inv = mx_inv_scale(e);
                 if ((tid & 3) == 0)
                     sbytes[r * 4 + cb] = static_cast<uint8_t>(e + 127);
@@ -552,10 +582,14 @@ __global__ __launch_bounds__(256) void mx_quant_kernel(const MxArgs a) {
                     am = fmaxf(am, abs_or_zero(v[i]));
             }
             if constexpr (COL2D) {
-                am = 0.f;
+                if (ROW && ROW2D && row_done) { // the register row pass has left the blocks' maxima
+                    am = amax_blk[rb * 4 + (c >> 5)];
+                } else {
+                    am = 0.f;
 #pragma unroll 8
-                for (int i = 0; i < 32; ++i)
-                    am = fmaxf(am, amax_rc[(rb * 32 + i) * 4 + (c >> 5)]);
+                    for (int i = 0; i < 32; ++i)
+                        am = fmaxf(am, amax_rc[(rb * 32 + i) * 4 + (c >> 5)]);
+                }
             }
             const int e = mx_exponent<FMT>(am);
             if (FMT == MX_E2M1 && (a.sr_mask & 2)) {
