@@ -52,6 +52,22 @@ def _randn_bf16(shape, seed, std):
     return (torch.randn(shape, generator=g, dtype=torch.float32) * std).to(torch.bfloat16)
 
 
+
+def gemm_parity(pairs):
+    """(ok, text) for (oracle, result) pairs of output samples: the four figures of the GEMM gate
+    (cosine >= 0.9999; max |err| / max |ref| <= 1e-2; |err|_F / |ref|_F <= 1e-2, the relative error of
+    the reference's own tests; element-wise |err| <= 2^-7 |ref| + 2^-7 rms(ref row))."""
+    from oracle import gemm as OG
+
+    rel = max(OG.max_rel_err(r, g) for r, g in pairs)
+    cos = min(OG.cosine(g, r) for r, g in pairs)
+    fro = max(OG.rel_fro(r, g) for r, g in pairs)
+    exc = max(OG.elementwise_excess(r, g) for r, g in pairs)
+    ok = bool(rel <= 1e-2 and cos >= 0.9999 and fro <= 1e-2 and exc <= 1.0)
+    return ok, (f"max|err|/max|ref| (relative to the output range)={rel:.2e}, cosine={cos:.6f}, |err|_F/|ref|_F={fro:.2e}, "
+                f"element-wise max |err|/(2^-7|ref|+2^-7 rms(row))={exc:.3f}")
+
+
 class _GemmBase:
     unit = "TFLOP/s"
     dtype = "fp8_e4m3 (fp32 accumulate)"
@@ -120,10 +136,8 @@ class GemmFp8Rowwise(_GemmBase):
         ref = OG.gemm_dequantized(Q.fp8_dequant(aq, asi, "e4m3"), Q.fp8_dequant(bq, bsi, "e4m3"), trans_b=True)
         # the product is rounded to bf16: compare against the bf16-rounded oracle
         ref_t = torch.from_numpy(np.ascontiguousarray(ref, dtype=np.float32)).to(torch.bfloat16).float().numpy()
-        rel = OG.max_rel_err(ref_t, out[rows])
-        cos = OG.cosine(out[rows], ref_t)
-        ok = bool(same and rel <= 1e-2 and cos >= 0.9999)
-        return ok, f"quantized bytes and activation scales bit-exact; 128 output rows vs oracle: max|err|/max|ref| (relative to the output range, not element-wise)={rel:.2e}, cosine={cos:.6f}"
+        ok, text = gemm_parity([(ref_t, out[rows])])
+        return bool(same and ok), f"quantized bytes and activation scales bit-exact: {same}; 128 output rows vs oracle: {text}"
 
     def cpu_baseline(self):
         """The reference's CPU formulas on an M-slice: rowwise quantize of the slice and of all of
@@ -204,10 +218,8 @@ class GemmFp8Blockwise(_GemmBase):
             Q.fp8_blockwise_dequant(aq, asi, 1, "e4m3", 128), Q.fp8_blockwise_weight_dequant(bq, bsi, "e4m3", 128), trans_b=True
         )
         ref_t = torch.from_numpy(np.ascontiguousarray(ref, dtype=np.float32)).to(torch.bfloat16).float().numpy()
-        rel = OG.max_rel_err(ref_t, out[rows])
-        cos = OG.cosine(out[rows], ref_t)
-        ok = bool(same and rel <= 1e-2 and cos >= 0.9999)
-        return ok, f"quantized bytes bit-exact; 128 output rows vs oracle: max|err|/max|ref| (relative to the output range, not element-wise)={rel:.2e}, cosine={cos:.6f}"
+        ok, text = gemm_parity([(ref_t, out[rows])])
+        return bool(same and ok), f"quantized bytes bit-exact: {same}; 128 output rows vs oracle: {text}"
 
     def cpu_baseline(self):
         from oracle import cpu_reference as R
@@ -300,10 +312,8 @@ class GemmMx(_GemmBase):
         b_deq = Q.mx_dequant(u8(self.bq)[:nb], u8(self.bs)[:nb], self.fmt)
         ref = OG.gemm_dequantized(Q.mx_dequant(aq, asc, self.fmt), b_deq, trans_b=True)
         ref_t = torch.from_numpy(np.ascontiguousarray(ref, dtype=np.float32)).to(torch.bfloat16).float().numpy()
-        rel = OG.max_rel_err(ref_t, out[rows][:, :nb])
-        cos = OG.cosine(out[rows][:, :nb], ref_t)
-        ok = bool(same and rel <= 1e-2 and cos >= 0.9999)
-        return ok, f"codes and E8M0 bytes bit-exact: {same}; 128 x 2048 outputs vs oracle: max|err|/max|ref| (relative to the output range, not element-wise)={rel:.2e}, cosine={cos:.6f}"
+        ok, text = gemm_parity([(ref_t, out[rows][:, :nb])])
+        return bool(same and ok), f"codes and E8M0 bytes bit-exact: {same}; 128 x 2048 outputs vs oracle: {text}"
 
     def cpu_baseline(self):
         """The oracle (numpy restatement of the reference's MX quantizer) plus an fp32 matmul on a
@@ -424,7 +434,7 @@ class GroupedGemmFp8(_GemmBase):
         out = self.dominant().float().cpu().numpy()
         offs = np.concatenate([[0], np.cumsum(self.lens)])
         live = [g for g in range(self.groups) if self.lens[g] > 0]
-        same, rel, cos = True, 0.0, 1.0
+        same, pairs = True, []
         for g in (live[0], live[-1]):
             r0, r1 = int(offs[g]), int(min(offs[g] + 64, offs[g + 1]))
             aq, asi = Q.fp8_blockwise(self.x_cpu.float().numpy()[r0:r1], 1, "e4m3", 128)
@@ -434,10 +444,9 @@ class GroupedGemmFp8(_GemmBase):
             ref = OG.gemm_dequantized(Q.fp8_blockwise_dequant(aq, asi, 1, "e4m3", 128),
                                       Q.fp8_blockwise_weight_dequant(bq, bsi, "e4m3", 128), trans_b=True)
             ref_t = torch.from_numpy(np.ascontiguousarray(ref, dtype=np.float32)).to(torch.bfloat16).float().numpy()
-            rel = max(rel, OG.max_rel_err(ref_t, out[r0:r1]))
-            cos = min(cos, OG.cosine(out[r0:r1], ref_t))
-        ok = bool(same and rel <= 1e-2 and cos >= 0.9999)
-        return ok, f"quantized bytes bit-exact: {same}; rows of two experts vs oracle: max|err|/max|ref| (relative to the output range, not element-wise)={rel:.2e}, cosine={cos:.6f}"
+            pairs.append((ref_t, out[r0:r1]))
+        ok, text = gemm_parity(pairs)
+        return bool(same and ok), f"quantized bytes bit-exact: {same}; rows of two experts vs oracle: {text}"
 
     def cpu_baseline(self):
         """The reference's CPU formulas (blockwise quantize, dequantize, per-expert fp32 matmul) for
@@ -565,7 +574,7 @@ class GroupedGemmMxfp8(_GemmBase):
         offs = np.concatenate([[0], np.cumsum(self.lens)])
         orow = self.offs_row.cpu().numpy()
         live = [g for g in range(self.groups) if self.lens[g] > 0]
-        same, rel, cos = True, 0.0, 1.0
+        same, pairs = True, []
         for g in (live[0], live[-1]):
             n = int(min(64, self.lens[g]))
             r0, p0 = int(offs[g]), int(orow[g])
@@ -574,10 +583,9 @@ class GroupedGemmMxfp8(_GemmBase):
             w_deq = Q.mx_dequant(u8(self.wq[g]), u8(self.ws[g]), self.fmt)
             ref = OG.gemm_dequantized(Q.mx_dequant(aq, asc, self.fmt), w_deq, trans_b=True)
             ref_t = torch.from_numpy(np.ascontiguousarray(ref, dtype=np.float32)).to(torch.bfloat16).float().numpy()
-            rel = max(rel, OG.max_rel_err(ref_t, out[r0 : r0 + n]))
-            cos = min(cos, OG.cosine(out[r0 : r0 + n], ref_t))
-        ok = bool(same and rel <= 1e-2 and cos >= 0.9999)
-        return ok, f"codes and E8M0 bytes bit-exact: {same}; rows of two experts vs oracle: max|err|/max|ref| (relative to the output range, not element-wise)={rel:.2e}, cosine={cos:.6f}"
+            pairs.append((ref_t, out[r0 : r0 + n]))
+        ok, text = gemm_parity(pairs)
+        return bool(same and ok), f"codes and E8M0 bytes bit-exact: {same}; rows of two experts vs oracle: {text}"
 
     def cpu_baseline(self):
         """The numpy oracle (MX quantize, de-quantize) plus an fp32 matmul for 256 tokens of the

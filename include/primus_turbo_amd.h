@@ -112,10 +112,11 @@ PT_API int pt_quantize_fp8_tensorwise_ex(const void *x, int x_dtype, int64_t num
  * it calls allocates or frees memory. Same kernels and results as
  * pt_quantize_fp8_tensorwise.
  *
- * Each stream that calls it on a device is given its own slot set, at most
- * PT_TENSORWISE_STATIC_MAX_STREAMS per device; one more stream is rejected with
- * PT_ERR_WORKSPACE, and numel above PT_TENSORWISE_STATIC_MAX_NUMEL with
- * PT_ERR_INVALID_ARGUMENT. Calls on one stream are ordered and share that stream's slot
+ * Each stream HANDLE that calls it on a device is given its own slot set and keeps it until
+ * pt_tensorwise_static_release (the limit counts handles that have called and not released,
+ * not streams in use at a time), at most PT_TENSORWISE_STATIC_MAX_STREAMS per device; one
+ * more is rejected with PT_ERR_WORKSPACE, and numel above PT_TENSORWISE_STATIC_MAX_NUMEL
+ * with PT_ERR_INVALID_ARGUMENT. Calls on one stream are ordered and share that stream's slot
  * set; the set keeps the last call's words (they are generation-tagged, so nothing has
  * to be cleared). Work that overlaps on one GPU while using ONE slot set races: a graph
  * captured on stream S and replayed on another stream while S is also calling, or the
@@ -126,6 +127,28 @@ PT_API int pt_quantize_fp8_tensorwise_ex(const void *x, int x_dtype, int64_t num
 PT_API int pt_quantize_fp8_tensorwise_static(const void *x, int x_dtype, int64_t numel, void *q,
                                              int q_dtype, const float *scale_in, float *scale_inv,
                                              int32_t *status, void *stream);
+
+/* Gives the slot set that pt_quantize_fp8_tensorwise_static keeps for `stream` on the current
+ * device back, so that another stream handle can take it (a process that cycles through
+ * stream handles would otherwise run out of the PT_TENSORWISE_STATIC_MAX_STREAMS sets). Every
+ * call made on `stream` through the static entry point must have completed. A stream that
+ * holds no set is not an error. Allocates nothing. No counterpart in Primus-Turbo. */
+PT_API int pt_tensorwise_static_release(void *stream);
+
+/* The same quantizer in two launches with no exchange between workgroups: per-workgroup
+ * abs-max into the workspace, then every workgroup of the second launch reduces those, forms
+ * the scale and casts. This is the launch structure of Primus-Turbo's own op
+ * (csrc/pytorch/quantization/quantization.cpp:44-90: reduce, compute scale, cast; kernels
+ * csrc/kernels/reduce/reduce_row.cuh:16-88, quantization_tensorwise.cu:51-111). Results are
+ * bit-identical with pt_quantize_fp8_tensorwise. Nothing in it depends on all workgroups
+ * of a launch being resident at once, so it is the form to use when other streams, CU
+ * masks or graph replays beside eager work may hold compute units; x is read twice.
+ * workspace : as for pt_quantize_fp8_tensorwise in size and alignment, but it needs NO
+ *             zero-fill and carries nothing from call to call; calls that may overlap
+ *             need separate buffers. */
+PT_API int pt_quantize_fp8_tensorwise_two_pass(const void *x, int x_dtype, int64_t numel, void *q,
+                                               int q_dtype, float *scale_inv, void *workspace,
+                                               size_t workspace_bytes, void *stream);
 
 /* Replaces torch.ops.primus_turbo_cpp_extension.dequantize_fp8_tensorwise
  * (csrc/pytorch/bindings_pytorch.cpp:38, quantization.cpp:211-230,
@@ -356,9 +379,11 @@ PT_API int pt_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const v
  * codes per byte, K counts codes). a_scale [M, >= K / 32] and b_scale [N, >= K / 32] are E8M0
  * bytes with row pitches sa_ld / sb_ld. K % 32 == 0; bytes of a row behind K must be zero
  * codes, as the MX quantizers leave them. Rows that are not whole 128-byte slabs (at least
- * four) are first copied into `workspace` (pt_gemm_mx_workspace_bytes, 16-byte aligned); for
- * large problems the workspace also receives a copy of both scale arrays with the 32-bit words
- * of one K position of all rows contiguous, which is what the kernel's scale copies then read.
+ * four) are first copied into `workspace` (16-byte aligned); a workspace of
+ * pt_gemm_mx_workspace_bytes also receives, for large problems, a copy of both scale arrays with
+ * the 32-bit words of one K position of all rows contiguous, which is what the kernel's scale
+ * copies then read (faster; with a smaller workspace, or none when no row copy is needed, the
+ * scales are read in place).
  * accumulate != 0 adds into C (beta = 1). tile_cfg as for pt_gemm_fp8; 4 = 256 x 256 tile with
  * eight wavefronts (the automatic choice for MXFP4 with M, N >= 2048), bit-identical results. */
 PT_API size_t pt_gemm_mx_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,

@@ -16,7 +16,8 @@ fp32 summation order and the final rounding to the output dtype:
 Pinned by (tests/test_oracle_gemm.py): float64 python-loop evaluation on tiny shapes in all
 four operand layouts, hand-computed values, exact small-integer cases where fp32 accumulation
 is exact, grouped cases with empty groups and rows past the last group, the adjoint identity
-between the grouped forward and the variable-K product, and hand values of the metrics.
+between the grouped forward and the variable-K product, and hand values of the metrics
+(cosine, range-relative maximum, Frobenius-relative error, element-wise bound, SNR).
 """
 
 from __future__ import annotations
@@ -89,6 +90,31 @@ def max_rel_err(ref: np.ndarray, y: np.ndarray) -> float:
     y = np.asarray(y, dtype=np.float64)
     den = np.max(np.abs(ref))
     return float(np.max(np.abs(y - ref)) / den) if den > 0 else float(np.max(np.abs(y)))
+
+
+def rel_fro(ref: np.ndarray, y: np.ndarray) -> float:
+    """|y - ref|_F / |ref|_F, the reference tests' relative error
+    (/root/reference/tests/pytorch/test_utils.py:43-45)."""
+    ref = np.asarray(ref, dtype=np.float64)
+    y = np.asarray(y, dtype=np.float64)
+    den = np.linalg.norm(ref)
+    return float(np.linalg.norm(y - ref) / den) if den > 0 else float(np.linalg.norm(y))
+
+
+def elementwise_excess(ref: np.ndarray, y: np.ndarray, rtol: float = 2.0 ** -7) -> float:
+    """max over elements of |y - ref| / (rtol |ref| + rtol rms(ref's row)); a result is inside the
+    element-wise bound when this is <= 1. Unlike the range-relative maximum, an error of a few
+    per cent of ONE small element (a wrong scale on one row block) fails it: every element is
+    held to its own size plus a share of its row's typical size (1-D input: one row)."""
+    ref = np.atleast_2d(np.asarray(ref, dtype=np.float64))
+    y = np.atleast_2d(np.asarray(y, dtype=np.float64))
+    ref2, y2 = ref.reshape(-1, ref.shape[-1]), y.reshape(-1, y.shape[-1])
+    rms = np.sqrt(np.mean(ref2 * ref2, axis=1, keepdims=True))
+    bound = rtol * np.abs(ref2) + rtol * rms
+    err = np.abs(y2 - ref2)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        ratio = np.where(bound > 0, err / bound, np.where(err > 0, np.inf, 0.0))
+    return float(ratio.max()) if ratio.size else 0.0
 
 
 def snr_db(ref: np.ndarray, y: np.ndarray) -> float:

@@ -151,29 +151,37 @@ __global__ __launch_bounds__(256) void transpose_words_kernel(const uint32_t *__
     __shared__ uint32_t t[32][33];
     in += static_cast<int64_t>(blockIdx.z) * R * pitch; // batch of matrices, each transposed on its own
     out += static_cast<int64_t>(blockIdx.z) * W * R;
-    const int64_t r0 = static_cast<int64_t>(blockIdx.y) * 32, w0 = static_cast<int64_t>(blockIdx.x) * 32;
+    const int64_t w0 = static_cast<int64_t>(blockIdx.x) * 32;
     const int     tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    // (the row tiles are walked with the grid's y extent as the stride: it is capped at 65535)
+    for (int64_t r0 = static_cast<int64_t>(blockIdx.y) * 32; r0 < R; r0 += static_cast<int64_t>(gridDim.y) * 32) {
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const int64_t r = r0 + ty + 8 * p, w = w0 + tx;
-        if (r < R && w < W)
-            t[ty + 8 * p][tx] = in[r * pitch + w];
-    }
-    __syncthreads();
+        for (int p = 0; p < 4; ++p) {
+            const int64_t r = r0 + ty + 8 * p, w = w0 + tx;
+            if (r < R && w < W)
+                t[ty + 8 * p][tx] = in[r * pitch + w];
+        }
+        __syncthreads();
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const int64_t w = w0 + ty + 8 * p, r = r0 + tx;
-        if (w < W && r < R)
-            out[w * R + r] = t[tx][ty + 8 * p];
+        for (int p = 0; p < 4; ++p) {
+            const int64_t w = w0 + ty + 8 * p, r = r0 + tx;
+            if (w < W && r < R)
+                out[w * R + r] = t[tx][ty + 8 * p];
+        }
+        __syncthreads();
     }
 }
 
-void launch_transpose_words(const uint32_t *in, uint32_t *out, int64_t R, int64_t W, int64_t pitch, hipStream_t st,
-                            int64_t batch) {
+int launch_transpose_words(const uint32_t *in, uint32_t *out, int64_t R, int64_t W, int64_t pitch, hipStream_t st,
+                           int64_t batch) {
     if (R * W * batch == 0)
-        return;
-    dim3 g(static_cast<unsigned>(cdiv(W, 32)), static_cast<unsigned>(cdiv(R, 32)), static_cast<unsigned>(batch));
+        return PT_OK;
+    if (batch > 65535)
+        return fail(PT_ERR_INVALID_ARGUMENT, "transpose_words: more than 65535 matrices in a batch");
+    const int64_t gy = cdiv(R, 32) < 65535 ? cdiv(R, 32) : 65535;
+    dim3 g(static_cast<unsigned>(cdiv(W, 32)), static_cast<unsigned>(gy), static_cast<unsigned>(batch));
     transpose_words_kernel<<<g, 256, 0, st>>>(in, out, R, W, pitch);
+    return check_launch("transpose_words_kernel");
 }
 
 template <int FA, int FB>
@@ -303,7 +311,8 @@ int pt_gemm_fp8(const void *a, int a_dtype, const float *a_scale, const void *b,
     const size_t  scale_area = block_scale_copy_pays(M, N, K) ? static_cast<size_t>(round_up(M * KB * 4, 256)) : 0;
     // per-row A scales stored [M, K / 128] (sa_k == 1): hand the kernel a [K / 128, M] copy
     if (have_ws && scale_area != 0 && scale_mode == SCALE_BLOCK && sa_block == 1 && sa_k == 1 && sa_m >= KB) {
-        launch_transpose_words(reinterpret_cast<const uint32_t *>(a_scale), static_cast<uint32_t *>(workspace), M, KB, sa_m, st);
+        if (const int rc = launch_transpose_words(reinterpret_cast<const uint32_t *>(a_scale), static_cast<uint32_t *>(workspace), M, KB, sa_m, st))
+            return rc;
         a_scale = static_cast<const float *>(workspace);
         sa_m    = 1;
         sa_k    = M;

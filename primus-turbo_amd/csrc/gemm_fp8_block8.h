@@ -19,9 +19,10 @@
 //   * two LDS stages. One barrier per slab, before row group 6: everyone's copies of the next
 //     slab have landed and everyone has finished reading the current stage. From there on
 //     the wavefront reads the next slab's first A fragments, its scales and (after its last
-//     use of each B fragment) the B fragments, and the copies of the slab after next go into
-//     the stage just freed: five of them (B rows, scales) in row groups 6 and 7, four (A
-//     rows) in row groups 0..3 of the following slab;
+//     use of each B fragment) the B fragments, and all nine copies of the slab after next (B
+//     rows, scales, A rows) go into the stage just freed during row groups 6 and 7: every
+//     copy a barrier waits for is then older than the stores of a result tile written in
+//     between, which is what lets that wait leave the stores in flight;
 //   * the slab sequence runs across tile boundaries (persistent grid), the loader changing
 //     tile by swapping uniform values as in the four-wavefront kernel.
 #pragma once
@@ -310,14 +311,10 @@ __global__ __launch_bounds__(B8_THREADS) void gemm_fp8_block8_kernel(const GemmA
         }
 
         const int64_t wm_base = cur_t.m0 + wm * (TM * 16), wn_base = cur_t.n0 + wn * (TN * 16);
-        epilogue<TM, TN, SCALE_BLOCK, false>(a, acc, cur_t.C, cur_t.sA, cur_t.sB, cur_t.m_end, wm_base, wn_base, lane);
-        // the straight-line store path (the condition of `epilogue`) issues one 16-byte store per pair
-        // of MFMA tiles (16-bit outputs) or per tile (fp32); other paths are not counted on
-        {
-            const bool fast = wm_base + TM * 16 <= cur_t.m_end && wn_base + TN * 16 <= a.N && (a.N & 7) == 0 &&
-                              (reinterpret_cast<uintptr_t>(cur_t.C) & 15) == 0;
-            pending = __builtin_amdgcn_readfirstlane(fast ? (a.out_dtype == PT_DTYPE_F32 ? TM * TN : TM * TN / 2) : 0);
-        }
+        // stores of the epilogue's straight-line path (0, 16 or 32: the cases of the barrier's wait)
+        pending = __builtin_amdgcn_readfirstlane(
+            epilogue<TM, TN, SCALE_BLOCK, false>(a, acc, cur_t.C, cur_t.sA, cur_t.sB, cur_t.m_end, wm_base, wn_base, lane));
+        static_assert(TM * TN == 32, "the barrier's wait distinguishes 16 and 32 stores in flight");
 
         if (next_tile >= total)
             break;

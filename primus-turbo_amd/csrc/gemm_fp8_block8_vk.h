@@ -288,12 +288,10 @@ __global__ __launch_bounds__(B8_THREADS) void gemm_fp8_block8_vk_kernel(const Ge
             PT_GEMM_TRACE_POINT(5);
             uint8_t *Cg = static_cast<uint8_t *>(a.C) + static_cast<int64_t>(g) * a.c_gstride * ES;
             const int64_t wm_base = m0 + wm * (TM * 16), wn_base = n0 + wn * (TN * 16);
-            epilogue<TM, TN, SCALE_BLOCK, false>(a, acc, Cg, a.sA, a.sB, a.M, wm_base, wn_base, lane);
-            // the straight-line store path (the condition of `epilogue`) issues one 16-byte store per
-            // pair of MFMA tiles (16-bit outputs) or per tile (fp32); other paths are not counted on
-            const bool fast = wm_base + TM * 16 <= a.M && wn_base + TN * 16 <= a.N && (a.N & 7) == 0 &&
-                              (reinterpret_cast<uintptr_t>(Cg) & 15) == 0;
-            pending = __builtin_amdgcn_readfirstlane(fast ? (ES == 2 ? TM * TN / 2 : TM * TN) : 0);
+            // stores of the epilogue's straight-line path (0, 16 or 32: the cases of the barrier's wait)
+            pending = __builtin_amdgcn_readfirstlane(
+                epilogue<TM, TN, SCALE_BLOCK, false>(a, acc, Cg, a.sA, a.sB, a.M, wm_base, wn_base, lane));
+            static_assert(TM * TN == 32, "the barrier's wait distinguishes 16 and 32 stores in flight");
             PT_GEMM_TRACE_POINT(6);
             pos  = g_hi;
             g_hi = nxt_hi;

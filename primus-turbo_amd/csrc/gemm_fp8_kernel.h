@@ -229,9 +229,13 @@ template <bool ACC_IN_AGPR> __device__ __forceinline__ f32x4 read_acc(const f32x
 // row and store instruction, so that no partially written 64-byte unit ever leaves the L2.
 // `row` points at C[m][wn_base + 16 (lg & 1) + 8 (lg >> 1)] for 16-bit outputs and at
 // C[m][wn_base + 4 lg] for fp32.
+// Returns the number of store instructions it has issued (every one of them younger than any
+// memory operation issued before the call): what a caller may leave in flight when it next waits
+// for older operations by count.
 template <typename T, int TM, int TN, int MODE, bool ACC_IN_AGPR>
-__device__ __forceinline__ void epilogue_inner(T *row, int64_t step, bool accu, const f32x4 (&acc)[TM][TN],
-                                               const float (&sa)[TM], const f32x4 (&sb)[TN]) {
+__device__ __forceinline__ int epilogue_inner(T *row, int64_t step, bool accu, const f32x4 (&acc)[TM][TN],
+                                              const float (&sa)[TM], const f32x4 (&sb)[TN]) {
+    int stores = 0;
     static_for<0, TM>([&](auto ic) {
         constexpr int i = ic;
         if constexpr (sizeof(T) == 4) {
@@ -259,6 +263,7 @@ __device__ __forceinline__ void epilogue_inner(T *row, int64_t step, bool accu, 
                     if (accu)
                         v += old[j - j0];
                     *reinterpret_cast<f32x4 *>(q) = v;
+                    ++stores;
                     // keep each accumulator's read next to its store (register pressure)
                     __builtin_amdgcn_sched_barrier(0);
                 });
@@ -299,11 +304,13 @@ __device__ __forceinline__ void epilogue_inner(T *row, int64_t step, bool accu, 
                 w.z = pack2<T>(y[0], y[1]);
                 w.w = pack2<T>(y[2], y[3]);
                 *reinterpret_cast<u32x4 *>(q) = w; // (streaming stores measured no faster here)
+                ++stores;
                 __builtin_amdgcn_sched_barrier(0);
             });
         }
         row += step;
     });
+    return stores; // (a compile-time constant after unrolling: TM * TN, or TM * TN / 2 for 16-bit outputs)
 }
 
 __device__ __forceinline__ void store_elem(float f, uint8_t *q, int out_dtype, bool accu) {
@@ -321,8 +328,13 @@ __device__ __forceinline__ void store_elem(float f, uint8_t *q, int out_dtype, b
 
 // `Cm` / `sAm` / `sBm` / `m_end` describe the matrix the tile belongs to (the whole problem,
 // or one group's share of it).
+// Returns (uniform over the wavefront) how many of the vector-memory operations it issued are
+// guaranteed to be younger than everything issued before the call and may still be in flight on
+// return: the store count of the straight-line path, 0 for the generic path. Kernels that wait
+// for older direct-to-LDS copies by count (memory operations retire in order) leave exactly
+// that many operations outstanding instead of waiting for the stores to be acknowledged.
 template <int TM, int TN, int MODE, bool ACC_IN_AGPR>
-__device__ __forceinline__ void epilogue(const GemmArgs &a, const f32x4 (&acc)[TM][TN], uint8_t *Cm,
+__device__ __forceinline__ int epilogue(const GemmArgs &a, const f32x4 (&acc)[TM][TN], uint8_t *Cm,
                                          const float *sAm, const float *sBm, int64_t m_end,
                                          int64_t wm_base, int64_t wn_base, int lane) {
     const int     ES = a.out_dtype == PT_DTYPE_F32 ? 4 : 2;
@@ -356,11 +368,10 @@ __device__ __forceinline__ void epilogue(const GemmArgs &a, const f32x4 (&acc)[T
         // 16-bit outputs: the lane's eight columns after the exchange between tile pairs
         uint8_t *rowp = C + (m0 * a.N + wn_base + 16 * (lg & 1) + 8 * (lg >> 1)) * 2;
         if (a.out_dtype == PT_DTYPE_BF16)
-            epilogue_inner<bf16_t, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<bf16_t *>(rowp), step, accu, acc, sa, sb);
-        else if (a.out_dtype == PT_DTYPE_F16)
-            epilogue_inner<f16_t, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<f16_t *>(rowp), step, accu, acc, sa, sb);
-        else
-            epilogue_inner<float, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<float *>(row), step, accu, acc, sa, sb);
+            return epilogue_inner<bf16_t, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<bf16_t *>(rowp), step, accu, acc, sa, sb);
+        if (a.out_dtype == PT_DTYPE_F16)
+            return epilogue_inner<f16_t, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<f16_t *>(rowp), step, accu, acc, sa, sb);
+        return epilogue_inner<float, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<float *>(row), step, accu, acc, sa, sb);
     } else {
         static_for<0, TM>([&](auto ic) {
             constexpr int i = ic;
@@ -383,6 +394,7 @@ __device__ __forceinline__ void epilogue(const GemmArgs &a, const f32x4 (&acc)[T
             row += step * ES;
         });
     }
+    return 0;
 }
 
 // Where a workgroup's tile lives. The second half only varies between tiles of grouped
@@ -1020,12 +1032,9 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
             if constexpr (MODE != SCALE_BLOCK)
                 asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
             PT_GEMM_TRACE_POINT(5);
-            epilogue<TM, TN, MODE, MODE != SCALE_BLOCK>(a, acc, cur_t.C, cur_t.sA, cur_t.sB, cur_t.m_end, wm_base, wn_base,
-                                                         lane);
-            // (the same test as the epilogue's: its straight-line path issues exactly this many stores)
-            const bool fast = wm_base + TM * 16 <= cur_t.m_end && wn_base + TN * 16 <= a.N && (a.N & 7) == 0 &&
-                              (reinterpret_cast<uintptr_t>(cur_t.C) & 15) == 0;
-            pending = __builtin_amdgcn_readfirstlane(fast ? (a.out_dtype == PT_DTYPE_F32 ? ST32 : ST16) : 0);
+            // (0, ST16 or ST32: the stores of the epilogue's straight-line path)
+            pending = __builtin_amdgcn_readfirstlane(epilogue<TM, TN, MODE, MODE != SCALE_BLOCK>(
+                a, acc, cur_t.C, cur_t.sA, cur_t.sB, cur_t.m_end, wm_base, wn_base, lane));
         } else {
             const int ES     = a.out_dtype == PT_DTYPE_F32 ? 4 : 2;
             int64_t   g_lo   = a.group_offs[cur_t.g0] >> (F4 ? 1 : 0);
@@ -1164,7 +1173,7 @@ void launch_pad_rows(const uint8_t *in, uint8_t *out, int64_t R, int64_t C, int6
 // in[R, C] with row pitch ldi -> out[R, ldo] (columns [C, ldo) zero-filled)
 void launch_pad_rows2(const uint8_t *in, uint8_t *out, int64_t R, int64_t C, int64_t ldi, int64_t ldo, hipStream_t st);
 // out[b][w * R + r] = in[b][r * pitch + w] for w < W (32-bit words): scale arrays made contiguous along their rows
-void launch_transpose_words(const uint32_t *in, uint32_t *out, int64_t R, int64_t W, int64_t pitch, hipStream_t st,
+int launch_transpose_words(const uint32_t *in, uint32_t *out, int64_t R, int64_t W, int64_t pitch, hipStream_t st,
                             int64_t batch = 1);
 int  launch_gemm_block(const GemmArgs &a, int fa, int fb, bool sb_vec, int tile_cfg, hipStream_t stream);
 

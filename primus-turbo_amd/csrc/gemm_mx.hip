@@ -76,22 +76,30 @@ int pt_gemm_mx(const void *a, const void *a_scale, const void *b, const void *b_
     // that carry anything but zeros behind K, into zero-padded rows
     const int64_t  need = mx_row_bytes(K, fp4);
     const uint8_t *A = static_cast<const uint8_t *>(a), *B = static_cast<const uint8_t *>(b);
-    // word-major scales need whole 32-bit words per row in the source
-    const bool     wordmajor = mx_wordmajor_pays(M, N, K) && sa_ld % 4 == 0 && sb_ld % 4 == 0 && aligned_to(a_scale, 4) &&
-                           aligned_to(b_scale, 4) && sa_ld >= mx_scale_words(K) * 4 && sb_ld >= mx_scale_words(K) * 4;
+    // word-major scales need whole 32-bit words per row in the source, and room in the workspace:
+    // without it (a caller that passes only what the operand copies need, or nothing) the scales
+    // are read in place
+    const bool     copies    = lda != need || ldb != need;
+    const size_t   want_copy = static_cast<size_t>((lda != need ? round_up(M * need, 256) : 0) + (ldb != need ? round_up(N * need, 256) : 0));
+    const size_t   want_all  = pt_gemm_mx_workspace_bytes(M, N, K, lda, ldb, fp4);
+    const bool     have_all  = workspace != nullptr && workspace_bytes >= want_all && aligned_to(workspace, 16);
+    const bool     wordmajor = have_all && mx_wordmajor_pays(M, N, K) && sa_ld % 4 == 0 && sb_ld % 4 == 0 &&
+                           aligned_to(a_scale, 4) && aligned_to(b_scale, 4) && sa_ld >= mx_scale_words(K) * 4 &&
+                           sb_ld >= mx_scale_words(K) * 4;
     const void *sa_use = a_scale, *sb_use = b_scale;
-    if (lda != need || ldb != need || wordmajor) {
-        const size_t want = pt_gemm_mx_workspace_bytes(M, N, K, lda, ldb, fp4);
-        if (workspace == nullptr || workspace_bytes < want || !aligned_to(workspace, 16))
+    if (copies || wordmajor) {
+        if (workspace == nullptr || workspace_bytes < want_copy || !aligned_to(workspace, 16))
             return fail(PT_ERR_WORKSPACE, "pt_gemm_mx: workspace missing, too small or misaligned");
         uint8_t *ws = static_cast<uint8_t *>(workspace);
         if (wordmajor) {
             const int64_t W = mx_scale_words(K);
             // in: [rows, sa_ld / 4] words (the first W of every row are used) -> out: [W, rows]
-            launch_transpose_words(static_cast<const uint32_t *>(a_scale), reinterpret_cast<uint32_t *>(ws), M, W, sa_ld / 4, st);
+            if (const int rc = launch_transpose_words(static_cast<const uint32_t *>(a_scale), reinterpret_cast<uint32_t *>(ws), M, W, sa_ld / 4, st))
+                return rc;
             sa_use = ws;
             ws += round_up(M * W * 4, 256);
-            launch_transpose_words(static_cast<const uint32_t *>(b_scale), reinterpret_cast<uint32_t *>(ws), N, W, sb_ld / 4, st);
+            if (const int rc = launch_transpose_words(static_cast<const uint32_t *>(b_scale), reinterpret_cast<uint32_t *>(ws), N, W, sb_ld / 4, st))
+                return rc;
             sb_use = ws;
             ws += round_up(N * W * 4, 256);
         }

@@ -133,8 +133,10 @@ int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, int64_t 
             workspace_bytes >= pt_grouped_gemm_mx_workspace_bytes(G, a_rows, N, K) && sa_ld >= 4 * W && sb_ld >= 4 * W) {
             uint32_t *wa = static_cast<uint32_t *>(workspace);
             uint32_t *wb = wa + round_up(a_rows * W * 4, 256) / 4;
-            launch_transpose_words(static_cast<const uint32_t *>(a_scale), wa, a_rows, W, sa_ld / 4, st);
-            launch_transpose_words(static_cast<const uint32_t *>(b_scale), wb, N, W, sb_ld / 4, st, G);
+            if (const int rc = launch_transpose_words(static_cast<const uint32_t *>(a_scale), wa, a_rows, W, sa_ld / 4, st))
+                return rc;
+            if (const int rc = launch_transpose_words(static_cast<const uint32_t *>(b_scale), wb, N, W, sb_ld / 4, st, G))
+                return rc;
             g.sA         = reinterpret_cast<const float *>(wa);
             g.sB         = reinterpret_cast<const float *>(wb);
             g.sa_wpitch  = a_rows * 4;
@@ -195,8 +197,10 @@ int pt_grouped_gemm_mx_variable_k(const void *lhs, int lhs_dtype, const void *lh
         auto      st = static_cast<hipStream_t>(stream);
         uint32_t *wa = static_cast<uint32_t *>(workspace);
         uint32_t *wb = wa + round_up(Ml * W * 4, 256) / 4;
-        launch_transpose_words(static_cast<const uint32_t *>(lhs_scale), wa, Ml, W, ld / 32 / 4, st);
-        launch_transpose_words(static_cast<const uint32_t *>(rhs_scale), wb, Nr, W, ld / 32 / 4, st);
+        if (const int rc = launch_transpose_words(static_cast<const uint32_t *>(lhs_scale), wa, Ml, W, ld / 32 / 4, st))
+            return rc;
+        if (const int rc = launch_transpose_words(static_cast<const uint32_t *>(rhs_scale), wb, Nr, W, ld / 32 / 4, st))
+            return rc;
         g.sA        = reinterpret_cast<const float *>(wa);
         g.sB        = reinterpret_cast<const float *>(wb);
         g.sa_wpitch = Ml * 4;

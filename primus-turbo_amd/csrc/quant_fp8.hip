@@ -366,6 +366,114 @@ static int launch_quant_tensorwise(const void *x, int64_t n, void *q, const floa
     return check_launch("quant_tensorwise_kernel");
 }
 
+// ---------------------------------------------------------------------------
+// Two-launch form of the tensorwise quantizer: per-workgroup abs-max into `partial`, then a
+// second launch in which every workgroup takes the maximum of all partials, forms the scale and
+// casts. No workgroup waits for another, so nothing depends on the launch being resident as a
+// whole (other streams may hold CUs, CU masks, HIP-graph replays beside eager work), at the
+// price of reading x twice (the second read finds a tensor of this size in the caches). The
+// launch structure of Primus-Turbo's own op (csrc/pytorch/quantization/quantization.cpp:44-90:
+// reduce, compute scale, cast) with the scale computation folded into the cast.
+// `partial` needs no clearing: launch 1 writes every word that launch 2 reads.
+// ---------------------------------------------------------------------------
+template <typename T, bool VEC16>
+__global__ __launch_bounds__(TW_THREADS) void tw_partial_amax_kernel(const T *__restrict__ x, const int64_t n,
+                                                                     float *__restrict__ partial) {
+    __shared__ float s_red[TW_THREADS / 64];
+    const int64_t    stride = static_cast<int64_t>(gridDim.x) * TW_THREADS;
+    const int64_t    tid0   = static_cast<int64_t>(blockIdx.x) * TW_THREADS + threadIdx.x;
+    float            amax   = 0.f;
+    if constexpr (VEC16) {
+        const int64_t units = n / TW_VEC;
+        const int64_t tail0 = units * TW_VEC;
+        constexpr int UNR   = 4; // loads requested together
+        int64_t       u     = tid0;
+        for (; u + (UNR - 1) * stride < units; u += UNR * stride) {
+            Unit16<T> t[UNR];
+#pragma unroll
+            for (int k = 0; k < UNR; ++k)
+                t[k].load(x + (u + k * stride) * TW_VEC);
+#pragma unroll
+            for (int k = 0; k < UNR; ++k)
+                amax = fmaxf(amax, t[k].amax());
+        }
+        for (; u < units; u += stride) {
+            Unit16<T> t;
+            t.load(x + u * TW_VEC);
+            amax = fmaxf(amax, t.amax());
+        }
+        if (blockIdx.x == 0 && tail0 + threadIdx.x < n)
+            amax = fmaxf(amax, fabsf(HP<T>::to_f32(x[tail0 + threadIdx.x])));
+    } else {
+        for (int64_t i = tid0; i < n; i += stride)
+            amax = fmaxf(amax, fabsf(HP<T>::to_f32(x[i])));
+    }
+    amax = block_max(amax, s_red);
+    if (threadIdx.x == 0)
+        partial[blockIdx.x] = amax;
+}
+
+template <typename T, bool E5M2, bool VEC16>
+__global__ __launch_bounds__(TW_THREADS) void tw_cast_from_partials_kernel(
+    const T *__restrict__ x, uint8_t *__restrict__ q, const int64_t n, const float *__restrict__ partial,
+    const int nparts, float *__restrict__ scale_inv_out, const float qmax) {
+    __shared__ float s_red[TW_THREADS / 64];
+    const int64_t    stride = static_cast<int64_t>(gridDim.x) * TW_THREADS;
+    const int64_t    tid0   = static_cast<int64_t>(blockIdx.x) * TW_THREADS + threadIdx.x;
+    float            amax   = 0.f;
+    for (int t = threadIdx.x; t < nparts; t += TW_THREADS)
+        amax = fmaxf(amax, partial[t]);
+    amax              = block_max(amax, s_red);
+    const float scale = qmax / fmaxf(amax, 1e-12f);
+    if (tid0 == 0)
+        scale_inv_out[0] = 1.0f / scale;
+    if constexpr (VEC16) {
+        const int64_t units = n / TW_VEC;
+        const int64_t tail0 = units * TW_VEC;
+        for (int64_t u = tid0; u < units; u += stride) {
+            Unit16<T> t;
+            t.load(x + u * TW_VEC);
+            st128_nt(q + u * TW_VEC, t.template quant<E5M2>(scale, qmax));
+        }
+        if (blockIdx.x == 0 && tail0 + threadIdx.x < n)
+            q[tail0 + threadIdx.x] = quant1<E5M2>(HP<T>::to_f32(x[tail0 + threadIdx.x]), scale, qmax);
+    } else {
+        for (int64_t i = tid0; i < n; i += stride)
+            q[i] = quant1<E5M2>(HP<T>::to_f32(x[i]), scale, qmax);
+    }
+}
+
+template <typename T, bool E5M2>
+static int launch_quant_tensorwise_two_pass(const void *x, int64_t n, void *q, float *scale_inv, float *partial,
+                                            hipStream_t stream) {
+    const float   qmax  = E5M2 ? 57344.0f : 448.0f;
+    const bool    vec   = aligned_to(x, 16) && aligned_to(q, 16);
+    const int     cus   = device_cu_count();
+    const int64_t units = vec ? n / TW_VEC : n;
+    const int64_t full  = cdiv(units, TW_THREADS);
+    int64_t       g1    = full < 1 ? 1 : (full > 2L * cus ? 2L * cus : full);
+    if (g1 > WS_MAX_BLOCKS)
+        g1 = WS_MAX_BLOCKS;
+    const int64_t g2 = full < 1 ? 1 : (full > 8L * cus ? 8L * cus : full);
+    const T      *xp = static_cast<const T *>(x);
+    auto         *qp = static_cast<uint8_t *>(q);
+    dim3          b(TW_THREADS);
+    if (vec)
+        tw_partial_amax_kernel<T, true><<<dim3(static_cast<unsigned>(g1)), b, 0, stream>>>(xp, n, partial);
+    else
+        tw_partial_amax_kernel<T, false><<<dim3(static_cast<unsigned>(g1)), b, 0, stream>>>(xp, n, partial);
+    const int rc = check_launch("tw_partial_amax_kernel");
+    if (rc != PT_OK)
+        return rc;
+    if (vec)
+        tw_cast_from_partials_kernel<T, E5M2, true>
+            <<<dim3(static_cast<unsigned>(g2)), b, 0, stream>>>(xp, qp, n, partial, static_cast<int>(g1), scale_inv, qmax);
+    else
+        tw_cast_from_partials_kernel<T, E5M2, false>
+            <<<dim3(static_cast<unsigned>(g2)), b, 0, stream>>>(xp, qp, n, partial, static_cast<int>(g1), scale_inv, qmax);
+    return check_launch("tw_cast_from_partials_kernel");
+}
+
 // y[8 u .. 8 u + 7] = T(fp8(q[8 u ..]) * s) for the pieces u = first, first + step, ... below
 // `units`: 8 code bytes in, 16 or 32 bytes out per lane (whole lines per wavefront on both sides),
 // four pieces per round requested together, streaming accesses (nothing here is read twice).
@@ -773,18 +881,20 @@ static int launch_dequant_rowwise(const void *q, int64_t B, int64_t M, int64_t N
 // neither it nor its caller allocates anything. One slot set per stream that has used the
 // entry point on the device (calls on one stream are ordered, calls on different streams
 // must not share slots), PT_TENSORWISE_STATIC_MAX_STREAMS of them: 66 KB per GPU, held
-// until the process ends.
+// until the process ends. A slot set belongs to a stream HANDLE from its first call until
+// pt_tensorwise_static_release(stream).
 // ---------------------------------------------------------------------------
 static __device__ __align__(256) uint64_t tw_scratch[PT_TENSORWISE_STATIC_MAX_STREAMS * WS_WORDS];
 
 // Device address of tw_scratch on the current device (the array's name is only a host-side
 // handle; every GPU holds its own copy at its own address) and the slot set of `stream`.
-static int static_scratch_for(hipStream_t stream, uint64_t **out) {
+// release = true: give the stream's slot set back instead (out is not written).
+static int static_scratch_for(hipStream_t stream, uint64_t **out, bool release = false) {
     constexpr int MAX_DEV = 64;
     struct PerDevice {
         uint64_t   *base = nullptr;
-        int         used = 0;
-        hipStream_t streams[PT_TENSORWISE_STATIC_MAX_STREAMS];
+        bool        taken[PT_TENSORWISE_STATIC_MAX_STREAMS]   = {};
+        hipStream_t streams[PT_TENSORWISE_STATIC_MAX_STREAMS] = {};
     };
     static PerDevice  table[MAX_DEV];
     static std::mutex mu;
@@ -802,17 +912,26 @@ static int static_scratch_for(hipStream_t stream, uint64_t **out) {
                                            hipGetErrorString(e));
         pd.base = static_cast<uint64_t *>(p);
     }
-    int idx = -1;
-    for (int i = 0; i < pd.used; ++i)
-        if (pd.streams[i] == stream)
+    int idx = -1, vacant = -1;
+    for (int i = 0; i < PT_TENSORWISE_STATIC_MAX_STREAMS; ++i) {
+        if (pd.taken[i] && pd.streams[i] == stream)
             idx = i;
+        if (!pd.taken[i] && vacant < 0)
+            vacant = i;
+    }
+    if (release) {
+        if (idx >= 0)
+            pd.taken[idx] = false; // the words stay as they are: generation tags need no clearing
+        return PT_OK;
+    }
     if (idx < 0) {
-        if (pd.used == PT_TENSORWISE_STATIC_MAX_STREAMS)
+        if (vacant < 0)
             return fail(PT_ERR_WORKSPACE,
-                        "pt_quantize_fp8_tensorwise_static: more distinct streams on this device "
-                        "than PT_TENSORWISE_STATIC_MAX_STREAMS; use pt_quantize_fp8_tensorwise "
-                        "with a workspace per stream");
-        idx             = pd.used++;
+                        "pt_quantize_fp8_tensorwise_static: PT_TENSORWISE_STATIC_MAX_STREAMS stream handles "
+                        "hold a slot set on this device; release one with pt_tensorwise_static_release, or "
+                        "use pt_quantize_fp8_tensorwise with a workspace per stream");
+        idx             = vacant;
+        pd.taken[idx]   = true;
         pd.streams[idx] = stream;
     }
     *out = pd.base + static_cast<size_t>(idx) * WS_WORDS;
@@ -898,6 +1017,27 @@ int pt_quantize_fp8_tensorwise_static(const void *x, int x_dtype, int64_t numel,
     }
     return quantize_fp8_tensorwise_common(x, x_dtype, numel, q, q_dtype, scale_in, scale_inv, ws,
                                           status, 0, 0, static_cast<hipStream_t>(stream));
+}
+
+int pt_tensorwise_static_release(void *stream) {
+    uint64_t *unused = nullptr;
+    return static_scratch_for(static_cast<hipStream_t>(stream), &unused, true);
+}
+
+int pt_quantize_fp8_tensorwise_two_pass(const void *x, int x_dtype, int64_t numel, void *q, int q_dtype,
+                                        float *scale_inv, void *workspace, size_t workspace_bytes,
+                                        void *stream) {
+    PT_TW_CHECK_ARGS();
+    if (workspace == nullptr || workspace_bytes < pt_quantize_fp8_tensorwise_workspace_bytes() ||
+        !aligned_to(workspace, 16))
+        return fail(PT_ERR_WORKSPACE,
+                    "pt_quantize_fp8_tensorwise_two_pass: workspace missing, too small or misaligned");
+    auto st = static_cast<hipStream_t>(stream);
+#define CALL(T, E5)                                                                                \
+    return launch_quant_tensorwise_two_pass<T, E5>(x, numel, q, scale_inv,                         \
+                                                   static_cast<float *>(workspace), st)
+    PT_DISPATCH_HP_FP8(x_dtype, q_dtype, CALL);
+#undef CALL
 }
 
 int pt_dequantize_fp8_tensorwise(const void *q, int q_dtype, int64_t numel, const float *scale_inv,

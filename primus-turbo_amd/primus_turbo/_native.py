@@ -67,6 +67,11 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_int, c_i64, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
     ),
+    "pt_tensorwise_static_release": (c_int, [c_void_p]),
+    "pt_quantize_fp8_tensorwise_two_pass": (
+        c_int,
+        [c_void_p, c_int, c_i64, c_void_p, c_int, c_void_p, c_void_p, c_size_t, c_void_p],
+    ),
     "pt_dequantize_fp8_tensorwise": (c_int, [c_void_p, c_int, c_i64, c_void_p, c_void_p, c_int, c_void_p]),
     "pt_quantize_fp8_rowwise": (
         c_int,

@@ -67,9 +67,11 @@ def _both_directions(x, dest_dtype, row: ScalingRecipe, col: ScalingRecipe, fp4:
     return list(fn(x, dest_dtype, None, 32, True, row, col))
 
 
-def _meta_pair(x, dest_dtype, rowwise: bool, fp4: bool):
+def _meta_pair(x, dest_dtype, rowwise: bool, fp4: bool, shuffle_scale: bool = False):
     shapes = Q._mx_shapes(x, dest_dtype, rowwise, not rowwise)
     q, s = (shapes[0], shapes[1]) if rowwise else (shapes[2], shapes[3])
+    if shuffle_scale:  # the shuffled scale of every matrix is padded (shuffle_scale_batched)
+        s = tuple(s[:-2]) + Q._scale_pad(s[-2], s[-1])
     mk = lambda shp, dt: torch.empty(shp, dtype=torch.uint8, device=x.device).view(dt)  # noqa: E731
     return [mk(q, dest_dtype), mk(s, _E8M0)]
 
@@ -99,7 +101,7 @@ def _quantize_mxfp8(input, dest_dtype, axis, padding_align_size, use_2d_block, s
 
 
 def _quantize_mxfp8_meta(input, dest_dtype, axis, padding_align_size, use_2d_block, shuffle_scale=False, shuffle_out=False):
-    return _meta_pair(input, dest_dtype, axis == input.dim() - 1, False)
+    return _meta_pair(input, dest_dtype, axis == input.dim() - 1, False, shuffle_scale)
 
 
 def _quantize_mxfp8_dual(input, dest_dtype, padding_align_size, rowwise_use_2d_block, colwise_use_2d_block,
@@ -111,8 +113,11 @@ def _quantize_mxfp8_dual(input, dest_dtype, padding_align_size, rowwise_use_2d_b
                             ScalingRecipe(colwise_use_2d_block, False, False, shuffle_colwise_scale, shuffle_colwise), False)
 
 
-def _quantize_mxfp8_dual_meta(input, dest_dtype, padding_align_size, *flags):
-    return _meta_pair(input, dest_dtype, True, False) + _meta_pair(input, dest_dtype, False, False)
+def _quantize_mxfp8_dual_meta(input, dest_dtype, padding_align_size, rowwise_use_2d_block, colwise_use_2d_block,
+                              shuffle_rowwise_scale=False, shuffle_rowwise=False, shuffle_colwise_scale=False,
+                              shuffle_colwise=False):
+    return (_meta_pair(input, dest_dtype, True, False, shuffle_rowwise_scale)
+            + _meta_pair(input, dest_dtype, False, False, shuffle_colwise_scale))
 
 
 def _quantize_mxfp4(input, dest_dtype, axis, padding_align_size, use_2d_block, use_sr, use_rht, shuffle_scale=False,
@@ -121,8 +126,9 @@ def _quantize_mxfp4(input, dest_dtype, axis, padding_align_size, use_2d_block, u
     return _one_direction(input, dest_dtype, axis, ScalingRecipe(use_2d_block, use_sr, use_rht, shuffle_scale, shuffle_out), True)
 
 
-def _quantize_mxfp4_meta(input, dest_dtype, axis, padding_align_size, *flags):
-    return _meta_pair(input, dest_dtype, axis == input.dim() - 1, True)
+def _quantize_mxfp4_meta(input, dest_dtype, axis, padding_align_size, use_2d_block, use_sr, use_rht, shuffle_scale=False,
+                         shuffle_out=False):
+    return _meta_pair(input, dest_dtype, axis == input.dim() - 1, True, shuffle_scale)
 
 
 def _quantize_mxfp4_dual(input, dest_dtype, padding_align_size, rowwise_use_2d_block, rowwise_use_sr, rowwise_use_rht,
@@ -135,8 +141,11 @@ def _quantize_mxfp4_dual(input, dest_dtype, padding_align_size, rowwise_use_2d_b
         ScalingRecipe(colwise_use_2d_block, colwise_use_sr, colwise_use_rht, shuffle_colwise_scale, shuffle_colwise), True)
 
 
-def _quantize_mxfp4_dual_meta(input, dest_dtype, padding_align_size, *flags):
-    return _meta_pair(input, dest_dtype, True, True) + _meta_pair(input, dest_dtype, False, True)
+def _quantize_mxfp4_dual_meta(input, dest_dtype, padding_align_size, rowwise_use_2d_block, rowwise_use_sr, rowwise_use_rht,
+                              colwise_use_2d_block, colwise_use_sr, colwise_use_rht, shuffle_rowwise_scale=False,
+                              shuffle_rowwise=False, shuffle_colwise_scale=False, shuffle_colwise=False):
+    return (_meta_pair(input, dest_dtype, True, True, shuffle_rowwise_scale)
+            + _meta_pair(input, dest_dtype, False, True, shuffle_colwise_scale))
 
 
 # ---------------------------------------------------------------------------------------------

@@ -11,6 +11,7 @@ libprimus_turbo_amd.so on the current stream.
 
 from __future__ import annotations
 
+import os
 from typing import List, Optional, Tuple
 
 import torch
@@ -54,6 +55,30 @@ def _bmn(shape, axis: int) -> Tuple[int, int, int]:
 _ext.define("quantize_fp8_tensorwise(Tensor input, ScalarType dest_dtype, Tensor? scale_opt=None) -> Tensor[]")
 
 
+# Which launch structure the dynamic tensorwise quantizer takes.
+#   "fused"    one launch with a grid-wide amax exchange (x read once). Needs every workgroup of the
+#              launch resident at once, which holds while nothing else keeps compute units busy
+#              for long; the exchange words of eager calls live in the library's static scratch.
+#   "two_pass" two launches, no exchange (x read twice): independent of what else runs on the GPU.
+# Default: fused for eager calls, two_pass under HIP-graph capture (a replay may run beside any
+# other work, and the static scratch is keyed by the capture stream, which every graph shares).
+# PRIMUS_TURBO_TENSORWISE_MODE=fused|two_pass or set_tensorwise_mode() override both.
+_TENSORWISE_MODES = ("auto", "fused", "two_pass")
+_tensorwise_mode = os.environ.get("PRIMUS_TURBO_TENSORWISE_MODE", "auto")
+if _tensorwise_mode not in _TENSORWISE_MODES:
+    raise RuntimeError(f"PRIMUS_TURBO_TENSORWISE_MODE must be one of {_TENSORWISE_MODES}")
+
+
+def set_tensorwise_mode(mode: str) -> str:
+    """Select the launch structure of the dynamic tensorwise quantizer; returns the previous mode.
+    Callers that run quantizers on several streams at once, or beside long kernels of other
+    streams, want "two_pass"."""
+    global _tensorwise_mode
+    _check(mode in _TENSORWISE_MODES, f"mode must be one of {_TENSORWISE_MODES}")
+    prev, _tensorwise_mode = _tensorwise_mode, mode
+    return prev
+
+
 def _quantize_fp8_tensorwise(input: torch.Tensor, dest_dtype: torch.dtype, scale_opt: Optional[torch.Tensor] = None):
     N.require_cuda(input, scale_opt)
     _check(input.dtype in _HP_DTYPES, "input must be bfloat16, float16 or float32")
@@ -66,35 +91,31 @@ def _quantize_fp8_tensorwise(input: torch.Tensor, dest_dtype: torch.dtype, scale
     if scale_opt is not None:
         _check(scale_opt.numel() == 1, "tensorwise scale must be scalar tensor")
         scale_in = scale_opt.to(torch.float32).contiguous()
-    # The grid exchange of the fused kernel keeps its words in the library's static device
-    # scratch (one slot set per stream): no per-call allocation or fill. A lost exchange shows
-    # as NaN in scale_inv (see the header), so nothing is read back here.
-    status = lib.pt_quantize_fp8_tensorwise_static(
-        N.ptr(input),
-        N.dtype_code(input.dtype),
-        input.numel(),
-        N.ptr(out),
-        N.dtype_code(dest_dtype),
-        N.ptr(scale_in),
-        N.ptr(scale_inv),
-        None,
-        N.stream_of(input),
-    )
+    capturing = torch.cuda.is_current_stream_capturing()
+    mode = _tensorwise_mode
+    if mode == "auto":
+        mode = "two_pass" if capturing else "fused"
+    head = (N.ptr(input), N.dtype_code(input.dtype), input.numel(), N.ptr(out), N.dtype_code(dest_dtype))
+    if scale_in is None and mode == "two_pass":
+        # (the partial maxima need no zero-fill; the buffer comes from the capture's own pool)
+        ws = torch.empty(lib.pt_quantize_fp8_tensorwise_workspace_bytes(), dtype=torch.uint8, device=input.device)
+        N.check(lib.pt_quantize_fp8_tensorwise_two_pass(*head, N.ptr(scale_inv), N.ptr(ws), ws.numel(), N.stream_of(input)))
+        return [out, scale_inv]
+    if scale_in is not None:  # static scale: one cast launch, no exchange and no workspace
+        N.check(lib.pt_quantize_fp8_tensorwise(*head, N.ptr(scale_in), N.ptr(scale_inv), None, 0, N.stream_of(input)))
+        return [out, scale_inv]
+    status = N.PT_ERR_WORKSPACE
+    if not capturing:
+        # The grid exchange of the fused kernel keeps its words in the library's static device
+        # scratch (one slot set per stream handle): no per-call allocation or fill. A lost exchange
+        # shows as NaN in scale_inv (see the header), so nothing is read back here.
+        status = lib.pt_quantize_fp8_tensorwise_static(*head, None, N.ptr(scale_inv), None, N.stream_of(input))
     if status == N.PT_ERR_WORKSPACE:
-        # more streams in use on this device than the static scratch has slot sets
+        # under capture (every graph captured on torch's capture stream would share that stream's
+        # static slot set, and replays of two graphs may overlap), or with more stream handles on
+        # this device than the static scratch has slot sets: a zero-filled workspace of this call
         ws = N.zeroed_workspace(input.device, lib.pt_quantize_fp8_tensorwise_workspace_bytes())
-        status = lib.pt_quantize_fp8_tensorwise(
-            N.ptr(input),
-            N.dtype_code(input.dtype),
-            input.numel(),
-            N.ptr(out),
-            N.dtype_code(dest_dtype),
-            N.ptr(scale_in),
-            N.ptr(scale_inv),
-            N.ptr(ws),
-            ws.numel(),
-            N.stream_of(input),
-        )
+        status = lib.pt_quantize_fp8_tensorwise(*head, None, N.ptr(scale_inv), N.ptr(ws), ws.numel(), N.stream_of(input))
     N.check(status)
     return [out, scale_inv]
 

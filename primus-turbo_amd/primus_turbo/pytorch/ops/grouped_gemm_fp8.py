@@ -108,8 +108,9 @@ def _block_forward_product(a_fp8_row, a_scale_row, b, group_lens, group_offs, tr
 
 
 def _block_backward_products(grad_out, a_fp8_col_t, a_scale_col, b_fp8, b_scale, group_lens, group_offs, trans_b, config,
-                             out_dtype, num_cu, b_ready, fuse_bgrad_accum, main_grad):
-    """dgrad and variable-K wgrad of the BLOCKWISE grouped layer -> ``(grad_a, grad_b)``."""
+                             dgrad_dtype, wgrad_dtype, num_cu, b_ready, fuse_bgrad_accum, main_grad):
+    """dgrad and variable-K wgrad of the BLOCKWISE grouped layer -> ``(grad_a, grad_b)``; the
+    activation gradient comes out in ``dgrad_dtype``, the weight gradient in ``wgrad_dtype``."""
     g_dtype = _get_fp8_dtype(config.format, False)
     gran = config.granularity.value
     g_row, g_col_t, g_scale_row, g_scale_col, var_k_lens, var_k_offs = quant_fp8_blockwise_segment_m_row_col_t_impl(
@@ -117,10 +118,10 @@ def _block_backward_products(grad_out, a_fp8_col_t, a_scale_col, b_fp8, b_scale,
     # grad_a = grad_out @ b^T: the saved weight copy is contiguous along the reduction already,
     # or (caller-quantized weight) the forward operand read the other way round
     grad_a = grouped_gemm_fp8_impl(g_row, b_fp8, g_scale_row, b_scale, group_lens, group_offs, False,
-                                   True if b_ready else not trans_b, out_dtype, gran, num_cu, _NATIVE)
+                                   True if b_ready else not trans_b, dgrad_dtype, gran, num_cu, _NATIVE)
     # grad_b[g] = a_g^T @ grad_out_g over the padded token ranges, both operands K-major
     grad_b = _grouped_gemm_fp8_variable_k_impl_wrapper(
-        a_fp8_col_t, g_col_t, a_scale_col, g_scale_col, var_k_lens, var_k_offs, False, True, trans_b, out_dtype, gran,
+        a_fp8_col_t, g_col_t, a_scale_col, g_scale_col, var_k_lens, var_k_offs, False, True, trans_b, wgrad_dtype, gran,
         num_cu, _NATIVE, inplace_add_to_out=fuse_bgrad_accum, out=main_grad,
     )
     return grad_a, grad_b
@@ -169,7 +170,8 @@ class FP8GroupedGemmBlockFunc(torch.autograd.Function):
         a_fp8_col_t, a_scale_col, b_fp8, b_scale, group_lens, group_offs = ctx.saved_tensors
         trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad, b_ready = ctx.meta
         grad_a, grad_b = _block_backward_products(grad_out, a_fp8_col_t, a_scale_col, b_fp8, b_scale, group_lens, group_offs,
-                                                  trans_b, config, out_dtype, num_cu, b_ready, fuse_bgrad_accum, main_grad)
+                                                  trans_b, config, out_dtype, out_dtype, num_cu, b_ready, fuse_bgrad_accum,
+                                                  main_grad)
         return grad_a, grad_b, None, None, None, None, None, None, None, None, None
 
 
@@ -208,7 +210,8 @@ class FP8GluGroupedGemmBlockFunc(torch.autograd.Function):
         x2, p1, row_mask, a_col_t, a_scale_col, b_fp8, b_scale, group_lens, group_offs = ctx.saved_tensors
         trans_b, config, out_dtype, num_cu, fuse_bgrad_accum, main_grad, b_ready, act_type, probs_shape = ctx.meta
         grad_act, grad_b = _block_backward_products(grad_out, a_col_t, a_scale_col, b_fp8, b_scale, group_lens, group_offs,
-                                                    trans_b, config, x2.dtype, num_cu, b_ready, fuse_bgrad_accum, main_grad)
+                                                    trans_b, config, x2.dtype, out_dtype, num_cu, b_ready, fuse_bgrad_accum,
+                                                    main_grad)
         grad_x, grad_probs = glu_bwd_with_probs(grad_act, x2, p1, row_mask, ACT_SILU if act_type == "silu" else ACT_GELU)
         return grad_x, grad_probs.view(probs_shape), None, None, grad_b, None, None, None, None, None, None, None
 
@@ -501,7 +504,8 @@ def glu_grouped_gemm_fp8(
     """``grouped_gemm_fp8(swiglu_with_probs(x, probs, row_mask), b, group_lens, ...)`` (``act_type="gelu"``:
     ``geglu_with_probs``) as one operation for the BLOCKWISE and MX_BLOCKWISE configurations: fc1's output ``x [tokens, 2 H]``
     is read once by a quantizer that applies the gated activation on load, so the bf16 activation
-    never goes through HBM; results and gradients are bit-identical with the two-step form. (The
+    never goes through HBM; results and gradients are bit-identical with the two-step form when ``x``, ``b`` and
+    ``out_dtype`` are one type (otherwise the activation gradient is written in ``x``'s type directly). (The
     reference has the two steps only: ops/activation.py:21-83, ops/grouped_gemm_fp8.py:99-265.)"""
     if config is None:
         config = Float8QuantConfig(granularity=ScalingGranularity.BLOCKWISE, block_size=128)

@@ -66,3 +66,17 @@ def group_lens(kind, G_, total, seed):
         lens[np.argmax(lens)] += total - lens.sum()
         return lens
     raise ValueError(kind)
+
+
+def gemm_gate(ref, got, what="", min_cos=0.9999, max_rel=1e-2, max_fro=1e-2, elementwise=True):
+    """The GEMM gate of the parity tests: cosine similarity, error relative to the output's range,
+    the Frobenius-relative error of the reference's own tests (tests/pytorch/test_utils.py:43-45) and
+    an element-wise bound |err| <= 2^-7 |ref| + 2^-7 rms(ref row), under which a wrong scale on one
+    row block cannot hide behind the output's range. Returns the four figures."""
+    from oracle import gemm as OG
+
+    cos, rel, fro = OG.cosine(ref, got), OG.max_rel_err(ref, got), OG.rel_fro(ref, got)
+    exc = OG.elementwise_excess(ref, got) if elementwise else 0.0
+    msg = f"{what}: cosine {cos:.6f}, max err / range {rel:.3e}, rel fro {fro:.3e}, element-wise excess {exc:.3f}"
+    assert cos >= min_cos and rel <= max_rel and fro <= max_fro and exc <= 1.0, msg
+    return {"cosine": cos, "max_rel_err": rel, "rel_fro": fro, "elementwise_excess": exc}

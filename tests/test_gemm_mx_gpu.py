@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import bf16_randn, codes_np, to_f32_np
+from helpers import bf16_randn, codes_np, gemm_gate, to_f32_np
 from oracle import gemm as OG
 from oracle import quantize as Q
 
@@ -34,8 +34,7 @@ def _turbo(native_lib):
 
 
 def _gate(ref, got, what=""):
-    cos, rel = OG.cosine(ref, got), OG.max_rel_err(ref, got)
-    assert cos >= MIN_COS and rel <= MAX_REL, f"{what}: cosine {cos:.6f}, max rel err {rel:.3e}"
+    return gemm_gate(ref, got, what)
 
 
 SHAPES = [(256, 256, 384), (512, 384, 1024), (130, 70, 160), (64, 96, 96), (1024, 2048, 512), (300, 260, 2080)]
@@ -103,6 +102,33 @@ def test_mx_gemm_eight_wavefront_tile(M, N, K, fmt):
     ref = OG.gemm_dequantized(Q.mx_dequant(codes_np(aq), codes_np(as_), fmt),
                               Q.mx_dequant(codes_np(bq), codes_np(bs), "e2m1" if fmt == "e2m1" else "e4m3"))
     _gate(ref, to_f32_np(got), f"mx8 {fmt} {M}x{N}x{K}")
+
+
+def test_mx_gemm_without_workspace_reads_scales_in_place():
+    """Whole-slab operand rows need no copy: pt_gemm_mx then works with no workspace at all (the
+    word-major scale copy of large problems is an option that a sufficient workspace buys), and
+    gives the same bits either way."""
+    from primus_turbo import _native as N
+
+    lib = N.lib()
+    M, Nn, K = 1024, 1280, 2048
+    a = bf16_randn((M, K), seed=73, outlier_frac=0.002).cuda()
+    b = bf16_randn((Nn, K), seed=74).cuda()
+    aq, as_ = qi.quantize_mxfp8_impl(a, torch.float8_e4m3fn, 1, 32)
+    bq, bs = qi.quantize_mxfp8_impl(b, torch.float8_e4m3fn, 1, 32)
+    want = lib.pt_gemm_mx_workspace_bytes(M, Nn, K, K, K, 0)
+    assert want > 0, "a problem of this size takes the word-major scale copy when it can"
+    outs = []
+    for ws in (torch.empty(want, dtype=torch.uint8, device="cuda"), None):
+        out = torch.empty((M, Nn), dtype=torch.bfloat16, device="cuda")
+        N.check(lib.pt_gemm_mx(N.ptr(aq), N.ptr(as_), N.ptr(bq), N.ptr(bs), N.dtype_code(aq.dtype), 0, 0, N.ptr(out),
+                               N.dtype_code(out.dtype), M, Nn, K, K, K, as_.shape[1], bs.shape[1], 0, N.ptr(ws),
+                               0 if ws is None else ws.numel(), 0, N.stream_of(aq)))
+        outs.append(out)
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1])
+    ref = OG.gemm_dequantized(Q.mx_dequant(codes_np(aq), codes_np(as_), "e4m3"), Q.mx_dequant(codes_np(bq), codes_np(bs), "e4m3"))
+    _gate(ref, to_f32_np(outs[1]), "mxfp8 without workspace")
 
 
 @pytest.mark.parametrize("tile_cfg", [0, 4])

@@ -109,6 +109,38 @@ def test_fused_activation_grouped_gemm_equals_the_two_step_layer(act, trans_b):
     assert torch.equal(out, a[0])
 
 
+def test_fused_activation_grouped_gemm_mixed_dtypes():
+    """fp16 activations, a bf16 weight and an explicit out_dtype: the activation gradient comes
+    back in the activation's type and the weight gradient in out_dtype."""
+    G_, M, H, N = 4, 1024, 256, 384
+    lens, gl, offs, x, probs, mask = _inputs("ragged", G_, M, H, torch.float16, 97, False)
+    w = bf16_randn((G_, N, H), seed=98, scale=0.05).cuda()
+    dy = bf16_randn((M, N), seed=99).cuda()
+    cfg = Float8QuantConfig(granularity=G.BLOCKWISE, block_size=128)
+
+    def run(fused):
+        xx, pp, ww = x.clone().requires_grad_(True), probs.clone().requires_grad_(True), w.clone().requires_grad_(True)
+        if fused:
+            out = turbo.ops.glu_grouped_gemm_fp8(xx, pp, ww, gl, offs, trans_b=True, config=cfg, act_type="silu",
+                                                 out_dtype=torch.bfloat16)
+        else:
+            out = turbo.ops.grouped_gemm_fp8(turbo.ops.swiglu_with_probs(xx, pp, None), ww, gl, offs, trans_b=True,
+                                             out_dtype=torch.bfloat16, config=cfg)
+        assert out.dtype == torch.bfloat16
+        out.backward(dy)
+        return out.detach(), xx.grad, pp.grad, ww.grad
+
+    a, b = run(True), run(False)
+    assert a[1].dtype == torch.float16 and a[3].dtype == torch.bfloat16
+    for name, u, v in zip(("out", "grad_x", "grad_probs", "grad_w"), a, b):
+        assert u.dtype == v.dtype, name
+    assert torch.equal(a[0], b[0]) and torch.equal(a[3], b[3]), "output and weight gradient: same GEMMs, same types"
+    # the two-step form rounds the activation gradient to out_dtype (bf16) before autograd casts it to
+    # fp16; the fused form writes fp16 from the fp32 sums directly: equal up to that bf16 rounding
+    for u, v in ((a[1], b[1]), (a[2], b[2])):
+        assert (u.float() - v.float()).norm() <= 2.0 ** -7 * v.float().norm()
+
+
 # ---- the grouped MX quantizers (MXFP8 / MXFP4) with the gated activation applied on load ----
 MX_CASES = [("balanced", 4, 1024, 512, False), ("ragged", 8, 3000, 384, True), ("zeros", 8, 2048, 256, False),
             ("ragged", 3, 77, 96, True), ("zipf", 32, 8192, 2048, True)]

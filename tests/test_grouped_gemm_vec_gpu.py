@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import bf16_randn, codes_np, group_lens, to_f32_np
+from helpers import bf16_randn, codes_np, gemm_gate, group_lens, to_f32_np
 from oracle import gemm as OG
 from oracle import quantize as Q
 
@@ -25,8 +25,7 @@ def _turbo(native_lib):
 
 
 def _gate(ref, got, what=""):
-    cos, rel = OG.cosine(ref, got), OG.max_rel_err(ref, got)
-    assert cos >= 0.9999 and rel <= 1e-2, f"{what}: cosine {cos:.6f}, max rel err {rel:.3e}"
+    return gemm_gate(ref, got, what)
 
 
 def _offs(lens):

@@ -59,6 +59,37 @@ def test_graph_tensorwise_quantize_dequantize():
     _replay_check(fn, lambda seed: (bf16_randn((1024, 1024), seed=100 + seed, outlier_frac=0.001) * (1 + seed),), 1)
 
 
+def test_two_graphs_on_the_capture_stream_tensorwise():
+    """Two graphs captured one after the other on torch's capture stream, each holding a dynamic
+    tensorwise quantizer, replayed in order (and the first again): neither may see the other's
+    abs-max. Nothing of a captured quantizer lives in per-stream state of the library."""
+    import numpy as np
+
+    from helpers import bits_np, codes_np, to_f32_np
+    from oracle import quantize as Q
+
+    xa = bf16_randn((1024, 1024), seed=170, outlier_frac=0.001).cuda()
+    xb = (bf16_randn((512, 2048), seed=171) * 37.0).cuda()
+    turbo.ops.quantize_fp8(xa, turbo.float8_e4m3, G.TENSORWISE)  # one-time set-up outside the captures
+    torch.cuda.synchronize()
+    ga, gb = torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()
+    with torch.cuda.graph(ga):
+        qa, sa = turbo.ops.quantize_fp8(xa, turbo.float8_e4m3, G.TENSORWISE)
+    with torch.cuda.graph(gb):
+        qb, sb = turbo.ops.quantize_fp8(xb, turbo.float8_e4m3, G.TENSORWISE)
+    for rep in range(3):
+        xa.mul_(1.5)
+        ga.replay()
+        gb.replay()
+        turbo.ops.quantize_fp8(xb, turbo.float8_e4m3, G.TENSORWISE)  # eager work on the same stream
+        ga.replay()
+        torch.cuda.synchronize()
+        for x, q, s in ((xa, qa, sa), (xb, qb, sb)):
+            oq, osinv = Q.fp8_tensorwise(to_f32_np(x.cpu()), "e4m3")
+            assert bits_np(s).item() == osinv.view(np.uint32).item(), rep
+            assert np.array_equal(codes_np(q), oq), rep
+
+
 @pytest.mark.parametrize("gran", ["ROWWISE", "BLOCKWISE", "MX_BLOCKWISE"])
 def test_graph_gemm_fp8_forward(gran):
     kw = {"BLOCKWISE": dict(block_size=128), "MX_BLOCKWISE": dict(block_size=32, scale_dtype=ScaleDtype.E8M0)}.get(gran, {})

@@ -91,6 +91,27 @@ def test_quantize_mxfp4_and_dual_and_dequantize():
     assert np.array_equal(codes_np(hq), rq) and np.array_equal(codes_np(hs), rs)
 
 
+def test_meta_shapes_with_shuffled_scales():
+    """shuffle_scale pads the scale of every matrix (rows to 256, columns to 8): the Meta
+    implementations have to say so too, also for 3-D input and where M is no multiple of 256."""
+    for shape in ((200, 320), (3, 136, 160)):
+        x = bf16_randn(shape, seed=73).cuda()
+        dt = torch.float8_e4m3fn
+        for axis in (x.dim() - 1, x.dim() - 2):
+            args = (x, dt, axis, 128, False, True, False)
+            outs = ext.quantize_mxfp8(*args)
+            assert tuple(outs[1].shape[-2:]) == Qi._scale_pad(*outs[1].shape[-2:])  # padded already
+            _same_meta(ext.quantize_mxfp8, args, outs)
+        for flags in ((True, False, False, False), (False, False, True, False), (True, False, True, False)):
+            args = (x, dt, 128, False, False) + flags
+            _same_meta(ext.quantize_mxfp8_dual, args, ext.quantize_mxfp8_dual(*args))
+        if F4 is not None:
+            args = (x, F4, x.dim() - 1, 128, False, False, False, True, False)
+            _same_meta(ext.quantize_mxfp4, args, ext.quantize_mxfp4(*args))
+            args = (x, F4, 128, False, False, False, False, False, False, True, False, True, False)
+            _same_meta(ext.quantize_mxfp4_dual, args, ext.quantize_mxfp4_dual(*args))
+
+
 def test_grouped_quantize_mxfp8_names():
     G_, M, N = 6, 700, 256
     lens = group_lens("ragged", G_, M, 73)

@@ -171,6 +171,27 @@ def test_metric_hand_values():
     assert OG.max_rel_err(np.zeros(3), np.array([0.0, 3.0, -1.0])) == 3.0
     assert OG.max_rel_err(y, ref) == 0.5 / 20.0 and OG.max_rel_err(2 * ref, 2 * y) == 0.5 / 20.0
 
+    # |y - ref|_F / |ref|_F: ref (3, 4), error (0.3, 0.4) -> 0.5 / 5
+    assert math.isclose(OG.rel_fro([3.0, 4.0], [3.3, 4.4]), 0.1, rel_tol=1e-12)
+    assert OG.rel_fro([3.0, 4.0], [3.0, 4.0]) == 0.0 and OG.rel_fro([0.0, 0.0], [3.0, 4.0]) == 5.0
+    assert math.isclose(OG.rel_fro(ref, y), math.sqrt(0.5) / math.sqrt(100 + 400 + 0.25), rel_tol=1e-12)
+
+    # element-wise bound |err| <= r |ref| + r rms(row): row (3, 4) has rms sqrt(12.5)
+    r = 2.0 ** -7
+    rms = math.sqrt(12.5)
+    assert math.isclose(OG.elementwise_excess([3.0, 4.0], [3.0, 4.0 + 0.01]), 0.01 / (r * 4 + r * rms), rel_tol=1e-12)
+    assert OG.elementwise_excess([3.0, 4.0], [3.0, 4.0]) == 0.0
+    # rows are judged on their own: the same 0.05 error passes in a row of large values and fails in a small one
+    big_small = np.array([[100.0, -100.0, 100.0], [0.1, -0.1, 0.1]])
+    e1, e2 = big_small.copy(), big_small.copy()
+    e1[0, 1] += 0.05
+    e2[1, 1] += 0.05
+    assert OG.elementwise_excess(big_small, e1) < 1 < OG.elementwise_excess(big_small, e2)
+    # what the range-relative gate cannot see: both read 5e-4 there
+    assert math.isclose(OG.max_rel_err(big_small, e1), 5e-4, rel_tol=1e-9) and math.isclose(OG.max_rel_err(big_small, e2), 5e-4, rel_tol=1e-9)
+    assert OG.elementwise_excess(np.zeros((2, 2)), np.zeros((2, 2))) == 0.0
+    assert OG.elementwise_excess(np.zeros((2, 2)), np.array([[0.0, 1e-30], [0.0, 0.0]])) == math.inf
+
     # 10 log10(|ref|^2 / |ref - y|^2): ref (3, 4), noise (0.3, 0.4) -> 25 / 0.25 = 100 -> 20 dB
     assert math.isclose(OG.snr_db([3.0, 4.0], [3.3, 4.4]), 20.0, abs_tol=1e-9)
     assert math.isclose(OG.snr_db([3.0, 4.0], [3.0 + 3, 4.0 + 4]), 0.0, abs_tol=1e-9)
@@ -192,6 +213,7 @@ def test_metrics_against_torch_formulas():
     assert math.isclose(OG.cosine(ref, y), cos, abs_tol=2e-6)
     assert math.isclose(OG.snr_db(ref, y), snr, abs_tol=1e-3)
     assert math.isclose(OG.max_rel_err(ref, y), (tr - ty).abs().max().item() / tr.abs().max().item(), rel_tol=1e-6)
+    assert math.isclose(OG.rel_fro(ref, y), (torch.norm(tr - ty) / torch.norm(tr)).item(), rel_tol=1e-5)
 
 
 # ---------------------------------------------------------------------------------------------

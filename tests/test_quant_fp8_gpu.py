@@ -209,3 +209,79 @@ def test_tensorwise_lost_grid_exchange_is_visible():
     torch.cuda.synchronize()
     oq, osinv = Q.fp8_tensorwise(to_f32_np(x), "e4m3")
     assert status.item() == 0 and np.array_equal(codes_np(q), oq)
+
+
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+@pytest.mark.parametrize("src", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(4096, 4096), (333, 257), (1,), (17,), (2881,), (256 * 1024 * 16 * 2 + 3,)])
+def test_tensorwise_two_pass_bit_exact(shape, src, dtype):
+    """The two-launch form (no exchange between workgroups) through the C ABI: same bytes and the
+    same scale as the oracle, hence as the fused kernel; its workspace is deliberately dirty."""
+    if (shape[0] >= 4096) and src != torch.bfloat16:
+        pytest.skip("large sizes only for bf16")
+    from primus_turbo import _native as N
+
+    lib = N.lib()
+    x = bf16_randn(shape, seed=21, outlier_frac=0.001, dtype=src)
+    xg = x.cuda()
+    q = torch.empty_like(xg, dtype=dtype)
+    sinv = torch.zeros((), dtype=torch.float32, device="cuda")
+    ws = torch.full((lib.pt_quantize_fp8_tensorwise_workspace_bytes(),), 0x7F, dtype=torch.uint8, device="cuda")
+    for _ in range(2):
+        N.check(lib.pt_quantize_fp8_tensorwise_two_pass(
+            N.ptr(xg), N.dtype_code(src), xg.numel(), N.ptr(q), N.dtype_code(dtype), N.ptr(sinv), N.ptr(ws), ws.numel(),
+            N.stream_of(xg)))
+    torch.cuda.synchronize()
+    oq, osinv = Q.fp8_tensorwise(to_f32_np(x), FMT[dtype])
+    assert bits_np(sinv).item() == osinv.view(np.uint32).item()
+    assert np.array_equal(codes_np(q), oq)
+
+
+def test_tensorwise_two_pass_special_values_and_unaligned():
+    from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+    prev = qi.set_tensorwise_mode("two_pass")
+    try:
+        x = torch.zeros(1000, dtype=torch.bfloat16)
+        _check_tensorwise(x, torch.float8_e4m3fn)
+        x = bf16_randn((4096,), 3)
+        x[5] = float("nan")
+        _check_tensorwise(x, torch.float8_e4m3fn)
+        x[9] = float("inf")
+        _check_tensorwise(x, torch.float8_e4m3fn)
+        base = bf16_randn((4096 * 8 + 16,), 5, outlier_frac=0.01)
+        for off in (1, 3, 8):
+            xg = base.cuda()[off : off + 4096 * 8]
+            q, sinv = turbo.ops.quantize_fp8(xg, torch.float8_e4m3fn, G.TENSORWISE)
+            oq, osinv = Q.fp8_tensorwise(to_f32_np(base[off : off + 4096 * 8]), "e4m3")
+            assert np.array_equal(codes_np(q), oq) and bits_np(sinv).item() == osinv.view(np.uint32).item()
+    finally:
+        qi.set_tensorwise_mode(prev)
+    with pytest.raises(RuntimeError):
+        qi.set_tensorwise_mode("three_pass")
+
+
+def test_tensorwise_quantizers_on_concurrent_streams_two_pass():
+    """Several streams quantizing at once: the two-launch form has no cross-workgroup wait, so
+    every stream's result is exact whatever the others hold of the GPU."""
+    from primus_turbo.pytorch.kernels.quantization import quantization_impl as qi
+
+    prev = qi.set_tensorwise_mode("two_pass")
+    try:
+        xs = [bf16_randn((2048, 2048), seed=40 + i, outlier_frac=0.001) * (1 + i) for i in range(4)]
+        xg = [x.cuda() for x in xs]
+        streams = [torch.cuda.Stream() for _ in xs]
+        torch.cuda.synchronize()
+        outs = []
+        for _ in range(3):
+            outs = []
+            for x, st in zip(xg, streams):
+                with torch.cuda.stream(st):
+                    outs.append(turbo.ops.quantize_fp8(x, torch.float8_e4m3fn, G.TENSORWISE))
+        torch.cuda.synchronize()
+        for x, (q, sinv) in zip(xs, outs):
+            oq, osinv = Q.fp8_tensorwise(to_f32_np(x), "e4m3")
+            assert bits_np(sinv).item() == osinv.view(np.uint32).item()
+            assert np.array_equal(codes_np(q), oq)
+    finally:
+        qi.set_tensorwise_mode(prev)

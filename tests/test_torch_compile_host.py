@@ -109,3 +109,16 @@ def test_grouped_linear_traces_fullgraph(turbo, gran):
     lens = torch.empty(4, device="meta", dtype=torch.int64)
     out = _trace(mod, x, lens)
     assert out.shape == (1024, 512) and x.grad.shape == x.shape and mod.weight.grad.shape == (4, 512, 512)
+
+
+def test_mx_dispatcher_meta_shapes_with_shuffled_scales(turbo):
+    """Shape functions of the dense MX quantizer operators with shuffle_scale: the scale of every
+    matrix is padded to (256, 8) multiples, as the device path returns it."""
+    ext = torch.ops.primus_turbo_cpp_extension
+    x = torch.empty(3, 136, 160, device="meta", dtype=torch.bfloat16)
+    q, s = ext.quantize_mxfp8(x, torch.float8_e4m3fn, 2, 128, False, True, False)
+    assert tuple(q.shape) == (3, 136, 256) and tuple(s.shape) == (3, 256, 8)
+    q, s = ext.quantize_mxfp8(x, torch.float8_e4m3fn, 2, 128, False, False, False)
+    assert tuple(s.shape) == (3, 136, 8)
+    rq, rs, cq, cs = ext.quantize_mxfp8_dual(x, torch.float8_e4m3fn, 128, False, False, False, False, True, False)
+    assert tuple(rs.shape) == (3, 136, 8) and tuple(cq.shape) == (3, 160, 256) and tuple(cs.shape) == (3, 256, 8)

@@ -85,3 +85,50 @@ def test_static_entry_point_on_a_side_stream_and_its_limits():
     too_many = ctypes.c_int64(1 << 38)
     rc = lib.pt_quantize_fp8_tensorwise_static(N.ptr(x), 0, too_many, N.ptr(q), 3, None, N.ptr(sinv), None, None)
     assert rc == N.PT_ERR_INVALID_ARGUMENT and b"MAX_NUMEL" in lib.pt_last_error()
+
+
+def test_static_slot_sets_are_released_and_reused():
+    """A stream handle keeps its slot set until pt_tensorwise_static_release: fill the table, see the
+    next handle refused, release one, see it served, and give every set of this test back."""
+    from primus_turbo import _native as N
+
+    lib = N.lib()
+    x = bf16_randn((256, 512), seed=16).cuda()
+    q_ref = torch.empty_like(x, dtype=torch.float8_e4m3fn)
+    sinv_ref = torch.zeros((), dtype=torch.float32, device="cuda")
+    ws = torch.zeros(lib.pt_quantize_fp8_tensorwise_workspace_bytes(), dtype=torch.uint8, device="cuda")
+    N.check(_call_workspace(lib, N, x, q_ref, sinv_ref, ws))
+    torch.cuda.synchronize()
+    streams, held, refused = [torch.cuda.Stream() for _ in range(10)], [], None
+    assert len({s.cuda_stream for s in streams}) == 10
+    try:
+        for st in streams:
+            with torch.cuda.stream(st):
+                q = torch.empty_like(x, dtype=torch.float8_e4m3fn)
+                sinv = torch.zeros((), dtype=torch.float32, device="cuda")
+                rc = _call_static(lib, N, x, q, sinv, None)
+            st.synchronize()
+            if rc == N.PT_ERR_WORKSPACE:
+                refused = st
+                break
+            N.check(rc)
+            held.append(st)
+            assert np.array_equal(codes_np(q), codes_np(q_ref)) and sinv.item() == sinv_ref.item()
+        assert refused is not None and len(held) <= 8, "the table holds eight stream handles per device"
+        # (earlier tests of the session may hold sets too: with none of this test's own, the idle
+        # default stream's set is the one given back)
+        victim = held[0].cuda_stream if held else torch.cuda.default_stream().cuda_stream
+        assert lib.pt_tensorwise_static_release(victim) == 0
+        assert lib.pt_tensorwise_static_release(victim) == 0  # holding nothing is no error
+        with torch.cuda.stream(refused):
+            q = torch.empty_like(x, dtype=torch.float8_e4m3fn)
+            sinv = torch.zeros((), dtype=torch.float32, device="cuda")
+            for _ in range(2):  # the set it inherits carries the previous owner's tags
+                N.check(_call_static(lib, N, x, q, sinv, None))
+        refused.synchronize()
+        held = held[1:] + [refused]
+        assert np.array_equal(codes_np(q), codes_np(q_ref)) and sinv.item() == sinv_ref.item()
+    finally:
+        torch.cuda.synchronize()
+        for st in held:
+            lib.pt_tensorwise_static_release(st.cuda_stream)
