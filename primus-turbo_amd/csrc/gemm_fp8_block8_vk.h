@@ -290,7 +290,7 @@ __global__ __launch_bounds__(B8_THREADS) void gemm_fp8_block8_vk_kernel(const Ge
             const int64_t wm_base = m0 + wm * (TM * 16), wn_base = n0 + wn * (TN * 16);
             // stores of the epilogue's straight-line path (0, 16 or 32: the cases of the barrier's wait)
             pending = __builtin_amdgcn_readfirstlane(
-                epilogue<TM, TN, SCALE_BLOCK, false>(a, acc, Cg, a.sA, a.sB, a.M, wm_base, wn_base, lane));
+                epilogue<TM, TN, SCALE_BLOCK, false, false>(a, acc, Cg, a.sA, a.sB, a.M, wm_base, wn_base, lane));
             static_assert(TM * TN == 32, "the barrier's wait distinguishes 16 and 32 stores in flight");
             PT_GEMM_TRACE_POINT(6);
             pos  = g_hi;

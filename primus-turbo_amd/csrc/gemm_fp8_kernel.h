@@ -197,6 +197,66 @@ __device__ __forceinline__ void tile_coords_local(int lid, int tiles_m, int tile
     tn                 = r / gsz;
 }
 
+// Tile coordinates inside one group of a row-grouped problem (gtm tile rows x tiles_n tile
+// columns, local = 0 .. gtm * tiles_n - 1). Workgroup ids, hence consecutive tiles, go to the
+// eight XCDs round-robin, and the tiles that run at the same time are a window of consecutive
+// ids: what matters for the traffic between the L2s and the fabric is which tiles share an XCD,
+// i.e. the tiles whose ids are congruent modulo 8. The group's tile rows are cut into panels of
+// 8, 4, 2 and 1 rows (binary decomposition of gtm), walked one after the other; inside a panel
+// of R x C tiles the eight residue classes each own a compact block of the panel (R = 8: 4 rows
+// x C / 4 columns; R = 4: 2 rows x C / 4 columns; R = 2: 2 rows x C / 8 columns), walked row-fastest, so that the tiles an
+// XCD works on at a time share A panels AND B panels in its L2. (With the plain row-fastest
+// numbering an XCD owns one tile row of the panel and every tile of it fetches a B panel of its
+// own: the forward launch of 32 Zipf-sized groups moved 4.2 times its operand bytes.)
+__device__ __forceinline__ void group_tile_coords(int local, int gtm, int tiles_n, int &tm, int &tn) {
+    const int C  = tiles_n;
+    const int n8 = gtm >> 3;
+    int       first_m, R, r;
+    if (local < n8 * 8 * C) {
+        first_m = (local / (8 * C)) * 8;
+        r       = local % (8 * C);
+        R       = 8;
+    } else {
+        r       = local - n8 * 8 * C;
+        first_m = n8 * 8;
+        R       = 1;
+        const int left = gtm - first_m; // 0 .. 7
+        if (left & 4) {
+            if (r < 4 * C) {
+                R = 4;
+            } else {
+                r -= 4 * C;
+                first_m += 4;
+            }
+        }
+        if (R == 1 && (left & 2)) {
+            if (r < 2 * C) {
+                R = 2;
+            } else {
+                r -= 2 * C;
+                first_m += 2;
+            }
+        }
+    }
+    const int k = r & 7, sl = r >> 3;
+    if (R == 8 && (C & 3) == 0) {
+        const int cw = C >> 2;
+        tm           = first_m + (k & 1) * 4 + (sl & 3);
+        tn           = (k >> 1) * cw + (sl >> 2);
+    } else if (R == 4 && (C & 3) == 0) {
+        const int cw = C >> 2;
+        tm           = first_m + (k & 1) * 2 + (sl & 1);
+        tn           = (k >> 1) * cw + (sl >> 1);
+    } else if (R == 2 && (C & 7) == 0) {
+        const int cw = C >> 3;
+        tm           = first_m + (sl & 1);
+        tn           = k * cw + (sl >> 1);
+    } else {
+        tm = first_m + r % R;
+        tn = r / R;
+    }
+}
+
 // Epilogue. A lane holds, for MFMA tile (i, j), C[wm_base + 16 i + lm][wn_base + 16 j + 4 lg + e],
 // e = 0..3. It scales, converts and stores those four values itself (8 bytes of bf16/fp16,
 // 16 bytes of fp32): per instruction the wavefront writes 16 rows x 32 (64) contiguous bytes,
@@ -232,12 +292,17 @@ template <bool ACC_IN_AGPR> __device__ __forceinline__ f32x4 read_acc(const f32x
 // Returns the number of store instructions it has issued (every one of them younger than any
 // memory operation issued before the call): what a caller may leave in flight when it next waits
 // for older operations by count.
-template <typename T, int TM, int TN, int MODE, bool ACC_IN_AGPR>
+// `rows_left`: rows of the matrix from this lane's first row on (its row of MFMA tile i is
+// 16 i): a lane skips the loads and stores of the row groups at or beyond it, so a sub-tile that
+// hangs over the end of its matrix (the last rows of a group) still leaves in 16-byte stores.
+// (ROWCHECK = false: every row group is stored; for callers whose sub-tile is known to lie inside.)
+template <typename T, int TM, int TN, int MODE, bool ACC_IN_AGPR, bool ROWCHECK>
 __device__ __forceinline__ int epilogue_inner(T *row, int64_t step, bool accu, const f32x4 (&acc)[TM][TN],
-                                              const float (&sa)[TM], const f32x4 (&sb)[TN]) {
+                                              const float (&sa)[TM], const f32x4 (&sb)[TN], const int64_t rows_left) {
     int stores = 0;
     static_for<0, TM>([&](auto ic) {
         constexpr int i = ic;
+        const bool    live = !ROWCHECK || 16 * i < rows_left;
         if constexpr (sizeof(T) == 4) {
             // accumulating: the old values of four tiles are requested together, then used (one
             // load at a time would pay the memory latency TN times per row)
@@ -245,7 +310,7 @@ __device__ __forceinline__ int epilogue_inner(T *row, int64_t step, bool accu, c
             static_for<0, TN / JB>([&](auto jbc) {
                 constexpr int j0 = JB * jbc;
                 f32x4         old[JB];
-                if (accu) {
+                if (accu && live) {
 #pragma unroll
                     for (int jj = 0; jj < JB; ++jj)
                         old[jj] = *reinterpret_cast<const f32x4 *>(row + (j0 + jj) * 16);
@@ -260,9 +325,10 @@ __device__ __forceinline__ int epilogue_inner(T *row, int64_t step, bool accu, c
                             v[e] = v[e] * sa[i] * sb[j][e];
                     }
                     T *q = row + j * 16;
-                    if (accu)
+                    if (accu && live)
                         v += old[j - j0];
-                    *reinterpret_cast<f32x4 *>(q) = v;
+                    if (live)
+                        *reinterpret_cast<f32x4 *>(q) = v;
                     ++stores;
                     // keep each accumulator's read next to its store (register pressure)
                     __builtin_amdgcn_sched_barrier(0);
@@ -290,7 +356,7 @@ __device__ __forceinline__ int epilogue_inner(T *row, int64_t step, bool accu, c
                 }
                 asm volatile("s_nop 1" ::: "memory");
                 T *q = row + j * 16;
-                if (accu) {
+                if (accu && live) {
                     const u32x4 old = *reinterpret_cast<const u32x4 *>(q);
                     float       o0, o1;
                     unpack2<T>(old.x, o0, o1); x[0] += o0; x[1] += o1;
@@ -303,7 +369,8 @@ __device__ __forceinline__ int epilogue_inner(T *row, int64_t step, bool accu, c
                 w.y = pack2<T>(x[2], x[3]);
                 w.z = pack2<T>(y[0], y[1]);
                 w.w = pack2<T>(y[2], y[3]);
-                *reinterpret_cast<u32x4 *>(q) = w; // (streaming stores measured no faster here)
+                if (live)
+                    *reinterpret_cast<u32x4 *>(q) = w; // (streaming stores measured no faster here)
                 ++stores;
                 __builtin_amdgcn_sched_barrier(0);
             });
@@ -333,7 +400,10 @@ __device__ __forceinline__ void store_elem(float f, uint8_t *q, int out_dtype, b
 // return: the store count of the straight-line path, 0 for the generic path. Kernels that wait
 // for older direct-to-LDS copies by count (memory operations retire in order) leave exactly
 // that many operations outstanding instead of waiting for the stores to be acknowledged.
-template <int TM, int TN, int MODE, bool ACC_IN_AGPR>
+// ROWCHECK = false keeps the 16-byte stores for sub-tiles that lie wholly inside the matrix only
+// (a hanging one takes the generic path): for kernels that cannot afford the registers of the
+// row test around their epilogue.
+template <int TM, int TN, int MODE, bool ACC_IN_AGPR, bool ROWCHECK = true>
 __device__ __forceinline__ int epilogue(const GemmArgs &a, const f32x4 (&acc)[TM][TN], uint8_t *Cm,
                                          const float *sAm, const float *sBm, int64_t m_end,
                                          int64_t wm_base, int64_t wn_base, int lane) {
@@ -359,19 +429,26 @@ __device__ __forceinline__ int epilogue(const GemmArgs &a, const f32x4 (&acc)[TM
                 sb[j][e]        = sBm[(n < a.N ? n : a.N - 1) * a.sb_n];
             }
     }
-    // whole sub-tile inside the matrix and every 16-byte group aligned: no per-element checks
-    const bool fast = wm_base + TM * 16 <= m_end && wn_base + TN * 16 <= a.N && (a.N & 7) == 0 &&
+    // all columns of the sub-tile inside the matrix and every 16-byte group aligned: 16-byte stores,
+    // with the row groups beyond the end of the matrix (the end of a group's rows) left out
+    // (only a sub-tile that lies wholly inside is certain to have issued every store it counts)
+    const bool whole = wm_base + TM * 16 <= m_end;
+    const bool fast  = (ROWCHECK || whole) && wn_base + TN * 16 <= a.N && (a.N & 7) == 0 &&
                       (reinterpret_cast<uintptr_t>(C) & 15) == 0;
     uint8_t      *row  = C + (m0 * a.N + n0) * ES;
     const int64_t step = 16 * a.N;
+    const int64_t rows_left = m_end - m0;
     if (fast) {
         // 16-bit outputs: the lane's eight columns after the exchange between tile pairs
         uint8_t *rowp = C + (m0 * a.N + wn_base + 16 * (lg & 1) + 8 * (lg >> 1)) * 2;
+        int stores;
         if (a.out_dtype == PT_DTYPE_BF16)
-            return epilogue_inner<bf16_t, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<bf16_t *>(rowp), step, accu, acc, sa, sb);
-        if (a.out_dtype == PT_DTYPE_F16)
-            return epilogue_inner<f16_t, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<f16_t *>(rowp), step, accu, acc, sa, sb);
-        return epilogue_inner<float, TM, TN, MODE, ACC_IN_AGPR>(reinterpret_cast<float *>(row), step, accu, acc, sa, sb);
+            stores = epilogue_inner<bf16_t, TM, TN, MODE, ACC_IN_AGPR, ROWCHECK>(reinterpret_cast<bf16_t *>(rowp), step, accu, acc, sa, sb, rows_left);
+        else if (a.out_dtype == PT_DTYPE_F16)
+            stores = epilogue_inner<f16_t, TM, TN, MODE, ACC_IN_AGPR, ROWCHECK>(reinterpret_cast<f16_t *>(rowp), step, accu, acc, sa, sb, rows_left);
+        else
+            stores = epilogue_inner<float, TM, TN, MODE, ACC_IN_AGPR, ROWCHECK>(reinterpret_cast<float *>(row), step, accu, acc, sa, sb, rows_left);
+        return whole ? stores : 0;
     } else {
         static_for<0, TM>([&](auto ic) {
             constexpr int i = ic;
@@ -438,7 +515,7 @@ __device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile, const 
         const int64_t hi = a.group_offs_out != nullptr ? lo + (a.group_offs_out[g + 1] - a.group_offs_out[g])
                                                        : a.group_offs[g + 1];
         const int     gtm = static_cast<int>((hi - lo + BM - 1) / BM);
-        tile_coords_local(local, gtm, a.tiles_n, tm, tn);
+        group_tile_coords(local, gtm, a.tiles_n, tm, tn);
         t.m0    = lo + static_cast<int64_t>(tm) * BM;
         t.m_end = hi;
         t.Ag    = a.A + t.m0 * a.lda;

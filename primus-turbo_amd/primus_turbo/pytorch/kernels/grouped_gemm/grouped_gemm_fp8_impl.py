@@ -144,9 +144,10 @@ def _grouped_mx(a, b, a_scales, b_scales, group_offs, group_offs_out, trans_a, t
     rows = a.shape[0]
     _check(a.shape[1] == kb, f"reduction dims differ: {a.shape[1]} vs {kb}")
     K = kb * 2 if fp4 else kb
+    # (any such K: rows shorter than four whole 128-byte slabs are copied once into zero-padded
+    # rows, _mx_pitch below; the reference's operators pad K to 128 and have no lower limit,
+    # csrc/pytorch/quantization/quantization.cpp:971-1100)
     _check(K % 32 == 0, "MX grouped GEMM needs K to be a multiple of 32")
-    if not fp4:
-        _check(K % 128 == 0 and K >= 512, "grouped MXFP8 GEMM needs K to be a multiple of 128 and at least 512")
     _check(group_offs.dtype == torch.int64 and group_offs.numel() == G + 1, "group_offs must be int64 [G + 1]")
     a_s, b_s = _u8(a_scales), _u8(b_scales)
     _check(a_s.dim() == 2 and a_s.shape[0] == rows and a_s.shape[1] >= K // 32, "a_scales must be [rows, K/32]")

@@ -128,7 +128,9 @@ def test_grouped_mx_quantizer_shuffled_outputs():
 
 
 GCASES = [("balanced", 4, 1024, 512, 512), ("ragged", 8, 3000, 384, 1024), ("zeros", 8, 2048, 256, 512),
-          ("zipf", 32, 8192, 1024, 768), ("ragged", 3, 77, 96, 640), ("zipf", 16, 4096, 2048, 512)]
+          ("zipf", 32, 8192, 1024, 768), ("ragged", 3, 77, 96, 640), ("zipf", 16, 4096, 2048, 512),
+          # K below four 128-byte slabs, and K that the quantizer pads to the next multiple of 128
+          ("ragged", 4, 600, 256, 128), ("zipf", 8, 1024, 384, 256), ("balanced", 2, 256, 128, 384), ("ragged", 3, 300, 256, 160)]
 
 
 @pytest.mark.parametrize("kind,G_,M,N,K", GCASES)
@@ -191,7 +193,8 @@ def test_grouped_mx_variable_k_product(kind, G_, M, N, K, trans_c):
 
 
 @pytest.mark.parametrize("fmt,gate", [("E4M3", 25), ("E5M2", 20), ("HYBRID", 20)])
-@pytest.mark.parametrize("kind,G_,M,N,K", [("zipf", 8, 4096, 1024, 512), ("ragged", 4, 1000, 512, 1024)])
+@pytest.mark.parametrize("kind,G_,M,N,K", [("zipf", 8, 4096, 1024, 512), ("ragged", 4, 1000, 512, 1024),
+                                           ("ragged", 4, 1000, 256, 128), ("zipf", 8, 2048, 128, 384)])
 def test_grouped_gemm_fp8_mx_autograd(fmt, gate, kind, G_, M, N, K):
     """The MX_BLOCKWISE op end to end (grouped quantizers, forward, dgrad, wgrad) against the
     unquantized grouped matmul; empty experts get a zero weight gradient; a forward-only call

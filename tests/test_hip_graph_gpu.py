@@ -123,6 +123,40 @@ def test_graph_grouped_gemm_forward_backward(kind):
                                     bf16_randn((1024, 512), seed=160 + seed)), 3)
 
 
+@pytest.mark.parametrize("kind", ["blockwise", "mxfp8", "mxfp4"])
+def test_graph_grouped_gemm_replays_with_other_group_lens(kind):
+    """The grouped kernels look their groups up on the device, so one captured graph serves any
+    split of the same token count: the static ``group_lens`` tensor is rewritten between replays
+    (another split, then one with an expert going empty, then the first again) and every replay
+    must equal the eager result for that split bit for bit, forward and backward (the reference
+    holds this test, skipped there: tests/pytorch/ops/test_grouped_gemm_fp8.py:1029)."""
+    import numpy as np
+
+    M, Gn = 1024, 4
+    splits = [group_lens("ragged", Gn, M, 131), group_lens("ragged", Gn, M, 977), np.array([700, 0, 24, 300], dtype=np.int64),
+              np.array([1, 1021, 1, 1], dtype=np.int64)]
+    assert all(int(x.sum()) == M for x in splits)
+    if kind == "mxfp4":
+        cfg, op = F4(), turbo.ops.grouped_gemm_fp4
+    else:
+        kw = dict(block_size=128) if kind == "blockwise" else dict(block_size=32, scale_dtype=ScaleDtype.E8M0)
+        cfg = F8(format=Format.E4M3, granularity=G.BLOCKWISE if kind == "blockwise" else G.MX_BLOCKWISE, **kw)
+        op = turbo.ops.grouped_gemm_fp8
+
+    def fn(a, b, dy, gl):
+        a = a.detach().requires_grad_(True)
+        b = b.detach().requires_grad_(True)
+        y = op(a, b, gl, trans_b=True, config=cfg)
+        da, db = torch.autograd.grad(y, (a, b), dy)
+        return y, da, db
+
+    def make(seed):
+        return (bf16_randn((M, 1024), seed=180 + seed), bf16_randn((Gn, 512, 1024), seed=190 + seed),
+                bf16_randn((M, 512), seed=200 + seed), torch.from_numpy(splits[seed % len(splits)]))
+
+    _replay_check(fn, make, 4, replays=5)
+
+
 def test_stochastic_rounding_refuses_graph_capture():
     """The stochastic-rounding seed is a host-side launch argument: captured, every replay would
     round with the same noise. The quantizer raises under capture instead (and works outside)."""
