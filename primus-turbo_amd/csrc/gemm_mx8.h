@@ -14,14 +14,16 @@
 // into B rows + scale words (row groups 6, 7) and A rows (row groups 0..3 of the next slab).
 // Scale words: wavefronts 0..3 copy the words of the tile's 256 rows (64 each), wavefronts 4..7
 // those of its 256 columns, one word per slab (two for MXFP4); every wavefront reads the bytes of
-// its 8 + 4 fragments from the current stage at the start of the slab.
+// its 8 + 4 fragments from the current stage at the start of the slab. GROUP_ROWS enumerates
+// (group, tile) pairs from the device-side offsets as gemm_fp8_block8.h does (MoE forward / dgrad).
 #pragma once
 #include "gemm_fp8_block8.h"
 
 namespace pt {
 
-template <int FA, int FB>
+template <int FA, int FB, int GMODE = GROUP_NONE>
 __global__ __launch_bounds__(B8_THREADS) void gemm_mx8_kernel(const GemmArgs a) {
+    static_assert(GMODE == GROUP_NONE || GMODE == GROUP_ROWS, "row groups or none");
     constexpr int  TM = B8_TM, TN = B8_TN, BM = B8_BM, BN = B8_BN;
     constexpr bool F4 = FA == 4;
     static_assert((FA == 4) == (FB == 4), "FP4 operands come in pairs");
@@ -41,13 +43,36 @@ __global__ __launch_bounds__(B8_THREADS) void gemm_mx8_kernel(const GemmArgs a) 
     const uint32_t frag_off_lo = lm * KSTEP + ((lg ^ swz(lm)) << 4);
     const uint32_t frag_off_hi = lm * KSTEP + (((4 + lg) ^ swz(lm)) << 4);
 
-    const int total  = a.tiles_m * a.tiles_n;
+    // ---- tile list (row groups: tiles before group g, from the device-side offsets) ----
+    int *prefix = reinterpret_cast<int *>(smem + B8_NSTAGE * STAGE);
+    int  total;
+    if constexpr (GMODE == GROUP_ROWS) {
+        for (int g = tid; g < a.G; g += B8_THREADS) {
+            const int64_t *o   = a.group_offs_out != nullptr ? a.group_offs_out : a.group_offs;
+            const int64_t rows = o[g + 1] - o[g];
+            prefix[g + 1]      = static_cast<int>((rows + BM - 1) / BM) * a.tiles_n;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            int run   = 0;
+            prefix[0] = 0;
+            for (int g = 1; g <= a.G; ++g) {
+                run += prefix[g];
+                prefix[g] = run;
+            }
+        }
+        __syncthreads();
+        total = __builtin_amdgcn_readfirstlane(prefix[a.G]);
+    } else {
+        total = a.tiles_m * a.tiles_n;
+    }
     const int KT_ALL = static_cast<int>(a.K / KSTEP); // >= 2
     int       tile   = blockIdx.x;
     if (tile >= total || KT_ALL < 2)
         return;
     int     g_cur = 0, g_nxt = 0;
-    TileCtx cur_t = make_tile<BM, BN, GROUP_NONE, F4>(a, tile, nullptr, g_cur);
+    TileCtx cur_t = make_tile<BM, BN, GMODE, F4>(a, tile, prefix, g_cur);
+    g_nxt         = g_cur;
     TileCtx nxt_t = cur_t;
 
     // ---- loader ----
@@ -187,7 +212,7 @@ __global__ __launch_bounds__(B8_THREADS) void gemm_mx8_kernel(const GemmArgs a) 
         const int next_tile = tile + gridDim.x;
         nxt_t               = cur_t;
         if (next_tile < total)
-            nxt_t = make_tile<BM, BN, GROUP_NONE, F4>(a, next_tile, nullptr, g_nxt);
+            nxt_t = make_tile<BM, BN, GMODE, F4>(a, next_tile, prefix, g_nxt);
 
         // one K slab per iteration; the body stays a single basic block
         for (int kt = 0; kt < KT_ALL; ++kt) {
@@ -257,31 +282,37 @@ __global__ __launch_bounds__(B8_THREADS) void gemm_mx8_kernel(const GemmArgs a) 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-template <int FA, int FB> static int launch_gemm_mx8(const GemmArgs &args_in, hipStream_t stream) {
-    constexpr int LDS = B8_NSTAGE * (B8_A_BYTES + B8_B_BYTES + (FA == 4 ? 2 : 1) * 2048);
-    static_assert(LDS <= 160 * 1024, "tile configuration does not fit the LDS");
+template <int FA, int FB, int GMODE = GROUP_NONE> static int launch_gemm_mx8(const GemmArgs &args_in, hipStream_t stream) {
+    constexpr int STAGES  = B8_NSTAGE * (B8_A_BYTES + B8_B_BYTES + (FA == 4 ? 2 : 1) * 2048);
+    constexpr int MAX_G   = 2048;
+    constexpr int LDS_MAX = STAGES + (GMODE == GROUP_ROWS ? (MAX_G + 2) * 4 : 0);
+    static_assert(LDS_MAX <= 160 * 1024, "tile configuration does not fit the LDS");
     GemmArgs a = args_in;
-    a.gmode    = GROUP_NONE;
+    a.gmode    = GMODE;
     a.tiles_m  = static_cast<int>(cdiv(a.M, B8_BM));
     a.tiles_n  = static_cast<int>(cdiv(a.N, B8_BN));
+    if (GMODE != GROUP_NONE && a.G > MAX_G)
+        return fail(PT_ERR_INVALID_ARGUMENT, "grouped gemm_mx: too many groups for this tile configuration");
     if (a.sa_shift != 0 || a.sb_shift != 0 || (a.sa_wpitch == 0 && (a.sa_m % 4 != 0 || a.sb_n % 4 != 0)) ||
         (a.sa_wpitch != 0) != (a.sb_wpitch != 0) || a.sa_wpitch % 4 != 0 || a.sb_wpitch % 4 != 0 ||
         reinterpret_cast<uintptr_t>(a.sA) % 4 != 0 || reinterpret_cast<uintptr_t>(a.sB) % 4 != 0)
         return fail(PT_ERR_INVALID_ARGUMENT, "gemm_mx: scale rows must be 4-byte aligned");
     if (a.K / KSTEP < 2)
         return fail(PT_ERR_INVALID_ARGUMENT, "gemm_mx: K too short for the 256x256 tile");
-    auto kern = gemm_mx8_kernel<FA, FB>;
+    auto kern = gemm_mx8_kernel<FA, FB, GMODE>;
     static std::atomic<unsigned long long> attr_set{0};
     int                                    dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
         return fail(PT_ERR_LAUNCH, "gemm_mx: no current device (or a device index beyond 63)");
     const unsigned long long dev_bit = 1ULL << dev;
     if (!(attr_set.load(std::memory_order_acquire) & dev_bit)) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess)
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_MAX) != hipSuccess)
             return fail(PT_ERR_LAUNCH, "gemm_mx: cannot raise the dynamic LDS limit");
         attr_set.fetch_or(dev_bit, std::memory_order_release);
     }
-    const int64_t total = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
+    const int     LDS   = STAGES + (GMODE == GROUP_ROWS ? (a.G + 2) * 4 : 0);
+    const int64_t total = GMODE == GROUP_ROWS ? (static_cast<int64_t>(a.tiles_m) + a.G) * a.tiles_n
+                                              : static_cast<int64_t>(a.tiles_m) * a.tiles_n;
     int64_t       grid  = device_cu_count(); // one workgroup per CU (LDS-limited), persistent
     if (grid > total)
         grid = total;

@@ -12,16 +12,21 @@
 // group_offs_out packing the result, wgrad is a variable-K NT product over the 128-padded
 // column-direction operands) and of its grouped MXFP4 path (ops/grouped_gemm_fp4.py:101-309:
 // the same three products over tight rows and 256-padded column-direction operands).
-#include "gemm_fp8_kernel.h"
+#include "gemm_mx8.h"
 
 namespace pt {
 
 template <int GMODE, int FA, int FB> static int launch_mxg_tiles(const GemmArgs &a, int tile_cfg, hipStream_t stream) {
-    // tile_cfg: 0 = auto, 1 = 256x256, 3 = 128x128 (two workgroups per CU)
+    // tile_cfg: 0 = auto, 1 = 256x256, 3 = 128x128 (two workgroups per CU), 4 = 256x256 with eight
+    // wavefronts (row groups only)
     if (tile_cfg == 0) {
         const bool big = GMODE == GROUP_K ? (a.M >= 1024 && a.N >= 1024)
                                           : (a.G > 0 && a.M / a.G >= 512 && a.N >= 1024);
         tile_cfg       = big ? 1 : 3;
+    }
+    if constexpr (GMODE == GROUP_ROWS) {
+        if (tile_cfg == 4)
+            return launch_gemm_mx8<FA, FB, GROUP_ROWS>(a, stream);
     }
     if (tile_cfg == 1 || tile_cfg == 2)
         return launch_gemm_cfg<8, 8, SCALE_MX, false, FA, FB, GMODE>(a, stream);
@@ -95,7 +100,7 @@ int pt_grouped_gemm_mx(const void *a, int a_dtype, const void *a_scale, int64_t 
     PT_REQUIRE(lda == ldb && lda >= kbytes && lda % KSTEP == 0 && lda >= GEMM_MIN_SLABS * KSTEP,
                "row pitches must be equal multiples of 128 bytes, at least 512, that hold K");
     PT_REQUIRE(lda < (1LL << 24), "K must be below 2^24");
-    PT_REQUIRE(tile_cfg >= 0 && tile_cfg <= 3, "tile_cfg must be 0..3");
+    PT_REQUIRE(tile_cfg >= 0 && tile_cfg <= 4, "tile_cfg must be 0..4");
     PT_REQUIRE(sa_ld >= K / 32 && sb_ld >= K / 32 && sa_ld % 4 == 0 && sb_ld % 4 == 0,
                "scale rows must hold K / 32 bytes and be 4-byte multiples");
     auto st = static_cast<hipStream_t>(stream);

@@ -21,7 +21,7 @@ from primus_turbo.pytorch.core.low_precision import ScalingGranularity
 _FP8 = (torch.float8_e4m3fn, torch.float8_e5m2)
 
 TILE_CFG = 0  # 0 = automatic; tests and the benchmark may pin 2 (256x128) or 3 (128x128)
-MX_TILE_CFG = 0  # MX path: 0 = automatic, 1 = 256x256, 3 = 128x128
+MX_TILE_CFG = 0  # MX path: 0 = automatic, 1 = 256x256, 3 = 128x128, 4 = 256x256 with eight wavefronts (row groups only)
 
 
 def _check(cond, msg):
@@ -74,7 +74,7 @@ def _grouped_vec(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, out_dty
         lib.pt_grouped_gemm_fp8_vec(
             N.ptr(a), N.dtype_code(a.dtype), N.ptr(a_scales), sa, N.ptr(b), N.dtype_code(b.dtype), N.ptr(b_scales), sb,
             Nn if sb else 0, N.ptr(out), N.dtype_code(out.dtype), N.ptr(group_offs.contiguous()), G, M, M, Nn, K,
-            int(trans_b), N.ptr(ws), ws_bytes, MX_TILE_CFG, N.stream_of(a),
+            int(trans_b), N.ptr(ws), ws_bytes, _cfg_without_eight_waves(), N.stream_of(a),
         )
     )
     return out
@@ -102,10 +102,15 @@ def _variable_k_vec(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, tran
         lib.pt_grouped_gemm_fp8_vec_variable_k(
             N.ptr(a), N.dtype_code(a.dtype), N.ptr(a_scales), sl, N.ptr(b), N.dtype_code(b.dtype), N.ptr(b_scales), sr,
             N.ptr(out), N.dtype_code(out.dtype), N.ptr(group_offs.contiguous()), G, M, Ml, Nr, int(trans_c),
-            int(accumulate), N.ptr(ws), ws_bytes, MX_TILE_CFG, N.stream_of(a),
+            int(accumulate), N.ptr(ws), ws_bytes, _cfg_without_eight_waves(), N.stream_of(a),
         )
     )
     return out
+
+
+def _cfg_without_eight_waves() -> int:
+    """The pinned MX tile configuration for the entry points that have no eight-wavefront tile."""
+    return 0 if MX_TILE_CFG == 4 else MX_TILE_CFG
 
 
 def _is_mx(granularity: int) -> bool:
@@ -200,7 +205,7 @@ def _variable_k_mx(a, b, a_scales, b_scales, group_offs, trans_a, trans_b, trans
         N.lib().pt_grouped_gemm_mx_variable_k(
             N.ptr(a), da, N.ptr(a_s), N.ptr(b), db, N.ptr(b_s), N.ptr(out),
             N.dtype_code(out.dtype), N.ptr(group_offs.contiguous()), G, Ml, Nr, ld, int(accumulate), N.ptr(ws), ws_bytes,
-            MX_TILE_CFG, N.stream_of(a),
+            _cfg_without_eight_waves(), N.stream_of(a),
         )
     )
     return out

@@ -159,6 +159,36 @@ def test_grouped_mx_forward_product(kind, G_, M, N, K, fa, fb):
     assert torch.equal(out2[:M], out[:M])
 
 
+@pytest.mark.parametrize("kind,G_,M,N,K", [("zipf", 32, 8192, 1024, 768), ("ragged", 8, 3000, 384, 1024), ("zeros", 8, 2048, 256, 512),
+                                           ("ragged", 3, 77, 96, 640), ("zipf", 16, 4096, 2048, 2048)])
+@pytest.mark.parametrize("padded", [False, True])
+def test_grouped_mx_eight_wavefront_tile(kind, G_, M, N, K, padded):
+    """tile_cfg 4 (256 x 256 tile, eight wavefronts, gemm_mx8.h with row groups) gives the bits of
+    the automatic configuration: the same products added in the same order, with the per-group
+    padded row layout of the grouped quantizer and with the tight one."""
+    lens = group_lens(kind, G_, M, 143)
+    gl, offs = _offs(lens)
+    x = bf16_randn((M, K), seed=144).cuda()
+    w = bf16_randn((G_, N, K), seed=145).cuda()
+    wq, ws = qimpl.quantize_mxfp8_impl(w, torch.float8_e4m3fn, 2, 32, scaling_recipe=ScalingRecipe(use_2d_block=True))
+    if padded:
+        rq, rs, _, orow = qimpl.grouped_quantize_mxfp8_impl(x, torch.float8_e4m3fn, 1, 32, gl, offs)
+        run = lambda: gimpl.grouped_gemm_fp8_impl(rq, wq, rs, ws, gl, orow, False, True, torch.bfloat16, G.MX_BLOCKWISE.value,  # noqa: E731
+                                                  None, 0, False, offs)
+    else:
+        rq, rs = qimpl.quantize_mxfp8_impl(x, torch.float8_e4m3fn, 1, 32)
+        run = lambda: gimpl.grouped_gemm_fp8_impl(rq, wq, rs, ws, gl, offs, False, True, torch.bfloat16, G.MX_BLOCKWISE.value,  # noqa: E731
+                                                  None, 0)
+    auto = run()
+    gimpl.MX_TILE_CFG = 4
+    try:
+        got = run()
+    finally:
+        gimpl.MX_TILE_CFG = 0
+    torch.cuda.synchronize()
+    assert torch.equal(got, auto)
+
+
 @pytest.mark.parametrize("kind,G_,M,N,K", GCASES)
 @pytest.mark.parametrize("trans_c", [False, True])
 def test_grouped_mx_variable_k_product(kind, G_, M, N, K, trans_c):

@@ -112,6 +112,31 @@ def test_grouped_mxfp4_forward_product(kind, G_, M, N, K):
     _gate(ref, to_f32_np(out), f"{kind} G={G_} {M}x{N}x{K}")
 
 
+@pytest.mark.parametrize("kind,G_,M,N,K", [("zipf", 32, 8192, 1024, 768), ("ragged", 8, 3000, 384, 1024), ("zeros", 8, 2048, 256, 512),
+                                           ("ragged", 3, 77, 96, 640), ("zipf", 16, 4096, 2048, 2048)])
+def test_grouped_mxfp4_eight_wavefront_tile(kind, G_, M, N, K):
+    """tile_cfg 4 (256 x 256 tile, eight wavefronts, row groups) against the automatic configuration:
+    the same products in the same order, so the same bits."""
+    from primus_turbo.pytorch.kernels.grouped_gemm import grouped_gemm_fp8_impl as g8
+
+    lens = group_lens(kind, G_, M, 163)
+    gl, offs = _offs(lens)
+    x = bf16_randn((M, K), seed=164).cuda()
+    w = bf16_randn((G_, N, K), seed=165).cuda()
+    rq, rs, _, orow = qimpl.grouped_quantize_mxfp4_impl(x, FP4, 1, 32, gl, offs)
+    wq, ws = qimpl.quantize_mxfp4_impl(w, FP4, 2, 32, scaling_recipe=ScalingRecipe(use_2d_block=True))
+    run = lambda: gimpl.grouped_gemm_fp4_impl(rq, wq, rs, ws, gl, orow, False, True, torch.bfloat16, G.MX_BLOCKWISE.value,  # noqa: E731
+                                              None, 0, False, offs)
+    auto = run()
+    g8.MX_TILE_CFG = 4
+    try:
+        got = run()
+    finally:
+        g8.MX_TILE_CFG = 0
+    torch.cuda.synchronize()
+    assert torch.equal(got, auto)
+
+
 @pytest.mark.parametrize("kind,G_,M,N,K", GCASES)
 @pytest.mark.parametrize("trans_c", [False, True])
 def test_grouped_mxfp4_variable_k_product(kind, G_, M, N, K, trans_c):
