@@ -173,7 +173,56 @@ class QuantTensorwise:
         )
 
 
-WORKLOADS = {"quant_tensorwise": QuantTensorwise}
+class QuantTensorwiseLarge(QuantTensorwise):
+    """The same quantizer on a 16384 x 16384 bf16 tensor (512 MiB): its rate away from the launch
+    ramp of the 32 MiB case. The fused kernel parks 32 MiB in registers across the grid exchange
+    and reads the rest a second time, so it moves 5 bytes per element for 3 algorithmic ones."""
+
+    name = "fp8_e4m3_tensorwise_quant_dequant_16384x16384_bf16"
+    traffic = None
+
+    def __init__(self, dev, side=16384):
+        import primus_turbo.pytorch as turbo
+        from primus_turbo.pytorch.core.low_precision import ScalingGranularity as G
+
+        self.turbo, self.G = turbo, G
+        g = torch.Generator().manual_seed(3)
+        self.x_cpu = torch.randn((side, side), generator=g, dtype=torch.float32).to(torch.bfloat16)
+        self.x_cpu.view(-1)[12345] = 300.0
+        self.x = self.x_cpu.to(dev)
+        self.n = self.x.numel()
+        self.q, self.sinv = turbo.ops.quantize_fp8(self.x, turbo.float8_e4m3, G.TENSORWISE)
+        self._ring = [self.x, self.x.clone()]
+        self._pos = 0
+
+    def check(self):
+        import numpy as np
+
+        from oracle import quantize as Q
+
+        # the scale from the whole tensor's abs-max, the bytes of the first and last 256 rows
+        amax = np.float32(self.x_cpu.abs().max().item())
+        _, osinv = Q.fp8_tensorwise(np.array([amax], dtype=np.float32), "e4m3")
+        same = self.sinv.cpu().view(torch.int32).item() == osinv.view(np.int32).item()
+        scale = np.float32(448.0) / max(amax, np.float32(1e-12))
+        for rows in (slice(0, 256), slice(-256, None)):
+            oq, _ = Q.fp8_tensorwise(self.x_cpu[rows].float().numpy(), "e4m3", scale=scale)
+            same = same and np.array_equal(self.q[rows].cpu().view(torch.uint8).numpy(), oq)
+        return bool(same), "scale_inv and the bytes of the first and last 256 rows bit-exact vs oracle"
+
+    def cpu_baseline(self):
+        from oracle import cpu_reference as R
+
+        x = self.x_cpu[:4096, :4096].contiguous()
+        t0 = time.perf_counter()
+        q, _, sinv = R.quantize_fp8_tensorwise_ref(x, torch.float8_e4m3fn)
+        R.dequantize_fp8_ref(q, torch.bfloat16, sinv)
+        dt = time.perf_counter() - t0
+        return dict(value=6.0 * x.numel() / dt / 1e9, unit="GB/s", cores=torch.get_num_threads(), kind="port",
+                    sample=f"a 4096x4096 corner, one run, {os.cpu_count()} logical CPUs visible")
+
+
+WORKLOADS = {"quant_tensorwise": QuantTensorwise, "quant_tensorwise_16384": QuantTensorwiseLarge}
 from bench_quant_workloads import register as _register_quant  # noqa: E402
 from bench_workloads import register as _register  # noqa: E402
 
@@ -186,7 +235,7 @@ DEFAULT_ORDER = ["gemm_fp8_blockwise_8192", "gemm_fp8_rowwise", "quant_tensorwis
 EXTRA_GEMM = ["gemm_fp8_rowwise", "gemm_fp8_blockwise", "gemm_fp8_blockwise_k7168", "grouped_gemm_fp8",
               "grouped_gemm_fp8_down", "gemm_mxfp4", "gemm_mxfp4_n28672", "gemm_mxfp8", "gemm_mxfp8_n28672",
               "grouped_gemm_mxfp8", "grouped_gemm_mxfp8_down", "grouped_gemm_mxfp4", "grouped_gemm_mxfp4_down"]
-EXTRA_QUANT = ["hbm_stream", "swiglu_with_probs", "moe_permute", "quant_tensorwise", "quant_rowwise", "quant_blockwise", "quant_blockwise_dual", "quant_blockwise_weight",
+EXTRA_QUANT = ["hbm_stream", "swiglu_with_probs", "moe_permute", "quant_tensorwise", "quant_tensorwise_16384", "quant_rowwise", "quant_blockwise", "quant_blockwise_dual", "quant_blockwise_weight",
                "quant_grouped", "glu_quant_grouped", "glu_quant_grouped_mxfp8", "quant_mxfp8", "quant_mxfp8_dual", "quant_mxfp4", "quant_mxfp4_dual"]
 EXTRA_BUDGET_S = 400.0  # no further extra workload is started after this many seconds of run time
 

@@ -71,8 +71,8 @@ class HbmStream(_QuantBase):
     """The yardstick of the HBM-bound kernels: what plain streaming kernels of the same traffic shape
     reach on this GPU, measured by the same harness (rotating inputs, graph replays). The dominant
     kernel reads a 16384 x 7168 bf16 tensor and writes one fp8-sized byte per element (the traffic
-    ratio of a quantizer, 3 bytes per element) with torch's elementwise cast; the other entry is a
-    same-size copy (2 + 2 bytes per element)."""
+    ratio of a quantizer, 3 bytes per element) with torch's elementwise cast; the other entries are a
+    same-size copy (2 + 2 bytes per element), a fill (writes only) and a reduction (reads only)."""
 
     name = "hbm_streaming_yardstick_16384x7168_bf16 (torch elementwise cast to fp8, copy)"
     metric = "plain streaming GB/s & fraction of HBM peak"
@@ -101,9 +101,20 @@ class HbmStream(_QuantBase):
         self.y.copy_(self.x)
         return self.y
 
+    def _fill(self):
+        self.y.zero_()
+        return self.y
+
+    def _read(self):
+        return self.x.view(torch.int32).amax()
+
     def kernels(self):
+        # a pure write stream and a pure read stream beside the copy: what the two directions of
+        # the memory system give on their own (a quantizer that emits two outputs, a gather that
+        # writes eight rows per row read, are write-heavy)
         n = float(self.M * self.N)
-        return [("copy_bf16_to_bf16", self._copy, 4.0 * n)]
+        return [("copy_bf16_to_bf16", self._copy, 4.0 * n), ("fill_write_only", self._fill, 2.0 * n),
+                ("amax_read_only", self._read, 2.0 * n)]
 
     def check(self):
         ok = torch.equal(self._copy(), self.x) and torch.equal(self.dominant().float(), self.x.to(torch.float8_e4m3fn).float())
