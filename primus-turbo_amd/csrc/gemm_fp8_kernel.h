@@ -309,30 +309,41 @@ __device__ __forceinline__ int epilogue_inner(T *row, int64_t step, bool accu, c
             constexpr int JB = TN < 4 ? TN : 4;
             static_for<0, TN / JB>([&](auto jbc) {
                 constexpr int j0 = JB * jbc;
-                f32x4         old[JB];
-                if (accu && live) {
-#pragma unroll
-                    for (int jj = 0; jj < JB; ++jj)
-                        old[jj] = *reinterpret_cast<const f32x4 *>(row + (j0 + jj) * 16);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                static_for<0, JB>([&](auto jjc) {
-                    constexpr int j = j0 + jjc;
+                // one branch holds the loads AND their uses: a load whose use sat behind a second
+                // test of the same condition would look outstanding, to the compiler's wait-count
+                // bookkeeping, on the path that skips that use, and the K loop of a persistent
+                // kernel would then open every slab with a full vmcnt(0) wait that drains its
+                // direct-to-LDS copies
+                auto tile_value = [&](auto jc2) {
+                    constexpr int j = jc2;
                     f32x4         v = read_acc<ACC_IN_AGPR>(acc[i][j]);
                     if constexpr (MODE == SCALE_VECTOR) {
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
                             v[e] = v[e] * sa[i] * sb[j][e];
                     }
-                    T *q = row + j * 16;
-                    if (accu && live)
-                        v += old[j - j0];
-                    if (live)
-                        *reinterpret_cast<f32x4 *>(q) = v;
-                    ++stores;
-                    // keep each accumulator's read next to its store (register pressure)
+                    return v;
+                };
+                if (accu && live) {
+                    f32x4 old[JB];
+#pragma unroll
+                    for (int jj = 0; jj < JB; ++jj)
+                        old[jj] = *reinterpret_cast<const f32x4 *>(row + (j0 + jj) * 16);
                     __builtin_amdgcn_sched_barrier(0);
-                });
+                    static_for<0, JB>([&](auto jjc) {
+                        constexpr int j = j0 + jjc;
+                        *reinterpret_cast<f32x4 *>(row + j * 16) = tile_value(std::integral_constant<int, j>{}) + old[j - j0];
+                        // keep each accumulator's read next to its store (register pressure)
+                        __builtin_amdgcn_sched_barrier(0);
+                    });
+                } else if (live) {
+                    static_for<0, JB>([&](auto jjc) {
+                        constexpr int j = j0 + jjc;
+                        *reinterpret_cast<f32x4 *>(row + j * 16) = tile_value(std::integral_constant<int, j>{});
+                        __builtin_amdgcn_sched_barrier(0);
+                    });
+                }
+                stores += JB;
             });
         } else {
             static_for<0, TN / 2>([&](auto jc) {
