@@ -346,45 +346,66 @@ __device__ __forceinline__ int epilogue_inner(T *row, int64_t step, bool accu, c
                 stores += JB;
             });
         } else {
-            static_for<0, TN / 2>([&](auto jc) {
-                constexpr int j = 2 * jc;
-                f32x4         x = read_acc<ACC_IN_AGPR>(acc[i][j]), y = read_acc<ACC_IN_AGPR>(acc[i][j + 1]);
+            // Two tiles (j, j + 1) give a lane eight consecutive columns after an exchange between
+            // lane groups (v_permlane16_swap, written out by hand: the compiler's builtin for this
+            // instruction loses track of vector elements; the wait states cover the VALU writes
+            // just before). One test of `live` per row group. The plain form packs first, so the
+            // exchange moves two registers per tile pair; the accumulating form exchanges the fp32
+            // values, requests the old values of the row group together and adds in fp32.
+            auto swap16 = [](auto &p, auto &q) { asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(p), "+v"(q)); };
+            auto scaled = [&](auto jc2) {
+                constexpr int j = jc2;
+                f32x4         v = read_acc<ACC_IN_AGPR>(acc[i][j]);
                 if constexpr (MODE == SCALE_VECTOR) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        x[e] = x[e] * sa[i] * sb[j][e];
-                        y[e] = y[e] * sa[i] * sb[j + 1][e];
-                    }
+                    for (int e = 0; e < 4; ++e)
+                        v[e] = v[e] * sa[i] * sb[j][e];
                 }
-                // (written out by hand: the compiler's builtin for this instruction loses track of
-                // vector elements; the wait states cover the VALU writes just before)
+                return v;
+            };
+            if (live) {
+                if (accu) {
+                    u32x4 old[TN / 2];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float xe = x[e], ye = y[e];
-                    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(xe), "+v"(ye));
-                    x[e] = xe;
-                    y[e] = ye;
+                    for (int jj = 0; jj < TN / 2; ++jj)
+                        old[jj] = *reinterpret_cast<const u32x4 *>(row + jj * 32);
+                    __builtin_amdgcn_sched_barrier(0);
+                    static_for<0, TN / 2>([&](auto jc) {
+                        constexpr int j = 2 * jc;
+                        f32x4         x = scaled(std::integral_constant<int, j>{}), y = scaled(std::integral_constant<int, j + 1>{});
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            float xe = x[e], ye = y[e];
+                            swap16(xe, ye);
+                            x[e] = xe;
+                            y[e] = ye;
+                        }
+                        asm volatile("s_nop 1" ::: "memory");
+                        const u32x4 &o = old[jc];
+                        float        o0, o1;
+                        unpack2<T>(o.x, o0, o1); x[0] += o0; x[1] += o1;
+                        unpack2<T>(o.y, o0, o1); x[2] += o0; x[3] += o1;
+                        unpack2<T>(o.z, o0, o1); y[0] += o0; y[1] += o1;
+                        unpack2<T>(o.w, o0, o1); y[2] += o0; y[3] += o1;
+                        *reinterpret_cast<u32x4 *>(row + j * 16) =
+                            u32x4{pack2<T>(x[0], x[1]), pack2<T>(x[2], x[3]), pack2<T>(y[0], y[1]), pack2<T>(y[2], y[3])};
+                        __builtin_amdgcn_sched_barrier(0);
+                    });
+                } else {
+                    static_for<0, TN / 2>([&](auto jc) {
+                        constexpr int j = 2 * jc;
+                        const f32x4   x = scaled(std::integral_constant<int, j>{}), y = scaled(std::integral_constant<int, j + 1>{});
+                        uint32_t      w0 = pack2<T>(x[0], x[1]), w1 = pack2<T>(x[2], x[3]);
+                        uint32_t      w2 = pack2<T>(y[0], y[1]), w3 = pack2<T>(y[2], y[3]);
+                        swap16(w0, w2);
+                        swap16(w1, w3);
+                        asm volatile("s_nop 1" ::: "memory");
+                        *reinterpret_cast<u32x4 *>(row + j * 16) = u32x4{w0, w1, w2, w3}; // (streaming stores measured no faster here)
+                        __builtin_amdgcn_sched_barrier(0);
+                    });
                 }
-                asm volatile("s_nop 1" ::: "memory");
-                T *q = row + j * 16;
-                if (accu && live) {
-                    const u32x4 old = *reinterpret_cast<const u32x4 *>(q);
-                    float       o0, o1;
-                    unpack2<T>(old.x, o0, o1); x[0] += o0; x[1] += o1;
-                    unpack2<T>(old.y, o0, o1); x[2] += o0; x[3] += o1;
-                    unpack2<T>(old.z, o0, o1); y[0] += o0; y[1] += o1;
-                    unpack2<T>(old.w, o0, o1); y[2] += o0; y[3] += o1;
-                }
-                u32x4 w;
-                w.x = pack2<T>(x[0], x[1]);
-                w.y = pack2<T>(x[2], x[3]);
-                w.z = pack2<T>(y[0], y[1]);
-                w.w = pack2<T>(y[2], y[3]);
-                if (live)
-                    *reinterpret_cast<u32x4 *>(q) = w; // (streaming stores measured no faster here)
-                ++stores;
-                __builtin_amdgcn_sched_barrier(0);
-            });
+            }
+            stores += TN / 2;
         }
         row += step;
     });

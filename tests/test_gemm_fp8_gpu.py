@@ -162,16 +162,26 @@ def _blockwise_nt_nn_tn(M, N, K):
     _gate(ref, to_f32_np(dw), "blockwise TN^T")
 
 
-def test_accumulate_epilogue():
-    M, N, K = 256, 384, 256
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M", [256, 200])
+def test_accumulate_epilogue(out_dtype, M):
+    """out += A B^T for every output type (16-bit outputs add in fp32 and round once); M = 200 leaves
+    row groups of the last tile outside the matrix."""
+    N, K = 384, 256
     a, b = bf16_randn((M, K), 38), bf16_randn((N, K), 39)
     aq, asi = turbo.ops.quantize_fp8(a.cuda(), torch.float8_e4m3fn, G.TENSORWISE)
     bq, bsi = turbo.ops.quantize_fp8(b.cuda(), torch.float8_e4m3fn, G.TENSORWISE)
-    base = bf16_randn((M, N), 40).float()
+    base = (bf16_randn((M, N), 40).float() * 8).to(out_dtype)
     out = base.cuda().clone()
-    impl.gemm_fp8_accum_impl(aq, asi, False, bq, bsi, True, torch.float32, False, G.TENSORWISE.value, out, 0)
-    ref = OG.gemm_dequantized(_deq_fp8(aq, asi, "e4m3"), _deq_fp8(bq, bsi, "e4m3")) + base.numpy()
-    _gate(ref, out.cpu().numpy(), "accumulate")
+    impl.gemm_fp8_accum_impl(aq, asi, False, bq, bsi, True, out_dtype, False, G.TENSORWISE.value, out, 0)
+    prod = OG.gemm_dequantized(_deq_fp8(aq, asi, "e4m3"), _deq_fp8(bq, bsi, "e4m3"))
+    ref = prod + base.float().numpy()
+    _gate(ref, out.float().cpu().numpy(), f"accumulate {out_dtype}")
+    # the old values really took part: without them the result is off by their norm
+    plain = torch.empty_like(out)
+    impl.gemm_fp8_accum_impl(aq, asi, False, bq, bsi, True, out_dtype, False, G.TENSORWISE.value, plain.zero_(), 0)
+    diff = (out.float() - plain.float()).cpu().numpy()
+    assert np.abs(diff - base.float().numpy()).max() <= 2.0 ** -6 * max(1.0, float(np.abs(ref).max()))
 
 
 def test_determinism():
