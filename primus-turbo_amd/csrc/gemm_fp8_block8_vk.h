@@ -159,7 +159,7 @@ __global__ __launch_bounds__(B8_THREADS) void gemm_fp8_block8_vk_kernel(const Ge
         const int64_t m0 = static_cast<int64_t>(tm) * BM, n0 = static_cast<int64_t>(tn) * BN;
         const int     rows_a = (a.M - m0) < BM ? static_cast<int>(a.M - m0) : BM;
         const int     rows_b = (a.N - n0) < BN ? static_cast<int>(a.N - n0) : BN;
-        const int64_t k_lo = a.group_offs[gs], k_hi = a.group_offs[ge];
+        const int64_t k_lo = uniform_load(a.group_offs + gs), k_hi = uniform_load(a.group_offs + ge);
 
         // ---- pipeline start: slabs 0 and 1 ----
         ld_S = static_cast<int>((k_hi - k_lo) / KSTEP);
@@ -187,11 +187,11 @@ __global__ __launch_bounds__(B8_THREADS) void gemm_fp8_block8_vk_kernel(const Ge
         }
 
         PT_GEMM_TRACE_POINT(7);
-        int64_t pos = k_lo, g_hi = a.group_offs[gs + 1];
+        int64_t pos = k_lo, g_hi = uniform_load(a.group_offs + gs + 1);
         for (int g = gs; g < ge; ++g) {
             const int KT = static_cast<int>((g_hi - pos) / KSTEP);
             // the end of the group after this one, fetched while this one is multiplied
-            const int64_t nxt_hi = g + 2 <= ge ? a.group_offs[g + 2] : g_hi;
+            const int64_t nxt_hi = g + 2 <= ge ? uniform_load(a.group_offs + g + 2) : g_hi;
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll

@@ -506,6 +506,38 @@ __device__ __forceinline__ int epilogue(const GemmArgs &a, const f32x4 (&acc)[TM
     return 0;
 }
 
+// Wavefront-uniform 64-bit loads of values written before the launch (group offsets), through the
+// scalar cache. Left to the compiler these are vector loads -- the kernel also stores to global
+// memory, so it cannot prove the location unclobbered -- and the wait for a vector load is also a
+// wait for every result-tile store issued before it (memory operations retire in order): each
+// tile of a grouped problem would begin by draining the previous tile's stores.
+__device__ __forceinline__ void uniform_load_pair(const int64_t *p, int64_t &v0, int64_t &v1) {
+#if defined(__HIP_DEVICE_COMPILE__) // the host pass cannot parse the scalar-register constraint
+    asm volatile("s_load_dwordx2 %0, %2, 0x0\n\t"
+                 "s_load_dwordx2 %1, %2, 0x8\n\t"
+                 "s_waitcnt lgkmcnt(0)"
+                 : "=&s"(v0), "=&s"(v1)
+                 : "s"(p)
+                 : "memory");
+#else
+    v0 = p[0];
+    v1 = p[1];
+#endif
+}
+__device__ __forceinline__ int64_t uniform_load(const int64_t *p) {
+    int64_t v;
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("s_load_dwordx2 %0, %1, 0x0\n\t"
+                 "s_waitcnt lgkmcnt(0)"
+                 : "=s"(v)
+                 : "s"(p)
+                 : "memory");
+#else
+    v = p[0];
+#endif
+    return v;
+}
+
 // Where a workgroup's tile lives. The second half only varies between tiles of grouped
 // problems; in the dense case it repeats the kernel arguments.
 struct TileCtx {
@@ -542,10 +574,13 @@ __device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile, const 
         while (g + 1 < a.G && tile >= __builtin_amdgcn_readfirstlane(prefix[g + 1]))
             ++g;
         const int     local = tile - __builtin_amdgcn_readfirstlane(prefix[g]);
-        const int64_t lo = a.group_offs[g];
+        int64_t lo, hi, out_lo = 0, out_hi = 0;
+        uniform_load_pair(a.group_offs + g, lo, hi);
         // with separate output offsets the group's row count is theirs (A may be padded per group)
-        const int64_t hi = a.group_offs_out != nullptr ? lo + (a.group_offs_out[g + 1] - a.group_offs_out[g])
-                                                       : a.group_offs[g + 1];
+        if (a.group_offs_out != nullptr) {
+            uniform_load_pair(a.group_offs_out + g, out_lo, out_hi);
+            hi = lo + (out_hi - out_lo);
+        }
         const int     gtm = static_cast<int>((hi - lo + BM - 1) / BM);
         group_tile_coords(local, gtm, a.tiles_n, tm, tn);
         t.m0    = lo + static_cast<int64_t>(tm) * BM;
@@ -556,7 +591,7 @@ __device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile, const 
         t.sB    = a.sB + g * a.sb_gstride;
         t.C     = static_cast<uint8_t *>(a.C);
         if (a.group_offs_out != nullptr) // the tile's rows keep their A numbering; C moves instead
-            t.C += (a.group_offs_out[g] - lo) * a.N * (a.out_dtype == PT_DTYPE_F32 ? 4 : 2);
+            t.C += (out_lo - lo) * a.N * (a.out_dtype == PT_DTYPE_F32 ? 4 : 2);
         t.KT    = static_cast<int>(a.K / KSTEP);
     } else {
         // unit = (chunk of consecutive groups, output position); the positions in XCD-contiguous
@@ -570,7 +605,7 @@ __device__ __forceinline__ TileCtx make_tile(const GemmArgs &a, int tile, const 
         t.g1 = __builtin_amdgcn_readfirstlane(prefix[chunk + 1]);
         g    = t.g0;
         // K ranges are given in elements; two E2M1 codes share a byte
-        const int64_t lo = a.group_offs[t.g0] >> (F4 ? 1 : 0), hi = a.group_offs[t.g1] >> (F4 ? 1 : 0);
+        const int64_t lo = uniform_load(a.group_offs + t.g0) >> (F4 ? 1 : 0), hi = uniform_load(a.group_offs + t.g1) >> (F4 ? 1 : 0);
         t.m0    = static_cast<int64_t>(tm) * BM;
         t.m_end = a.M;
         t.Ag    = a.A + t.m0 * a.lda + lo;
@@ -1146,9 +1181,9 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                 a, acc, cur_t.C, cur_t.sA, cur_t.sB, cur_t.m_end, wm_base, wn_base, lane));
         } else {
             const int ES     = a.out_dtype == PT_DTYPE_F32 ? 4 : 2;
-            int64_t   g_lo   = a.group_offs[cur_t.g0] >> (F4 ? 1 : 0);
+            int64_t   g_lo   = uniform_load(a.group_offs + cur_t.g0) >> (F4 ? 1 : 0);
             for (int g = cur_t.g0; g < cur_t.g1; ++g) {
-                const int64_t g_hi = a.group_offs[g + 1] >> (F4 ? 1 : 0);
+                const int64_t g_hi = uniform_load(a.group_offs + g + 1) >> (F4 ? 1 : 0);
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -1171,6 +1206,8 @@ __global__ __launch_bounds__(256) void gemm_fp8_nt_kernel(const GemmArgs a) {
                     asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
                 PT_GEMM_TRACE_POINT(5);
                 uint8_t *Cg = cur_t.C + static_cast<int64_t>(g) * a.c_gstride * ES;
+                // (the stores of a group's result are waited for at the next barrier here: leaving them in
+                // flight, as the row-group mode does, measured no faster in this mode)
                 epilogue<TM, TN, MODE, MODE != SCALE_BLOCK>(a, acc, Cg, cur_t.sA, cur_t.sB, cur_t.m_end, wm_base, wn_base, lane);
             }
             if (cur_t.g0 >= cur_t.g1 && next_tile < total && nxt_t.KT > 0)
