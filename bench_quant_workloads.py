@@ -85,6 +85,7 @@ class HbmStream(_QuantBase):
         self.x = self.x_cpu.to(dev)
         self.q = torch.empty((M, N), dtype=torch.float8_e4m3fn, device=dev)
         self.y = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+        self.big = torch.empty((4 * M, N), dtype=torch.bfloat16, device=dev)
 
     def dominant_work(self):
         return 3.0 * self.M * self.N
@@ -105,6 +106,10 @@ class HbmStream(_QuantBase):
         self.y.zero_()
         return self.y
 
+    def _fill_big(self):
+        self.big.zero_()
+        return self.big
+
     def _read(self):
         return self.x.view(torch.int32).amax()
 
@@ -113,8 +118,10 @@ class HbmStream(_QuantBase):
         # the memory system give on their own (a quantizer that emits two outputs, a gather that
         # writes eight rows per row read, are write-heavy)
         n = float(self.M * self.N)
+        # (the 235 MB fill fits the 256 MB Infinity Cache, which absorbs repeated writes of the same
+        # lines; the fill of four times that size has to reach HBM)
         return [("copy_bf16_to_bf16", self._copy, 4.0 * n), ("fill_write_only", self._fill, 2.0 * n),
-                ("amax_read_only", self._read, 2.0 * n)]
+                ("fill_write_only_940MB", self._fill_big, 8.0 * n), ("amax_read_only", self._read, 2.0 * n)]
 
     def check(self):
         ok = torch.equal(self._copy(), self.x) and torch.equal(self.dominant().float(), self.x.to(torch.float8_e4m3fn).float())
