@@ -7,8 +7,8 @@ compiler's own wait-count bookkeeping does not see those; if it believes that a 
 the epilogue may still be outstanding when the K loop of the next tile begins (a load and its use
 in two separately guarded blocks are enough), it puts an ``s_waitcnt vmcnt(0)`` in front of the
 first instruction of the loop that overwrites the load's register -- and every slab then begins by
-waiting for all copies in flight (dense MXFP8 16384^3: 3.2 -> 3.7 ms). The test compiles one
-translation unit to assembly (no GPU needed) and looks at every MFMA loop."""
+waiting for all copies in flight (dense MXFP8 16384^3: 3.2 -> 3.7 ms). The test compiles two
+translation units to assembly (no GPU needed) and looks at the MFMA loops of their kernels."""
 
 import re
 import subprocess
@@ -64,24 +64,49 @@ def test_scanner_sees_a_compiler_wait():
     assert _compiler_vmcnt_waits(body[s:e]) == ["s_waitcnt vmcnt(0)"]
 
 
-def test_mx_gemm_loops_have_no_compiler_inserted_vmcnt_wait(tmp_path):
+# translation unit -> which of its kernels are looked at: the dense MX kernels (gemm_mx8_kernel and
+# gemm_fp8_nt_kernel<TM, TN, 2 = MX, ...>) and the block-scaled eight-wavefront kernel of the
+# headline workload (the four-wavefront block kernels of that unit load their scales into
+# registers inside the loop and wait for them legitimately)
+UNITS = {
+    "gemm_mx.hip": (lambda n: "gemm_mx8_kernel" in n or re.search(r"gemm_fp8_nt_kernelILi\dELi\dELi2E", n), 8),
+    "gemm_fp8_block.hip": (lambda n: "gemm_fp8_block8_kernel" in n, 4),
+}
+
+
+@pytest.fixture(scope="module")
+def assembly(tmp_path_factory):
+    """Device assembly of the units, compiled side by side (about two minutes of hipcc)."""
+    from concurrent.futures import ThreadPoolExecutor
+
     import build_native
 
     try:
         hipcc = build_native.hipcc_path()
     except RuntimeError:
         pytest.skip("hipcc not found")
-    src = build_native.CSRC / "gemm_mx.hip"
-    asm = tmp_path / "gemm_mx.s"
+    out = tmp_path_factory.mktemp("asm")
     flags = [f for f in build_native.HIPCC_FLAGS if f != "-fPIC"]
-    cmd = [hipcc, *flags, *build_native._extra_flags(src), "-S", "--cuda-device-only", "-o", str(asm), str(src)]
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    assert res.returncode == 0, res.stderr[-2000:]
-    lines = asm.read_text().split("\n")
+
+    def one(unit):
+        src = build_native.CSRC / unit
+        asm = out / (src.stem + ".s")
+        cmd = [hipcc, *flags, *build_native._extra_flags(src), "-S", "--cuda-device-only", "-o", str(asm), str(src)]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        assert res.returncode == 0, res.stderr[-2000:]
+        return unit, asm.read_text().split("\n")
+
+    with ThreadPoolExecutor(max_workers=len(UNITS)) as ex:
+        return dict(ex.map(one, UNITS))
+
+
+@pytest.mark.parametrize("unit", sorted(UNITS))
+def test_mfma_loops_have_no_compiler_inserted_vmcnt_wait(assembly, unit):
+    lines = assembly[unit]
+    wanted, least = UNITS[unit]
     seen, bad = 0, []
     for name, a, b in _functions(lines):
-        # the dense MX kernels: gemm_mx8_kernel<FA, FB, 0> and gemm_fp8_nt_kernel<TM, TN, 2 (MX), ...>
-        if not ("gemm_mx8_kernel" in name or re.search(r"gemm_fp8_nt_kernelILi\dELi\dELi2E", name)):
+        if not wanted(name):
             continue
         body = lines[a:b]
         for s, e in _innermost_mfma_loops(body):
@@ -89,5 +114,5 @@ def test_mx_gemm_loops_have_no_compiler_inserted_vmcnt_wait(tmp_path):
             waits = _compiler_vmcnt_waits(body[s:e])
             if waits:
                 bad.append((name, waits))
-    assert seen >= 8, f"only {seen} MFMA loops found: the scanner no longer matches the compiler's output"
+    assert seen >= least, f"only {seen} MFMA loops found: the scanner no longer matches the compiler's output"
     assert not bad, bad
