@@ -460,6 +460,16 @@ __device__ __forceinline__ int epilogue(const GemmArgs &a, const f32x4 (&acc)[TM
                 const int64_t n = n0 + j * 16 + e;
                 sb[j][e]        = sBm[(n < a.N ? n : a.N - 1) * a.sb_n];
             }
+        // The scales are used inside the row tests below. On a path that skipped every one of those
+        // blocks the loads would still count as outstanding in the compiler's wait-count bookkeeping
+        // when the K loop of the next tile begins, and it would open every slab with a full
+        // vmcnt(0) wait: an (empty) use of each value here makes the loads complete on every path.
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+            asm volatile("" ::"v"(sa[i]));
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            asm volatile("" ::"v"(sb[j]));
     }
     // all columns of the sub-tile inside the matrix and every 16-byte group aligned: 16-byte stores,
     // with the row groups beyond the end of the matrix (the end of a group's rows) left out

@@ -7,7 +7,7 @@ compiler's own wait-count bookkeeping does not see those; if it believes that a 
 the epilogue may still be outstanding when the K loop of the next tile begins (a load and its use
 in two separately guarded blocks are enough), it puts an ``s_waitcnt vmcnt(0)`` in front of the
 first instruction of the loop that overwrites the load's register -- and every slab then begins by
-waiting for all copies in flight (dense MXFP8 16384^3: 3.2 -> 3.7 ms). The test compiles two
+waiting for all copies in flight (dense MXFP8 16384^3: 3.2 -> 3.7 ms). The test compiles three
 translation units to assembly (no GPU needed) and looks at the MFMA loops of their kernels."""
 
 import re
@@ -65,12 +65,14 @@ def test_scanner_sees_a_compiler_wait():
 
 
 # translation unit -> which of its kernels are looked at: the dense MX kernels (gemm_mx8_kernel and
-# gemm_fp8_nt_kernel<TM, TN, 2 = MX, ...>) and the block-scaled eight-wavefront kernel of the
+# gemm_fp8_nt_kernel<TM, TN, 2 = MX, ...>), the block-scaled eight-wavefront kernel of the
 # headline workload (the four-wavefront block kernels of that unit load their scales into
-# registers inside the loop and wait for them legitimately)
+# registers inside the loop and wait for them legitimately) and the grouped vector-scale kernels
 UNITS = {
     "gemm_mx.hip": (lambda n: "gemm_mx8_kernel" in n or re.search(r"gemm_fp8_nt_kernelILi\dELi\dELi2E", n), 8),
     "gemm_fp8_block.hip": (lambda n: "gemm_fp8_block8_kernel" in n, 4),
+    # vector scales (tensorwise / rowwise), row groups and variable K: the epilogue loads its scales
+    "gemm_fp8_grouped_vec.hip": (lambda n: re.search(r"gemm_fp8_nt_kernelILi\dELi\dELi0E", n), 8),
 }
 
 
